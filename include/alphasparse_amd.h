@@ -1,0 +1,192 @@
+/*
+ * C-ABI of the MI355X (gfx950) CSR SpMV / SpMM path.
+ *
+ * Plain pointers and sizes only.  Every `d_*` pointer is device memory owned by the
+ * caller; `stream` is a hipStream_t passed as void* (NULL = the default stream).  All
+ * entry points return an alphasparseStatus_t value (0 = success) and launch
+ * asynchronously on `stream` unless stated otherwise.  Indices are int32, zero based.
+ *
+ * The C++ entry points of the generic API (alphasparseSpMV, alphasparseSpMM and
+ * friends, declared in alphasparse.h next to this file) are thin host wrappers over
+ * the functions below and live in the same shared library.
+ *
+ * Each declaration cites the reference interface it stands in for
+ * (paths relative to the AlphaSparse source tree).
+ */
+#ifndef ALPHASPARSE_AMD_H
+#define ALPHASPARSE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* status codes: include/alphasparse/spdef.h:10-22 */
+enum {
+    ASX_STATUS_SUCCESS = 0,
+    ASX_STATUS_NOT_INITIALIZED = 1,
+    ASX_STATUS_ALLOC_FAILED = 2,
+    ASX_STATUS_INVALID_VALUE = 3,
+    ASX_STATUS_EXECUTION_FAILED = 4,
+    ASX_STATUS_INTERNAL_ERROR = 5,
+    ASX_STATUS_NOT_SUPPORTED = 6,
+    ASX_STATUS_INVALID_POINTER = 7,
+    ASX_STATUS_INVALID_HANDLE = 8,
+    ASX_STATUS_INVALID_KERNEL_PARAM = 9,
+    ASX_STATUS_INVALID_SIZE = 10
+};
+
+/* value types: include/alphasparse/spdef.h:144-155 (ALPHA_R_32F = 0, ALPHA_R_64F = 1) */
+enum { ASX_R_32F = 0, ASX_R_64F = 1 };
+
+/* SpMV kernels.  Numeric values of the first group are alphasparseSpMVAlg_t values
+ * (include/alphasparse/spdef.h:345-365); how each reference algorithm id maps onto these
+ * kernels is decided by asx_spmv_resolve_alg. */
+enum {
+    ASX_SPMV_DEFAULT = 0, /* pick from the row-length histogram (plan) or from m, nnz */
+    ASX_SPMV_VECTOR = 6,  /* wave64 sub-groups, one group per row */
+    ASX_SPMV_STREAM = 3,  /* LDS-staged row blocks, segmented reduction */
+    ASX_SPMV_MERGE = 9    /* merge-path tiles + ordered carry fix-up */
+};
+
+/* SpMM kernels (alphasparseSpMMAlg_t values, include/alphasparse/spdef.h:390-402) */
+enum {
+    ASX_SPMM_DEFAULT = 0,
+    ASX_SPMM_ROW = 5,    /* CSR_ALG1: one wave per (row, 64-column tile) */
+    ASX_SPMM_MERGE = 7,  /* CSR_ALG3: merge-path segments per wave + ordered carry fix-up */
+    ASX_SPMM_BLOCKED = 10 /* CSR_ALG6: 16x4-blocked MFMA variant (needs a plan) */
+};
+
+/* ------------------------------------------------------------------------------------
+ * Library / device
+ * ---------------------------------------------------------------------------------- */
+
+/* Version string "major.minor". */
+const char *asx_version(void);
+/* Number of compute units and wavefront size of the current device (host query).
+ * Stands in for the device query in alphasparseGetHandle, hip/util/handle.hip:67-83. */
+int asx_device_info(int *compute_units, int *wavefront_size);
+
+/* ------------------------------------------------------------------------------------
+ * CSR analysis: integer outputs, bit-identical to the reference functions cited.
+ * ---------------------------------------------------------------------------------- */
+
+/* Row-length histogram.  d_hist[b], b in [0,32]: b = 0 counts empty rows, b >= 1 counts rows
+ * with 2^(b-1) <= len < 2^b.  d_stats[0] = max row length, [1] = rows with len < 2,
+ * [2] = rows with 2 <= len < 1024, [3] = rows with len >= 1024 (the three bins of find_rows,
+ * hip/kernel/level2/alphasparse_spmv_csr_adaptive2.h:5-47).  d_hist: 33 x int64,
+ * d_stats: 4 x int64; both are overwritten. */
+int asx_row_length_histogram(const int32_t *d_row_ptr, int32_t m, int64_t *d_hist, int64_t *d_stats,
+                             void *stream);
+
+/* balanced_partition_row_by_nnz, hygon/util/partition.cpp:83-96 (device twins:
+ * dcu/kernel/level2/csrmv/dcu_gemv_row_partition.h:10-40).  d_partition: nparts+1 int32. */
+int asx_partition_rows_by_nnz(const int32_t *d_row_ptr, int32_t m, int32_t nparts, int32_t *d_partition,
+                              void *stream);
+
+/* Row holding stored element t*items, t in [0, ceil(nnz/items)); out[ceil(nnz/items)] = m.
+ * elebalance_partition_kernel, hip/kernel/level3/alphasparse_spmm_csr_nnz_split.h:7-47;
+ * adaptive_partition_kernel, hip/kernel/level3/alphasparse_spmm_csr_adaptive.h:7-43;
+ * flat_partition_kernel, hip/kernel/level3/alphasparse_spmm_csr_flat.h:6-25;
+ * balanced_partition_row_by_nnz_flat (items = 1024),
+ * hip/kernel/level2/alphasparse_spmv_csr_flat.h:7-38. */
+int asx_nnz_split_rows(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t items, int32_t *d_out,
+                       void *stream);
+
+/* Merge-path split points on diagonals g*items, g in [0, ceil((m+nnz)/items)]:
+ * d_xs[g] rows consumed, d_ys[g] stored elements consumed.
+ * abstract_merge_path_search, hip/kernel/level2/alphasparse_spmv_csr_merge_ginkgo.h:10-33,132-157
+ * (items = 4096); merge_path_search_kernel,
+ * hip/kernel/level3/alphasparse_spmm_csr_merge.h:6-30,32-75. */
+int asx_merge_path_search(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t items, int32_t *d_xs,
+                          int32_t *d_ys, void *stream);
+
+/* clac_size, hip/kernel/level2/alphasparse_spmv_csr_row_partition_ginkgo.h:93-122 (host). */
+int64_t asx_loadbalance_nwarps(int64_t nnz, int64_t warp_size, int64_t nwarps_base);
+/* balanced_partition_row_by_nnz<T,warp_size>,
+ * hip/kernel/level2/alphasparse_spmv_csr_row_partition_ginkgo.h:15-42 as launched at :419-424.
+ * d_out: nwarps int32. */
+int asx_loadbalance_partition(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t warp_size,
+                              int32_t nwarps, int32_t *d_out, void *stream);
+
+/* ComputeRowBlocks, hip/kernel/level2/alphasparse_spmv_csr_adaptive.h:354-568.  HOST routine on a
+ * HOST row_ptr, as in the reference.  Writes up to cap packed entries, returns through *count the
+ * number of entries the full result has (call with cap = 0 to size the array). */
+int asx_csr_adaptive_row_blocks(const int32_t *h_row_ptr, int32_t m, uint64_t *h_out, size_t cap,
+                                size_t *count);
+
+/* ------------------------------------------------------------------------------------
+ * Plans: analysis results kept across calls (the reference recomputes them inside every
+ * SpMV/SpMM call; its alphasparseSpMV_analysis is a stub, hip/kernel/level2/alphasparse_spmv.hip:
+ * 229-247, and _alphasparse_csrmv_info, include/alphasparse/handle.h:147-198, is never filled).
+ * A plan owns device memory (allocated at creation, freed at destruction) and is bound to the
+ * row_ptr contents it was built from.
+ * ---------------------------------------------------------------------------------- */
+typedef struct asx_plan asx_plan;
+
+/* Builds a plan for SpMV (ncols_dense = 1) or SpMM (ncols_dense = N > 1).  `alg` is one of
+ * the ASX_SPMV_* / ASX_SPMM_* values; DEFAULT reads the row-length histogram back (one small
+ * synchronous copy) and picks a kernel.  Synchronises `stream` before returning. */
+int asx_plan_create(asx_plan **plan, int is_spmm, int alg, int value_type, int32_t m, int32_t n,
+                    int32_t nnz, const int32_t *d_row_ptr, int32_t ncols_dense, void *stream);
+int asx_plan_destroy(asx_plan *plan);
+/* Kernel the plan resolved to, and bytes of per-call workspace its launches need. */
+int asx_plan_alg(const asx_plan *plan);
+size_t asx_plan_workspace_bytes(const asx_plan *plan);
+/* Copies the plan's histogram (33 bins) and stats (4) to host arrays. */
+int asx_plan_histogram(const asx_plan *plan, int64_t h_hist[33], int64_t h_stats[4]);
+
+/* ------------------------------------------------------------------------------------
+ * SpMV  y = alpha*A*x + beta*y      (alphasparseSpMV, include/alphasparse/spapi.h:6895-6905;
+ *                                    CPU twin alphasparse_?_mv, spapi.h:1000-1020)
+ * ---------------------------------------------------------------------------------- */
+
+/* Kernel an alphasparseSpMVAlg_t value runs as when no plan is given. */
+int asx_spmv_resolve_alg(int alg, int32_t m, int32_t nnz);
+/* Workspace bytes for a plan-less call (analysis metadata + carries).
+ * alphasparseSpMV_bufferSize, hip/kernel/level2/alphasparse_spmv.hip:258-338. */
+size_t asx_spmv_workspace_bytes(int alg, int value_type, int32_t m, int32_t nnz);
+
+/* With plan != NULL the kernel and its split points come from the plan and d_workspace only
+ * holds carries (asx_plan_workspace_bytes).  With plan == NULL the split points are computed
+ * into d_workspace by this call (asx_spmv_workspace_bytes), as the reference does on every
+ * call.  beta == 0 never reads y. */
+int asx_spmv_csr_f64(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, double alpha,
+                     const int32_t *d_row_ptr, const int32_t *d_col, const double *d_val,
+                     const double *d_x, double beta, double *d_y, void *d_workspace,
+                     size_t workspace_bytes, void *stream);
+int asx_spmv_csr_f32(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, float alpha,
+                     const int32_t *d_row_ptr, const int32_t *d_col, const float *d_val,
+                     const float *d_x, float beta, float *d_y, void *d_workspace,
+                     size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * SpMM  C = alpha*A*B + beta*C, B (k x ncols) and C (m x ncols) row-major
+ *       (alphasparseSpMM, include/alphasparse/spapi.h:6963-6974; CPU twin alphasparse_?_mm,
+ *        spapi.h:1272-1306)
+ * ---------------------------------------------------------------------------------- */
+int asx_spmm_resolve_alg(int alg, int32_t m, int32_t nnz, int32_t ncols);
+/* alphasparseSpMM_bufferSize, hip/kernel/level3/alphasparse_spmm.hip:699-850. */
+size_t asx_spmm_workspace_bytes(int alg, int value_type, int32_t m, int32_t nnz, int32_t ncols);
+
+int asx_spmm_csr_f32(const asx_plan *plan, int alg, int32_t m, int32_t k, int32_t nnz, int32_t ncols,
+                     float alpha, const int32_t *d_row_ptr, const int32_t *d_col, const float *d_val,
+                     const float *d_B, int64_t ldb, float beta, float *d_C, int64_t ldc,
+                     void *d_workspace, size_t workspace_bytes, void *stream);
+int asx_spmm_csr_f64(const asx_plan *plan, int alg, int32_t m, int32_t k, int32_t nnz, int32_t ncols,
+                     double alpha, const int32_t *d_row_ptr, const int32_t *d_col, const double *d_val,
+                     const double *d_B, int64_t ldb, double beta, double *d_C, int64_t ldc,
+                     void *d_workspace, size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * Measurement helpers (used by the benchmark; plain HIP underneath)
+ * ---------------------------------------------------------------------------------- */
+/* A coalesced copy kernel of `bytes` bytes (multiple of 16): calibration for bandwidth counters. */
+int asx_copy_bytes(const void *d_src, void *d_dst, size_t bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,236 @@
+"""ctypes view of the C-ABI in include/alphasparse_amd.h (used by tests and the benchmark).
+
+Device buffers are torch tensors; only their ``data_ptr()`` crosses into the library.  There
+is no fallback: if the shared library is missing, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libalphasparse_amd.so")
+
+R_32F, R_64F = 0, 1
+SPMV_DEFAULT, SPMV_STREAM, SPMV_VECTOR, SPMV_MERGE = 0, 3, 6, 9
+SPMM_DEFAULT, SPMM_ROW, SPMM_MERGE, SPMM_BLOCKED = 0, 5, 7, 10
+
+STATUS = {0: "SUCCESS", 1: "NOT_INITIALIZED", 2: "ALLOC_FAILED", 3: "INVALID_VALUE",
+          4: "EXECUTION_FAILED", 5: "INTERNAL_ERROR", 6: "NOT_SUPPORTED", 7: "INVALID_POINTER",
+          8: "INVALID_HANDLE", 9: "INVALID_KERNEL_PARAM", 10: "INVALID_SIZE"}
+
+# every symbol include/alphasparse_amd.h declares
+EXPORTS = [
+    "asx_version", "asx_device_info", "asx_row_length_histogram", "asx_partition_rows_by_nnz",
+    "asx_nnz_split_rows", "asx_merge_path_search", "asx_loadbalance_nwarps",
+    "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_plan_create",
+    "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
+    "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
+    "asx_spmm_resolve_alg", "asx_spmm_workspace_bytes", "asx_spmm_csr_f32", "asx_spmm_csr_f64",
+    "asx_copy_bytes",
+]
+
+
+class AsxError(RuntimeError):
+    def __init__(self, code, where):
+        super().__init__(f"{where}: status {code} ({STATUS.get(code, '?')})")
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f"{LIB_PATH} is not built (python -m library_amd.build); there is no fallback path")
+    L = C.CDLL(LIB_PATH)
+    vp, i32, i64, sz = C.c_void_p, C.c_int32, C.c_int64, C.c_size_t
+    L.asx_version.restype = C.c_char_p
+    L.asx_device_info.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_int)]
+    L.asx_row_length_histogram.argtypes = [vp, i32, vp, vp, vp]
+    L.asx_partition_rows_by_nnz.argtypes = [vp, i32, i32, vp, vp]
+    L.asx_nnz_split_rows.argtypes = [vp, i32, i32, i32, vp, vp]
+    L.asx_merge_path_search.argtypes = [vp, i32, i32, i32, vp, vp, vp]
+    L.asx_loadbalance_nwarps.argtypes = [i64, i64, i64]
+    L.asx_loadbalance_nwarps.restype = i64
+    L.asx_loadbalance_partition.argtypes = [vp, i32, i32, i32, i32, vp, vp]
+    L.asx_csr_adaptive_row_blocks.argtypes = [vp, i32, vp, sz, C.POINTER(sz)]
+    L.asx_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, C.c_int, i32, i32, i32, vp, i32, vp]
+    L.asx_plan_destroy.argtypes = [vp]
+    L.asx_plan_alg.argtypes = [vp]
+    L.asx_plan_workspace_bytes.argtypes = [vp]
+    L.asx_plan_workspace_bytes.restype = sz
+    L.asx_plan_histogram.argtypes = [vp, vp, vp]
+    L.asx_spmv_resolve_alg.argtypes = [C.c_int, i32, i32]
+    L.asx_spmv_workspace_bytes.argtypes = [C.c_int, C.c_int, i32, i32]
+    L.asx_spmv_workspace_bytes.restype = sz
+    L.asx_spmv_csr_f64.argtypes = [vp, C.c_int, i32, i32, i32, C.c_double, vp, vp, vp, vp, C.c_double, vp, vp, sz, vp]
+    L.asx_spmv_csr_f32.argtypes = [vp, C.c_int, i32, i32, i32, C.c_float, vp, vp, vp, vp, C.c_float, vp, vp, sz, vp]
+    L.asx_spmm_resolve_alg.argtypes = [C.c_int, i32, i32, i32]
+    L.asx_spmm_workspace_bytes.argtypes = [C.c_int, C.c_int, i32, i32, i32]
+    L.asx_spmm_workspace_bytes.restype = sz
+    L.asx_spmm_csr_f32.argtypes = [vp, C.c_int, i32, i32, i32, i32, C.c_float, vp, vp, vp, vp, i64, C.c_float, vp, i64, vp, sz, vp]
+    L.asx_spmm_csr_f64.argtypes = [vp, C.c_int, i32, i32, i32, i32, C.c_double, vp, vp, vp, vp, i64, C.c_double, vp, i64, vp, sz, vp]
+    L.asx_copy_bytes.argtypes = [vp, vp, sz, vp]
+    _lib = L
+    return L
+
+
+def _check(code, where):
+    if code != 0:
+        raise AsxError(code, where)
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def value_type(dtype):
+    import torch
+    return {torch.float32: R_32F, torch.float64: R_64F, np.dtype(np.float32): R_32F,
+            np.dtype(np.float64): R_64F}[dtype]
+
+
+# ------------------------------------------------------------------------------ analysis
+def row_length_histogram(row_ptr):
+    import torch
+    m = row_ptr.numel() - 1
+    hist = torch.empty(33, dtype=torch.int64, device=row_ptr.device)
+    stats = torch.empty(4, dtype=torch.int64, device=row_ptr.device)
+    _check(lib().asx_row_length_histogram(_ptr(row_ptr), m, _ptr(hist), _ptr(stats), _stream()), "asx_row_length_histogram")
+    return hist, stats
+
+
+def partition_rows_by_nnz(row_ptr, nparts):
+    import torch
+    m = row_ptr.numel() - 1
+    out = torch.empty(nparts + 1, dtype=torch.int32, device=row_ptr.device)
+    _check(lib().asx_partition_rows_by_nnz(_ptr(row_ptr), m, nparts, _ptr(out), _stream()), "asx_partition_rows_by_nnz")
+    return out
+
+
+def nnz_split_rows(row_ptr, nnz, items):
+    import torch
+    m = row_ptr.numel() - 1
+    nseg = (nnz + items - 1) // items
+    out = torch.empty(nseg + 1, dtype=torch.int32, device=row_ptr.device)
+    _check(lib().asx_nnz_split_rows(_ptr(row_ptr), m, nnz, items, _ptr(out), _stream()), "asx_nnz_split_rows")
+    return out
+
+
+def merge_path_search(row_ptr, nnz, items):
+    import torch
+    m = row_ptr.numel() - 1
+    nblk = (m + nnz + items - 1) // items
+    xs = torch.empty(nblk + 1, dtype=torch.int32, device=row_ptr.device)
+    ys = torch.empty(nblk + 1, dtype=torch.int32, device=row_ptr.device)
+    _check(lib().asx_merge_path_search(_ptr(row_ptr), m, nnz, items, _ptr(xs), _ptr(ys), _stream()), "asx_merge_path_search")
+    return xs, ys
+
+
+def loadbalance_nwarps(nnz, warp_size, nwarps_base):
+    return int(lib().asx_loadbalance_nwarps(nnz, warp_size, nwarps_base))
+
+
+def loadbalance_partition(row_ptr, nnz, warp_size, nwarps):
+    import torch
+    m = row_ptr.numel() - 1
+    out = torch.empty(max(nwarps, 1), dtype=torch.int32, device=row_ptr.device)
+    _check(lib().asx_loadbalance_partition(_ptr(row_ptr), m, nnz, warp_size, nwarps, _ptr(out), _stream()), "asx_loadbalance_partition")
+    return out[:nwarps]
+
+
+def csr_adaptive_row_blocks(row_ptr_host):
+    """Host routine on a host (numpy int32) row_ptr."""
+    rp = np.ascontiguousarray(row_ptr_host, dtype=np.int32)
+    m = rp.size - 1
+    n = C.c_size_t(0)
+    _check(lib().asx_csr_adaptive_row_blocks(rp.ctypes.data_as(C.c_void_p), m, None, 0, C.byref(n)), "asx_csr_adaptive_row_blocks")
+    out = np.zeros(n.value, dtype=np.uint64)
+    n2 = C.c_size_t(0)
+    _check(lib().asx_csr_adaptive_row_blocks(rp.ctypes.data_as(C.c_void_p), m, out.ctypes.data_as(C.c_void_p), out.size, C.byref(n2)), "asx_csr_adaptive_row_blocks")
+    assert n2.value == n.value
+    return out
+
+
+# ------------------------------------------------------------------------------ plans
+class Plan:
+    def __init__(self, is_spmm, alg, dtype, m, n, nnz, row_ptr, ncols=1):
+        h = C.c_void_p()
+        _check(lib().asx_plan_create(C.byref(h), int(is_spmm), alg, value_type(dtype), m, n, nnz, _ptr(row_ptr), ncols, _stream()), "asx_plan_create")
+        self.h = h
+        self._row_ptr = row_ptr  # keep alive
+
+    @property
+    def alg(self):
+        return lib().asx_plan_alg(self.h)
+
+    @property
+    def workspace_bytes(self):
+        return lib().asx_plan_workspace_bytes(self.h)
+
+    def histogram(self):
+        hist = np.zeros(33, dtype=np.int64)
+        stats = np.zeros(4, dtype=np.int64)
+        _check(lib().asx_plan_histogram(self.h, hist.ctypes.data_as(C.c_void_p), stats.ctypes.data_as(C.c_void_p)), "asx_plan_histogram")
+        return hist, stats
+
+    def destroy(self):
+        if self.h:
+            lib().asx_plan_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+def _workspace(nbytes, device):
+    import torch
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+# ------------------------------------------------------------------------------ SpMV / SpMM
+def spmv(row_ptr, col, val, x, y, alpha, beta, alg=SPMV_DEFAULT, plan=None, workspace=None, n=None):
+    """y <- alpha*A*x + beta*y in place (torch CUDA tensors).  Returns y."""
+    m = row_ptr.numel() - 1
+    n = x.numel() if n is None else n
+    nnz = col.numel()
+    vt = value_type(val.dtype)
+    need = plan.workspace_bytes if plan is not None else lib().asx_spmv_workspace_bytes(alg, vt, m, nnz)
+    if workspace is None:
+        workspace = _workspace(need, val.device)
+    fn = lib().asx_spmv_csr_f64 if vt == R_64F else lib().asx_spmv_csr_f32
+    _check(fn(plan.h if plan is not None else None, alg, m, n, nnz, alpha, _ptr(row_ptr), _ptr(col), _ptr(val),
+              _ptr(x), beta, _ptr(y), _ptr(workspace), workspace.numel(), _stream()), "asx_spmv_csr")
+    return y
+
+
+def spmm(row_ptr, col, val, B, Cm, ncols, alpha, beta, alg=SPMM_DEFAULT, plan=None, workspace=None,
+         ldb=None, ldc=None, k=None):
+    """C <- alpha*A*B + beta*C in place; B (k x ncols), C (m x ncols) row-major torch CUDA tensors."""
+    m = row_ptr.numel() - 1
+    nnz = col.numel()
+    ldb = ncols if ldb is None else ldb
+    ldc = ncols if ldc is None else ldc
+    k = B.numel() // ldb if k is None else k
+    vt = value_type(val.dtype)
+    need = plan.workspace_bytes if plan is not None else lib().asx_spmm_workspace_bytes(alg, vt, m, nnz, ncols)
+    if workspace is None:
+        workspace = _workspace(need, val.device)
+    fn = lib().asx_spmm_csr_f64 if vt == R_64F else lib().asx_spmm_csr_f32
+    _check(fn(plan.h if plan is not None else None, alg, m, k, nnz, ncols, alpha, _ptr(row_ptr), _ptr(col), _ptr(val),
+              _ptr(B), ldb, beta, _ptr(Cm), ldc, _ptr(workspace), workspace.numel(), _stream()), "asx_spmm_csr")
+    return Cm

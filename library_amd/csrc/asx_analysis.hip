@@ -1,0 +1,239 @@
+// CSR analysis kernels for gfx950: row-length histogram, row partitions, nnz-split rows,
+// merge-path split points.  All outputs are integers and are defined to be bit-identical to
+// the reference functions cited at each launcher (and in include/alphasparse_amd.h).
+// One thread per output element; every search is a binary search over row_ptr in global
+// memory (row_ptr is small next to the matrix and stays in L2 across the searches).
+#include "asx_internal.hpp"
+
+namespace asx {
+
+// -------------------------------------------------------------------------------------------
+// Row-length histogram: 33 log2 bins + max + the three find_rows bins
+// (hip/kernel/level2/alphasparse_spmv_csr_adaptive2.h:5-47: len < 2, len < 1024, else).
+// -------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_zero_i64(int64_t *p, int n)
+{
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+__global__ __launch_bounds__(256) void k_row_histogram(const int32_t *__restrict__ row_ptr, int32_t m,
+                                                       unsigned long long *hist /*33*/,
+                                                       unsigned long long *stats /*4*/)
+{
+    __shared__ unsigned int s_hist[33];
+    __shared__ unsigned int s_bins[3];
+    __shared__ int s_max;
+    if (threadIdx.x < 33) s_hist[threadIdx.x] = 0;
+    if (threadIdx.x < 3) s_bins[threadIdx.x] = 0;
+    if (threadIdx.x == 0) s_max = 0;
+    __syncthreads();
+    int local_max = 0;
+    for (int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; r < m;
+         r += (int64_t)gridDim.x * blockDim.x) {
+        int len = row_ptr[r + 1] - row_ptr[r];
+        int bin = len <= 0 ? 0 : 32 - __clz(len);
+        atomicAdd(&s_hist[bin], 1u);
+        atomicAdd(&s_bins[len < 2 ? 0 : (len < 1024 ? 1 : 2)], 1u);
+        local_max = len > local_max ? len : local_max;
+    }
+    atomicMax(&s_max, local_max);
+    __syncthreads();
+    if (threadIdx.x < 33 && s_hist[threadIdx.x])
+        atomicAdd(&hist[threadIdx.x], (unsigned long long)s_hist[threadIdx.x]);
+    if (threadIdx.x < 3 && s_bins[threadIdx.x])
+        atomicAdd(&stats[1 + threadIdx.x], (unsigned long long)s_bins[threadIdx.x]);
+    if (threadIdx.x == 0) atomicMax(&stats[0], (unsigned long long)s_max);
+}
+
+int launch_row_histogram(const int32_t *d_row_ptr, int32_t m, int64_t *d_hist, int64_t *d_stats,
+                         hipStream_t s)
+{
+    // counters are cleared with a kernel (not a memset node) so the call can sit in a graph
+    hipLaunchKernelGGL(k_zero_i64, dim3(1), dim3(256), 0, s, d_hist, 33);
+    hipLaunchKernelGGL(k_zero_i64, dim3(1), dim3(256), 0, s, d_stats, 4);
+    if (m > 0) {
+        int grid = (int)ceil_div64(m, 256 * 8);
+        if (grid > 4096) grid = 4096;
+        hipLaunchKernelGGL(k_row_histogram, dim3(grid), dim3(256), 0, s, d_row_ptr, m,
+                           (unsigned long long *)d_hist, (unsigned long long *)d_stats);
+    }
+    return check_launch();
+}
+
+// -------------------------------------------------------------------------------------------
+// hygon/util/partition.cpp:83-96: partition[i] = first p in [0, m-1) with row_end[p] >= ave*i,
+// or m-1 when there is none; ave = nnz / nparts in 32-bit integer arithmetic.
+// -------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_partition_rows_by_nnz(const int32_t *__restrict__ row_ptr,
+                                                               int32_t m, int32_t nparts,
+                                                               int32_t *__restrict__ out)
+{
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i > nparts) return;
+    if (i == 0) {
+        out[0] = 0;
+        return;
+    }
+    if (i == nparts) {
+        out[nparts] = m;
+        return;
+    }
+    const int32_t *row_end = row_ptr + 1;
+    int32_t nnz = row_end[m - 1];
+    int32_t ave = nnz / nparts;
+    int32_t target = (int32_t)((uint32_t)ave * (uint32_t)i);  // wraps as the 32-bit product does
+    int32_t lo = 0, hi = m - 1;
+    while (lo < hi) {
+        int32_t mid = (lo + hi) / 2;
+        if (row_end[mid] < target)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    out[i] = lo;
+}
+
+int launch_partition_rows_by_nnz(const int32_t *d_row_ptr, int32_t m, int32_t nparts, int32_t *d_out,
+                                 hipStream_t s)
+{
+    int grid = (int)ceil_div64((int64_t)nparts + 1, 256);
+    hipLaunchKernelGGL(k_partition_rows_by_nnz, dim3(grid), dim3(256), 0, s, d_row_ptr, m, nparts,
+                       d_out);
+    return check_launch();
+}
+
+// -------------------------------------------------------------------------------------------
+// Row holding stored element t*items (largest r with row_ptr[r] <= t*items); out[nseg] = m.
+// hip/kernel/level3/alphasparse_spmm_csr_nnz_split.h:7-47 reaches the same row through a
+// two-level search; hip/kernel/level2/alphasparse_spmv_csr_flat.h:7-38 through one.
+// -------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_nnz_split_rows(const int32_t *__restrict__ row_ptr, int32_t m,
+                                                        int32_t nseg, int32_t items,
+                                                        int32_t *__restrict__ out)
+{
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t > nseg) return;
+    if (t == nseg) {
+        out[nseg] = m;
+        return;
+    }
+    int64_t e = t * items;
+    int32_t lo = 0, hi = m;  // invariant row_ptr[lo] <= e
+    while (lo < hi) {
+        int32_t mid = lo + (hi - lo + 1) / 2;
+        if ((int64_t)row_ptr[mid] <= e)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    out[t] = lo;
+}
+
+int launch_nnz_split_rows(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t items,
+                          int32_t *d_out, hipStream_t s)
+{
+    int32_t nseg = (int32_t)ceil_div64(nnz, items);
+    int grid = (int)ceil_div64((int64_t)nseg + 1, 256);
+    hipLaunchKernelGGL(k_nnz_split_rows, dim3(grid), dim3(256), 0, s, d_row_ptr, m, nseg, items, d_out);
+    return check_launch();
+}
+
+// -------------------------------------------------------------------------------------------
+// Merge-path split points (hip/kernel/level2/alphasparse_spmv_csr_merge_ginkgo.h:10-33,132-157):
+// diagonal d = min(g*items, m+nnz); x = least p in [max(d-nnz,0), min(d,m)] with
+// row_end[p] >= d-p (else the window's upper end); y = d-x.
+// -------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_merge_path_search(const int32_t *__restrict__ row_ptr,
+                                                           int32_t m, int32_t nnz, int32_t items,
+                                                           int32_t nblk, int32_t *__restrict__ xs,
+                                                           int32_t *__restrict__ ys)
+{
+    int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g > nblk) return;
+    const int32_t *row_end = row_ptr + 1;
+    int64_t total = (int64_t)m + nnz;
+    int64_t d = g * items;
+    if (d > total) d = total;
+    int64_t lo = d - nnz > 0 ? d - nnz : 0;
+    int64_t hi = d < m ? d : m;
+    while (lo < hi) {
+        int64_t p = (lo + hi) / 2;
+        if ((int64_t)row_end[p] < d - p)
+            lo = p + 1;
+        else
+            hi = p;
+    }
+    xs[g] = (int32_t)lo;
+    ys[g] = (int32_t)(d - lo);
+}
+
+int launch_merge_path_search(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t items,
+                             int32_t *d_xs, int32_t *d_ys, hipStream_t s)
+{
+    int32_t nblk = (int32_t)ceil_div64((int64_t)m + nnz, items);
+    int grid = (int)ceil_div64((int64_t)nblk + 1, 256);
+    hipLaunchKernelGGL(k_merge_path_search, dim3(grid), dim3(256), 0, s, d_row_ptr, m, nnz, items, nblk,
+                       d_xs, d_ys);
+    return check_launch();
+}
+
+// -------------------------------------------------------------------------------------------
+// hip/kernel/level2/alphasparse_spmv_csr_row_partition_ginkgo.h:15-42 as launched at :419-424:
+// closed-range search over acc = row_ptr+1, indices [0, m-1]; the answer may be m.
+// -------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_loadbalance_partition(const int32_t *__restrict__ row_ptr,
+                                                               int32_t m, int64_t ave,
+                                                               int32_t warp_size, int32_t nwarps,
+                                                               int32_t *__restrict__ out)
+{
+    int g = blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= nwarps) return;
+    const int32_t *acc = row_ptr + 1;
+    int64_t target = ave * g;
+    int32_t l = 0, r = m - 1;
+    while (l <= r) {
+        int32_t mid = (l + r) / 2;
+        int64_t chunks = ((int64_t)acc[mid] + warp_size - 1) / warp_size;
+        if (chunks * nwarps < target)
+            l = mid + 1;
+        else
+            r = mid - 1;
+    }
+    out[g] = l;
+}
+
+int launch_loadbalance_partition(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t warp_size,
+                                 int32_t nwarps, int32_t *d_out, hipStream_t s)
+{
+    if (nwarps <= 0) return ASX_STATUS_SUCCESS;
+    int64_t ave = ceil_div64(nnz, warp_size);
+    int grid = (int)ceil_div64(nwarps, 256);
+    hipLaunchKernelGGL(k_loadbalance_partition, dim3(grid), dim3(256), 0, s, d_row_ptr, m, ave,
+                       warp_size, nwarps, d_out);
+    return check_launch();
+}
+
+// -------------------------------------------------------------------------------------------
+// Calibration copy: 16 bytes per lane per iteration, grid-stride.
+// -------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
+                                                size_t n16)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16;
+         i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
+int launch_copy_bytes(const void *d_src, void *d_dst, size_t bytes, hipStream_t s)
+{
+    size_t n16 = bytes / 16;
+    if (n16 == 0) return ASX_STATUS_SUCCESS;
+    size_t grid = (n16 + 255) / 256;
+    if (grid > 256 * 32) grid = 256 * 32;
+    hipLaunchKernelGGL(k_copy16, dim3((unsigned)grid), dim3(256), 0, s, (const uint4 *)d_src,
+                       (uint4 *)d_dst, n16);
+    return check_launch();
+}
+
+}  // namespace asx

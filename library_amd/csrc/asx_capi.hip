@@ -1,0 +1,480 @@
+// extern "C" entry points of libalphasparse_amd.so: argument checks, workspace layout, plans,
+// kernel selection.  No arithmetic lives here.  There is no CPU fallback: every compute entry
+// point launches HIP kernels or returns an error status.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <new>
+
+#include "asx_internal.hpp"
+
+using namespace asx;
+
+namespace {
+
+constexpr size_t kAlign = 256;
+
+size_t vsize(int value_type) { return value_type == ASX_R_64F ? 8 : 4; }
+
+struct MergeLayout {  // [xs | ys | carry] inside a workspace
+    size_t xs_off, ys_off, carry_off, bytes;
+};
+MergeLayout spmv_merge_layout(int32_t m, int32_t nnz, size_t sv, bool with_split)
+{
+    MergeLayout L{};
+    const size_t nt = (size_t)merge_tiles(m, nnz);
+    size_t off = 0;
+    if (with_split) {
+        L.xs_off = off;
+        off = align_up(off + (nt + 1) * 4, kAlign);
+        L.ys_off = off;
+        off = align_up(off + (nt + 1) * 4, kAlign);
+    }
+    L.carry_off = off;
+    off = align_up(off + std::max<size_t>(nt, 1) * sv, kAlign);
+    L.bytes = off;
+    return L;
+}
+
+struct SpmmLayout {  // [xs | ys | carry_row | carry]
+    size_t xs_off, ys_off, crow_off, carry_off, bytes;
+};
+SpmmLayout spmm_merge_layout(int32_t m, int32_t nnz, int32_t ncols, size_t sv, bool with_split)
+{
+    SpmmLayout L{};
+    const size_t ns = (size_t)spmm_segments(m, nnz);
+    size_t off = 0;
+    if (with_split) {
+        L.xs_off = off;
+        off = align_up(off + (ns + 1) * 4, kAlign);
+        L.ys_off = off;
+        off = align_up(off + (ns + 1) * 4, kAlign);
+    }
+    L.crow_off = off;
+    off = align_up(off + std::max<size_t>(ns, 1) * 4, kAlign);
+    L.carry_off = off;
+    off = align_up(off + std::max<size_t>(ns, 1) * (size_t)ncols * sv, kAlign);
+    L.bytes = off;
+    return L;
+}
+
+// Kernel choice from the row-length histogram: the stream kernel never lets a row leave its
+// workgroup, so one very long row would serialise on one workgroup; past a few windows the
+// merge-path kernel's even split wins.
+int choose_spmv_from_stats(const int64_t stats[4], int32_t m, int32_t nnz)
+{
+    const int64_t max_len = stats[0];
+    if (max_len > 4 * kStreamTile) return ASX_SPMV_MERGE;
+    (void)m;
+    (void)nnz;
+    return ASX_SPMV_STREAM;
+}
+
+template <typename T>
+int spmv_impl(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, T alpha,
+              const int32_t *row_ptr, const int32_t *col, const T *val, const T *x, T beta, T *y,
+              void *ws, size_t ws_bytes, hipStream_t s)
+{
+    if (m < 0 || n < 0 || nnz < 0) return ASX_STATUS_INVALID_SIZE;
+    if (m == 0) return ASX_STATUS_SUCCESS;
+    if (!row_ptr || !y || (nnz > 0 && (!col || !val || !x))) return ASX_STATUS_INVALID_POINTER;
+    const int vt = sizeof(T) == 8 ? ASX_R_64F : ASX_R_32F;
+    int kernel;
+    if (plan) {
+        if (plan->is_spmm || plan->m != m || plan->nnz != nnz || plan->value_type != vt)
+            return ASX_STATUS_INVALID_VALUE;
+        kernel = plan->alg;
+    } else {
+        kernel = asx_spmv_resolve_alg(alg, m, nnz);
+        if (kernel < 0) return ASX_STATUS_NOT_SUPPORTED;
+    }
+    char *w = (char *)ws;
+    switch (kernel) {
+    case ASX_SPMV_VECTOR:
+        return launch_spmv_vector<T>(m, nnz, alpha, row_ptr, col, val, x, beta, y, s);
+    case ASX_SPMV_STREAM: {
+        const int32_t *blocks;
+        if (plan) {
+            blocks = plan->d_meta;
+        } else {
+            const size_t need = asx_spmv_workspace_bytes(kernel, vt, m, nnz);
+            if (!ws) return ASX_STATUS_INVALID_POINTER;
+            if (ws_bytes < need) return ASX_STATUS_INVALID_SIZE;
+            int st = launch_stream_row_blocks(row_ptr, m, nnz, (int32_t *)w, s);
+            if (st) return st;
+            blocks = (const int32_t *)w;
+        }
+        return launch_spmv_stream<T>(m, nnz, alpha, row_ptr, col, val, x, beta, y, blocks, s);
+    }
+    case ASX_SPMV_MERGE: {
+        const MergeLayout L = spmv_merge_layout(m, nnz, sizeof(T), plan == nullptr);
+        if (!ws) return ASX_STATUS_INVALID_POINTER;
+        if (ws_bytes < L.bytes) return ASX_STATUS_INVALID_SIZE;
+        const int32_t *xs, *ys;
+        if (plan) {
+            const size_t nt = (size_t)merge_tiles(m, nnz);
+            xs = plan->d_meta;
+            ys = plan->d_meta + (nt + 1);
+        } else {
+            int st = launch_merge_path_search(row_ptr, m, nnz, kMergeTile, (int32_t *)(w + L.xs_off),
+                                              (int32_t *)(w + L.ys_off), s);
+            if (st) return st;
+            xs = (const int32_t *)(w + L.xs_off);
+            ys = (const int32_t *)(w + L.ys_off);
+        }
+        return launch_spmv_merge<T>(m, nnz, alpha, row_ptr, col, val, x, beta, y, xs, ys,
+                                    (T *)(w + L.carry_off), s);
+    }
+    default: return ASX_STATUS_NOT_SUPPORTED;
+    }
+}
+
+template <typename T>
+int spmm_impl(const asx_plan *plan, int alg, int32_t m, int32_t k, int32_t nnz, int32_t ncols, T alpha,
+              const int32_t *row_ptr, const int32_t *col, const T *val, const T *B, int64_t ldb, T beta,
+              T *C, int64_t ldc, void *ws, size_t ws_bytes, hipStream_t s)
+{
+    if (m < 0 || k < 0 || nnz < 0 || ncols < 0) return ASX_STATUS_INVALID_SIZE;
+    if (m == 0 || ncols == 0) return ASX_STATUS_SUCCESS;
+    if (ldb < ncols || ldc < ncols) return ASX_STATUS_INVALID_SIZE;
+    if (!row_ptr || !C || (nnz > 0 && (!col || !val || !B))) return ASX_STATUS_INVALID_POINTER;
+    const int vt = sizeof(T) == 8 ? ASX_R_64F : ASX_R_32F;
+    int kernel;
+    if (plan) {
+        if (!plan->is_spmm || plan->m != m || plan->nnz != nnz || plan->value_type != vt ||
+            plan->ncols != ncols)
+            return ASX_STATUS_INVALID_VALUE;
+        kernel = plan->alg;
+    } else {
+        kernel = asx_spmm_resolve_alg(alg, m, nnz, ncols);
+        if (kernel < 0) return ASX_STATUS_NOT_SUPPORTED;
+    }
+    char *w = (char *)ws;
+    switch (kernel) {
+    case ASX_SPMM_ROW:
+        return launch_spmm_row<T>(m, ncols, alpha, row_ptr, col, val, B, ldb, beta, C, ldc, s);
+    case ASX_SPMM_MERGE: {
+        const SpmmLayout L = spmm_merge_layout(m, nnz, ncols, sizeof(T), plan == nullptr);
+        if (!ws) return ASX_STATUS_INVALID_POINTER;
+        if (ws_bytes < L.bytes) return ASX_STATUS_INVALID_SIZE;
+        const int32_t *xs, *ys;
+        if (plan) {
+            const size_t ns = (size_t)spmm_segments(m, nnz);
+            xs = plan->d_meta;
+            ys = plan->d_meta + (ns + 1);
+        } else {
+            int st = launch_merge_path_search(row_ptr, m, nnz, kSpmmSegment, (int32_t *)(w + L.xs_off),
+                                              (int32_t *)(w + L.ys_off), s);
+            if (st) return st;
+            xs = (const int32_t *)(w + L.xs_off);
+            ys = (const int32_t *)(w + L.ys_off);
+        }
+        return launch_spmm_merge<T>(m, nnz, ncols, alpha, row_ptr, col, val, B, ldb, beta, C, ldc, xs,
+                                    ys, (T *)(w + L.carry_off), (int32_t *)(w + L.crow_off), s);
+    }
+    default: return ASX_STATUS_NOT_SUPPORTED;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *asx_version(void) { return "0.1"; }
+
+int asx_device_info(int *compute_units, int *wavefront_size)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return status_of(e);
+    int cu = 0, wf = 0;
+    e = hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return status_of(e);
+    e = hipDeviceGetAttribute(&wf, hipDeviceAttributeWarpSize, dev);
+    if (e != hipSuccess) return status_of(e);
+    if (compute_units) *compute_units = cu;
+    if (wavefront_size) *wavefront_size = wf;
+    return ASX_STATUS_SUCCESS;
+}
+
+// ---------------------------------------------------------------- analysis
+int asx_row_length_histogram(const int32_t *d_row_ptr, int32_t m, int64_t *d_hist, int64_t *d_stats,
+                             void *stream)
+{
+    if (m < 0) return ASX_STATUS_INVALID_SIZE;
+    if (!d_hist || !d_stats || (m > 0 && !d_row_ptr)) return ASX_STATUS_INVALID_POINTER;
+    return launch_row_histogram(d_row_ptr, m, d_hist, d_stats, (hipStream_t)stream);
+}
+
+int asx_partition_rows_by_nnz(const int32_t *d_row_ptr, int32_t m, int32_t nparts, int32_t *d_partition,
+                              void *stream)
+{
+    if (m < 1 || nparts < 1) return ASX_STATUS_INVALID_SIZE;
+    if (!d_row_ptr || !d_partition) return ASX_STATUS_INVALID_POINTER;
+    return launch_partition_rows_by_nnz(d_row_ptr, m, nparts, d_partition, (hipStream_t)stream);
+}
+
+int asx_nnz_split_rows(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t items, int32_t *d_out,
+                       void *stream)
+{
+    if (m < 0 || nnz < 0 || items < 1) return ASX_STATUS_INVALID_SIZE;
+    if (!d_row_ptr || !d_out) return ASX_STATUS_INVALID_POINTER;
+    return launch_nnz_split_rows(d_row_ptr, m, nnz, items, d_out, (hipStream_t)stream);
+}
+
+int asx_merge_path_search(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t items, int32_t *d_xs,
+                          int32_t *d_ys, void *stream)
+{
+    if (m < 0 || nnz < 0 || items < 1) return ASX_STATUS_INVALID_SIZE;
+    if (!d_row_ptr || !d_xs || !d_ys) return ASX_STATUS_INVALID_POINTER;
+    return launch_merge_path_search(d_row_ptr, m, nnz, items, d_xs, d_ys, (hipStream_t)stream);
+}
+
+int64_t asx_loadbalance_nwarps(int64_t nnz, int64_t warp_size, int64_t nwarps_base)
+{
+    if (warp_size <= 0) return 0;
+    int64_t mult = 8;
+    if (nnz >= (int64_t)2e8)
+        mult = 2048;
+    else if (nnz >= (int64_t)2e7)
+        mult = 512;
+    else if (nnz >= (int64_t)2e6)
+        mult = 128;
+    else if (nnz >= (int64_t)2e5)
+        mult = 32;
+    return std::min(ceil_div64(nnz, warp_size), nwarps_base * mult);
+}
+
+int asx_loadbalance_partition(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t warp_size,
+                              int32_t nwarps, int32_t *d_out, void *stream)
+{
+    if (m < 1 || nnz < 0 || warp_size < 1 || nwarps < 0) return ASX_STATUS_INVALID_SIZE;
+    if (!d_row_ptr || (nwarps > 0 && !d_out)) return ASX_STATUS_INVALID_POINTER;
+    return launch_loadbalance_partition(d_row_ptr, m, nnz, warp_size, nwarps, d_out,
+                                        (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------- plans
+int asx_plan_create(asx_plan **out, int is_spmm, int alg, int value_type, int32_t m, int32_t n,
+                    int32_t nnz, const int32_t *d_row_ptr, int32_t ncols_dense, void *stream)
+{
+    if (!out) return ASX_STATUS_INVALID_POINTER;
+    *out = nullptr;
+    if (m < 0 || n < 0 || nnz < 0 || ncols_dense < 1) return ASX_STATUS_INVALID_SIZE;
+    if (value_type != ASX_R_32F && value_type != ASX_R_64F) return ASX_STATUS_NOT_SUPPORTED;
+    if (m > 0 && !d_row_ptr) return ASX_STATUS_INVALID_POINTER;
+    hipStream_t s = (hipStream_t)stream;
+    asx_plan *p = new (std::nothrow) asx_plan();
+    if (!p) return ASX_STATUS_ALLOC_FAILED;
+    std::memset(p, 0, sizeof(*p));
+    p->is_spmm = is_spmm ? 1 : 0;
+    p->value_type = value_type;
+    p->m = m;
+    p->n = n;
+    p->nnz = nnz;
+    p->ncols = is_spmm ? ncols_dense : 1;
+    p->row_ptr = d_row_ptr;
+
+    // histogram (always: it is cheap and callers may ask for it)
+    int64_t *d_cnt = nullptr;
+    int st = status_of(hipMalloc((void **)&d_cnt, 37 * sizeof(int64_t)));
+    if (st) {
+        delete p;
+        return st;
+    }
+    st = launch_row_histogram(d_row_ptr, m, d_cnt, d_cnt + 33, s);
+    if (!st) st = status_of(hipMemcpyAsync(p->hist, d_cnt, 33 * sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    if (!st) st = status_of(hipMemcpyAsync(p->stats, d_cnt + 33, 4 * sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    if (!st) st = status_of(hipStreamSynchronize(s));
+    (void)hipFree(d_cnt);
+    if (st) {
+        delete p;
+        return st;
+    }
+
+    const size_t sv = vsize(value_type);
+    if (!is_spmm) {
+        int kernel = alg;
+        if (alg == ASX_SPMV_DEFAULT)
+            kernel = choose_spmv_from_stats(p->stats, m, nnz);
+        else
+            kernel = asx_spmv_resolve_alg(alg, m, nnz);
+        if (kernel < 0) {
+            delete p;
+            return ASX_STATUS_NOT_SUPPORTED;
+        }
+        p->alg = kernel;
+        if (kernel == ASX_SPMV_STREAM) {
+            int32_t nb = std::max(stream_blocks(nnz), 1);
+            p->nunits = nb;
+            p->meta_bytes = ((size_t)nb + 1) * 4;
+            st = status_of(hipMalloc((void **)&p->d_meta, p->meta_bytes));
+            if (!st) st = launch_stream_row_blocks(d_row_ptr, m, nnz, p->d_meta, s);
+            p->workspace_bytes = 0;
+        } else if (kernel == ASX_SPMV_MERGE) {
+            const size_t nt = (size_t)merge_tiles(m, nnz);
+            p->nunits = (int32_t)nt;
+            p->meta_bytes = 2 * (nt + 1) * 4;
+            st = status_of(hipMalloc((void **)&p->d_meta, p->meta_bytes));
+            if (!st)
+                st = launch_merge_path_search(d_row_ptr, m, nnz, kMergeTile, p->d_meta,
+                                              p->d_meta + (nt + 1), s);
+            p->workspace_bytes = spmv_merge_layout(m, nnz, sv, false).bytes;
+        } else {
+            p->workspace_bytes = 0;
+        }
+    } else {
+        int kernel = asx_spmm_resolve_alg(alg, m, nnz, ncols_dense);
+        if (kernel < 0) {
+            delete p;
+            return ASX_STATUS_NOT_SUPPORTED;
+        }
+        p->alg = kernel;
+        if (kernel == ASX_SPMM_MERGE) {
+            const size_t ns = (size_t)spmm_segments(m, nnz);
+            p->nunits = (int32_t)ns;
+            p->meta_bytes = 2 * (ns + 1) * 4;
+            st = status_of(hipMalloc((void **)&p->d_meta, p->meta_bytes));
+            if (!st)
+                st = launch_merge_path_search(d_row_ptr, m, nnz, kSpmmSegment, p->d_meta,
+                                              p->d_meta + (ns + 1), s);
+            p->workspace_bytes = spmm_merge_layout(m, nnz, ncols_dense, sv, false).bytes;
+        } else {
+            p->workspace_bytes = 0;
+        }
+    }
+    if (!st) st = status_of(hipStreamSynchronize(s));
+    if (st) {
+        if (p->d_meta) (void)hipFree(p->d_meta);
+        delete p;
+        return st;
+    }
+    *out = p;
+    return ASX_STATUS_SUCCESS;
+}
+
+int asx_plan_destroy(asx_plan *plan)
+{
+    if (!plan) return ASX_STATUS_SUCCESS;
+    int st = ASX_STATUS_SUCCESS;
+    if (plan->d_meta) st = status_of(hipFree(plan->d_meta));
+    delete plan;
+    return st;
+}
+
+int asx_plan_alg(const asx_plan *plan) { return plan ? plan->alg : -1; }
+size_t asx_plan_workspace_bytes(const asx_plan *plan) { return plan ? plan->workspace_bytes : 0; }
+int asx_plan_histogram(const asx_plan *plan, int64_t h_hist[33], int64_t h_stats[4])
+{
+    if (!plan || !h_hist || !h_stats) return ASX_STATUS_INVALID_POINTER;
+    std::memcpy(h_hist, plan->hist, sizeof(plan->hist));
+    std::memcpy(h_stats, plan->stats, sizeof(plan->stats));
+    return ASX_STATUS_SUCCESS;
+}
+
+// ---------------------------------------------------------------- SpMV
+// Reference algorithm ids (include/alphasparse/spdef.h:345-365) onto the three kernels here:
+// the reference's scalar/vector/line-enhance families are one-row-per-lane-group kernels, its
+// adaptive/stream/flat/acc families stage row blocks through LDS, its merge/row-partition/
+// load-balance families split work evenly whatever the row lengths.
+int asx_spmv_resolve_alg(int alg, int32_t m, int32_t nnz)
+{
+    (void)m;
+    (void)nnz;
+    switch (alg) {
+    case 0: return ASX_SPMV_MERGE;   /* DEFAULT without a histogram: the kernel with no bad case */
+    case 5:                          /* SCALAR */
+    case 6:                          /* VECTOR */
+    case 10:                         /* LINE */
+    case 16: return ASX_SPMV_VECTOR; /* LINE_ENHANCE */
+    case 2:                          /* CSR_ADAPTIVE */
+    case 3:                          /* CSR_STREAM */
+    case 8:                          /* ADAPTIVE */
+    case 11:
+    case 12:
+    case 13: /* FLAT1/4/8 */
+    case 14: /* ACC */
+    case 15: /* FLAT */
+    case 18: return ASX_SPMV_STREAM; /* PFLAT */
+    case 7:                          /* ROW_PARTITION */
+    case 9:                          /* MERGE */
+    case 17: return ASX_SPMV_MERGE;  /* LOAD_BALANCE */
+    default: return -1;              /* COO (1), ELL (4): other formats */
+    }
+}
+
+size_t asx_spmv_workspace_bytes(int alg, int value_type, int32_t m, int32_t nnz)
+{
+    const int kernel = asx_spmv_resolve_alg(alg, m, nnz);
+    if (kernel == ASX_SPMV_MERGE) return spmv_merge_layout(m, nnz, vsize(value_type), true).bytes;
+    if (kernel == ASX_SPMV_STREAM)
+        return align_up(((size_t)std::max(stream_blocks(nnz), 1) + 1) * 4, kAlign);
+    return 0;
+}
+
+int asx_spmv_csr_f64(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, double alpha,
+                     const int32_t *d_row_ptr, const int32_t *d_col, const double *d_val,
+                     const double *d_x, double beta, double *d_y, void *d_workspace,
+                     size_t workspace_bytes, void *stream)
+{
+    return spmv_impl<double>(plan, alg, m, n, nnz, alpha, d_row_ptr, d_col, d_val, d_x, beta, d_y,
+                             d_workspace, workspace_bytes, (hipStream_t)stream);
+}
+int asx_spmv_csr_f32(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, float alpha,
+                     const int32_t *d_row_ptr, const int32_t *d_col, const float *d_val,
+                     const float *d_x, float beta, float *d_y, void *d_workspace,
+                     size_t workspace_bytes, void *stream)
+{
+    return spmv_impl<float>(plan, alg, m, n, nnz, alpha, d_row_ptr, d_col, d_val, d_x, beta, d_y,
+                            d_workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------- SpMM
+int asx_spmm_resolve_alg(int alg, int32_t m, int32_t nnz, int32_t ncols)
+{
+    (void)m;
+    (void)nnz;
+    (void)ncols;
+    switch (alg) {
+    case 0: return ASX_SPMM_MERGE; /* DEFAULT */
+    case 5: return ASX_SPMM_ROW;   /* CSR_ALG1 row split */
+    case 6:                        /* CSR_ALG2 nnz split */
+    case 7:                        /* CSR_ALG3 merge */
+    case 8:                        /* CSR_ALG4 adaptive */
+    case 9: return ASX_SPMM_MERGE; /* CSR_ALG5 flat */
+    default: return -1;            /* COO algorithms; CSR_ALG6 needs a blocked plan */
+    }
+}
+
+size_t asx_spmm_workspace_bytes(int alg, int value_type, int32_t m, int32_t nnz, int32_t ncols)
+{
+    const int kernel = asx_spmm_resolve_alg(alg, m, nnz, ncols);
+    if (kernel == ASX_SPMM_MERGE) return spmm_merge_layout(m, nnz, ncols, vsize(value_type), true).bytes;
+    return 0;
+}
+
+int asx_spmm_csr_f32(const asx_plan *plan, int alg, int32_t m, int32_t k, int32_t nnz, int32_t ncols,
+                     float alpha, const int32_t *d_row_ptr, const int32_t *d_col, const float *d_val,
+                     const float *d_B, int64_t ldb, float beta, float *d_C, int64_t ldc,
+                     void *d_workspace, size_t workspace_bytes, void *stream)
+{
+    return spmm_impl<float>(plan, alg, m, k, nnz, ncols, alpha, d_row_ptr, d_col, d_val, d_B, ldb, beta,
+                            d_C, ldc, d_workspace, workspace_bytes, (hipStream_t)stream);
+}
+int asx_spmm_csr_f64(const asx_plan *plan, int alg, int32_t m, int32_t k, int32_t nnz, int32_t ncols,
+                     double alpha, const int32_t *d_row_ptr, const int32_t *d_col, const double *d_val,
+                     const double *d_B, int64_t ldb, double beta, double *d_C, int64_t ldc,
+                     void *d_workspace, size_t workspace_bytes, void *stream)
+{
+    return spmm_impl<double>(plan, alg, m, k, nnz, ncols, alpha, d_row_ptr, d_col, d_val, d_B, ldb,
+                             beta, d_C, ldc, d_workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int asx_copy_bytes(const void *d_src, void *d_dst, size_t bytes, void *stream)
+{
+    if (!d_src || !d_dst) return ASX_STATUS_INVALID_POINTER;
+    if (bytes % 16) return ASX_STATUS_INVALID_SIZE;
+    return launch_copy_bytes(d_src, d_dst, bytes, (hipStream_t)stream);
+}
+
+}  // extern "C"

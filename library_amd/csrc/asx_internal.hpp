@@ -1,0 +1,92 @@
+// Internal declarations shared by the HIP translation units of libalphasparse_amd.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/alphasparse_amd.h"
+#include "asx_device.hpp"
+
+namespace asx {
+
+// Tile geometry of the SpMV kernels (one workgroup of 256 threads per tile).
+constexpr int kBlock = 256;
+constexpr int kMergeItemsPerThread = 8;
+constexpr int kMergeTile = kBlock * kMergeItemsPerThread;  // rows + stored elements per tile
+constexpr int kStreamTile = 2048;                          // stored elements per row block
+// SpMM: merge items (rows + stored elements) per wave
+constexpr int kSpmmSegment = 128;
+
+inline int status_of(hipError_t e)
+{
+    switch (e) {
+    case hipSuccess: return ASX_STATUS_SUCCESS;
+    case hipErrorOutOfMemory: return ASX_STATUS_ALLOC_FAILED;
+    case hipErrorInvalidValue: return ASX_STATUS_INVALID_VALUE;
+    case hipErrorInvalidDevicePointer: return ASX_STATUS_INVALID_POINTER;
+    case hipErrorInvalidDevice:
+    case hipErrorInvalidResourceHandle: return ASX_STATUS_INVALID_HANDLE;
+    default: return ASX_STATUS_INTERNAL_ERROR;
+    }
+}
+inline int check_launch() { return status_of(hipGetLastError()); }
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// ---- analysis launchers (asx_analysis.hip) ----
+int launch_row_histogram(const int32_t *d_row_ptr, int32_t m, int64_t *d_hist, int64_t *d_stats,
+                         hipStream_t s);
+int launch_partition_rows_by_nnz(const int32_t *d_row_ptr, int32_t m, int32_t nparts, int32_t *d_out,
+                                 hipStream_t s);
+int launch_nnz_split_rows(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t items,
+                          int32_t *d_out, hipStream_t s);
+int launch_merge_path_search(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t items,
+                             int32_t *d_xs, int32_t *d_ys, hipStream_t s);
+int launch_loadbalance_partition(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t warp_size,
+                                 int32_t nwarps, int32_t *d_out, hipStream_t s);
+int launch_stream_row_blocks(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t *d_blocks,
+                             hipStream_t s);
+int launch_copy_bytes(const void *d_src, void *d_dst, size_t bytes, hipStream_t s);
+
+// ---- SpMV launchers (asx_spmv.hip) ----
+template <typename T>
+int launch_spmv_vector(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, const int32_t *col,
+                       const T *val, const T *x, T beta, T *y, hipStream_t s);
+template <typename T>
+int launch_spmv_merge(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, const int32_t *col,
+                      const T *val, const T *x, T beta, T *y, const int32_t *xs, const int32_t *ys,
+                      T *carry, hipStream_t s);
+template <typename T>
+int launch_spmv_stream(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, const int32_t *col,
+                       const T *val, const T *x, T beta, T *y, const int32_t *blocks, hipStream_t s);
+
+// ---- SpMM launchers (asx_spmm.hip) ----
+template <typename T>
+int launch_spmm_row(int32_t m, int32_t ncols, T alpha, const int32_t *row_ptr, const int32_t *col,
+                    const T *val, const T *B, int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t s);
+template <typename T>
+int launch_spmm_merge(int32_t m, int32_t nnz, int32_t ncols, T alpha, const int32_t *row_ptr,
+                      const int32_t *col, const T *val, const T *B, int64_t ldb, T beta, T *C,
+                      int64_t ldc, const int32_t *xs, const int32_t *ys, T *carry, int32_t *carry_row,
+                      hipStream_t s);
+
+inline int32_t merge_tiles(int32_t m, int32_t nnz) { return (int32_t)ceil_div64((int64_t)m + nnz, kMergeTile); }
+inline int32_t stream_blocks(int32_t nnz) { return (int32_t)ceil_div64(nnz, kStreamTile); }
+inline int32_t spmm_segments(int32_t m, int32_t nnz) { return (int32_t)ceil_div64((int64_t)m + nnz, kSpmmSegment); }
+
+}  // namespace asx
+
+// Plan: analysis results kept on the device across calls.
+struct asx_plan {
+    int is_spmm;
+    int alg;  // resolved kernel
+    int value_type;
+    int32_t m, n, nnz, ncols;
+    const int32_t *row_ptr;  // the device array the plan was built from (identity check only)
+    int32_t *d_meta;         // split points / row blocks (layout depends on alg)
+    size_t meta_bytes;
+    int32_t nunits;  // tiles / row blocks / segments
+    int64_t hist[33];
+    int64_t stats[4];
+    size_t workspace_bytes;
+};

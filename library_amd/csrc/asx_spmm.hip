@@ -1,0 +1,209 @@
+// CSR x dense SpMM for gfx950, C = alpha*A*B + beta*C with B (k x N) and C (m x N) row-major.
+//
+// Lanes of a wavefront are the 64 columns of a column tile, so every read of a row of B and
+// every access to a row of C is one fully coalesced 256-byte (fp32) / 512-byte (fp64) access.
+// The stored elements of A are read 64 at a time, one per lane, and broadcast lane by lane
+// through v_readlane, which also makes the row address of B wave-uniform (scalar base +
+// lane offset).
+//
+//   row   : one wave per (row, column tile).  Simple; long rows serialise.
+//   merge : one wave per kSpmmSegment consecutive items of the merge path over
+//           (row ends, stored elements): bounded work per wave whatever the row lengths.
+//           Rows that end inside a segment are written by that segment; the part of a row
+//           that runs past a segment end is kept as a carry row and added by an ordered
+//           pass afterwards.  No atomics (the reference's default SpMM,
+//           hip/kernel/level3/alphasparse_spmm_csr_nnz_split.h:283-409, scales C in a
+//           separate pass and joins segments with atomicAdd).
+#include "asx_internal.hpp"
+
+namespace asx {
+
+template <typename T>
+__device__ __forceinline__ T readlane_t(T v, int l);
+template <>
+__device__ __forceinline__ float readlane_t<float>(float v, int l)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
+}
+template <>
+__device__ __forceinline__ double readlane_t<double>(double v, int l)
+{
+    int lo = __builtin_amdgcn_readlane(__double2loint(v), l);
+    int hi = __builtin_amdgcn_readlane(__double2hiint(v), l);
+    return __hiloint2double(hi, lo);
+}
+
+// acc += sum over stored elements [k_begin, k_end) of one row: a * B[col, c]
+template <typename T>
+__device__ __forceinline__ T spmm_accumulate(T acc, int32_t k_begin, int32_t k_end, int lane, bool col_ok,
+                                             int64_t c, const int32_t *__restrict__ col,
+                                             const T *__restrict__ val, const T *__restrict__ B,
+                                             int64_t ldb)
+{
+    for (int32_t k0 = k_begin; k0 < k_end; k0 += kWave) {
+        const int32_t kk = k0 + lane;
+        const int32_t cl = kk < k_end ? col[kk] : 0;
+        const T vl = kk < k_end ? val[kk] : T(0);
+        const int cnt = k_end - k0 < kWave ? k_end - k0 : kWave;
+        int j = 0;
+        for (; j + 4 <= cnt; j += 4) {
+            const int32_t c0 = __builtin_amdgcn_readlane(cl, j);
+            const int32_t c1 = __builtin_amdgcn_readlane(cl, j + 1);
+            const int32_t c2 = __builtin_amdgcn_readlane(cl, j + 2);
+            const int32_t c3 = __builtin_amdgcn_readlane(cl, j + 3);
+            T b0 = T(0), b1 = T(0), b2 = T(0), b3 = T(0);
+            if (col_ok) {
+                b0 = B[(int64_t)c0 * ldb + c];
+                b1 = B[(int64_t)c1 * ldb + c];
+                b2 = B[(int64_t)c2 * ldb + c];
+                b3 = B[(int64_t)c3 * ldb + c];
+            }
+            acc = fma_t<T>(readlane_t<T>(vl, j), b0, acc);
+            acc = fma_t<T>(readlane_t<T>(vl, j + 1), b1, acc);
+            acc = fma_t<T>(readlane_t<T>(vl, j + 2), b2, acc);
+            acc = fma_t<T>(readlane_t<T>(vl, j + 3), b3, acc);
+        }
+        for (; j < cnt; ++j) {
+            const int32_t c0 = __builtin_amdgcn_readlane(cl, j);
+            T b0 = col_ok ? B[(int64_t)c0 * ldb + c] : T(0);
+            acc = fma_t<T>(readlane_t<T>(vl, j), b0, acc);
+        }
+    }
+    return acc;
+}
+
+template <typename T>
+__device__ __forceinline__ T scaled_out(T alpha, T acc, T beta, const T *C, int64_t idx)
+{
+    return beta == T(0) ? alpha * acc : fma_t<T>(alpha, acc, beta * C[idx]);
+}
+
+// ===========================================================================================
+// row: one wave per (row, column tile)
+// ===========================================================================================
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_spmm_row(int32_t m, int32_t ncols, T alpha,
+                                                     const int32_t *__restrict__ row_ptr,
+                                                     const int32_t *__restrict__ col,
+                                                     const T *__restrict__ val, const T *__restrict__ B,
+                                                     int64_t ldb, T beta, T *__restrict__ C,
+                                                     int64_t ldc)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    if (row >= m) return;  // wave-uniform
+    const int64_t c = (int64_t)blockIdx.y * kWave + lane;
+    const bool col_ok = c < ncols;
+    const int32_t s = __builtin_amdgcn_readfirstlane(row_ptr[row]);
+    const int32_t e = __builtin_amdgcn_readfirstlane(row_ptr[row + 1]);
+    T acc = spmm_accumulate<T>(T(0), s, e, lane, col_ok, c, col, val, B, ldb);
+    if (col_ok) C[row * ldc + c] = scaled_out<T>(alpha, acc, beta, C, row * ldc + c);
+}
+
+template <typename T>
+int launch_spmm_row(int32_t m, int32_t ncols, T alpha, const int32_t *row_ptr, const int32_t *col,
+                    const T *val, const T *B, int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t s)
+{
+    if (m <= 0 || ncols <= 0) return ASX_STATUS_SUCCESS;
+    dim3 grid((unsigned)ceil_div64(m, kBlock / kWave), (unsigned)ceil_div64(ncols, kWave));
+    hipLaunchKernelGGL((k_spmm_row<T>), grid, dim3(kBlock), 0, s, m, ncols, alpha, row_ptr, col, val, B,
+                       ldb, beta, C, ldc);
+    return check_launch();
+}
+
+// ===========================================================================================
+// merge: one wave per kSpmmSegment merge items
+// ===========================================================================================
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_spmm_merge(int32_t m, int32_t nnz, int32_t nseg,
+                                                       int32_t ncols, T alpha,
+                                                       const int32_t *__restrict__ row_ptr,
+                                                       const int32_t *__restrict__ col,
+                                                       const T *__restrict__ val,
+                                                       const T *__restrict__ B, int64_t ldb, T beta,
+                                                       T *__restrict__ C, int64_t ldc,
+                                                       const int32_t *__restrict__ xs,
+                                                       const int32_t *__restrict__ ys,
+                                                       T *__restrict__ carry,
+                                                       int32_t *__restrict__ carry_row)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t seg = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    if (seg >= nseg) return;  // wave-uniform
+    const int64_t c = (int64_t)blockIdx.y * kWave + lane;
+    const bool col_ok = c < ncols;
+    const int32_t x0 = __builtin_amdgcn_readfirstlane(xs[seg]);
+    const int32_t y0 = __builtin_amdgcn_readfirstlane(ys[seg]);
+    const int32_t x1 = __builtin_amdgcn_readfirstlane(xs[seg + 1]);
+    const int32_t y1 = __builtin_amdgcn_readfirstlane(ys[seg + 1]);
+
+    int32_t k = y0;
+    T acc = T(0);
+    for (int32_t row = x0; row < x1; ++row) {  // rows whose end lies inside this segment
+        const int32_t e = __builtin_amdgcn_readfirstlane(row_ptr[row + 1]);
+        acc = spmm_accumulate<T>(acc, k, e, lane, col_ok, c, col, val, B, ldb);
+        k = e;
+        if (col_ok) {
+            const int64_t idx = (int64_t)row * ldc + c;
+            C[idx] = scaled_out<T>(alpha, acc, beta, C, idx);
+        }
+        acc = T(0);
+    }
+    // row x1 continues past the segment end: keep what this segment saw of it
+    const bool has_tail = y1 > k;
+    if (has_tail) {
+        acc = spmm_accumulate<T>(T(0), k, y1, lane, col_ok, c, col, val, B, ldb);
+        if (col_ok) carry[seg * ncols + c] = acc;
+    }
+    if (lane == 0 && blockIdx.y == 0) carry_row[seg] = has_tail ? x1 : -1;
+}
+
+// One wave per segment that opens a run of segments ending inside the same row: sums the
+// run's carry rows in segment order and adds them to C.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_spmm_merge_fixup(int32_t m, int32_t nseg, int32_t ncols,
+                                                             T alpha, const T *__restrict__ carry,
+                                                             const int32_t *__restrict__ carry_row,
+                                                             T *__restrict__ C, int64_t ldc)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t seg = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    if (seg >= nseg) return;
+    const int32_t row = carry_row[seg];
+    if (row < 0 || row >= m) return;
+    if (seg > 0 && carry_row[seg - 1] == row) return;
+    const int64_t c = (int64_t)blockIdx.y * kWave + lane;
+    if (c >= ncols) return;
+    T sum = carry[seg * ncols + c];
+    for (int64_t j = seg + 1; j < nseg && carry_row[j] == row; ++j) sum += carry[j * ncols + c];
+    const int64_t idx = (int64_t)row * ldc + c;
+    C[idx] = fma_t<T>(alpha, sum, C[idx]);
+}
+
+template <typename T>
+int launch_spmm_merge(int32_t m, int32_t nnz, int32_t ncols, T alpha, const int32_t *row_ptr,
+                      const int32_t *col, const T *val, const T *B, int64_t ldb, T beta, T *C,
+                      int64_t ldc, const int32_t *xs, const int32_t *ys, T *carry, int32_t *carry_row,
+                      hipStream_t s)
+{
+    if (m <= 0 || ncols <= 0) return ASX_STATUS_SUCCESS;
+    const int32_t nseg = spmm_segments(m, nnz);
+    dim3 grid((unsigned)ceil_div64(nseg, kBlock / kWave), (unsigned)ceil_div64(ncols, kWave));
+    hipLaunchKernelGGL((k_spmm_merge<T>), grid, dim3(kBlock), 0, s, m, nnz, nseg, ncols, alpha, row_ptr,
+                       col, val, B, ldb, beta, C, ldc, xs, ys, carry, carry_row);
+    hipLaunchKernelGGL((k_spmm_merge_fixup<T>), grid, dim3(kBlock), 0, s, m, nseg, ncols, alpha, carry,
+                       carry_row, C, ldc);
+    return check_launch();
+}
+
+#define ASX_INST(T)                                                                                  \
+    template int launch_spmm_row<T>(int32_t, int32_t, T, const int32_t *, const int32_t *, const T *, \
+                                    const T *, int64_t, T, T *, int64_t, hipStream_t);               \
+    template int launch_spmm_merge<T>(int32_t, int32_t, int32_t, T, const int32_t *, const int32_t *, \
+                                      const T *, const T *, int64_t, T, T *, int64_t, const int32_t *, \
+                                      const int32_t *, T *, int32_t *, hipStream_t);
+ASX_INST(float)
+ASX_INST(double)
+#undef ASX_INST
+
+}  // namespace asx

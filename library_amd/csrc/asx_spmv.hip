@@ -1,0 +1,415 @@
+// CSR SpMV kernels for gfx950 (wave64), y = alpha*A*x + beta*y.
+//
+//   vector : aligned sub-groups of a wavefront (2..64 lanes) own one row each; DPP reduction.
+//   stream : a workgroup owns the rows that start inside a window of kStreamTile stored
+//            elements; products are staged through LDS once (coalesced), rows are reduced
+//            from LDS by 1..64 lanes each; the one row that may run past the window is
+//            finished by the whole workgroup.  No atomics, no inter-workgroup traffic.
+//   merge  : a workgroup owns kMergeTile consecutive items of the merge path over
+//            (row ends, stored elements); each thread walks exactly kMergeItemsPerThread
+//            items; partial rows are joined by a segmented scan inside the workgroup and by
+//            an ordered carry pass between workgroups.  No atomics: results do not depend on
+//            scheduling.
+//
+// The reference's kernels for the same job (hip/kernel/level2/alphasparse_spmv_csr_vector.h,
+// _flat.h, _merge_ginkgo.h, _adaptive.h) join partial rows with floating-point atomicAdd and
+// recompute their split points in every call; neither is done here.
+#include "asx_internal.hpp"
+
+namespace asx {
+
+// Workgroups are dealt to the 8 XCDs round-robin by the hardware.  Mapping workgroup id ->
+// tile so that each XCD walks one contiguous eighth of the tiles keeps the x entries shared
+// by neighbouring rows in that XCD's own L2.
+__device__ __forceinline__ int xcd_contiguous_tile(int bid, int ntiles)
+{
+    const int per = (ntiles + 7) >> 3;
+    return (bid & 7) * per + (bid >> 3);
+}
+inline int xcd_grid(int ntiles) { return ((ntiles + 7) >> 3) << 3; }
+
+template <typename T>
+__device__ __forceinline__ T axpby_out(T alpha, T sum, T beta, const T *y, int64_t r)
+{
+    return beta == T(0) ? alpha * sum : fma_t<T>(alpha, sum, beta * y[r]);
+}
+
+// ===========================================================================================
+// vector
+// ===========================================================================================
+template <typename T, int LANES>
+__global__ __launch_bounds__(kBlock) void k_spmv_vector(int32_t m, T alpha,
+                                                        const int32_t *__restrict__ row_ptr,
+                                                        const int32_t *__restrict__ col,
+                                                        const T *__restrict__ val,
+                                                        const T *__restrict__ x, T beta,
+                                                        T *__restrict__ y)
+{
+    const int lane = threadIdx.x & (LANES - 1);
+    const int64_t row = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / LANES;
+    T sum = T(0);
+    if (row < m) {
+        const int32_t e = row_ptr[row + 1];
+        int32_t k = row_ptr[row] + lane;
+        // two independent chains per lane keep more gathers in flight on long rows
+        T s0 = T(0), s1 = T(0);
+        for (; k + LANES < e; k += 2 * LANES) {
+            s0 = fma_t<T>(val[k], x[col[k]], s0);
+            s1 = fma_t<T>(val[k + LANES], x[col[k + LANES]], s1);
+        }
+        if (k < e) s0 = fma_t<T>(val[k], x[col[k]], s0);
+        sum = s0 + s1;
+    }
+    sum = group_sum<LANES>(sum);  // all lanes stay active for the cross-lane moves
+    if (row < m && lane == 0) y[row] = axpby_out<T>(alpha, sum, beta, y, row);
+}
+
+template <typename T>
+int launch_spmv_vector(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, const int32_t *col,
+                       const T *val, const T *x, T beta, T *y, hipStream_t s)
+{
+    if (m <= 0) return ASX_STATUS_SUCCESS;
+    const double mean = (double)nnz / (double)m;
+#define ASX_VEC(L)                                                                                   \
+    hipLaunchKernelGGL((k_spmv_vector<T, L>), dim3((unsigned)ceil_div64((int64_t)m * L, kBlock)),    \
+                       dim3(kBlock), 0, s, m, alpha, row_ptr, col, val, x, beta, y)
+    if (mean <= 2.0)
+        ASX_VEC(2);
+    else if (mean <= 4.0)
+        ASX_VEC(4);
+    else if (mean <= 8.0)
+        ASX_VEC(8);
+    else if (mean <= 16.0)
+        ASX_VEC(16);
+    else if (mean <= 32.0)
+        ASX_VEC(32);
+    else
+        ASX_VEC(64);
+#undef ASX_VEC
+    return check_launch();
+}
+
+// ===========================================================================================
+// stream
+// ===========================================================================================
+// LDS index with one pad slot per 32 entries: rows whose length is a multiple of 16 or 32
+// would otherwise put every lane of a wave on the same few banks.
+__device__ __forceinline__ int pad32(int j) { return j + (j >> 5); }
+constexpr int kStreamLds = kStreamTile + kStreamTile / 32 + 1;
+
+template <int G, typename T>
+__device__ __forceinline__ void stream_reduce_rows(const T *s_prod, int32_t r0, int32_t nrows,
+                                                   int32_t a, int32_t c1, int32_t last_row,
+                                                   T extra, T alpha, T beta,
+                                                   const int32_t *__restrict__ row_ptr,
+                                                   T *__restrict__ y)
+{
+    const int lane = threadIdx.x & (G - 1);
+    const int rows_per_pass = kBlock / G;
+    // every lane runs the same number of passes so the cross-lane moves see full waves
+    for (int base = 0; base < nrows; base += rows_per_pass) {
+        const int g = base + (int)threadIdx.x / G;
+        T sum = T(0);
+        int32_t r = r0 + g;
+        if (g < nrows) {
+            int32_t s = row_ptr[r] - a;
+            int32_t e = row_ptr[r + 1];
+            e = (e < c1 ? e : c1) - a;
+            for (int32_t j = s + lane; j < e; j += G) sum += s_prod[pad32(j)];
+        }
+        sum = group_sum<G>(sum);
+        if (g < nrows && lane == 0) {
+            if (r == last_row) sum += extra;
+            y[r] = axpby_out<T>(alpha, sum, beta, y, r);
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_spmv_stream(int32_t m, int32_t nblocks, T alpha,
+                                                        const int32_t *__restrict__ row_ptr,
+                                                        const int32_t *__restrict__ col,
+                                                        const T *__restrict__ val,
+                                                        const T *__restrict__ x, T beta,
+                                                        T *__restrict__ y,
+                                                        const int32_t *__restrict__ blocks)
+{
+    __shared__ T s_prod[kStreamLds];
+    __shared__ T s_part[kBlock / kWave];
+    const int t = xcd_contiguous_tile(blockIdx.x, nblocks);
+    if (t >= nblocks) return;
+    const int32_t r0 = blocks[t], r1 = blocks[t + 1];
+    const int32_t nrows = r1 - r0;
+    if (nrows <= 0) return;
+    const int32_t a = row_ptr[r0];
+    const int32_t bend = row_ptr[r1];
+    const int32_t c1 = bend - a > kStreamTile ? a + kStreamTile : bend;
+    const int32_t n1 = c1 - a;
+    const int tid = threadIdx.x;
+
+    // ---- stage the window's products (coalesced; all loads issued before first use) ----
+    constexpr int IPT = kStreamTile / kBlock;
+    int32_t cj[IPT];
+    T vj[IPT];
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+        const int j = tid + i * kBlock;
+        cj[i] = j < n1 ? col[(int64_t)a + j] : 0;
+        vj[i] = j < n1 ? val[(int64_t)a + j] : T(0);
+    }
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+        const int j = tid + i * kBlock;
+        if (j < n1) s_prod[pad32(j)] = vj[i] * x[cj[i]];
+    }
+
+    // ---- the last row may run past the window: finish it with the whole workgroup ----
+    T extra = T(0);
+    if (bend > c1) {  // uniform over the workgroup
+        T p0 = T(0), p1 = T(0);
+        int64_t k = (int64_t)c1 + tid;
+        for (; k + kBlock < bend; k += 2 * kBlock) {
+            p0 = fma_t<T>(val[k], x[col[k]], p0);
+            p1 = fma_t<T>(val[k + kBlock], x[col[k + kBlock]], p1);
+        }
+        if (k < bend) p0 = fma_t<T>(val[k], x[col[k]], p0);
+        T p = group_sum<kWave>(p0 + p1);
+        if ((tid & (kWave - 1)) == 0) s_part[tid / kWave] = p;
+    }
+    __syncthreads();
+    if (bend > c1) extra = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+
+    const int32_t last_row = r1 - 1;
+#define ASX_RED(G) stream_reduce_rows<G, T>(s_prod, r0, nrows, a, c1, last_row, extra, alpha, beta, row_ptr, y)
+    if (nrows > 128)
+        ASX_RED(1);
+    else if (nrows > 64)
+        ASX_RED(2);
+    else if (nrows > 32)
+        ASX_RED(4);
+    else if (nrows > 16)
+        ASX_RED(8);
+    else if (nrows > 8)
+        ASX_RED(16);
+    else if (nrows > 4)
+        ASX_RED(32);
+    else
+        ASX_RED(64);
+#undef ASX_RED
+}
+
+// Row blocks of the stream kernel: blocks[t] = first row whose first stored element lies at or
+// after t*kStreamTile (t < nb), blocks[nb] = m, nb = max(1, ceil(nnz / kStreamTile)).
+__global__ __launch_bounds__(kBlock) void k_stream_row_blocks(const int32_t *__restrict__ row_ptr,
+                                                              int32_t m, int32_t nb,
+                                                              int32_t *__restrict__ blocks)
+{
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t > nb) return;
+    if (t == nb) {
+        blocks[nb] = m;
+        return;
+    }
+    const int64_t target = t * kStreamTile;
+    int32_t lo = 0, hi = m;  // first r in [0,m] with row_ptr[r] >= target
+    while (lo < hi) {
+        int32_t mid = (lo + hi) / 2;
+        if ((int64_t)row_ptr[mid] < target)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    blocks[t] = lo;
+}
+
+int launch_stream_row_blocks(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t *d_blocks,
+                             hipStream_t s)
+{
+    int32_t nb = stream_blocks(nnz);
+    if (nb < 1) nb = 1;
+    hipLaunchKernelGGL(k_stream_row_blocks, dim3((unsigned)ceil_div64((int64_t)nb + 1, kBlock)),
+                       dim3(kBlock), 0, s, d_row_ptr, m, nb, d_blocks);
+    return check_launch();
+}
+
+template <typename T>
+int launch_spmv_stream(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, const int32_t *col,
+                       const T *val, const T *x, T beta, T *y, const int32_t *blocks, hipStream_t s)
+{
+    if (m <= 0) return ASX_STATUS_SUCCESS;
+    int32_t nb = stream_blocks(nnz);
+    if (nb < 1) nb = 1;
+    hipLaunchKernelGGL((k_spmv_stream<T>), dim3((unsigned)xcd_grid(nb)), dim3(kBlock), 0, s, m, nb,
+                       alpha, row_ptr, col, val, x, beta, y, blocks);
+    return check_launch();
+}
+
+// ===========================================================================================
+// merge path
+// ===========================================================================================
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_spmv_merge(int32_t m, int32_t nnz, int32_t ntiles, T alpha,
+                                                       const int32_t *__restrict__ row_ptr,
+                                                       const int32_t *__restrict__ col,
+                                                       const T *__restrict__ val,
+                                                       const T *__restrict__ x, T beta,
+                                                       T *__restrict__ y,
+                                                       const int32_t *__restrict__ xs,
+                                                       const int32_t *__restrict__ ys,
+                                                       T *__restrict__ carry)
+{
+    constexpr int IPT = kMergeItemsPerThread;
+    // s_val[0..nz) = products, s_val[nz..nz+nr) = finished row sums (nz + nr <= kMergeTile)
+    __shared__ T s_val[kMergeTile];
+    __shared__ int32_t s_rend[kMergeTile + 1];
+    __shared__ T s_wv[kBlock / kWave];
+    __shared__ int32_t s_wk[kBlock / kWave];
+
+    const int b = xcd_contiguous_tile(blockIdx.x, ntiles);
+    if (b >= ntiles) return;
+    const int tid = threadIdx.x;
+    const int32_t x0 = xs[b], y0 = ys[b], x1 = xs[b + 1], y1 = ys[b + 1];
+    const int32_t nr = x1 - x0, nz = y1 - y0, total = nr + nz;
+
+    // ---- stage: stored elements first (the long-latency part), then row ends ----
+    int32_t cj[IPT];
+    T vj[IPT];
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+        const int j = tid + i * kBlock;
+        cj[i] = j < nz ? col[(int64_t)y0 + j] : 0;
+        vj[i] = j < nz ? val[(int64_t)y0 + j] : T(0);
+    }
+    for (int i = tid; i <= nr; i += kBlock) {
+        const int32_t r = x0 + i;
+        s_rend[i] = (r < m ? row_ptr[r + 1] : nnz) - y0;
+    }
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+        const int j = tid + i * kBlock;
+        if (j < nz) s_val[j] = vj[i] * x[cj[i]];
+    }
+    __syncthreads();
+
+    // ---- this thread's start on the tile's merge path ----
+    int32_t diag = tid * IPT;
+    if (diag > total) diag = total;
+    int32_t lo = diag - nz > 0 ? diag - nz : 0;
+    int32_t hi = diag < nr ? diag : nr;
+    while (lo < hi) {
+        const int32_t p = (lo + hi) >> 1;
+        if (s_rend[p] < diag - p)
+            lo = p + 1;
+        else
+            hi = p;
+    }
+    int32_t row = lo, k = diag - lo;
+    const int32_t first_row = row;
+    int32_t cur_end = s_rend[row];
+    bool emitted = false;
+    T run = T(0);
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+        if (diag + i < total) {
+            if (k < cur_end) {
+                run += s_val[k];
+                ++k;
+            } else {
+                s_val[nz + row] = run;
+                emitted = true;
+                run = T(0);
+                ++row;
+                cur_end = s_rend[row];
+            }
+        }
+    }
+
+    // ---- join rows that span threads: segmented scan of (row in progress, partial) ----
+    const int lane = tid & (kWave - 1), w = tid / kWave;
+    const T incl = wave_segscan_incl<T>(row, run);
+    const int32_t k0 = __shfl(row, 0, kWave);
+    if (lane == kWave - 1) {
+        s_wk[w] = row;
+        s_wv[w] = incl;
+    }
+    __syncthreads();
+    int32_t pk = -1;
+    T pv = T(0);
+    for (int j = 0; j < w; ++j) {
+        const int32_t kj = s_wk[j];
+        const T vjj = s_wv[j];
+        if (kj == pk)
+            pv += vjj;
+        else {
+            pk = kj;
+            pv = vjj;
+        }
+    }
+    const int32_t up_k = __shfl_up(row, 1, kWave);
+    T carry_in = __shfl_up(incl, 1, kWave);
+    if (lane == 0) {
+        carry_in = (w > 0 && pk == first_row) ? pv : T(0);
+    } else {
+        if (up_k != first_row) carry_in = T(0);  // cannot happen on a consistent path; keeps it safe
+        if (up_k == k0 && pk == up_k) carry_in += pv;
+    }
+    if (emitted) s_val[nz + first_row] += carry_in;
+    if (tid == kBlock - 1) {
+        T out = incl;
+        if (row == k0 && pk == row) out += pv;
+        carry[b] = out;  // partial of row x1 gathered in this tile (0 when none of it is here)
+    }
+    __syncthreads();
+
+    // ---- finished rows, coalesced ----
+    for (int i = tid; i < nr; i += kBlock) {
+        const int64_t r = (int64_t)x0 + i;
+        y[r] = axpby_out<T>(alpha, s_val[nz + i], beta, y, r);
+    }
+}
+
+// Adds the carries to the rows that continue past a tile end, in tile order.  The thread of the
+// first tile of each run of tiles that end inside the same row sums the run sequentially.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_spmv_merge_fixup(int32_t m, int32_t ntiles, T alpha,
+                                                             const int32_t *__restrict__ xs,
+                                                             const T *__restrict__ carry,
+                                                             T *__restrict__ y)
+{
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= ntiles) return;
+    const int32_t row = xs[b + 1];
+    if (row >= m) return;
+    if (b > 0 && xs[b] == row) return;  // the previous tile ended inside the same row
+    T sum = carry[b];
+    for (int j = b + 1; j < ntiles && xs[j + 1] == row; ++j) sum += carry[j];
+    if (sum != T(0)) y[row] = fma_t<T>(alpha, sum, y[row]);
+}
+
+template <typename T>
+int launch_spmv_merge(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, const int32_t *col,
+                      const T *val, const T *x, T beta, T *y, const int32_t *xs, const int32_t *ys,
+                      T *carry, hipStream_t s)
+{
+    if (m <= 0) return ASX_STATUS_SUCCESS;
+    const int32_t ntiles = merge_tiles(m, nnz);
+    hipLaunchKernelGGL((k_spmv_merge<T>), dim3((unsigned)xcd_grid(ntiles)), dim3(kBlock), 0, s, m, nnz,
+                       ntiles, alpha, row_ptr, col, val, x, beta, y, xs, ys, carry);
+    hipLaunchKernelGGL((k_spmv_merge_fixup<T>), dim3((unsigned)ceil_div64(ntiles, kBlock)),
+                       dim3(kBlock), 0, s, m, ntiles, alpha, xs, carry, y);
+    return check_launch();
+}
+
+#define ASX_INST(T)                                                                                  \
+    template int launch_spmv_vector<T>(int32_t, int32_t, T, const int32_t *, const int32_t *,        \
+                                       const T *, const T *, T, T *, hipStream_t);                   \
+    template int launch_spmv_stream<T>(int32_t, int32_t, T, const int32_t *, const int32_t *,        \
+                                       const T *, const T *, T, T *, const int32_t *, hipStream_t);  \
+    template int launch_spmv_merge<T>(int32_t, int32_t, T, const int32_t *, const int32_t *,         \
+                                      const T *, const T *, T, T *, const int32_t *, const int32_t *, \
+                                      T *, hipStream_t);
+ASX_INST(float)
+ASX_INST(double)
+#undef ASX_INST
+
+}  // namespace asx

@@ -1,0 +1,228 @@
+// A caller written the way the reference's own GPU tests drive the generic API
+// (hip/test/level2/spmv_csr_r_f64_test.hip:143-217, hip/test/level3/spmm_csr_row_r_f32_test.hip):
+// get a handle, put the CSR arrays on the device, wrap them in descriptors, ask for the buffer
+// size, allocate it, call alphasparseSpMV / alphasparseSpMM, copy the result back.  It compiles
+// against include/alphasparse.h of this repository and links libalphasparse_amd.so only.
+//
+//   generic_api_caller <case_dir>     run the case described by <case_dir>/meta.txt, write out.bin
+//   generic_api_caller --selftest     error-path and life-cycle checks of the API on the device
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "alphasparse.h"
+
+#define HIP_OK(e)                                                                          \
+    do {                                                                                   \
+        hipError_t _e = (e);                                                               \
+        if (_e != hipSuccess) {                                                            \
+            std::fprintf(stderr, "HIP error %s at %s:%d\n", hipGetErrorString(_e), __FILE__, __LINE__); \
+            std::exit(2);                                                                  \
+        }                                                                                  \
+    } while (0)
+#define EXPECT(cond)                                                                       \
+    do {                                                                                   \
+        if (!(cond)) {                                                                     \
+            std::fprintf(stderr, "selftest failed: %s (%s:%d)\n", #cond, __FILE__, __LINE__); \
+            std::exit(3);                                                                  \
+        }                                                                                  \
+    } while (0)
+
+template <typename T>
+static std::vector<T> read_bin(const std::string &path, size_t n)
+{
+    std::vector<T> v(n);
+    FILE *f = std::fopen(path.c_str(), "rb");
+    if (!f || std::fread(v.data(), sizeof(T), n, f) != n) {
+        std::fprintf(stderr, "cannot read %zu items from %s\n", n, path.c_str());
+        std::exit(2);
+    }
+    std::fclose(f);
+    return v;
+}
+template <typename T>
+static T *to_device(const std::vector<T> &h)
+{
+    T *d = nullptr;
+    HIP_OK(hipMalloc((void **)&d, (h.size() ? h.size() : 1) * sizeof(T)));
+    if (!h.empty()) HIP_OK(hipMemcpy(d, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice));
+    return d;
+}
+
+template <typename T>
+static int run_case(const std::string &dir, const char *op, long m, long n, long nnz, long ncols, int alg,
+                    double alpha_d, double beta_d, int analysis, alphasparseDataType dt)
+{
+    auto rp = read_bin<int>(dir + "/row_ptr.bin", m + 1);
+    auto col = read_bin<int>(dir + "/col.bin", nnz);
+    auto val = read_bin<T>(dir + "/val.bin", nnz);
+    const bool mm = std::strcmp(op, "spmm") == 0;
+    auto xin = read_bin<T>(dir + "/x.bin", mm ? n * ncols : n);
+    auto yin = read_bin<T>(dir + "/y.bin", mm ? m * ncols : m);
+    int *d_rp = to_device(rp), *d_col = to_device(col);
+    T *d_val = to_device(val), *d_x = to_device(xin), *d_y = to_device(yin);
+    const T alpha = (T)alpha_d, beta = (T)beta_d;
+
+    alphasparseHandle_t handle = nullptr;
+    if (alphasparseGetHandle(&handle) != ALPHA_SPARSE_STATUS_SUCCESS) return 4;
+    alphasparseSpMatDescr_t A;
+    if (alphasparseCreateCsr(&A, (int)m, (int)n, (int)nnz, d_rp, d_col, d_val, ALPHA_SPARSE_INDEXTYPE_I32,
+                             ALPHA_SPARSE_INDEXTYPE_I32, ALPHA_SPARSE_INDEX_BASE_ZERO, dt))
+        return 5;
+    size_t bytes = 0;
+    void *buffer = nullptr;
+    alphasparseStatus_t s;
+    if (!mm) {
+        alphasparseDnVecDescr_t X, Y;
+        if (alphasparseCreateDnVec(&X, n, d_x, dt) || alphasparseCreateDnVec(&Y, m, d_y, dt)) return 6;
+        s = alphasparseSpMV_bufferSize(handle, ALPHA_SPARSE_OPERATION_NON_TRANSPOSE, &alpha, A, X, &beta, Y, dt,
+                                       (alphasparseSpMVAlg_t)alg, &bytes);
+        if (s) return 10 + (int)s;
+        HIP_OK(hipMalloc(&buffer, bytes ? bytes : 1));
+        if (analysis) {
+            s = alphasparseSpMV_analysis(handle, ALPHA_SPARSE_OPERATION_NON_TRANSPOSE, A, (alphasparseSpMVAlg_t)alg);
+            if (s) return 30 + (int)s;
+        }
+        for (int rep = 0; rep < 2; ++rep) {  // twice: the second call must not depend on the first
+            HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
+            s = alphasparseSpMV(handle, ALPHA_SPARSE_OPERATION_NON_TRANSPOSE, &alpha, A, X, &beta, Y, dt,
+                                (alphasparseSpMVAlg_t)alg, buffer);
+            if (s) return 50 + (int)s;
+        }
+        if (analysis && alphasparseSpMV_clear(handle, (alphasparseSpMVAlg_t)alg)) return 7;
+        alphasparseDestroyDnVec(X);
+        alphasparseDestroyDnVec(Y);
+    } else {
+        alphasparseDnMatDescr_t B, C;
+        if (alphasparseCreateDnMat(&B, n, ncols, ncols, d_x, dt, ALPHASPARSE_ORDER_ROW) ||
+            alphasparseCreateDnMat(&C, m, ncols, ncols, d_y, dt, ALPHASPARSE_ORDER_ROW))
+            return 6;
+        const auto N = ALPHA_SPARSE_OPERATION_NON_TRANSPOSE;
+        s = alphasparseSpMM_bufferSize(handle, N, N, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, &bytes);
+        if (s) return 10 + (int)s;
+        HIP_OK(hipMalloc(&buffer, bytes ? bytes : 1));
+        if (analysis) {
+            size_t b2 = 0;
+            s = alphasparseSpMM_preprocess(handle, N, N, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, &b2);
+            if (s) return 30 + (int)s;
+            if (b2 > bytes) return 8;
+        }
+        for (int rep = 0; rep < 2; ++rep) {
+            HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
+            s = alphasparseSpMM(handle, N, N, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, buffer);
+            if (s) return 50 + (int)s;
+        }
+        alphasparseDestroyDnMat(B);
+        alphasparseDestroyDnMat(C);
+    }
+    HIP_OK(hipStreamSynchronize(handle->stream));
+    std::vector<T> out(yin.size());
+    HIP_OK(hipMemcpy(out.data(), d_y, out.size() * sizeof(T), hipMemcpyDeviceToHost));
+    FILE *f = std::fopen((dir + "/out.bin").c_str(), "wb");
+    if (!f || std::fwrite(out.data(), sizeof(T), out.size(), f) != out.size()) return 9;
+    std::fclose(f);
+    alphasparseDestroySpMat(A);
+    alphasparse_destory_handle(handle);
+    for (void *p : {(void *)buffer, (void *)d_rp, (void *)d_col, (void *)d_val, (void *)d_x, (void *)d_y}) (void)hipFree(p);
+    return 0;
+}
+
+static int selftest()
+{
+    alphasparseHandle_t h = nullptr;
+    EXPECT(alphasparseGetHandle(&h) == ALPHA_SPARSE_STATUS_SUCCESS);
+    EXPECT(h && h->wavefront_size == 64 && h->buffer && h->buffer_size >= (1u << 20));
+    std::vector<int> rp = {0, 2, 3}, col = {0, 1, 1};
+    std::vector<double> val = {1, 2, 3}, x = {1, 10}, y = {100, 100};
+    int *d_rp = to_device(rp), *d_col = to_device(col);
+    double *d_val = to_device(val), *d_x = to_device(x), *d_y = to_device(y);
+    alphasparseSpMatDescr_t A;
+    EXPECT(alphasparseCreateCsr(&A, 2, 2, 3, d_rp, d_col, d_val, ALPHA_SPARSE_INDEXTYPE_I32, ALPHA_SPARSE_INDEXTYPE_I32,
+                                ALPHA_SPARSE_INDEX_BASE_ZERO, ALPHA_R_64F) == 0);
+    EXPECT(A->format == ALPHA_SPARSE_FORMAT_CSR && A->rows == 2 && A->nnz == 3 && A->row_data == d_rp && A->descr);
+    alphasparseDnVecDescr_t X, Y, Xf;
+    EXPECT(alphasparseCreateDnVec(&X, 2, d_x, ALPHA_R_64F) == 0 && alphasparseCreateDnVec(&Y, 2, d_y, ALPHA_R_64F) == 0);
+    EXPECT(alphasparseCreateDnVec(&Xf, 2, d_x, ALPHA_R_32F) == 0);
+    const double alpha = 2.0, beta = 0.5;
+    const auto N = ALPHA_SPARSE_OPERATION_NON_TRANSPOSE;
+    size_t bytes = 123;
+    // DEFAULT runs a kernel and the handle's own scratch serves a call without a caller's buffer
+    EXPECT(alphasparseSpMV(h, N, &alpha, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) == 0);
+    HIP_OK(hipDeviceSynchronize());
+    HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
+    EXPECT(y[0] == 2.0 * 21.0 + 50.0 && y[1] == 2.0 * 30.0 + 50.0);
+    // what is not supported says so
+    EXPECT(alphasparseSpMV(h, ALPHA_SPARSE_OPERATION_TRANSPOSE, &alpha, A, X, &beta, Y, ALPHA_R_64F,
+                           ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) == ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
+    EXPECT(alphasparseSpMV(h, N, &alpha, A, Xf, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) ==
+           ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
+    EXPECT(alphasparseSpMV(h, N, &alpha, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_COO, nullptr) ==
+           ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
+    EXPECT(alphasparseSpMV(nullptr, N, &alpha, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) ==
+           ALPHA_SPARSE_STATUS_INVALID_HANDLE);
+    EXPECT(alphasparseSpMV(h, N, nullptr, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) ==
+           ALPHA_SPARSE_STATUS_INVALID_POINTER);
+    EXPECT(alphasparseSpMV_bufferSize(h, N, &alpha, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_VECTOR, &bytes) == 0 &&
+           bytes == 0);
+    EXPECT(alphasparseSpMV_bufferSize(h, N, &alpha, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_MERGE, &bytes) == 0 &&
+           bytes > 0);
+    A->idx_base = ALPHA_SPARSE_INDEX_BASE_ONE;
+    EXPECT(alphasparseSpMV(h, N, &alpha, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) ==
+           ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
+    A->idx_base = ALPHA_SPARSE_INDEX_BASE_ZERO;
+    // analysis is kept on the handle, found again, and cleared
+    EXPECT(alphasparseSpMV_analysis(h, N, A, ALPHA_SPARSE_SPMV_ALG_DEFAULT) == 0 && A->analysed);
+    EXPECT(alphasparseSpMV_analysis(h, N, A, ALPHA_SPARSE_SPMV_ALG_DEFAULT) == 0);
+    HIP_OK(hipMemcpy(d_y, x.data(), sizeof(double) * 2, hipMemcpyHostToDevice));
+    EXPECT(alphasparseSpMV(h, N, &alpha, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) == 0);
+    HIP_OK(hipDeviceSynchronize());
+    HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
+    EXPECT(y[0] == 42.5 && y[1] == 65.0);
+    EXPECT(alphasparseSpMV_clear(h, ALPHA_SPARSE_SPMV_ALG_DEFAULT) == 0);
+    // SpMM: column-major operands are refused, row-major run
+    alphasparseDnMatDescr_t B, C, Bc;
+    EXPECT(alphasparseCreateDnMat(&B, 2, 1, 1, d_x, ALPHA_R_64F, ALPHASPARSE_ORDER_ROW) == 0);
+    EXPECT(alphasparseCreateDnMat(&C, 2, 1, 1, d_y, ALPHA_R_64F, ALPHASPARSE_ORDER_ROW) == 0);
+    EXPECT(alphasparseCreateDnMat(&Bc, 2, 1, 2, d_x, ALPHA_R_64F, ALPHASPARSE_ORDER_COL) == 0);
+    EXPECT(alphasparseSpMM(h, N, N, &alpha, A, Bc, &beta, C, ALPHA_R_64F, ALPHASPARSE_SPMM_ALG_DEFAULT, nullptr) ==
+           ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
+    EXPECT(alphasparseSpMM(h, N, N, &alpha, A, B, &beta, C, ALPHA_R_64F, ALPHASPARSE_SPMM_COO_ALG1, nullptr) ==
+           ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
+    HIP_OK(hipMemcpy(d_y, x.data(), sizeof(double) * 2, hipMemcpyHostToDevice));
+    EXPECT(alphasparseSpMM(h, N, N, &alpha, A, B, &beta, C, ALPHA_R_64F, ALPHASPARSE_SPMM_ALG_DEFAULT, nullptr) == 0);
+    HIP_OK(hipDeviceSynchronize());
+    HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
+    EXPECT(y[0] == 42.5 && y[1] == 65.0);
+    EXPECT(alphasparse_destory_handle(h) == 0);
+    std::printf("selftest ok\n");
+    return 0;
+}
+
+int main(int argc, char **argv)
+{
+    if (argc != 2) {
+        std::fprintf(stderr, "usage: %s <case_dir> | --selftest\n", argv[0]);
+        return 1;
+    }
+    if (std::strcmp(argv[1], "--selftest") == 0) return selftest();
+    const std::string dir = argv[1];
+    FILE *f = std::fopen((dir + "/meta.txt").c_str(), "r");
+    if (!f) return 1;
+    char op[16], dtype[16];
+    long m, n, nnz, ncols;
+    int alg, analysis;
+    double alpha, beta;
+    if (std::fscanf(f, "%15s %15s %ld %ld %ld %ld %d %lf %lf %d", op, dtype, &m, &n, &nnz, &ncols, &alg, &alpha, &beta,
+                    &analysis) != 10)
+        return 1;
+    std::fclose(f);
+    int rc = std::strcmp(dtype, "f64") == 0
+                 ? run_case<double>(dir, op, m, n, nnz, ncols, alg, alpha, beta, analysis, ALPHA_R_64F)
+                 : run_case<float>(dir, op, m, n, nnz, ncols, alg, alpha, beta, analysis, ALPHA_R_32F);
+    std::printf("rc %d\n", rc);
+    return rc;
+}

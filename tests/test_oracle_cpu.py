@@ -1,0 +1,320 @@
+"""Pins the CPU oracle: against the reference's own compiled CPU path where it is built,
+against committed golden vectors the reference produced, and against what the mathematics
+fixes (closed forms, exact-integer inputs, brute force on small inputs, a library routine)."""
+import math
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+from conftest import analysis_shapes, csr_from_lengths, row_ptr_from_lengths
+from library_amd import workloads as W
+
+
+# ------------------------------------------------------------------ oracle vs compiled reference
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("threads", [1, 3, 8])
+def test_spmv_matches_reference_build(oracle, ref, dtype, threads):
+    rng = np.random.default_rng(3)
+    lens = np.minimum(rng.zipf(1.8, 4000), 3000)
+    lens[rng.random(lens.size) < 0.05] = 0
+    rp, col, val = csr_from_lengths(lens, 5000, 4, dtype)
+    x = rng.uniform(-1, 1, 5000).astype(dtype)
+    y0 = rng.uniform(-1, 1, lens.size).astype(dtype)
+    for alpha, beta in ((1.0, 0.0), (1.5, 0.5), (2.0, 3.0)):
+        a = oracle.spmv(rp, col, val, x, alpha, beta, y0, threads)
+        b = ref.spmv(rp, col, val, x, alpha, beta, y0, threads)
+        assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n", [1, 7, 8, 64, 65, 600])
+def test_spmm_matches_reference_build(oracle, ref, dtype, n):
+    rng = np.random.default_rng(n)
+    lens = rng.integers(0, 12, 97)
+    lens[5] = 300
+    rp, col, val = csr_from_lengths(lens, 700, 6, dtype)
+    B = rng.uniform(-1, 1, 700 * n).astype(dtype)
+    C0 = rng.uniform(-1, 1, lens.size * n).astype(dtype)
+    a = oracle.spmm(rp, col, val, B, n, 2.0, 3.0, C0, 3)
+    b = ref.spmm(rp, col, val, B, n, 2.0, 3.0, C0, 3)
+    assert np.array_equal(a, b)
+
+
+def test_partition_matches_reference_build(oracle, ref):
+    for name, lens in analysis_shapes().items():
+        rp = row_ptr_from_lengths(lens)
+        for t in (1, 2, 3, 8, 25, 64, 1000):
+            assert np.array_equal(oracle.partition_rows_by_nnz(rp, t), ref.partition_rows_by_nnz(rp, t)), (name, t)
+
+
+def test_row_blocks_match_reference_build(oracle, ref):
+    rng = np.random.default_rng(77)
+    shapes = dict(analysis_shapes())
+    for i in range(20):
+        shapes[f"mix{i}"] = np.r_[rng.integers(0, 40, rng.integers(1, 400)), rng.integers(100, 1500, rng.integers(0, 30)),
+                                  rng.integers(0, 200, rng.integers(1, 300))]
+    for name, lens in shapes.items():
+        rp = row_ptr_from_lengths(lens)
+        assert np.array_equal(oracle.csr_adaptive_row_blocks(rp), ref.csr_adaptive_row_blocks(rp)), name
+
+
+# ------------------------------------------------------------------ oracle vs golden vectors
+def test_golden_banded(oracle, golden):
+    g = golden("banded_f64.npz")
+    w = W.banded_f64()
+    assert w.nnz == 24230 and w.bytes_algorithmic() == 316364
+    assert np.array_equal(oracle.spmv(w.row_ptr, w.col, w.val, w.x, 1.0, 0.0, w.y, 2), g["y_a1_b0"])
+    assert np.array_equal(oracle.spmv(w.row_ptr, w.col, w.val, w.x, 2.0, 3.0, w.y, 5), g["y_a2_b3"])
+
+
+@pytest.mark.parametrize("tag", ["f64", "f32"])
+def test_golden_rows(oracle, golden, tag):
+    g = golden(f"rows_{tag}.npz")
+    y = oracle.spmv(g["row_ptr"], g["col"], g["val"], g["x"], float(g["alpha"]), float(g["beta"]), g["y0"], 1)
+    assert np.array_equal(y, g["y"])
+
+
+def test_golden_spmm(oracle, golden):
+    g = golden("spmm_f32.npz")
+    for n in (1, 7, 8, 64, 65):
+        c = oracle.spmm(g["row_ptr"], g["col"], g["val"], g[f"B{n}"], n, float(g["alpha"]), float(g["beta"]), g[f"C0_{n}"], 2)
+        assert np.array_equal(c, g[f"C{n}"]), n
+    g = golden("spmm_f64.npz")
+    for n in (1, 8, 13):
+        c = oracle.spmm(g["row_ptr"], g["col"], g["val"], g[f"B{n}"], n, float(g["alpha"]), float(g["beta"]), g[f"C0_{n}"], 2)
+        assert np.array_equal(c, g[f"C{n}"]), n
+
+
+def test_golden_partition(oracle, golden):
+    g = golden("partition.npz")
+    names = sorted({k.split("__")[0] for k in g.files})
+    for name in names:
+        rp = g[f"{name}__row_ptr"]
+        for t in (1, 2, 3, 8, 25, 64):
+            assert np.array_equal(oracle.partition_rows_by_nnz(rp, t), g[f"{name}__T{t}"]), (name, t)
+
+
+def test_golden_row_blocks(oracle, golden):
+    g = golden("row_blocks.npz")
+    for name in sorted({k.split("__")[0] for k in g.files}):
+        assert np.array_equal(oracle.csr_adaptive_row_blocks(g[f"{name}__row_ptr"]), g[f"{name}__blocks"]), name
+
+
+# ------------------------------------------------------------------ what the mathematics fixes
+def _exact_fma_row_f64(a, x):
+    """The asm kernel's summation tree in exact rational arithmetic, one rounding per fma/add."""
+    def rnd(fr):
+        return float(fr)  # Fraction -> nearest double (correctly rounded)
+    acc = [0.0] * 4
+    k, n = 0, len(a)
+    s = 0.0
+    if n >= 4:
+        while k < n - 3:
+            for l in range(4):
+                acc[l] = rnd(Fraction(a[k + l]) * Fraction(x[k + l]) + Fraction(acc[l]))
+            k += 4
+        lo = rnd(Fraction(acc[2]) + Fraction(acc[0]))
+        hi = rnd(Fraction(acc[3]) + Fraction(acc[1]))
+        s = rnd(Fraction(hi) + Fraction(lo))
+    while k < n:
+        s = rnd(Fraction(a[k]) * Fraction(x[k]) + Fraction(s))
+        k += 1
+    return s
+
+
+def test_fp64_row_tree_against_exact_rationals(oracle):
+    rng = np.random.default_rng(5)
+    lens = list(range(0, 14)) + [17, 31, 64, 65]
+    rp, col, val = csr_from_lengths(lens, 200, 8, np.float64)
+    x = rng.uniform(-1, 1, 200)
+    y0 = rng.uniform(-1, 1, len(lens))
+    alpha, beta = 1.5, 0.5
+    y = oracle.spmv(rp, col, val, x, alpha, beta, y0, 1)
+    for r in range(len(lens)):
+        s = _exact_fma_row_f64(val[rp[r]:rp[r + 1]], x[col[rp[r]:rp[r + 1]]])
+        by = float(Fraction(beta) * Fraction(y0[r]))
+        expect = float(Fraction(alpha) * Fraction(s) + Fraction(by))
+        assert y[r] == expect, r
+
+
+def test_integer_inputs_are_order_independent(oracle):
+    # small integers: every partial sum is exact, so any correct kernel gives the same bits
+    rng = np.random.default_rng(2)
+    lens = rng.integers(0, 70, 500)
+    for dtype in (np.float64, np.float32):
+        rp, col, _ = csr_from_lengths(lens, 900, 3, dtype)
+        val = rng.integers(-8, 9, col.size).astype(dtype)
+        x = rng.integers(-8, 9, 900).astype(dtype)
+        y0 = rng.integers(-8, 9, lens.size).astype(dtype)
+        y = oracle.spmv(rp, col, val, x, 2.0, 3.0, y0, 2)
+        expect = np.array([2 * int(np.dot(val[rp[r]:rp[r + 1]].astype(np.int64), x[col[rp[r]:rp[r + 1]]].astype(np.int64)))
+                           + 3 * int(y0[r]) for r in range(lens.size)], dtype=dtype)
+        assert np.array_equal(y, expect)
+        n = 9
+        B = rng.integers(-4, 5, 900 * n).astype(dtype)
+        C0 = rng.integers(-4, 5, lens.size * n).astype(dtype)
+        Cm = oracle.spmm(rp, col, val, B, n, 2.0, 3.0, C0, 2)
+        A = sp.csr_matrix((val.astype(np.int64), col, rp), shape=(lens.size, 900))
+        expectC = 2 * (A @ B.reshape(900, n).astype(np.int64)) + 3 * C0.reshape(-1, n).astype(np.int64)
+        assert np.array_equal(Cm.reshape(-1, n), expectC.astype(dtype))
+
+
+def test_laplacian_closed_form(oracle):
+    nx = ny = 64
+    rp, col, val = W.csr_stencil5(nx, ny)
+    assert rp[-1] == 5 * nx * ny - 2 * nx - 2 * ny
+    ones = np.ones(nx * ny)
+    y = oracle.spmv(rp, col, val, ones, 1.0, 0.0, np.full(nx * ny, 7.0), 2)
+    deg = np.diff(rp) - 1
+    assert np.array_equal(y, 4.0 - deg)  # 0 interior, 1 edges, 2 corners
+    ix = np.tile(np.arange(nx, dtype=np.float64), ny)
+    y = oracle.spmv(rp, col, val, ix, 1.0, 0.0, np.zeros(nx * ny), 1).reshape(ny, nx)
+    assert np.all(y[1:-1, 1:-1] == 0.0)  # a linear ramp is harmonic away from the boundary
+
+
+def test_diagonal_and_beta(oracle):
+    n = 257
+    rp = np.arange(n + 1, dtype=np.int32)
+    col = np.arange(n, dtype=np.int32)
+    rng = np.random.default_rng(0)
+    a, x, y0 = rng.uniform(-1, 1, n), rng.uniform(-1, 1, n), rng.uniform(-1, 1, n)
+    y = oracle.spmv(rp, col, a, x, 1.5, 0.5, y0, 1)
+    expect = np.array([math.fma(1.5, math.fma(a[i], x[i], 0.0), 0.5 * y0[i]) for i in range(n)]) \
+        if hasattr(math, "fma") else None
+    if expect is not None:
+        assert np.array_equal(y, expect)
+    assert np.allclose(y, 1.5 * a * x + 0.5 * y0, rtol=1e-15, atol=1e-16)
+    # the reference CPU kernel multiplies y by beta even when beta == 0: NaN in y propagates
+    ynan = oracle.spmv(rp, col, a, x, 1.0, 0.0, np.full(n, np.nan), 1)
+    assert np.all(np.isnan(ynan))
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float64, 1e-13), (np.float32, 1e-5)])
+def test_against_scipy_and_fsum(oracle, dtype, tol):
+    rng = np.random.default_rng(9)
+    lens = np.minimum(rng.zipf(1.7, 2000), 1500)
+    rp, col, val = csr_from_lengths(lens, 3000, 10, dtype)
+    x = rng.uniform(-1, 1, 3000).astype(dtype)
+    y0 = rng.uniform(-1, 1, lens.size).astype(dtype)
+    y = oracle.spmv(rp, col, val, x, 1.5, 0.5, y0, 4).astype(np.float64)
+    A = sp.csr_matrix((val.astype(np.float64), col, rp), shape=(lens.size, 3000))
+    exact = np.array([1.5 * math.fsum(val[rp[r]:rp[r + 1]].astype(np.float64) * x[col[rp[r]:rp[r + 1]]].astype(np.float64))
+                      + 0.5 * float(y0[r]) for r in range(lens.size)])
+    scale = 1.5 * (abs(A) @ np.abs(x.astype(np.float64))) + 0.5 * np.abs(y0.astype(np.float64))
+    assert np.all(np.abs(y - exact) <= tol * np.maximum(scale, 1e-300))
+    assert np.all(np.abs(A @ x.astype(np.float64) * 1.5 + 0.5 * y0 - exact) <= 1e-12 * np.maximum(scale, 1e-300))
+
+
+def test_spmm_columns_equal_spmv_of_columns(oracle):
+    # ties the SpMM restatement to the SpMV one: same products, sums differ only in order
+    rng = np.random.default_rng(4)
+    lens = rng.integers(0, 30, 300)
+    rp, col, val = csr_from_lengths(lens, 500, 5, np.float64)
+    n = 5
+    B = rng.uniform(-1, 1, 500 * n)
+    C0 = rng.uniform(-1, 1, lens.size * n)
+    Cm = oracle.spmm(rp, col, val, B, n, 1.5, 0.5, C0, 2).reshape(-1, n)
+    for j in range(n):
+        yj = oracle.spmv(rp, col, val, np.ascontiguousarray(B.reshape(500, n)[:, j]), 1.5, 0.5,
+                         np.ascontiguousarray(C0.reshape(-1, n)[:, j]), 1)
+        assert np.allclose(Cm[:, j], yj, rtol=0, atol=1e-13)
+
+
+# ------------------------------------------------------------------ integer analysis: brute force
+def _brute_partition(rp, t):
+    m = rp.size - 1
+    acc = rp[1:]
+    nnz = int(acc[m - 1])
+    ave = nnz // t
+    out = [0]
+    for i in range(1, t):
+        target = np.int32(np.int64(ave) * i & 0xFFFFFFFF) if ave * i > 2**31 - 1 else ave * i
+        p = next((p for p in range(0, m - 1) if acc[p] >= target), m - 1)
+        out.append(p)
+    out.append(m)
+    return np.array(out, dtype=np.int32)
+
+
+def test_partition_brute_force(oracle):
+    for name, lens in analysis_shapes().items():
+        rp = row_ptr_from_lengths(lens)
+        for t in (1, 2, 5, 16, 300):
+            got = oracle.partition_rows_by_nnz(rp, t)
+            assert np.array_equal(got, _brute_partition(rp, t)), (name, t)
+            assert got[0] == 0 and got[-1] == rp.size - 1 and np.all(np.diff(got) >= 0)
+
+
+def test_nnz_split_brute_force(oracle):
+    for name, lens in analysis_shapes().items():
+        rp = row_ptr_from_lengths(lens)
+        m, nnz = rp.size - 1, int(rp[-1])
+        for items in (1, 7, 64, 1024):
+            got = oracle.nnz_split_rows(rp, items)
+            nseg = (nnz + items - 1) // items
+            assert got.size == nseg + 1 and got[-1] == m
+            for t in range(nseg):
+                e = t * items
+                r = got[t]
+                assert rp[r] <= e < rp[r + 1], (name, items, t)  # the row that holds element e
+
+
+def test_merge_path_brute_force(oracle):
+    for name, lens in analysis_shapes().items():
+        rp = row_ptr_from_lengths(lens)
+        m, nnz = rp.size - 1, int(rp[-1])
+        row_end = rp[1:].astype(np.int64)
+        for items in (1, 5, 128, 2048, 4096):
+            xs, ys = oracle.merge_path_search(rp, items)
+            nblk = (m + nnz + items - 1) // items
+            assert xs.size == nblk + 1
+            # walk the merge path item by item: consume a stored element while one of the current
+            # row is left, else consume the row end
+            x = y = 0
+            g = 0
+            for d in range(m + nnz + 1):
+                while g <= nblk and min(g * items, m + nnz) == d:
+                    assert (xs[g], ys[g]) == (x, y), (name, items, g)
+                    g += 1
+                if d == m + nnz:
+                    break
+                if x < m and y < row_end[x]:
+                    y += 1
+                elif x < m:
+                    x += 1
+                else:
+                    y += 1
+            assert g == nblk + 1
+            assert xs[-1] == m and ys[-1] == nnz
+
+
+def test_loadbalance_brute_force(oracle):
+    table = {0: 8, 199999: 8, 200000: 32, 1999999: 32, 2000000: 128, 19999999: 128, 20000000: 512,
+             199999999: 512, 200000000: 2048}
+    for nnz, mult in table.items():
+        assert oracle.loadbalance_nwarps(nnz, 32, 160) == min((nnz + 31) // 32, 160 * mult)
+    assert oracle.loadbalance_nwarps(16777216, 32, 160) == 20480
+    for name, lens in analysis_shapes().items():
+        rp = row_ptr_from_lengths(lens)
+        m, nnz = rp.size - 1, int(rp[-1])
+        if nnz == 0:
+            continue
+        for ws, base in ((32, 2), (64, 1)):
+            nw = oracle.loadbalance_nwarps(nnz, ws, base)
+            got = oracle.loadbalance_partition(rp, ws, nw)
+            ave = (nnz + ws - 1) // ws
+            acc = rp[1:].astype(np.int64)
+            chunks = (acc + ws - 1) // ws * nw
+            for g in range(nw):
+                expect = int(np.searchsorted(chunks, ave * g, side="left"))  # first p with chunks[p] >= target, else m
+                assert got[g] == expect, (name, ws, g)
+
+
+def test_find_rows_brute_force(oracle):
+    for name, lens in analysis_shapes().items():
+        rp = row_ptr_from_lengths(lens)
+        counts, mid = oracle.find_rows_counts(rp, 2, 1024)
+        lens = np.asarray(lens)
+        assert list(counts) == [int((lens < 2).sum()), int(((lens >= 2) & (lens < 1024)).sum()), int((lens >= 1024).sum())]
+        assert mid == int(lens[(lens >= 2) & (lens < 1024)].sum())
