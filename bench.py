@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of the CSR SpMV / SpMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only]
+
+A step is one SpMV (or SpMM) call through the C-ABI on a synthetic workload that is already
+resident in HBM; analysis (split points) is done once, outside the timed region, and reported
+separately.  Prints ONE JSON line.  `value` is effective GB/s = algorithmic bytes / time, with
+    SpMV bytes = nnz*(sv+4) + (m+1)*4 + n*sv   + m*sv  *(beta != 0 ? 2 : 1)
+    SpMM bytes = nnz*(sv+4) + (m+1)*4 + k*N*sv + m*N*sv*(beta != 0 ? 2 : 1)
+All five benchmark configurations are measured (unless --only); the one named by --workload
+supplies the headline fields, the others are listed under "workloads".
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
+ORDER = ["banded_f64", "uniform16_f32", "powerlaw_f64", "stencil5_f64", "spmm_zipf_f32"]
+KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 5: "k_spmm_row", 7: "k_spmm_merge"}
+
+# HBM traffic per call measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; see profiles/),
+# scaled by the same counters' reading for a plain copy of known size.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="powerlaw_f64", choices=ORDER)
+    ap.add_argument("--only", action="store_true", help="measure only --workload")
+    ap.add_argument("--alg", type=int, default=0, help="kernel id (0 = pick from the histogram)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
+    return ap.parse_args()
+
+
+def measure(w, steps, warmup, alg):
+    """Returns a dict of measurements for workload w (arrays on host)."""
+    import numpy as np
+    import torch
+    from library_amd import capi
+
+    dev = lambda a: torch.from_numpy(a).cuda()
+    d_rp, d_col, d_val, d_x = dev(w.row_ptr), dev(w.col), dev(w.val), dev(w.x)
+    d_y = dev(w.y.copy())
+    spmm = w.kind == "spmm"
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    plan = capi.Plan(spmm, alg, w.val.dtype, w.m, w.n, w.nnz, d_rp, ncols=w.ncols)
+    torch.cuda.synchronize()
+    analysis_ms = (time.perf_counter() - t0) * 1e3
+    ws = torch.empty(max(plan.workspace_bytes, 256), dtype=torch.uint8, device="cuda")
+
+    def step():
+        if spmm:
+            capi.spmm(d_rp, d_col, d_val, d_x, d_y, w.ncols, w.alpha, w.beta, plan=plan, workspace=ws, k=w.n)
+        else:
+            capi.spmv(d_rp, d_col, d_val, d_x, d_y, w.alpha, w.beta, plan=plan, workspace=ws)
+
+    for _ in range(warmup):
+        step()
+    # (a) K steps back to back, bracketed by synchronisation: the whole-job figure
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # (b) one HIP event pair per call on the launch stream: per-call device time
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    for i in range(steps):
+        starts[i].record()
+        step()
+        ends[i].record()
+    torch.cuda.synchronize()
+    per_call = np.array([s.elapsed_time(e) for s, e in zip(starts, ends)])
+    nbytes = w.bytes_algorithmic()
+    res = {
+        "workload": w.name, "kind": w.kind, "dtype": "f64" if w.dtype.itemsize == 8 else "f32",
+        "m": w.m, "n": w.n, "nnz": w.nnz, "ncols": w.ncols, "alpha": w.alpha, "beta": w.beta,
+        "max_row": int(np.diff(w.row_ptr).max()) if w.m else 0,
+        "kernel": KERNEL_NAMES.get(plan.alg, str(plan.alg)),
+        "bytes": nbytes, "bytes_y_twice": w.bytes_algorithmic(y_twice=True), "flops": w.flops,
+        "analysis_ms": round(analysis_ms, 3),
+        "ms_per_step": wall_ms,
+        "event_ms_mean": float(per_call.mean()), "event_ms_median": float(np.median(per_call)),
+        "event_ms_min": float(per_call.min()),
+    }
+    res["gbs"] = nbytes / (wall_ms * 1e-3) / 1e9
+    res["gflops"] = w.flops / (wall_ms * 1e-3) / 1e9
+    res["gbs_event"] = nbytes / (res["event_ms_mean"] * 1e-3) / 1e9
+    res["frac_hbm_peak"] = res["gbs_event"] / HBM_PEAK_GBS
+    plan.destroy()
+    del d_rp, d_col, d_val, d_x, d_y, ws
+    torch.cuda.empty_cache()
+    return res
+
+
+def cpu_baseline(w, budget_s):
+    """The reference's own CPU path (oracle/_ref, kind "reference") or, where that is not
+    built, the C restatement (kind "port"), timed on this host for the same workload."""
+    import numpy as np
+    from oracle.bindings import Oracle, Ref
+
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 16)
+    nbytes = w.bytes_algorithmic()
+    times = []
+    if Ref.available():
+        kind = "reference"
+        ref = Ref()
+        h = ref.create(w.row_ptr, w.col, w.val, w.n)
+        y = w.y.copy()
+
+        def call():
+            if w.kind == "spmm":
+                ref.mm(h, w.x, w.ncols, w.alpha, w.beta, y, threads)
+            else:
+                ref.mv(h, w.x, w.alpha, w.beta, y, threads)
+    else:
+        kind = "port"
+        orc = Oracle()
+
+        def call():
+            if w.kind == "spmm":
+                orc.spmm(w.row_ptr, w.col, w.val, w.x, w.ncols, w.alpha, w.beta, w.y, threads)
+            else:
+                orc.spmv(w.row_ptr, w.col, w.val, w.x, w.alpha, w.beta, w.y, threads)
+    t_start = time.perf_counter()
+    call()  # warm-up (first touch, thread pool)
+    warm = time.perf_counter() - t_start
+    reps = 0
+    while reps < 20 and (time.perf_counter() - t_start) < budget_s and (reps < 3 or warm * (reps + 2) < budget_s):
+        t0 = time.perf_counter()
+        call()
+        times.append(time.perf_counter() - t0)
+        reps += 1
+    if not times:
+        times = [warm]
+    t = float(np.median(times))
+    if kind == "reference":
+        ref.destroy(h)
+    return {"value": nbytes / t / 1e9, "unit": "GB/s", "cores": threads, "kind": kind,
+            "sample": f"{w.name} at full size, median of {len(times)} calls after 1 warm-up, {threads} OpenMP threads",
+            "ms_per_call": t * 1e3, "gflops": w.flops / t / 1e9}
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {a.gpus} is not supported "
+              "(the path has no multi-GPU part: rows shard by nnz with an all-gather of x, see DESIGN.md)",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from library_amd import capi, workloads as W
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    capi.lib()
+
+    names = [a.workload] if a.only else ORDER
+    results = {}
+    head_w = None
+    for name in names:
+        w = W.CONFIGS[name]()
+        results[name] = measure(w, a.steps, a.warmup, a.alg if name == a.workload else 0)
+        if name == a.workload:
+            head_w = w
+        else:
+            del w
+    head = results[a.workload]
+    cpu = None
+    if not a.no_cpu:
+        try:
+            cpu = cpu_baseline(head_w, a.cpu_seconds)
+        except Exception as e:  # the baseline is a reported extra; never lose the GPU line to it
+            cpu = {"value": None, "unit": "GB/s", "cores": 0, "kind": "unavailable", "sample": repr(e)}
+    traffic = MEASURED_TRAFFIC_BYTES.get(a.workload)
+    line = {
+        "metric": "effective HBM GB/s, CSR " + ("SpMM N=64 fp32" if head["kind"] == "spmm" else f"SpMV {head['dtype']}")
+                  + " (algorithmic bytes / time)",
+        "value": head["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": head["dtype"], "data": "synthetic",
+        "config": {"workload": a.workload, "m": head["m"], "n": head["n"], "nnz": head["nnz"], "ncols": head["ncols"],
+                   "alpha": head["alpha"], "beta": head["beta"], "max_row": head["max_row"], "kernel": head["kernel"],
+                   "analysis_ms": head["analysis_ms"]},
+        "gflops": head["gflops"], "pct_hbm_peak": 100.0 * head["gbs"] / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "achieved": head["gbs_event"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": head["frac_hbm_peak"], "traffic": traffic, "kernel": head["kernel"],
+                     "bytes_per_launch": head["bytes"], "launch_ms": head["event_ms_mean"]},
+        "cpu_baseline": cpu,
+        "workloads": [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in results[n].items()} for n in names],
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -64,7 +64,7 @@ SpmmLayout spmm_merge_layout(int32_t m, int32_t nnz, int32_t ncols, size_t sv, b
 int choose_spmv_from_stats(const int64_t stats[4], int32_t m, int32_t nnz)
 {
     const int64_t max_len = stats[0];
-    if (max_len > 4 * kStreamTile) return ASX_SPMV_MERGE;
+    if (max_len > kStreamMaxRow) return ASX_SPMV_MERGE;
     (void)m;
     (void)nnz;
     return ASX_SPMV_STREAM;
@@ -307,7 +307,7 @@ int asx_plan_create(asx_plan **out, int is_spmm, int alg, int value_type, int32_
         if (kernel == ASX_SPMV_STREAM) {
             int32_t nb = std::max(stream_blocks(nnz), 1);
             p->nunits = nb;
-            p->meta_bytes = ((size_t)nb + 1) * 4;
+            p->meta_bytes = ((size_t)nb + 1) * 8;
             st = status_of(hipMalloc((void **)&p->d_meta, p->meta_bytes));
             if (!st) st = launch_stream_row_blocks(d_row_ptr, m, nnz, p->d_meta, s);
             p->workspace_bytes = 0;
@@ -408,7 +408,7 @@ size_t asx_spmv_workspace_bytes(int alg, int value_type, int32_t m, int32_t nnz)
     const int kernel = asx_spmv_resolve_alg(alg, m, nnz);
     if (kernel == ASX_SPMV_MERGE) return spmv_merge_layout(m, nnz, vsize(value_type), true).bytes;
     if (kernel == ASX_SPMV_STREAM)
-        return align_up(((size_t)std::max(stream_blocks(nnz), 1) + 1) * 4, kAlign);
+        return align_up(((size_t)std::max(stream_blocks(nnz), 1) + 1) * 8, kAlign);
     return 0;
 }
 

@@ -13,7 +13,8 @@ namespace asx {
 constexpr int kBlock = 256;
 constexpr int kMergeItemsPerThread = 8;
 constexpr int kMergeTile = kBlock * kMergeItemsPerThread;  // rows + stored elements per tile
-constexpr int kStreamTile = 2048;                          // stored elements per row block
+constexpr int kStreamTile = 1024;                          // stored elements per row block
+constexpr int kStreamMaxRow = 8192;  // DEFAULT picks the stream kernel only below this row length
 // SpMM: merge items (rows + stored elements) per wave
 constexpr int kSpmmSegment = 128;
 

@@ -158,8 +158,10 @@ __global__ __launch_bounds__(kBlock) void k_spmm_merge(int32_t m, int32_t nnz, i
     if (lane == 0 && blockIdx.y == 0) carry_row[seg] = has_tail ? x1 : -1;
 }
 
-// One wave per segment that opens a run of segments ending inside the same row: sums the
-// run's carry rows in segment order and adds them to C.
+// One wave per segment that opens a run of segments ending inside the same row: finds the
+// length of the run (64 segments per step, one ballot each), then sums the run's carry rows in
+// segment order with a counted, unrolled loop (many independent loads in flight; a loop that
+// tests carry_row before every add would pay one memory round trip per segment).
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_spmm_merge_fixup(int32_t m, int32_t nseg, int32_t ncols,
                                                              T alpha, const T *__restrict__ carry,
@@ -168,14 +170,32 @@ __global__ __launch_bounds__(kBlock) void k_spmm_merge_fixup(int32_t m, int32_t 
 {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t seg = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
-    if (seg >= nseg) return;
-    const int32_t row = carry_row[seg];
+    if (seg >= nseg) return;  // wave-uniform from here on
+    const int32_t row = __builtin_amdgcn_readfirstlane(carry_row[seg]);
     if (row < 0 || row >= m) return;
-    if (seg > 0 && carry_row[seg - 1] == row) return;
+    if (seg > 0 && __builtin_amdgcn_readfirstlane(carry_row[seg - 1]) == row) return;
+    int64_t len = 1;
+    for (int64_t base = seg + 1;; base += kWave) {
+        const int64_t idx = base + lane;
+        const bool same = idx < nseg && carry_row[idx] == row;
+        const unsigned long long mask = __ballot(same);
+        const int n = mask == ~0ull ? kWave : __ffsll((unsigned long long)~mask) - 1;
+        len += n;
+        if (n < kWave) break;
+    }
     const int64_t c = (int64_t)blockIdx.y * kWave + lane;
     if (c >= ncols) return;
-    T sum = carry[seg * ncols + c];
-    for (int64_t j = seg + 1; j < nseg && carry_row[j] == row; ++j) sum += carry[j * ncols + c];
+    const T *p = carry + seg * ncols + c;
+    T sum = T(0);
+    int64_t j = 0;
+    for (; j + 16 <= len; j += 16) {
+        T v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v[u] = p[(j + u) * ncols];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) sum += v[u];
+    }
+    for (; j < len; ++j) sum += p[j * ncols];
     const int64_t idx = (int64_t)row * ldc + c;
     C[idx] = fma_t<T>(alpha, sum, C[idx]);
 }

@@ -18,15 +18,37 @@
 
 namespace asx {
 
-// Workgroups are dealt to the 8 XCDs round-robin by the hardware.  Mapping workgroup id ->
-// tile so that each XCD walks one contiguous eighth of the tiles keeps the x entries shared
-// by neighbouring rows in that XCD's own L2.
-__device__ __forceinline__ int xcd_contiguous_tile(int bid, int ntiles)
+// Tile order: tile = workgroup id.  Workgroups are dealt to the 8 XCDs round-robin, so
+// neighbouring tiles run at the same time on different XCDs.  The alternative (each XCD walks
+// one contiguous eighth of the tiles, so that x entries shared by neighbouring rows stay in
+// one L2) measured 0-5 % slower on the benchmark workloads (5-point stencil 326 vs 312 us,
+// power-law 586 vs 580 us, uniform 16/row equal): the shared x lines are served by the
+// Infinity Cache either way, and eight far-apart streams cost more than they save.
+
+// Streaming operands (stored elements, column indices, y) are touched once per call.  When
+// they are larger than the Infinity Cache can hold from one call to the next, loading and
+// storing them with the non-temporal hint keeps x cached (stencil: 312 -> 305 us); when the
+// whole working set fits that cache the hint costs its hits (uniform 16/row fp32, 151 MB:
+// 96 -> 114 us), so it is chosen per call from the size of the streamed arrays.
+template <bool NT, typename T>
+__device__ __forceinline__ T stream_load(const T *p)
 {
-    const int per = (ntiles + 7) >> 3;
-    return (bid & 7) * per + (bid >> 3);
+    return NT ? __builtin_nontemporal_load(p) : *p;
 }
-inline int xcd_grid(int ntiles) { return ((ntiles + 7) >> 3) << 3; }
+template <bool NT, typename T>
+__device__ __forceinline__ void stream_store(T *p, T v)
+{
+    if (NT)
+        __builtin_nontemporal_store(v, p);
+    else
+        *p = v;
+}
+
+constexpr int64_t kNonTemporalAboveBytes = (int64_t)128 << 20;
+inline bool use_nontemporal(int64_t nnz, size_t sv)
+{
+    return nnz * (int64_t)(sv + 4) > kNonTemporalAboveBytes;
+}
 
 template <typename T>
 __device__ __forceinline__ T axpby_out(T alpha, T sum, T beta, const T *y, int64_t r)
@@ -96,11 +118,20 @@ int launch_spmv_vector(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, 
 // would otherwise put every lane of a wave on the same few banks.
 __device__ __forceinline__ int pad32(int j) { return j + (j >> 5); }
 constexpr int kStreamLds = kStreamTile + kStreamTile / 32 + 1;
+constexpr int kStreamRowCap = kStreamTile / 2;  // row pointers kept in LDS per block (+1)
 
-template <int G, typename T>
-__device__ __forceinline__ void stream_reduce_rows(const T *s_prod, int32_t r0, int32_t nrows,
-                                                   int32_t a, int32_t c1, int32_t last_row,
-                                                   T extra, T alpha, T beta,
+// Row pointer i of the block (relative to the block's first stored element): from LDS for the
+// first kStreamRowCap+1 rows, from memory for the (rare) rows past that.
+__device__ __forceinline__ int32_t stream_rp(const int32_t *s_rp, const int32_t *__restrict__ row_ptr,
+                                             int32_t r0, int32_t a, int i)
+{
+    return i <= kStreamRowCap ? s_rp[i] : row_ptr[r0 + i] - a;
+}
+
+template <int G, bool NT, typename T>
+__device__ __forceinline__ void stream_reduce_rows(const T *s_prod, const int32_t *s_rp, int32_t r0,
+                                                   int32_t nrows, int32_t a, int32_t n1, T extra,
+                                                   T alpha, T beta, T y_first, bool y_first_ok,
                                                    const int32_t *__restrict__ row_ptr,
                                                    T *__restrict__ y)
 {
@@ -110,22 +141,27 @@ __device__ __forceinline__ void stream_reduce_rows(const T *s_prod, int32_t r0, 
     for (int base = 0; base < nrows; base += rows_per_pass) {
         const int g = base + (int)threadIdx.x / G;
         T sum = T(0);
-        int32_t r = r0 + g;
         if (g < nrows) {
-            int32_t s = row_ptr[r] - a;
-            int32_t e = row_ptr[r + 1];
-            e = (e < c1 ? e : c1) - a;
+            const int32_t s = stream_rp(s_rp, row_ptr, r0, a, g);
+            int32_t e = stream_rp(s_rp, row_ptr, r0, a, g + 1);
+            e = e < n1 ? e : n1;
             for (int32_t j = s + lane; j < e; j += G) sum += s_prod[pad32(j)];
         }
         sum = group_sum<G>(sum);
         if (g < nrows && lane == 0) {
-            if (r == last_row) sum += extra;
-            y[r] = axpby_out<T>(alpha, sum, beta, y, r);
+            const int64_t r = (int64_t)r0 + g;
+            if (g == nrows - 1) sum += extra;
+            T out;
+            if (beta == T(0))
+                out = alpha * sum;
+            else
+                out = fma_t<T>(alpha, sum, beta * ((base == 0 && y_first_ok) ? y_first : y[r]));
+            stream_store<NT>(y + r, out);
         }
     }
 }
 
-template <typename T>
+template <typename T, bool NT>
 __global__ __launch_bounds__(kBlock) void k_spmv_stream(int32_t m, int32_t nblocks, T alpha,
                                                         const int32_t *__restrict__ row_ptr,
                                                         const int32_t *__restrict__ col,
@@ -135,32 +171,60 @@ __global__ __launch_bounds__(kBlock) void k_spmv_stream(int32_t m, int32_t nbloc
                                                         const int32_t *__restrict__ blocks)
 {
     __shared__ T s_prod[kStreamLds];
+    __shared__ int32_t s_rp[kStreamRowCap + 1];
     __shared__ T s_part[kBlock / kWave];
-    const int t = xcd_contiguous_tile(blockIdx.x, nblocks);
-    if (t >= nblocks) return;
-    const int32_t r0 = blocks[t], r1 = blocks[t + 1];
+    const int t = blockIdx.x;
+    // blocks[2t] = first row of block t, blocks[2t+1] = its first stored element: one hop
+    const int2 lo = reinterpret_cast<const int2 *>(blocks)[t];
+    const int2 hi = reinterpret_cast<const int2 *>(blocks)[t + 1];
+    const int32_t r0 = lo.x, r1 = hi.x;
     const int32_t nrows = r1 - r0;
     if (nrows <= 0) return;
-    const int32_t a = row_ptr[r0];
-    const int32_t bend = row_ptr[r1];
+    const int32_t a = lo.y;
+    const int32_t bend = hi.y;
     const int32_t c1 = bend - a > kStreamTile ? a + kStreamTile : bend;
     const int32_t n1 = c1 - a;
     const int tid = threadIdx.x;
 
-    // ---- stage the window's products (coalesced; all loads issued before first use) ----
+    // ---- issue every load of the block up front: stored elements, row pointers, y ----
     constexpr int IPT = kStreamTile / kBlock;
     int32_t cj[IPT];
     T vj[IPT];
 #pragma unroll
     for (int i = 0; i < IPT; ++i) {
         const int j = tid + i * kBlock;
-        cj[i] = j < n1 ? col[(int64_t)a + j] : 0;
-        vj[i] = j < n1 ? val[(int64_t)a + j] : T(0);
+        cj[i] = j < n1 ? stream_load<NT>(col + (int64_t)a + j) : 0;
     }
 #pragma unroll
     for (int i = 0; i < IPT; ++i) {
         const int j = tid + i * kBlock;
+        vj[i] = j < n1 ? stream_load<NT>(val + (int64_t)a + j) : T(0);
+    }
+    constexpr int RPI = (kStreamRowCap + 1 + kBlock - 1) / kBlock;
+    const int32_t rp_n = nrows < kStreamRowCap ? nrows : kStreamRowCap;  // pointers 0..rp_n
+    int32_t rpv[RPI];
+#pragma unroll
+    for (int i = 0; i < RPI; ++i) {
+        const int j = tid + i * kBlock;
+        rpv[i] = j <= rp_n ? row_ptr[r0 + j] : 0;
+    }
+    // the row this thread writes in the first reduction pass (lanes-per-row is decided below
+    // from nrows alone, so the mapping is known here)
+    int g_shift = 0;
+    if (nrows <= 128) g_shift = nrows > 64 ? 1 : nrows > 32 ? 2 : nrows > 16 ? 3 : nrows > 8 ? 4 : nrows > 4 ? 5 : 6;
+    const int my_g = tid >> g_shift;
+    const bool y_first_ok = beta != T(0) && my_g < nrows && (tid & ((1 << g_shift) - 1)) == 0;
+    const T y_first = y_first_ok ? y[(int64_t)r0 + my_g] : T(0);
+
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+        const int j = tid + i * kBlock;
         if (j < n1) s_prod[pad32(j)] = vj[i] * x[cj[i]];
+    }
+#pragma unroll
+    for (int i = 0; i < RPI; ++i) {
+        const int j = tid + i * kBlock;
+        if (j <= rp_n) s_rp[j] = rpv[i] - a;
     }
 
     // ---- the last row may run past the window: finish it with the whole workgroup ----
@@ -179,27 +243,23 @@ __global__ __launch_bounds__(kBlock) void k_spmv_stream(int32_t m, int32_t nbloc
     __syncthreads();
     if (bend > c1) extra = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
 
-    const int32_t last_row = r1 - 1;
-#define ASX_RED(G) stream_reduce_rows<G, T>(s_prod, r0, nrows, a, c1, last_row, extra, alpha, beta, row_ptr, y)
-    if (nrows > 128)
-        ASX_RED(1);
-    else if (nrows > 64)
-        ASX_RED(2);
-    else if (nrows > 32)
-        ASX_RED(4);
-    else if (nrows > 16)
-        ASX_RED(8);
-    else if (nrows > 8)
-        ASX_RED(16);
-    else if (nrows > 4)
-        ASX_RED(32);
-    else
-        ASX_RED(64);
+#define ASX_RED(G) \
+    stream_reduce_rows<G, NT, T>(s_prod, s_rp, r0, nrows, a, n1, extra, alpha, beta, y_first, y_first_ok, row_ptr, y)
+    switch (g_shift) {
+    case 0: ASX_RED(1); break;
+    case 1: ASX_RED(2); break;
+    case 2: ASX_RED(4); break;
+    case 3: ASX_RED(8); break;
+    case 4: ASX_RED(16); break;
+    case 5: ASX_RED(32); break;
+    default: ASX_RED(64); break;
+    }
 #undef ASX_RED
 }
 
-// Row blocks of the stream kernel: blocks[t] = first row whose first stored element lies at or
-// after t*kStreamTile (t < nb), blocks[nb] = m, nb = max(1, ceil(nnz / kStreamTile)).
+// Row blocks of the stream kernel, as (row, row_ptr[row]) pairs: pair t = first row whose first
+// stored element lies at or after t*kStreamTile (t < nb), pair nb = (m, nnz),
+// nb = max(1, ceil(nnz / kStreamTile)).  2*(nb+1) int32, 8-byte aligned.
 __global__ __launch_bounds__(kBlock) void k_stream_row_blocks(const int32_t *__restrict__ row_ptr,
                                                               int32_t m, int32_t nb,
                                                               int32_t *__restrict__ blocks)
@@ -207,7 +267,8 @@ __global__ __launch_bounds__(kBlock) void k_stream_row_blocks(const int32_t *__r
     int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t > nb) return;
     if (t == nb) {
-        blocks[nb] = m;
+        blocks[2 * nb] = m;
+        blocks[2 * nb + 1] = row_ptr[m];
         return;
     }
     const int64_t target = t * kStreamTile;
@@ -219,7 +280,8 @@ __global__ __launch_bounds__(kBlock) void k_stream_row_blocks(const int32_t *__r
         else
             hi = mid;
     }
-    blocks[t] = lo;
+    blocks[2 * t] = lo;
+    blocks[2 * t + 1] = row_ptr[lo];
 }
 
 int launch_stream_row_blocks(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t *d_blocks,
@@ -239,15 +301,19 @@ int launch_spmv_stream(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, 
     if (m <= 0) return ASX_STATUS_SUCCESS;
     int32_t nb = stream_blocks(nnz);
     if (nb < 1) nb = 1;
-    hipLaunchKernelGGL((k_spmv_stream<T>), dim3((unsigned)xcd_grid(nb)), dim3(kBlock), 0, s, m, nb,
-                       alpha, row_ptr, col, val, x, beta, y, blocks);
+    if (use_nontemporal(nnz, sizeof(T)))
+        hipLaunchKernelGGL((k_spmv_stream<T, true>), dim3((unsigned)nb), dim3(kBlock), 0, s, m, nb, alpha,
+                           row_ptr, col, val, x, beta, y, blocks);
+    else
+        hipLaunchKernelGGL((k_spmv_stream<T, false>), dim3((unsigned)nb), dim3(kBlock), 0, s, m, nb, alpha,
+                           row_ptr, col, val, x, beta, y, blocks);
     return check_launch();
 }
 
 // ===========================================================================================
 // merge path
 // ===========================================================================================
-template <typename T>
+template <typename T, bool NT>
 __global__ __launch_bounds__(kBlock) void k_spmv_merge(int32_t m, int32_t nnz, int32_t ntiles, T alpha,
                                                        const int32_t *__restrict__ row_ptr,
                                                        const int32_t *__restrict__ col,
@@ -265,8 +331,7 @@ __global__ __launch_bounds__(kBlock) void k_spmv_merge(int32_t m, int32_t nnz, i
     __shared__ T s_wv[kBlock / kWave];
     __shared__ int32_t s_wk[kBlock / kWave];
 
-    const int b = xcd_contiguous_tile(blockIdx.x, ntiles);
-    if (b >= ntiles) return;
+    const int b = blockIdx.x;
     const int tid = threadIdx.x;
     const int32_t x0 = xs[b], y0 = ys[b], x1 = xs[b + 1], y1 = ys[b + 1];
     const int32_t nr = x1 - x0, nz = y1 - y0, total = nr + nz;
@@ -277,8 +342,8 @@ __global__ __launch_bounds__(kBlock) void k_spmv_merge(int32_t m, int32_t nnz, i
 #pragma unroll
     for (int i = 0; i < IPT; ++i) {
         const int j = tid + i * kBlock;
-        cj[i] = j < nz ? col[(int64_t)y0 + j] : 0;
-        vj[i] = j < nz ? val[(int64_t)y0 + j] : T(0);
+        cj[i] = j < nz ? stream_load<NT>(col + (int64_t)y0 + j) : 0;
+        vj[i] = j < nz ? stream_load<NT>(val + (int64_t)y0 + j) : T(0);
     }
     for (int i = tid; i <= nr; i += kBlock) {
         const int32_t r = x0 + i;
@@ -364,7 +429,7 @@ __global__ __launch_bounds__(kBlock) void k_spmv_merge(int32_t m, int32_t nnz, i
     // ---- finished rows, coalesced ----
     for (int i = tid; i < nr; i += kBlock) {
         const int64_t r = (int64_t)x0 + i;
-        y[r] = axpby_out<T>(alpha, s_val[nz + i], beta, y, r);
+        stream_store<NT>(y + r, axpby_out<T>(alpha, s_val[nz + i], beta, y, r));
     }
 }
 
@@ -393,8 +458,12 @@ int launch_spmv_merge(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, c
 {
     if (m <= 0) return ASX_STATUS_SUCCESS;
     const int32_t ntiles = merge_tiles(m, nnz);
-    hipLaunchKernelGGL((k_spmv_merge<T>), dim3((unsigned)xcd_grid(ntiles)), dim3(kBlock), 0, s, m, nnz,
-                       ntiles, alpha, row_ptr, col, val, x, beta, y, xs, ys, carry);
+    if (use_nontemporal(nnz, sizeof(T)))
+        hipLaunchKernelGGL((k_spmv_merge<T, true>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, m, nnz,
+                           ntiles, alpha, row_ptr, col, val, x, beta, y, xs, ys, carry);
+    else
+        hipLaunchKernelGGL((k_spmv_merge<T, false>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, m, nnz,
+                           ntiles, alpha, row_ptr, col, val, x, beta, y, xs, ys, carry);
     hipLaunchKernelGGL((k_spmv_merge_fixup<T>), dim3((unsigned)ceil_div64(ntiles, kBlock)),
                        dim3(kBlock), 0, s, m, ntiles, alpha, xs, carry, y);
     return check_launch();
