@@ -26,7 +26,12 @@ KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 5: "k
 
 # HBM traffic per call measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; see profiles/),
 # scaled by the same counters' reading for a plain copy of known size.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    "powerlaw_f64": (2034745.4 * 2 + 34144.8) * 1024,    # profiles/spmv_merge_powerlaw_f64.md
+    "stencil5_f64": (694107.6 * 2 + 134039.3) * 1024,    # profiles/spmv_stream_stencil5_f64.md
+    "uniform16_f32": (220068.2 * 2 + 4096.1) * 1024,     # profiles/spmv_stream_uniform16_f32.md
+    "spmm_zipf_f32": (2319893.4 * 2 + 297719.3) * 1024,  # profiles/spmm_merge_spmm_zipf_f32.md
+}
 
 
 def parse():
@@ -39,6 +44,11 @@ def parse():
     ap.add_argument("--alg", type=int, default=0, help="kernel id (0 = pick from the histogram)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
+    ap.add_argument("--probe", action="store_true",
+                    help="only run the stream / stream+gather probes on --workload (what the chip sustains "
+                         "for this matrix without reduction and write)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run the plain copy kernel on 1 GiB (known traffic, for scaling profiler counters)")
     return ap.parse_args()
 
 
@@ -105,6 +115,57 @@ def measure(w, steps, warmup, alg):
     return res
 
 
+def copy_calibration(steps, nbytes=1 << 30):
+    """Plain device copy of nbytes (reads nbytes, writes nbytes): the practical streaming
+    ceiling of this chip, and a launch of known traffic for scaling FETCH_SIZE / WRITE_SIZE."""
+    import torch
+    from library_amd import capi
+    src = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(3):
+        capi.lib().asx_copy_bytes(src.data_ptr(), dst.data_ptr(), nbytes, stream)
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(steps):
+        capi.lib().asx_copy_bytes(src.data_ptr(), dst.data_ptr(), nbytes, stream)
+    e.record()
+    torch.cuda.synchronize()
+    ms = s.elapsed_time(e) / steps
+    return {"copy_bytes_read": nbytes, "copy_bytes_written": nbytes, "ms": ms,
+            "read_plus_write_gbs": 2 * nbytes / (ms * 1e-3) / 1e9}
+
+
+def probe(w, steps):
+    """Stream-only and stream+gather rates for workload w (no reduction, no output)."""
+    import torch
+    from library_amd import capi
+    dev = lambda a: torch.from_numpy(a).cuda()
+    d_col, d_val, d_x = dev(w.col), dev(w.val), dev(w.x)
+    sink = torch.zeros(16, dtype=d_val.dtype, device="cuda")
+    vt = capi.value_type(w.val.dtype)
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {"workload": w.name, "nnz": w.nnz, "stream_bytes": w.nnz * (w.dtype.itemsize + 4)}
+    for mode, key in ((0, "stream"), (1, "stream_gather")):
+        call = lambda: capi.lib().asx_probe_stream_gather(vt, mode, w.nnz, d_col.data_ptr(), d_val.data_ptr(),
+                                                          d_x.data_ptr(), sink.data_ptr(), stream)
+        for _ in range(3):
+            call()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(steps):
+            call()
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e) / steps
+        out[key + "_us"] = ms * 1e3
+        out[key + "_gbs_of_col_val"] = out["stream_bytes"] / (ms * 1e-3) / 1e9
+        out[key + "_gnnz_per_s"] = w.nnz / (ms * 1e-3) / 1e9
+    return out
+
+
 def cpu_baseline(w, budget_s):
     """The reference's own CPU path (oracle/_ref, kind "reference") or, where that is not
     built, the C restatement (kind "port"), timed on this host for the same workload."""
@@ -165,6 +226,12 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     capi.lib()
 
+    if a.calibrate_copy:
+        print(json.dumps(copy_calibration(a.steps)))
+        return
+    if a.probe:
+        print(json.dumps(probe(W.CONFIGS[a.workload](), a.steps)))
+        return
     names = [a.workload] if a.only else ORDER
     results = {}
     head_w = None
@@ -197,6 +264,9 @@ def main():
                      "frac": head["frac_hbm_peak"], "traffic": traffic, "kernel": head["kernel"],
                      "bytes_per_launch": head["bytes"], "launch_ms": head["event_ms_mean"]},
         "cpu_baseline": cpu,
+        "roofline_by_workload": {n: {"kernel": results[n]["kernel"], "achieved": round(results[n]["gbs_event"], 1),
+                                     "frac": round(results[n]["frac_hbm_peak"], 4),
+                                     "traffic": MEASURED_TRAFFIC_BYTES.get(n)} for n in names},
         "workloads": [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in results[n].items()} for n in names],
     }
     print(json.dumps(line))

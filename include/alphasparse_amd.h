@@ -185,6 +185,11 @@ int asx_spmm_csr_f64(const asx_plan *plan, int alg, int32_t m, int32_t k, int32_
  * ---------------------------------------------------------------------------------- */
 /* A coalesced copy kernel of `bytes` bytes (multiple of 16): calibration for bandwidth counters. */
 int asx_copy_bytes(const void *d_src, void *d_dst, size_t bytes, void *stream);
+/* The memory side of a CSR SpMV without reduction and without output: mode 0 streams d_col and
+ * d_val only, mode 1 also gathers d_x[col].  Gives the rates the chip sustains for a given
+ * column pattern.  d_sink: one value of the value type (never written in practice). */
+int asx_probe_stream_gather(int value_type, int mode, int64_t nnz, const int32_t *d_col,
+                            const void *d_val, const void *d_x, void *d_sink, void *stream);
 
 #ifdef __cplusplus
 }
