@@ -22,7 +22,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 ORDER = ["banded_f64", "uniform16_f32", "powerlaw_f64", "stencil5_f64", "spmm_zipf_f32"]
-KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 5: "k_spmm_row", 7: "k_spmm_merge"}
+EXTRA = ["spmm_banded_f32"]  # not a BASELINE configuration: dense-block matrix for the MFMA SpMM variant
+KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 5: "k_spmm_row", 7: "k_spmm_merge",
+                10: "k_spmm_blocked"}
 
 # HBM traffic per call measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; see profiles/),
 # scaled by the same counters' reading for a plain copy of known size.  None = not measured.
@@ -39,7 +41,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="powerlaw_f64", choices=ORDER)
+    ap.add_argument("--workload", default="powerlaw_f64", choices=ORDER + EXTRA)
     ap.add_argument("--only", action="store_true", help="measure only --workload")
     ap.add_argument("--alg", type=int, default=0, help="kernel id (0 = pick from the histogram)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -64,7 +66,7 @@ def measure(w, steps, warmup, alg):
     spmm = w.kind == "spmm"
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    plan = capi.Plan(spmm, alg, w.val.dtype, w.m, w.n, w.nnz, d_rp, ncols=w.ncols)
+    plan = capi.Plan(spmm, alg, w.val.dtype, w.m, w.n, w.nnz, d_rp, ncols=w.ncols, col=d_col, val=d_val)
     torch.cuda.synchronize()
     analysis_ms = (time.perf_counter() - t0) * 1e3
     ws = torch.empty(max(plan.workspace_bytes, 256), dtype=torch.uint8, device="cuda")
@@ -232,7 +234,7 @@ def main():
     if a.probe:
         print(json.dumps(probe(W.CONFIGS[a.workload](), a.steps)))
         return
-    names = [a.workload] if a.only else ORDER
+    names = [a.workload] if (a.only or a.workload in EXTRA) else ORDER
     results = {}
     head_w = None
     for name in names:

@@ -56,7 +56,7 @@ enum {
     ASX_SPMM_DEFAULT = 0,
     ASX_SPMM_ROW = 5,    /* CSR_ALG1: one wave per (row, 64-column tile) */
     ASX_SPMM_MERGE = 7,  /* CSR_ALG3: merge-path segments per wave + ordered carry fix-up */
-    ASX_SPMM_BLOCKED = 10 /* CSR_ALG6: 16x4-blocked MFMA variant (needs a plan) */
+    ASX_SPMM_BLOCKED = 10 /* CSR_ALG6: 16x4-blocked MFMA variant (needs asx_spmm_plan_create) */
 };
 
 /* ------------------------------------------------------------------------------------
@@ -131,6 +131,17 @@ typedef struct asx_plan asx_plan;
  * synchronous copy) and picks a kernel.  Synchronises `stream` before returning. */
 int asx_plan_create(asx_plan **plan, int is_spmm, int alg, int value_type, int32_t m, int32_t n,
                     int32_t nnz, const int32_t *d_row_ptr, int32_t ncols_dense, void *stream);
+/* SpMM plan that may look at A's columns and values.  alg = ASX_SPMM_BLOCKED re-tiles A into
+ * zero-filled 16x4 blocks for the MFMA kernel (tc_preprocess,
+ * hip/kernel/level3/alphasparse_spmm_tc4csr.h:38-153; the plan then holds a COPY of the values:
+ * rebuild it when they change).  alg = ASX_SPMM_DEFAULT measures the block fill
+ * nnz / (64 * blocks) and picks the blocked kernel when it is at least 1/8, else the merge
+ * kernel.  Other algorithms behave as asx_plan_create.  Synchronises `stream`. */
+int asx_spmm_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, int32_t k, int32_t nnz,
+                         const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, int32_t ncols,
+                         void *stream);
+/* Number of 16x4 blocks and their fill of a blocked plan. */
+int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill);
 int asx_plan_destroy(asx_plan *plan);
 /* Kernel the plan resolved to, and bytes of per-call workspace its launches need. */
 int asx_plan_alg(const asx_plan *plan);

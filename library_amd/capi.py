@@ -26,7 +26,7 @@ EXPORTS = [
     "asx_version", "asx_device_info", "asx_row_length_histogram", "asx_partition_rows_by_nnz",
     "asx_nnz_split_rows", "asx_merge_path_search", "asx_loadbalance_nwarps",
     "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_plan_create",
-    "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
+    "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
     "asx_spmm_resolve_alg", "asx_spmm_workspace_bytes", "asx_spmm_csr_f32", "asx_spmm_csr_f64",
     "asx_copy_bytes", "asx_probe_stream_gather",
@@ -61,6 +61,8 @@ def lib():
     L.asx_loadbalance_partition.argtypes = [vp, i32, i32, i32, i32, vp, vp]
     L.asx_csr_adaptive_row_blocks.argtypes = [vp, i32, vp, sz, C.POINTER(sz)]
     L.asx_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, C.c_int, i32, i32, i32, vp, i32, vp]
+    L.asx_spmm_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, i32, i32, i32, vp, vp, vp, i32, vp]
+    L.asx_plan_block_stats.argtypes = [vp, C.POINTER(i64), C.POINTER(C.c_double)]
     L.asx_plan_destroy.argtypes = [vp]
     L.asx_plan_alg.argtypes = [vp]
     L.asx_plan_workspace_bytes.argtypes = [vp]
@@ -166,11 +168,21 @@ def csr_adaptive_row_blocks(row_ptr_host):
 
 # ------------------------------------------------------------------------------ plans
 class Plan:
-    def __init__(self, is_spmm, alg, dtype, m, n, nnz, row_ptr, ncols=1):
+    def __init__(self, is_spmm, alg, dtype, m, n, nnz, row_ptr, ncols=1, col=None, val=None):
         h = C.c_void_p()
-        _check(lib().asx_plan_create(C.byref(h), int(is_spmm), alg, value_type(dtype), m, n, nnz, _ptr(row_ptr), ncols, _stream()), "asx_plan_create")
+        if is_spmm and col is not None and val is not None:
+            _check(lib().asx_spmm_plan_create(C.byref(h), alg, value_type(dtype), m, n, nnz, _ptr(row_ptr), _ptr(col),
+                                              _ptr(val), ncols, _stream()), "asx_spmm_plan_create")
+        else:
+            _check(lib().asx_plan_create(C.byref(h), int(is_spmm), alg, value_type(dtype), m, n, nnz, _ptr(row_ptr),
+                                         ncols, _stream()), "asx_plan_create")
         self.h = h
-        self._row_ptr = row_ptr  # keep alive
+        self._keep = (row_ptr, col, val)  # keep alive
+
+    def block_stats(self):
+        n, f = C.c_int64(0), C.c_double(0.0)
+        _check(lib().asx_plan_block_stats(self.h, C.byref(n), C.byref(f)), "asx_plan_block_stats")
+        return n.value, f.value
 
     @property
     def alg(self):

@@ -430,9 +430,11 @@ alphasparseStatus_t alphasparseSpMM_bufferSize(alphasparseHandle_t handle, alpha
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
-// Builds and keeps the split points for (matA, N = matC->cols, alg).  *bufferSize, when given,
-// receives the workspace a later alphasparseSpMM call needs (never more than
-// alphasparseSpMM_bufferSize reports).
+// Builds and keeps the analysis for (matA, N = matC->cols, alg): merge split points, or for
+// ALPHASPARSE_SPMM_CSR_ALG6 (and for DEFAULT when the 16x4 blocks of A are at least 1/8 full) the
+// blocked copy of A for the MFMA kernel, which holds A's values: call again after changing them.
+// *bufferSize, when given, receives the workspace a later alphasparseSpMM call needs (never more
+// than alphasparseSpMM_bufferSize reports).
 alphasparseStatus_t alphasparseSpMM_preprocess(alphasparseHandle_t handle, alphasparseOperation_t opA,
                                                alphasparseOperation_t opB, const void *alpha,
                                                alphasparseSpMatDescr_t matA,
@@ -451,9 +453,9 @@ alphasparseStatus_t alphasparseSpMM_preprocess(alphasparseHandle_t handle, alpha
         HandlePlans *hp = plans_of(handle, true);
         if (!hp) return ALPHA_SPARSE_STATUS_ALLOC_FAILED;
         asx_plan *plan = nullptr;
-        int rc = asx_plan_create(&plan, 1, (int)alg, (int)matA->data_type, (int32_t)matA->rows,
-                                 (int32_t)matA->cols, (int32_t)matA->nnz, matA->row_data, ncols,
-                                 (void *)handle->stream);
+        int rc = asx_spmm_plan_create(&plan, (int)alg, (int)matA->data_type, (int32_t)matA->rows,
+                                      (int32_t)matA->cols, (int32_t)matA->nnz, matA->row_data,
+                                      matA->col_data, matA->val_data, ncols, (void *)handle->stream);
         if (rc) return st(rc);
         hp->plans.push_back(KeptPlan{true, (int)alg, matA->row_data, matA->rows, matA->nnz,
                                      (int)matA->data_type, ncols, plan});

@@ -172,6 +172,10 @@ int spmm_impl(const asx_plan *plan, int alg, int32_t m, int32_t k, int32_t nnz, 
         return launch_spmm_merge<T>(m, nnz, ncols, alpha, row_ptr, col, val, B, ldb, beta, C, ldc, xs,
                                     ys, (T *)(w + L.carry_off), (int32_t *)(w + L.crow_off), s);
     }
+    case ASX_SPMM_BLOCKED:
+        // the blocks hold a copy of A's values and are built by asx_spmm_plan_create
+        if (!plan || !plan->blocked.brow_ptr) return ASX_STATUS_NOT_INITIALIZED;
+        return launch_spmm_blocked<T>(m, k, ncols, alpha, &plan->blocked, B, ldb, beta, C, ldc, s);
     default: return ASX_STATUS_NOT_SUPPORTED;
     }
 }
@@ -325,7 +329,7 @@ int asx_plan_create(asx_plan **out, int is_spmm, int alg, int value_type, int32_
         }
     } else {
         int kernel = asx_spmm_resolve_alg(alg, m, nnz, ncols_dense);
-        if (kernel < 0) {
+        if (kernel < 0 || kernel == ASX_SPMM_BLOCKED) {  // blocked plans need col and val too
             delete p;
             return ASX_STATUS_NOT_SUPPORTED;
         }
@@ -358,8 +362,70 @@ int asx_plan_destroy(asx_plan *plan)
     if (!plan) return ASX_STATUS_SUCCESS;
     int st = ASX_STATUS_SUCCESS;
     if (plan->d_meta) st = status_of(hipFree(plan->d_meta));
+    free_blocked(&plan->blocked);
     delete plan;
     return st;
+}
+
+// Blocks are worth it when they are at least this full (bytes moved per stored element fall
+// below the merge kernel's from about 1/8 upwards, see asx_blocked.hip).
+static const double kBlockedMinFill = 0.125;
+static const int32_t kBlockedProbeMaxNnz = 1 << 28;
+
+int asx_spmm_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int32_t k, int32_t nnz,
+                         const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, int32_t ncols,
+                         void *stream)
+{
+    if (!out) return ASX_STATUS_INVALID_POINTER;
+    *out = nullptr;
+    const int kernel = asx_spmm_resolve_alg(alg, m, nnz, ncols);
+    if (kernel < 0) return ASX_STATUS_NOT_SUPPORTED;
+    const bool want_blocked = kernel == ASX_SPMM_BLOCKED;
+    const bool probe_blocked = alg == ASX_SPMM_DEFAULT && nnz > 0 && nnz <= kBlockedProbeMaxNnz;
+    if (!want_blocked && !probe_blocked)
+        return asx_plan_create(out, 1, alg, value_type, m, k, nnz, d_row_ptr, ncols, stream);
+    if (m < 0 || k < 0 || nnz < 0 || ncols < 1) return ASX_STATUS_INVALID_SIZE;
+    if (value_type != ASX_R_32F && value_type != ASX_R_64F) return ASX_STATUS_NOT_SUPPORTED;
+    if ((m > 0 && !d_row_ptr) || (nnz > 0 && (!d_col || !d_val))) return ASX_STATUS_INVALID_POINTER;
+    hipStream_t s = (hipStream_t)stream;
+    BlockedMatrix bm{};
+    int st = value_type == ASX_R_64F
+                 ? build_blocked<double>(m, k, nnz, d_row_ptr, d_col, (const double *)d_val, &bm, s)
+                 : build_blocked<float>(m, k, nnz, d_row_ptr, d_col, (const float *)d_val, &bm, s);
+    if (st) return st;
+    const double fill = bm.nblocks > 0 ? (double)nnz / (64.0 * (double)bm.nblocks) : 0.0;
+    if (!want_blocked && fill < kBlockedMinFill) {
+        free_blocked(&bm);
+        return asx_plan_create(out, 1, alg, value_type, m, k, nnz, d_row_ptr, ncols, stream);
+    }
+    asx_plan *p = new (std::nothrow) asx_plan();
+    if (!p) {
+        free_blocked(&bm);
+        return ASX_STATUS_ALLOC_FAILED;
+    }
+    std::memset(p, 0, sizeof(*p));
+    p->is_spmm = 1;
+    p->alg = ASX_SPMM_BLOCKED;
+    p->value_type = value_type;
+    p->m = m;
+    p->n = k;
+    p->nnz = nnz;
+    p->ncols = ncols;
+    p->row_ptr = d_row_ptr;
+    p->blocked = bm;
+    p->nunits = bm.nblocks;
+    p->workspace_bytes = 0;
+    *out = p;
+    return ASX_STATUS_SUCCESS;
+}
+
+int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill)
+{
+    if (!plan || !nblocks || !fill) return ASX_STATUS_INVALID_POINTER;
+    if (plan->alg != ASX_SPMM_BLOCKED) return ASX_STATUS_INVALID_VALUE;
+    *nblocks = plan->blocked.nblocks;
+    *fill = plan->blocked.nblocks > 0 ? (double)plan->nnz / (64.0 * (double)plan->blocked.nblocks) : 0.0;
+    return ASX_STATUS_SUCCESS;
 }
 
 int asx_plan_alg(const asx_plan *plan) { return plan ? plan->alg : -1; }
@@ -442,7 +508,8 @@ int asx_spmm_resolve_alg(int alg, int32_t m, int32_t nnz, int32_t ncols)
     case 7:                        /* CSR_ALG3 merge */
     case 8:                        /* CSR_ALG4 adaptive */
     case 9: return ASX_SPMM_MERGE; /* CSR_ALG5 flat */
-    default: return -1;            /* COO algorithms; CSR_ALG6 needs a blocked plan */
+    case 10: return ASX_SPMM_BLOCKED; /* CSR_ALG6: needs a plan from asx_spmm_plan_create */
+    default: return -1;            /* COO algorithms */
     }
 }
 

@@ -71,6 +71,22 @@ int launch_spmm_merge(int32_t m, int32_t nnz, int32_t ncols, T alpha, const int3
                       int64_t ldc, const int32_t *xs, const int32_t *ys, T *carry, int32_t *carry_row,
                       hipStream_t s);
 
+// ---- blocked (MFMA) SpMM (asx_blocked.hip) ----
+struct BlockedMatrix {
+    int32_t nbrows;     // ceil(m / 16)
+    int32_t nblocks;    // non-empty 16x4 blocks
+    int32_t *brow_ptr;  // nbrows + 1
+    int32_t *bcol;      // column quad of each block
+    void *bval;         // nblocks * 64 values, lane order of the MFMA A operand
+};
+template <typename T>
+int build_blocked(int32_t m, int32_t k, int32_t nnz, const int32_t *row_ptr, const int32_t *col,
+                  const T *val, BlockedMatrix *out, hipStream_t s);
+void free_blocked(BlockedMatrix *b);
+template <typename T>
+int launch_spmm_blocked(int32_t m, int32_t k, int32_t ncols, T alpha, const BlockedMatrix *bm, const T *B,
+                        int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t s);
+
 inline int32_t merge_tiles(int32_t m, int32_t nnz) { return (int32_t)ceil_div64((int64_t)m + nnz, kMergeTile); }
 inline int32_t stream_blocks(int32_t nnz) { return (int32_t)ceil_div64(nnz, kStreamTile); }
 inline int32_t spmm_segments(int32_t m, int32_t nnz) { return (int32_t)ceil_div64((int64_t)m + nnz, kSpmmSegment); }
@@ -90,4 +106,5 @@ struct asx_plan {
     int64_t hist[33];
     int64_t stats[4];
     size_t workspace_bytes;
+    asx::BlockedMatrix blocked;  // only for ASX_SPMM_BLOCKED plans
 };

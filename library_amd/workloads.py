@@ -182,10 +182,20 @@ def spmm_zipf_f32(m=1 << 20, ncols=64, max_len=50000, seed=0, scale=SPMM_ZIPF_SC
                     1.0, B, Cm, ncols, {"scale": scale})
 
 
+def spmm_banded_f32(m=1 << 20, half_bw=32, ncols=64, seed=0):
+    """Not a BASELINE configuration: a banded A (dense 16x4 blocks) for the blocked MFMA SpMM."""
+    rp, col, val = csr_banded(m, half_bw, np.float32, seed)
+    B = uniform(m * ncols, np.float32, -1.0, 1.0, seed, S_B)
+    Cm = uniform(m * ncols, np.float32, -1.0, 1.0, seed, S_C)
+    return Workload("spmm_banded_f32", "spmm", np.dtype(np.float32), m, m, int(rp[-1]), rp, col, val, 1.0,
+                    1.0, B, Cm, ncols, {"half_bw": half_bw})
+
+
 CONFIGS = {
     "banded_f64": banded_f64,
     "uniform16_f32": uniform16_f32,
     "powerlaw_f64": powerlaw_f64,
     "stencil5_f64": stencil5_f64,
     "spmm_zipf_f32": spmm_zipf_f32,
+    "spmm_banded_f32": spmm_banded_f32,
 }

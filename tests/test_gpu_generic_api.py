@@ -59,6 +59,6 @@ def test_spmm_through_generic_api(tmp_path, oracle):
     alpha, beta = 2.0, 3.0  # hip/test/level3/spmm_csr_row_r_f32_test.hip:45-46
     ref = oracle.spmm(rp, col, val, B, n, alpha, beta, C0, 4)
     scale = spmm_scale(rp, col, val, B, n, alpha, beta, C0)
-    for alg, analysis in ((0, 0), (0, 1), (5, 0), (6, 0), (7, 1), (8, 0), (9, 0)):
+    for alg, analysis in ((0, 0), (0, 1), (5, 0), (6, 0), (7, 1), (8, 0), (9, 0), (10, 1)):
         got = _run_case(tmp_path, "spmm", np.float32, rp, col, val, B, C0, n, alg, alpha, beta, analysis)
         assert_close(got, ref, scale, np.float32, f"spmm alg {alg} analysis {analysis}")

@@ -336,3 +336,69 @@ def test_benchmark_configs_full_size(torch, capi, oracle):
     scale = spmm_scale(w.row_ptr, w.col, w.val, w.x, w.ncols, w.alpha, w.beta, w.y)
     got = run_spmm(torch, capi, w.row_ptr, w.col, w.val, w.x, w.y, w.ncols, w.alpha, w.beta, capi.SPMM_DEFAULT, True)
     assert_close(got, ref, scale, np.float32, "spmm_zipf_f32")
+
+
+# ------------------------------------------------------------------ blocked (MFMA) SpMM
+def _block_structured(rng, m, k, dtype, density=0.7):
+    """Rows in groups of 16 share column quads: most 16x4 blocks are well filled."""
+    rows, cols = [], []
+    for br in range((m + 15) // 16):
+        nq = (k + 3) // 4
+        quads = rng.choice(nq, size=min(nq, int(rng.integers(1, 6))), replace=False)
+        for r in range(br * 16, min(br * 16 + 16, m)):
+            for q in quads:
+                for c in range(q * 4, min(q * 4 + 4, k)):
+                    if rng.random() < density:
+                        rows.append(r)
+                        cols.append(c)
+    import scipy.sparse as sp
+    A = sp.csr_matrix((rng.uniform(-1, 1, len(rows)).astype(dtype), (rows, cols)), shape=(m, k))
+    A.sort_indices()
+    return A.indptr.astype(np.int32), A.indices.astype(np.int32), A.data.astype(dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_spmm_blocked_mfma(torch, capi, oracle, dtype):
+    rng = np.random.default_rng(61)
+    for m, k in ((1000, 1003), (16, 4), (37, 9), (4096, 2048)):
+        rp, col, val = _block_structured(rng, m, k, dtype)
+        d = [dev(torch, a) for a in (rp, col, val)]
+        for n in (64, 16, 7, 130):
+            B = rng.uniform(-1, 1, k * n).astype(dtype)
+            C0 = rng.uniform(-1, 1, m * n).astype(dtype)
+            plan = capi.Plan(True, capi.SPMM_BLOCKED, np.dtype(dtype), m, k, col.size, d[0], ncols=n, col=d[1], val=d[2])
+            assert plan.alg == capi.SPMM_BLOCKED
+            nblocks, fill = plan.block_stats()
+            keys = np.unique((np.repeat(np.arange(m), np.diff(rp)) // 16).astype(np.int64) * (1 << 31) + col // 4)
+            assert nblocks == keys.size and abs(fill - col.size / (64.0 * keys.size)) < 1e-12
+            for alpha, beta in ((1.0, 1.0), (2.0, 0.0)):
+                ref = oracle.spmm(rp, col, val, B, n, alpha, beta, C0, 4)
+                scale = spmm_scale(rp, col, val, B, n, alpha, beta, C0)
+                Cm = dev(torch, C0)
+                capi.spmm(d[0], d[1], d[2], dev(torch, B), Cm, n, alpha, beta, alg=capi.SPMM_BLOCKED, plan=plan, k=k)
+                torch.cuda.synchronize()
+                assert_close(Cm.cpu().numpy(), ref, scale, dtype, f"blocked m={m} k={k} n={n} a={alpha} b={beta}")
+            plan.destroy()
+
+
+def test_spmm_default_picks_blocked_only_for_dense_blocks(torch, capi, oracle):
+    rng = np.random.default_rng(62)
+    # dense blocks: DEFAULT -> MFMA kernel
+    rp, col, val = _block_structured(rng, 2048, 2048, np.float32, density=0.9)
+    d = [dev(torch, a) for a in (rp, col, val)]
+    plan = capi.Plan(True, capi.SPMM_DEFAULT, np.dtype(np.float32), 2048, 2048, col.size, d[0], ncols=64, col=d[1], val=d[2])
+    assert plan.alg == capi.SPMM_BLOCKED and plan.block_stats()[1] > 0.5
+    plan.destroy()
+    # uniform random columns: blocks hold ~1 element, DEFAULT -> merge kernel
+    lens = rng.integers(1, 20, 3000)
+    rp, col, val = csr_from_lengths(lens, 100000, 9, np.float32)
+    d = [dev(torch, a) for a in (rp, col, val)]
+    plan = capi.Plan(True, capi.SPMM_DEFAULT, np.dtype(np.float32), 3000, 100000, col.size, d[0], ncols=64, col=d[1], val=d[2])
+    assert plan.alg == capi.SPMM_MERGE
+    plan.destroy()
+    # asking for the blocked kernel without its plan is an error, not a silent fallback
+    B = dev(torch, np.zeros(100000 * 64, dtype=np.float32))
+    Cm = dev(torch, np.zeros(3000 * 64, dtype=np.float32))
+    with pytest.raises(capi.AsxError) as e:
+        capi.spmm(d[0], d[1], d[2], B, Cm, 64, 1.0, 0.0, alg=capi.SPMM_BLOCKED, k=100000)
+    assert e.value.code == 1
