@@ -272,6 +272,13 @@ alphasparseStatus_t alphasparseCreateCsr(alphasparseSpMatDescr_t *spMatDescr, co
                                        (void *)val_data, csrRowOffsetsType, csrColIndType, idxBase,
                                        valueType);
 }
+// COO row indices (sorted) -> CSR row offsets, device arrays (hip/format/coo2csr.h:7-16).
+template <typename T>
+alphasparseStatus_t alphasparseXcoo2csr(const int *row_data, int nnz, int m, T *csrRowPtr)
+{
+    static_assert(sizeof(T) == sizeof(int32_t), "32-bit row offsets only");
+    return (alphasparseStatus_t)asx_coo2csr(row_data, nnz, m, (int32_t *)csrRowPtr, nullptr);
+}
 // Extensions: the reference has no way to release these descriptors (they leak there).
 alphasparseStatus_t alphasparseDestroySpMat(alphasparseSpMatDescr_t descr);
 alphasparseStatus_t alphasparseDestroyDnVec(alphasparseDnVecDescr_t descr);

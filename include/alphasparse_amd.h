@@ -117,6 +117,16 @@ int asx_loadbalance_partition(const int32_t *d_row_ptr, int32_t m, int32_t nnz, 
 int asx_csr_adaptive_row_blocks(const int32_t *h_row_ptr, int32_t m, uint64_t *h_out, size_t cap,
                                 size_t *count);
 
+/* COO -> CSR row offsets from row indices sorted ascending: d_row_ptr[r] = first i with
+ * d_row_ind[i] >= r, r in [0, m].  alphasparseXcoo2csr, hip/format/coo2csr.h:7-16 (which
+ * forwards to hipsparseXcoo2csr). */
+int asx_coo2csr(const int32_t *d_row_ind, int32_t nnz, int32_t m, int32_t *d_row_ptr, void *stream);
+/* Sorts device COO triplets by (row, column) in place (stable for equal keys).  Device twin of
+ * the host qsort in coo_order, hip/format/coo_order.h:24-43.  Allocates temporaries and
+ * synchronises `stream`. */
+int asx_coo_sort(int value_type, int32_t *d_row_ind, int32_t *d_col_ind, void *d_val, int32_t nnz,
+                 void *stream);
+
 /* ------------------------------------------------------------------------------------
  * Plans: analysis results kept across calls (the reference recomputes them inside every
  * SpMV/SpMM call; its alphasparseSpMV_analysis is a stub, hip/kernel/level2/alphasparse_spmv.hip:

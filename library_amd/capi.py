@@ -25,7 +25,7 @@ STATUS = {0: "SUCCESS", 1: "NOT_INITIALIZED", 2: "ALLOC_FAILED", 3: "INVALID_VAL
 EXPORTS = [
     "asx_version", "asx_device_info", "asx_row_length_histogram", "asx_partition_rows_by_nnz",
     "asx_nnz_split_rows", "asx_merge_path_search", "asx_loadbalance_nwarps",
-    "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_plan_create",
+    "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_coo2csr", "asx_coo_sort", "asx_plan_create",
     "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
     "asx_spmm_resolve_alg", "asx_spmm_workspace_bytes", "asx_spmm_csr_f32", "asx_spmm_csr_f64",
@@ -60,6 +60,8 @@ def lib():
     L.asx_loadbalance_nwarps.restype = i64
     L.asx_loadbalance_partition.argtypes = [vp, i32, i32, i32, i32, vp, vp]
     L.asx_csr_adaptive_row_blocks.argtypes = [vp, i32, vp, sz, C.POINTER(sz)]
+    L.asx_coo2csr.argtypes = [vp, i32, i32, vp, vp]
+    L.asx_coo_sort.argtypes = [C.c_int, vp, vp, vp, i32, vp]
     L.asx_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, C.c_int, i32, i32, i32, vp, i32, vp]
     L.asx_spmm_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, i32, i32, i32, vp, vp, vp, i32, vp]
     L.asx_plan_block_stats.argtypes = [vp, C.POINTER(i64), C.POINTER(C.c_double)]
@@ -151,6 +153,18 @@ def loadbalance_partition(row_ptr, nnz, warp_size, nwarps):
     out = torch.empty(max(nwarps, 1), dtype=torch.int32, device=row_ptr.device)
     _check(lib().asx_loadbalance_partition(_ptr(row_ptr), m, nnz, warp_size, nwarps, _ptr(out), _stream()), "asx_loadbalance_partition")
     return out[:nwarps]
+
+
+def coo2csr(row_ind, m):
+    import torch
+    out = torch.empty(m + 1, dtype=torch.int32, device=row_ind.device)
+    _check(lib().asx_coo2csr(_ptr(row_ind), row_ind.numel(), m, _ptr(out), _stream()), "asx_coo2csr")
+    return out
+
+
+def coo_sort(row_ind, col_ind, val):
+    _check(lib().asx_coo_sort(value_type(val.dtype), _ptr(row_ind), _ptr(col_ind), _ptr(val), row_ind.numel(), _stream()),
+           "asx_coo_sort")
 
 
 def csr_adaptive_row_blocks(row_ptr_host):

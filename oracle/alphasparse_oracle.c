@@ -425,3 +425,15 @@ size_t orc_csr_adaptive_row_blocks(const int32_t *row_ptr, int32_t m, uint64_t *
 #undef TAG_PREV
     return n;
 }
+
+/* ---- hip/format/coo2csr.h:7-16 -> hipsparseXcoo2csr: counting form of the contract ---- */
+void orc_coo2csr(const int32_t *row_ind, int32_t nnz, int32_t m, int32_t *row_ptr)
+{
+    for (int32_t r = 0; r <= m; ++r)
+        row_ptr[r] = 0;
+    for (int32_t i = 0; i < nnz; ++i)
+        if (row_ind[i] >= 0 && row_ind[i] < m)
+            row_ptr[row_ind[i] + 1]++;
+    for (int32_t r = 0; r < m; ++r)
+        row_ptr[r + 1] += row_ptr[r];
+}

@@ -18,6 +18,7 @@
  *   orc_find_rows_counts        brute force
  *   orc_csr_adaptive_row_blocks bit-exact vs the reference's host routine compiled from its header
  *                               (oracle/_ref) + golden fixtures
+ *   orc_coo2csr                 numpy searchsorted / bincount (the reference forwards to hipSPARSE)
  */
 #ifndef ALPHASPARSE_ORACLE_H
 #define ALPHASPARSE_ORACLE_H
@@ -83,6 +84,11 @@ void orc_find_rows_counts(const int32_t *row_ptr, int32_t m, int32_t thr1, int32
  * include/alphasparse/common.h:12-20,192-200.  Returns the number of entries written
  * (the reference reports twice that as its array size).  cap = capacity of out. */
 size_t orc_csr_adaptive_row_blocks(const int32_t *row_ptr, int32_t m, uint64_t *out, size_t cap);
+
+/* hip/format/coo2csr.h:7-16 forwards to hipsparseXcoo2csr (hipSPARSE, a system install the
+ * reference does not pin and that is not part of its tree).  Its documented contract, restated:
+ * for row indices sorted ascending, row_ptr[r] = number of entries with row index < r. */
+void orc_coo2csr(const int32_t *row_ind, int32_t nnz, int32_t m, int32_t *row_ptr);
 
 #ifdef __cplusplus
 }

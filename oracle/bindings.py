@@ -51,6 +51,8 @@ class Oracle:
         L.orc_find_rows_counts.argtypes = [i32p, C.c_int32, C.c_int32, C.c_int32, i32p, C.POINTER(C.c_int64)]
         L.orc_csr_adaptive_row_blocks.argtypes = [i32p, C.c_int32, u64p, C.c_size_t]
         L.orc_csr_adaptive_row_blocks.restype = C.c_size_t
+        L.orc_coo2csr.argtypes = [i32p, C.c_int32, C.c_int32, i32p]
+        L.orc_coo2csr.restype = None
         for name in ("orc_partition_rows_by_nnz", "orc_spmv_csr_f64", "orc_spmv_csr_f32",
                      "orc_spmm_csr_row_f32", "orc_spmm_csr_row_f64", "orc_nnz_split_rows",
                      "orc_merge_path_search", "orc_loadbalance_partition", "orc_find_rows_counts"):
@@ -108,6 +110,12 @@ class Oracle:
         n = self.L.orc_csr_adaptive_row_blocks(_p(row_ptr, C.c_int32), m, _p(out, C.c_uint64), cap)
         assert n <= cap
         return out[:n].copy()
+
+    def coo2csr(self, row_ind, m):
+        row_ind = _i32(row_ind)
+        out = np.empty(m + 1, dtype=np.int32)
+        self.L.orc_coo2csr(_p(row_ind, C.c_int32), row_ind.size, m, _p(out, C.c_int32))
+        return out
 
     # ---- values ----
     def spmv(self, row_ptr, col, val, x, alpha, beta, y, nthreads=1):

@@ -402,3 +402,23 @@ def test_spmm_default_picks_blocked_only_for_dense_blocks(torch, capi, oracle):
     with pytest.raises(capi.AsxError) as e:
         capi.spmm(d[0], d[1], d[2], B, Cm, 64, 1.0, 0.0, alg=capi.SPMM_BLOCKED, k=100000)
     assert e.value.code == 1
+
+
+# ------------------------------------------------------------------ COO -> CSR
+def test_coo_sort_and_coo2csr(torch, capi, oracle):
+    rng = np.random.default_rng(71)
+    for name, lens in analysis_shapes().items():
+        ncols = int(max(np.max(lens), 64)) + 3
+        rp, col, val = csr_from_lengths(lens, ncols, 11, np.float64)
+        m = rp.size - 1
+        row_ind = np.repeat(np.arange(m, dtype=np.int32), np.diff(rp))
+        assert np.array_equal(capi.coo2csr(dev(torch, row_ind), m).cpu().numpy(), oracle.coo2csr(row_ind, m)), name
+        if col.size == 0:
+            continue
+        perm = rng.permutation(col.size)
+        for dtype in (np.float64, np.float32):
+            r, c, v = dev(torch, row_ind[perm]), dev(torch, col[perm]), dev(torch, val[perm].astype(dtype))
+            capi.coo_sort(r, c, v)
+            torch.cuda.synchronize()
+            assert np.array_equal(r.cpu().numpy(), row_ind) and np.array_equal(c.cpu().numpy(), col)
+            assert np.array_equal(v.cpu().numpy(), val.astype(dtype))

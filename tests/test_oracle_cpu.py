@@ -318,3 +318,14 @@ def test_find_rows_brute_force(oracle):
         lens = np.asarray(lens)
         assert list(counts) == [int((lens < 2).sum()), int(((lens >= 2) & (lens < 1024)).sum()), int((lens >= 1024).sum())]
         assert mid == int(lens[(lens >= 2) & (lens < 1024)].sum())
+
+
+def test_coo2csr_against_numpy(oracle):
+    rng = np.random.default_rng(3)
+    for name, lens in analysis_shapes().items():
+        rp = row_ptr_from_lengths(lens)
+        m = rp.size - 1
+        row_ind = np.repeat(np.arange(m, dtype=np.int32), np.diff(rp))
+        got = oracle.coo2csr(row_ind, m)
+        assert np.array_equal(got, rp), name
+        assert np.array_equal(got, np.searchsorted(row_ind, np.arange(m + 1), side="left").astype(np.int32))
