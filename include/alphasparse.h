@@ -134,6 +134,25 @@ typedef enum {  // spdef.h:390-402
 
 typedef enum { ALPHASPARSE_DIRECTION_ROW = 0, ALPHASPARSE_DIRECTION_COLUMN = 1 } alphasparseDirection_t;
 
+typedef enum {  // spdef.h:175-184
+    ALPHA_SPARSE_DATATYPE_FLOAT = 0,
+    ALPHA_SPARSE_DATATYPE_DOUBLE = 1,
+    ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX = 2,
+    ALPHA_SPARSE_DATATYPE_DOUBLE_COMPLEX = 3,
+    ALPHA_SPARSE_DATATYPE_HALF_FLOAT = 4,
+    ALPHA_SPARSE_DATATYPE_HALF_DOUBLE = 5,
+    ALPHA_SPARSE_DATATYPE_HALF_FLOAT_COMPLEX = 6,
+    ALPHA_SPARSE_DATATYPE_HALF_DOUBLE_COMPLEX = 7
+} alphasparse_datatype_t;
+
+typedef enum {  // spdef.h:560-566
+    ALPHA_SPARSE_DCU_SPMV_ALG_DEFAULT = 0,
+    ALPHA_SPARSE_DCU_SPMV_ALG_COO = 1,
+    ALPHA_SPARSE_DCU_SPMV_ALG_CSR_ADAPTIVE = 2,
+    ALPHA_SPARSE_DCU_SPMV_ALG_CSR_STREAM = 3,
+    ALPHA_SPARSE_DCU_SPMV_ALG_ELL = 4
+} alphasparse_dcu_spmv_alg_t;
+
 // ---- handle (include/alphasparse/handle.h:26-87) ---------------------------------------------
 typedef struct alphasparse_handle_s {
     int device;
@@ -299,6 +318,16 @@ alphasparseStatus_t alphasparseSpMV_bufferSize(alphasparseHandle_t handle, alpha
 alphasparseStatus_t alphasparseSpMV_analysis(alphasparseHandle_t handle, alphasparseOperation_t opA,
                                              alphasparseSpMatDescr_t matA, alphasparseSpMVAlg_t alg);
 alphasparseStatus_t alphasparseSpMV_clear(alphasparseHandle_t handle, alphasparseSpMVAlg_t alg);
+
+// The two-phase form declared (and never defined) in include/alphasparse/spapi_dcu.h:4440-4450:
+// with temp_buffer == nullptr only *buffer_size is written; otherwise the product is computed
+// with temp_buffer as workspace.
+alphasparseStatus_t alphasparse_spmv(alphasparseHandle_t handle, alphasparseOperation_t trans,
+                                     const void *alpha, const alphasparseSpMatDescr_t mat,
+                                     const alphasparseDnVecDescr_t x, const void *beta,
+                                     const alphasparseDnVecDescr_t y, alphasparse_datatype_t compute_type,
+                                     alphasparse_dcu_spmv_alg_t alg, size_t *buffer_size,
+                                     void *temp_buffer);
 
 // ---- generic SpMM (include/alphasparse/spapi.h:6963-6974,7004-7028) ------------------------------
 alphasparseStatus_t alphasparseSpMM(alphasparseHandle_t handle, alphasparseOperation_t opA,

@@ -411,6 +411,28 @@ alphasparseStatus_t alphasparseSpMV(alphasparseHandle_t handle, alphasparseOpera
     return st(rc);
 }
 
+alphasparseStatus_t alphasparse_spmv(alphasparseHandle_t handle, alphasparseOperation_t trans,
+                                     const void *alpha, const alphasparseSpMatDescr_t mat,
+                                     const alphasparseDnVecDescr_t x, const void *beta,
+                                     const alphasparseDnVecDescr_t y, alphasparse_datatype_t compute_type,
+                                     alphasparse_dcu_spmv_alg_t alg, size_t *buffer_size,
+                                     void *temp_buffer)
+{
+    alphasparseDataType ct;
+    switch (compute_type) {
+    case ALPHA_SPARSE_DATATYPE_FLOAT: ct = ALPHA_R_32F; break;
+    case ALPHA_SPARSE_DATATYPE_DOUBLE: ct = ALPHA_R_64F; break;
+    default: return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    // the five ids of this enumeration carry the same values in alphasparseSpMVAlg_t
+    const alphasparseSpMVAlg_t a = (alphasparseSpMVAlg_t)(int)alg;
+    if (temp_buffer == nullptr) {
+        if (!buffer_size) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+        return alphasparseSpMV_bufferSize(handle, trans, alpha, mat, x, beta, y, ct, a, buffer_size);
+    }
+    return alphasparseSpMV(handle, trans, alpha, mat, x, beta, y, ct, a, temp_buffer);
+}
+
 // ------------------------------------------------------------------------------------ SpMM
 alphasparseStatus_t alphasparseSpMM_bufferSize(alphasparseHandle_t handle, alphasparseOperation_t opA,
                                                alphasparseOperation_t opB, const void *alpha,

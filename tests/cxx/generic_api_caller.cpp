@@ -183,6 +183,36 @@ static int selftest()
     HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
     EXPECT(y[0] == 42.5 && y[1] == 65.0);
     EXPECT(alphasparseSpMV_clear(h, ALPHA_SPARSE_SPMV_ALG_DEFAULT) == 0);
+    // two-phase form: size query, then compute
+    {
+        size_t need = 0;
+        EXPECT(alphasparse_spmv(h, N, &alpha, A, X, &beta, Y, ALPHA_SPARSE_DATATYPE_DOUBLE,
+                                ALPHA_SPARSE_DCU_SPMV_ALG_CSR_ADAPTIVE, &need, nullptr) == 0);
+        void *tb = nullptr;
+        HIP_OK(hipMalloc(&tb, need ? need : 1));
+        HIP_OK(hipMemcpy(d_y, x.data(), sizeof(double) * 2, hipMemcpyHostToDevice));
+        EXPECT(alphasparse_spmv(h, N, &alpha, A, X, &beta, Y, ALPHA_SPARSE_DATATYPE_DOUBLE,
+                                ALPHA_SPARSE_DCU_SPMV_ALG_CSR_ADAPTIVE, &need, tb) == 0);
+        HIP_OK(hipDeviceSynchronize());
+        HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
+        EXPECT(y[0] == 42.5 && y[1] == 65.0);
+        EXPECT(alphasparse_spmv(h, N, &alpha, A, X, &beta, Y, ALPHA_SPARSE_DATATYPE_FLOAT_COMPLEX,
+                                ALPHA_SPARSE_DCU_SPMV_ALG_DEFAULT, &need, nullptr) == ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
+        (void)hipFree(tb);
+    }
+    // COO -> CSR through the reference's name
+    {
+        std::vector<int> ri = {0, 0, 1};
+        int *d_ri = to_device(ri), *d_out = nullptr;
+        HIP_OK(hipMalloc((void **)&d_out, 3 * sizeof(int)));
+        EXPECT(alphasparseXcoo2csr(d_ri, 3, 2, d_out) == 0);
+        HIP_OK(hipDeviceSynchronize());
+        int out[3];
+        HIP_OK(hipMemcpy(out, d_out, sizeof out, hipMemcpyDeviceToHost));
+        EXPECT(out[0] == 0 && out[1] == 2 && out[2] == 3);
+        (void)hipFree(d_ri);
+        (void)hipFree(d_out);
+    }
     // SpMM: column-major operands are refused, row-major run
     alphasparseDnMatDescr_t B, C, Bc;
     EXPECT(alphasparseCreateDnMat(&B, 2, 1, 1, d_x, ALPHA_R_64F, ALPHASPARSE_ORDER_ROW) == 0);

@@ -26,6 +26,7 @@ MANGLED = [
     "_Z21alphasparseSpMV_clearP20alphasparse_handle_s20alphasparseSpMVAlg_t",
     "_Z26alphasparseSpMM_bufferSizeP20alphasparse_handle_s22alphasparseOperation_tS1_PKvP22_alphasparseSpMatDescrP24_alphasparse_dnmat_descrS3_S7_19alphasparseDataType20alphasparseSpMMAlg_tPm",
     "_Z26alphasparseSpMM_preprocessP20alphasparse_handle_s22alphasparseOperation_tS1_PKvP22_alphasparseSpMatDescrP24_alphasparse_dnmat_descrS3_S7_19alphasparseDataType20alphasparseSpMMAlg_tPm",
+    "_Z16alphasparse_spmvP20alphasparse_handle_s22alphasparseOperation_tPKvP22_alphasparseSpMatDescrP24_alphasparse_dnvec_descrS3_S7_22alphasparse_datatype_t26alphasparse_dcu_spmv_alg_tPmPv",
     "_Z15alphasparseSpMMP20alphasparse_handle_s22alphasparseOperation_tS1_PKvP22_alphasparseSpMatDescrP24_alphasparse_dnmat_descrS3_S7_19alphasparseDataType20alphasparseSpMMAlg_tPv",
 ]
 
