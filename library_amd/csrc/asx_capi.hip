@@ -308,7 +308,10 @@ int asx_plan_create(asx_plan **out, int is_spmm, int alg, int value_type, int32_
             return ASX_STATUS_NOT_SUPPORTED;
         }
         p->alg = kernel;
-        if (kernel == ASX_SPMV_STREAM) {
+        if (m == 0) {
+            // nothing to analyse (and no row_ptr to read): calls with m == 0 return before any launch
+            p->workspace_bytes = 0;
+        } else if (kernel == ASX_SPMV_STREAM) {
             int32_t nb = std::max(stream_blocks(nnz), 1);
             p->nunits = nb;
             p->meta_bytes = ((size_t)nb + 1) * 8;
@@ -334,7 +337,9 @@ int asx_plan_create(asx_plan **out, int is_spmm, int alg, int value_type, int32_
             return ASX_STATUS_NOT_SUPPORTED;
         }
         p->alg = kernel;
-        if (kernel == ASX_SPMM_MERGE) {
+        if (m == 0) {
+            p->workspace_bytes = 0;
+        } else if (kernel == ASX_SPMM_MERGE) {
             const size_t ns = (size_t)spmm_segments(m, nnz);
             p->nunits = (int32_t)ns;
             p->meta_bytes = 2 * (ns + 1) * 4;

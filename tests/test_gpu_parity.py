@@ -212,8 +212,16 @@ def test_spmv_errors_and_empty(torch, capi):
         capi.spmv(rp, col, val, x, y, 1.0, 0.0, plan=plan)
     assert e.value.code == 3
     plan.destroy()
-    # m == 0 is a no-op; a matrix with no stored elements scales y
+    # m == 0 is a no-op (also through a plan built without a row_ptr); a matrix with no stored elements scales y
     assert L.asx_spmv_csr_f64(None, 0, 0, 0, 0, 1.0, None, None, None, None, 0.0, None, None, 0, None) == 0
+    for alg in (capi.SPMV_DEFAULT, capi.SPMV_STREAM, capi.SPMV_MERGE, capi.SPMV_VECTOR):
+        h = capi.C.c_void_p()
+        assert L.asx_plan_create(capi.C.byref(h), 0, alg, capi.R_64F, 0, 0, 0, None, 1, None) == 0
+        assert L.asx_spmv_csr_f64(h, alg, 0, 0, 0, 1.0, None, None, None, None, 0.0, None, None, 0, None) == 0
+        assert L.asx_plan_destroy(h) == 0
+    h = capi.C.c_void_p()
+    assert L.asx_plan_create(capi.C.byref(h), 1, capi.SPMM_MERGE, capi.R_32F, 0, 0, 0, None, 64, None) == 0
+    assert L.asx_plan_destroy(h) == 0
     rp0 = dev(torch, np.zeros(4, dtype=np.int32))
     e0 = torch.empty(0, dtype=torch.int32, device="cuda")
     v0 = torch.empty(0, dtype=torch.float64, device="cuda")
