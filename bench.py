@@ -23,7 +23,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 ORDER = ["banded_f64", "uniform16_f32", "powerlaw_f64", "stencil5_f64", "spmm_zipf_f32"]
 EXTRA = ["spmm_banded_f32"]  # not a BASELINE configuration: dense-block matrix for the MFMA SpMM variant
-KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 5: "k_spmm_row", 7: "k_spmm_merge",
+KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "k_spmv_flat", 5: "k_spmm_row", 7: "k_spmm_merge",
                 10: "k_spmm_blocked"}
 
 # HBM traffic per call measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; see profiles/),
@@ -95,6 +95,32 @@ def measure(w, steps, warmup, alg):
         ends[i].record()
     torch.cuda.synchronize()
     per_call = np.array([s.elapsed_time(e) for s, e in zip(starts, ends)])
+    # (c) the same call without kept analysis (split points recomputed inside every call, as the
+    #     reference does): what a caller that never calls *_analysis / *_preprocess sees
+    vt = capi.value_type(w.val.dtype)
+    if spmm:
+        need = capi.lib().asx_spmm_workspace_bytes(0, vt, w.m, w.nnz, w.ncols)
+    else:
+        need = capi.lib().asx_spmv_workspace_bytes(0, vt, w.m, w.nnz)
+    ws2 = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+
+    def step_noplan():
+        if spmm:
+            capi.spmm(d_rp, d_col, d_val, d_x, d_y, w.ncols, w.alpha, w.beta, alg=0, workspace=ws2, k=w.n)
+        else:
+            capi.spmv(d_rp, d_col, d_val, d_x, d_y, w.alpha, w.beta, alg=0, workspace=ws2)
+
+    for _ in range(3):
+        step_noplan()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    nrep = max(5, steps // 5)
+    e0.record()
+    for _ in range(nrep):
+        step_noplan()
+    e1.record()
+    torch.cuda.synchronize()
+    noplan_ms = e0.elapsed_time(e1) / nrep
     nbytes = w.bytes_algorithmic()
     res = {
         "workload": w.name, "kind": w.kind, "dtype": "f64" if w.dtype.itemsize == 8 else "f32",
@@ -106,13 +132,14 @@ def measure(w, steps, warmup, alg):
         "ms_per_step": wall_ms,
         "event_ms_mean": float(per_call.mean()), "event_ms_median": float(np.median(per_call)),
         "event_ms_min": float(per_call.min()),
+        "noplan_ms": float(noplan_ms),
     }
     res["gbs"] = nbytes / (wall_ms * 1e-3) / 1e9
     res["gflops"] = w.flops / (wall_ms * 1e-3) / 1e9
     res["gbs_event"] = nbytes / (res["event_ms_mean"] * 1e-3) / 1e9
     res["frac_hbm_peak"] = res["gbs_event"] / HBM_PEAK_GBS
     plan.destroy()
-    del d_rp, d_col, d_val, d_x, d_y, ws
+    del d_rp, d_col, d_val, d_x, d_y, ws, ws2
     torch.cuda.empty_cache()
     return res
 

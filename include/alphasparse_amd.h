@@ -48,7 +48,8 @@ enum {
     ASX_SPMV_DEFAULT = 0, /* pick from the row-length histogram (plan) or from m, nnz */
     ASX_SPMV_VECTOR = 6,  /* wave64 sub-groups, one group per row */
     ASX_SPMV_STREAM = 3,  /* LDS-staged row blocks, segmented reduction */
-    ASX_SPMV_MERGE = 9    /* merge-path tiles + ordered carry fix-up */
+    ASX_SPMV_MERGE = 9,   /* merge-path tiles + ordered carry fix-up */
+    ASX_SPMV_FLAT = 15    /* tiles of 1024 stored elements, register walk + ordered carry fix-up */
 };
 
 /* SpMM kernels (alphasparseSpMMAlg_t values, include/alphasparse/spdef.h:390-402) */

@@ -130,6 +130,15 @@ __global__ __launch_bounds__(256) void k_nnz_split_rows(const int32_t *__restric
     out[t] = lo;
 }
 
+// same kernel for a caller-chosen segment count (nseg >= ceil(nnz/items))
+int launch_nnz_split_rows_n(const int32_t *d_row_ptr, int32_t m, int32_t nseg, int32_t items, int32_t *d_out,
+                            hipStream_t s)
+{
+    int grid = (int)ceil_div64((int64_t)nseg + 1, 256);
+    hipLaunchKernelGGL(k_nnz_split_rows, dim3(grid), dim3(256), 0, s, d_row_ptr, m, nseg, items, d_out);
+    return check_launch();
+}
+
 int launch_nnz_split_rows(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t items,
                           int32_t *d_out, hipStream_t s)
 {

@@ -36,6 +36,24 @@ MergeLayout spmv_merge_layout(int32_t m, int32_t nnz, size_t sv, bool with_split
     return L;
 }
 
+struct FlatLayout {  // [seg_row | carry]
+    size_t seg_off, carry_off, bytes;
+};
+FlatLayout spmv_flat_layout(int32_t nnz, size_t sv, bool with_split)
+{
+    FlatLayout L{};
+    const size_t nt = (size_t)flat_tiles(nnz);
+    size_t off = 0;
+    if (with_split) {
+        L.seg_off = off;
+        off = align_up(off + (nt + 1) * 4, kAlign);
+    }
+    L.carry_off = off;
+    off = align_up(off + nt * sv, kAlign);
+    L.bytes = off;
+    return L;
+}
+
 struct SpmmLayout {  // [xs | ys | carry_row | carry]
     size_t xs_off, ys_off, crow_off, carry_off, bytes;
 };
@@ -58,16 +76,15 @@ SpmmLayout spmm_merge_layout(int32_t m, int32_t nnz, int32_t ncols, size_t sv, b
     return L;
 }
 
-// Kernel choice from the row-length histogram: the stream kernel never lets a row leave its
-// workgroup, so one very long row would serialise on one workgroup; past a few windows the
-// merge-path kernel's even split wins.
+// DEFAULT with a plan: the flat kernel, except for matrices with very long rows, where the
+// merge-path kernel measured about 1 % faster (power-law: 569 vs 576 us).  Elsewhere flat is the
+// fastest of the four or within 1 % of it (5-point stencil 300 us vs stream 305; uniform 16/row
+// 95 vs stream 96), and it has no bad case: work per tile is bounded whatever the row lengths.
 int choose_spmv_from_stats(const int64_t stats[4], int32_t m, int32_t nnz)
 {
-    const int64_t max_len = stats[0];
-    if (max_len > kStreamMaxRow) return ASX_SPMV_MERGE;
     (void)m;
     (void)nnz;
-    return ASX_SPMV_STREAM;
+    return stats[0] > kLongRow ? ASX_SPMV_MERGE : ASX_SPMV_FLAT;
 }
 
 template <typename T>
@@ -124,6 +141,21 @@ int spmv_impl(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, 
         }
         return launch_spmv_merge<T>(m, nnz, alpha, row_ptr, col, val, x, beta, y, xs, ys,
                                     (T *)(w + L.carry_off), s);
+    }
+    case ASX_SPMV_FLAT: {
+        const FlatLayout L = spmv_flat_layout(nnz, sizeof(T), plan == nullptr);
+        if (!ws) return ASX_STATUS_INVALID_POINTER;
+        if (ws_bytes < L.bytes) return ASX_STATUS_INVALID_SIZE;
+        const int32_t *seg;
+        if (plan) {
+            seg = plan->d_meta;
+        } else {
+            int st = launch_flat_seg_rows(row_ptr, m, nnz, (int32_t *)(w + L.seg_off), s);
+            if (st) return st;
+            seg = (const int32_t *)(w + L.seg_off);
+        }
+        return launch_spmv_flat<T>(m, nnz, alpha, row_ptr, col, val, x, beta, y, seg, (T *)(w + L.carry_off),
+                                   plan ? plan->carry_pass != 0 : true, s);
     }
     default: return ASX_STATUS_NOT_SUPPORTED;
     }
@@ -318,6 +350,26 @@ int asx_plan_create(asx_plan **out, int is_spmm, int alg, int value_type, int32_
             st = status_of(hipMalloc((void **)&p->d_meta, p->meta_bytes));
             if (!st) st = launch_stream_row_blocks(d_row_ptr, m, nnz, p->d_meta, s);
             p->workspace_bytes = 0;
+        } else if (kernel == ASX_SPMV_FLAT) {
+            const size_t nt = (size_t)flat_tiles(nnz);
+            p->nunits = (int32_t)nt;
+            p->meta_bytes = (nt + 1) * 4;
+            st = status_of(hipMalloc((void **)&p->d_meta, p->meta_bytes));
+            if (!st) st = launch_flat_seg_rows(d_row_ptr, m, nnz, p->d_meta, s);
+            p->workspace_bytes = spmv_flat_layout(nnz, sv, false).bytes;
+            p->carry_pass = 1;
+            if (!st) {  // is any row cut by a tile boundary?  (one int read back; creation syncs anyway)
+                int32_t *d_flag = nullptr, h_flag = 1;
+                st = status_of(hipMalloc((void **)&d_flag, sizeof(int32_t)));
+                if (!st) {
+                    st = status_of(hipMemsetAsync(d_flag, 0, sizeof(int32_t), s));
+                    if (!st) st = launch_flat_has_carry(d_row_ptr, m, nnz, p->d_meta, d_flag, s);
+                    if (!st) st = status_of(hipMemcpyAsync(&h_flag, d_flag, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+                    if (!st) st = status_of(hipStreamSynchronize(s));
+                    (void)hipFree(d_flag);
+                    if (!st) p->carry_pass = h_flag != 0;
+                }
+            }
         } else if (kernel == ASX_SPMV_MERGE) {
             const size_t nt = (size_t)merge_tiles(m, nnz);
             p->nunits = (int32_t)nt;
@@ -446,27 +498,28 @@ int asx_plan_histogram(const asx_plan *plan, int64_t h_hist[33], int64_t h_stats
 // ---------------------------------------------------------------- SpMV
 // Reference algorithm ids (include/alphasparse/spdef.h:345-365) onto the three kernels here:
 // the reference's scalar/vector/line-enhance families are one-row-per-lane-group kernels, its
-// adaptive/stream/flat/acc families stage row blocks through LDS, its merge/row-partition/
-// load-balance families split work evenly whatever the row lengths.
+// adaptive/stream families stage row blocks through LDS, its flat/acc families cut the stored
+// elements into equal tiles of 1024, its merge/row-partition/load-balance families split work
+// evenly whatever the row lengths.
 int asx_spmv_resolve_alg(int alg, int32_t m, int32_t nnz)
 {
     (void)m;
     (void)nnz;
     switch (alg) {
-    case 0: return ASX_SPMV_MERGE;   /* DEFAULT without a histogram: the kernel with no bad case */
+    case 0: return ASX_SPMV_FLAT;    /* DEFAULT without a histogram: even work per tile, no bad case */
     case 5:                          /* SCALAR */
     case 6:                          /* VECTOR */
     case 10:                         /* LINE */
     case 16: return ASX_SPMV_VECTOR; /* LINE_ENHANCE */
     case 2:                          /* CSR_ADAPTIVE */
     case 3:                          /* CSR_STREAM */
-    case 8:                          /* ADAPTIVE */
+    case 8: return ASX_SPMV_STREAM;  /* ADAPTIVE */
     case 11:
     case 12:
     case 13: /* FLAT1/4/8 */
     case 14: /* ACC */
     case 15: /* FLAT */
-    case 18: return ASX_SPMV_STREAM; /* PFLAT */
+    case 18: return ASX_SPMV_FLAT;   /* PFLAT */
     case 7:                          /* ROW_PARTITION */
     case 9:                          /* MERGE */
     case 17: return ASX_SPMV_MERGE;  /* LOAD_BALANCE */
@@ -478,6 +531,7 @@ size_t asx_spmv_workspace_bytes(int alg, int value_type, int32_t m, int32_t nnz)
 {
     const int kernel = asx_spmv_resolve_alg(alg, m, nnz);
     if (kernel == ASX_SPMV_MERGE) return spmv_merge_layout(m, nnz, vsize(value_type), true).bytes;
+    if (kernel == ASX_SPMV_FLAT) return spmv_flat_layout(nnz, vsize(value_type), true).bytes;
     if (kernel == ASX_SPMV_STREAM)
         return align_up(((size_t)std::max(stream_blocks(nnz), 1) + 1) * 8, kAlign);
     return 0;

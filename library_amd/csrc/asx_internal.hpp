@@ -14,7 +14,8 @@ constexpr int kBlock = 256;
 constexpr int kMergeItemsPerThread = 8;
 constexpr int kMergeTile = kBlock * kMergeItemsPerThread;  // rows + stored elements per tile
 constexpr int kStreamTile = 1024;                          // stored elements per row block
-constexpr int kStreamMaxRow = 8192;  // DEFAULT picks the stream kernel only below this row length
+constexpr int kFlatTile = 1024;                            // stored elements per flat tile
+constexpr int kLongRow = 8192;  // DEFAULT (with a plan) switches to the merge-path kernel above this row length
 // SpMM: merge items (rows + stored elements) per wave
 constexpr int kSpmmSegment = 128;
 
@@ -41,6 +42,9 @@ int launch_partition_rows_by_nnz(const int32_t *d_row_ptr, int32_t m, int32_t np
                                  hipStream_t s);
 int launch_nnz_split_rows(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t items,
                           int32_t *d_out, hipStream_t s);
+int launch_nnz_split_rows_n(const int32_t *d_row_ptr, int32_t m, int32_t nseg, int32_t items, int32_t *d_out,
+                            hipStream_t s);
+int launch_flat_seg_rows(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t *d_seg_row, hipStream_t s);
 int launch_merge_path_search(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t items,
                              int32_t *d_xs, int32_t *d_ys, hipStream_t s);
 int launch_loadbalance_partition(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t warp_size,
@@ -60,6 +64,13 @@ int launch_spmv_merge(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, c
 template <typename T>
 int launch_spmv_stream(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, const int32_t *col,
                        const T *val, const T *x, T beta, T *y, const int32_t *blocks, hipStream_t s);
+
+template <typename T>
+int launch_spmv_flat(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, const int32_t *col,
+                     const T *val, const T *x, T beta, T *y, const int32_t *seg_row, T *carry,
+                     bool carry_pass, hipStream_t s);
+int launch_flat_has_carry(const int32_t *d_row_ptr, int32_t m, int32_t nnz, const int32_t *d_seg_row,
+                          int32_t *d_flag, hipStream_t s);
 
 // ---- SpMM launchers (asx_spmm.hip) ----
 template <typename T>
@@ -88,6 +99,7 @@ int launch_spmm_blocked(int32_t m, int32_t k, int32_t ncols, T alpha, const Bloc
                         int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t s);
 
 inline int32_t merge_tiles(int32_t m, int32_t nnz) { return (int32_t)ceil_div64((int64_t)m + nnz, kMergeTile); }
+inline int32_t flat_tiles(int32_t nnz) { int32_t t = (int32_t)ceil_div64(nnz, kFlatTile); return t < 1 ? 1 : t; }
 inline int32_t stream_blocks(int32_t nnz) { return (int32_t)ceil_div64(nnz, kStreamTile); }
 inline int32_t spmm_segments(int32_t m, int32_t nnz) { return (int32_t)ceil_div64((int64_t)m + nnz, kSpmmSegment); }
 
@@ -103,6 +115,7 @@ struct asx_plan {
     int32_t *d_meta;         // split points / row blocks (layout depends on alg)
     size_t meta_bytes;
     int32_t nunits;  // tiles / row blocks / segments
+    int carry_pass;  // flat kernel: 0 when no row is cut by a tile boundary
     int64_t hist[33];
     int64_t stats[4];
     size_t workspace_bytes;

@@ -5,6 +5,10 @@
 //            elements; products are staged through LDS once (coalesced), rows are reduced
 //            from LDS by 1..64 lanes each; the one row that may run past the window is
 //            finished by the whole workgroup.  No atomics, no inter-workgroup traffic.
+//   flat   : a workgroup owns exactly kFlatTile consecutive stored elements (aligned vector
+//            loads, no metadata needed to start them); each thread walks its 4 products in
+//            registers, rows spanning threads are joined by a segmented scan, rows spanning
+//            tiles by the ordered carry pass.
 //   merge  : a workgroup owns kMergeTile consecutive items of the merge path over
 //            (row ends, stored elements); each thread walks exactly kMergeItemsPerThread
 //            items; partial rows are joined by a segmented scan inside the workgroup and by
@@ -483,6 +487,307 @@ int launch_spmv_merge(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, c
     return check_launch();
 }
 
+// ===========================================================================================
+// flat: tiles of exactly kFlatTile stored elements
+// ===========================================================================================
+// Tile t owns stored elements [t*kFlatTile, (t+1)*kFlatTile): its loads need no metadata and are
+// 16-byte vector loads on aligned addresses.  seg_row[t] (the row holding the tile's first
+// element, asx_nnz_split_rows) arrives while the loads are in flight.  Each thread keeps its 4
+// consecutive products in registers and walks them against the tile's row ends (LDS); rows that
+// end inside a thread are stored to an LDS row buffer, rows that span threads are joined by a
+// segmented scan, the row still open at the tile end leaves a carry that the same ordered pass
+// as the merge kernel's adds afterwards.  Work per tile is bounded whatever the row lengths;
+// a tile that meets more rows than the LDS row buffer holds (a flood of empty rows) takes a
+// slower thread-per-row path.
+constexpr int kFlatItemsPerThread = kFlatTile / kBlock;
+static_assert(kFlatItemsPerThread == 4, "the vector loads below read 4 elements per thread");
+constexpr int kFlatRowCap = 1024;  // rows of one tile kept in LDS
+
+template <typename T>
+struct Vec4;
+template <>
+struct Vec4<float> {
+    template <bool NT>
+    static __device__ __forceinline__ void load(const float *p, float v[4])
+    {
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        const f32x4 *q = reinterpret_cast<const f32x4 *>(p);
+        const f32x4 t = NT ? __builtin_nontemporal_load(q) : *q;
+        v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+    }
+};
+template <>
+struct Vec4<double> {
+    template <bool NT>
+    static __device__ __forceinline__ void load(const double *p, double v[4])
+    {
+        typedef double f64x2 __attribute__((ext_vector_type(2)));
+        const f64x2 *q = reinterpret_cast<const f64x2 *>(p);
+        const f64x2 a = NT ? __builtin_nontemporal_load(q) : q[0];
+        const f64x2 b = NT ? __builtin_nontemporal_load(q + 1) : q[1];
+        v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
+    }
+};
+
+// Row mode of the flat kernel: aligned groups of G lanes own one row each.
+template <int G, bool NT, typename T>
+__device__ __forceinline__ void flat_reduce_rows(const T *s_prod, const int32_t *s_rend, bool fits, int32_t rs,
+                                                 int32_t rcount, int32_t nwritten, int64_t base, int32_t n1,
+                                                 int t, T alpha, T beta, const int32_t *__restrict__ row_ptr,
+                                                 T *__restrict__ y, T *__restrict__ carry)
+{
+    const int lane = threadIdx.x & (G - 1);
+    const int rows_per_pass = kBlock / G;
+    for (int first = 0; first < rcount; first += rows_per_pass) {  // same trip count for every lane
+        const int i = first + (int)threadIdx.x / G;
+        T sum = T(0);
+        if (i < rcount) {
+            int32_t s, e;
+            if (fits) {
+                s = i > 0 ? s_rend[i - 1] : 0;
+                e = s_rend[i];
+            } else {
+                const int64_t gs = (int64_t)row_ptr[rs + i] - base, ge = (int64_t)row_ptr[rs + i + 1] - base;
+                s = gs < 0 ? 0 : (int32_t)gs;
+                e = ge > n1 ? n1 : (int32_t)ge;
+            }
+            s = s < 0 ? 0 : s;
+            e = e > n1 ? n1 : e;
+            for (int32_t k = s + lane; k < e; k += G) sum += s_prod[k + (k >> 5)];
+        }
+        sum = group_sum<G>(sum);
+        if (i < rcount && lane == 0) {
+            const int64_t r = (int64_t)rs + i;
+            if (i < nwritten)
+                stream_store<NT>(y + r, axpby_out<T>(alpha, sum, beta, y, r));
+            else
+                carry[t] = sum;
+        }
+    }
+}
+
+// Rows no longer than this are summed one thread per row from LDS; a tile that meets a longer
+// row takes the register walk, whose cost does not depend on row lengths.
+constexpr int kFlatRowModeMaxLen = 32;
+
+template <typename T, bool VEC, bool NT>
+__global__ __launch_bounds__(kBlock) void k_spmv_flat(int32_t m, int32_t nnz, int32_t ntiles, T alpha,
+                                                      const int32_t *__restrict__ row_ptr,
+                                                      const int32_t *__restrict__ col,
+                                                      const T *__restrict__ val,
+                                                      const T *__restrict__ x, T beta,
+                                                      T *__restrict__ y,
+                                                      const int32_t *__restrict__ seg_row,
+                                                      T *__restrict__ carry)
+{
+    __shared__ int32_t s_rend[kFlatRowCap + 1];
+    __shared__ T s_out[kFlatRowCap + 1];
+    __shared__ T s_prod[kFlatTile + kFlatTile / 32];  // row mode (padded against bank conflicts)
+    __shared__ T s_wv[kBlock / kWave];
+    __shared__ int32_t s_wk[kBlock / kWave];
+
+    const int t = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int64_t base = (int64_t)t * kFlatTile;
+    const int32_t n1 = nnz - base < kFlatTile ? (int32_t)(nnz - base) : kFlatTile;
+    const int32_t k0 = tid * 4;
+
+    // ---- this thread's 4 consecutive stored elements ----
+    int32_t c[4];
+    T p[4];
+    if (VEC && n1 == kFlatTile) {
+        typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+        const i32x4 *cp = reinterpret_cast<const i32x4 *>(col + base + k0);
+        const i32x4 cc = NT ? __builtin_nontemporal_load(cp) : *cp;
+        c[0] = cc.x, c[1] = cc.y, c[2] = cc.z, c[3] = cc.w;
+        Vec4<T>::template load<NT>(val + base + k0, p);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            c[j] = k0 + j < n1 ? col[base + k0 + j] : 0;
+            p[j] = k0 + j < n1 ? val[base + k0 + j] : T(0);
+        }
+    }
+    // ---- rows met by the tile: rs .. re; re (if < m) continues into the next tile ----
+    const int32_t rs = t == 0 ? 0 : seg_row[t];
+    const int32_t re = seg_row[t + 1];
+    const int32_t nwritten = re - rs;                   // rows that end inside this tile
+    const int32_t rcount = nwritten + (re < m ? 1 : 0);  // plus the one left open
+    const bool fits = rcount <= kFlatRowCap;
+    int has_long = 0;
+    if (fits) {
+        for (int i = tid; i < rcount; i += kBlock) {
+            const int32_t lo = row_ptr[rs + i], hi = row_ptr[rs + i + 1];
+            s_rend[i] = (int32_t)(hi - base);
+            s_out[i] = T(0);
+            has_long |= (hi - lo) > kFlatRowModeMaxLen;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        if (k0 + j < n1) p[j] *= x[c[j]];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) s_prod[k0 + j + ((k0 + j) >> 5)] = k0 + j < n1 ? p[j] : T(0);
+    const bool walk = fits && __syncthreads_or(has_long);  // also the barrier after staging
+    if (!fits) __syncthreads();
+
+    if (!walk) {
+        // ---- row mode: 1..64 lanes per row (from the tile's row count) over the products in LDS ----
+#define ASX_FLAT_ROWS(G)                                                                              \
+    flat_reduce_rows<G, NT, T>(s_prod, s_rend, fits, rs, rcount, nwritten, base, n1, t, alpha, beta, row_ptr, \
+                               y, carry)
+        if (rcount > 128)
+            ASX_FLAT_ROWS(1);
+        else if (rcount > 64)
+            ASX_FLAT_ROWS(2);
+        else if (rcount > 32)
+            ASX_FLAT_ROWS(4);
+        else if (rcount > 16)
+            ASX_FLAT_ROWS(8);
+        else
+            ASX_FLAT_ROWS(16);
+#undef ASX_FLAT_ROWS
+        if (re >= m && tid == 0) carry[t] = T(0);
+        return;
+    }
+
+    // ---- walk mode.  Row holding this thread's first element: first i with s_rend[i] > k0 ----
+    int32_t lo = 0, hi = rcount;
+    while (lo < hi) {
+        const int32_t mid = (lo + hi) >> 1;
+        if (s_rend[mid] > k0)
+            hi = mid;
+        else
+            lo = mid + 1;
+    }
+    int32_t row = lo;
+    const int32_t first_row = row;
+    bool emitted = false;
+    T run = T(0);
+    int32_t cur_end = row < rcount ? s_rend[row] : 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int32_t k = k0 + j;
+        if (k < n1) {
+            while (k >= cur_end) {  // the row ended before k (and any empty rows after it)
+                s_out[row] = run;
+                emitted = true;
+                run = T(0);
+                ++row;
+                cur_end = row < rcount ? s_rend[row] : 0x7fffffff;
+            }
+            run += p[j];
+        }
+    }
+    // the row ends exactly where this thread's elements end: nobody after us will see its end
+    if (k0 < n1 && (k0 + 4 < n1 ? k0 + 4 : n1) >= cur_end) {
+        s_out[row] = run;
+        emitted = true;
+        run = T(0);
+    }
+
+    // ---- join rows that span threads ----
+    const int lane = tid & (kWave - 1), w = tid / kWave;
+    const T incl = wave_segscan_incl<T>(row, run);
+    const int32_t key0 = __shfl(row, 0, kWave);
+    if (lane == kWave - 1) {
+        s_wk[w] = row;
+        s_wv[w] = incl;
+    }
+    __syncthreads();
+    int32_t pk = -1;
+    T pv = T(0);
+    for (int j = 0; j < w; ++j) {
+        const int32_t kj = s_wk[j];
+        const T vj = s_wv[j];
+        if (kj == pk)
+            pv += vj;
+        else {
+            pk = kj;
+            pv = vj;
+        }
+    }
+    const int32_t up_k = __shfl_up(row, 1, kWave);
+    T carry_in = __shfl_up(incl, 1, kWave);
+    if (lane == 0) {
+        carry_in = (w > 0 && pk == first_row) ? pv : T(0);
+    } else {
+        if (up_k != first_row)
+            carry_in = T(0);
+        else if (up_k == key0 && pk == up_k)
+            carry_in += pv;
+    }
+    if (emitted) s_out[first_row] += carry_in;
+    if (tid == kBlock - 1) {
+        T out = T(0);
+        if (re < m && row == nwritten) {  // the open row: everything the tile saw of it
+            out = incl;
+            if (row == key0 && pk == row) out += pv;
+        }
+        carry[t] = out;
+    }
+    __syncthreads();
+
+    for (int i = tid; i < nwritten; i += kBlock) {
+        const int64_t r = (int64_t)rs + i;
+        stream_store<NT>(y + r, axpby_out<T>(alpha, s_out[i], beta, y, r));
+    }
+}
+
+// seg_row[t] = row holding stored element t*kFlatTile for t < nt, seg_row[nt] = m,
+// nt = max(1, ceil(nnz / kFlatTile)): the reference's flat partition
+// (hip/kernel/level2/alphasparse_spmv_csr_flat.h:7-38) for 1024 elements per workgroup.
+int launch_flat_seg_rows(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t *d_seg_row, hipStream_t s)
+{
+    return launch_nnz_split_rows_n(d_row_ptr, m, flat_tiles(nnz), kFlatTile, d_seg_row, s);
+}
+
+// flag[0] = 1 if any row is cut by a tile boundary (then the carry pass is needed)
+__global__ __launch_bounds__(kBlock) void k_flat_has_carry(const int32_t *__restrict__ row_ptr, int32_t m,
+                                                           const int32_t *__restrict__ seg_row, int32_t ntiles,
+                                                           int32_t *__restrict__ flag)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x + 1;
+    if (t >= ntiles) return;
+    const int32_t r = seg_row[t];
+    if (r < m && (int64_t)row_ptr[r] < t * kFlatTile) flag[0] = 1;
+}
+
+int launch_flat_has_carry(const int32_t *d_row_ptr, int32_t m, int32_t nnz, const int32_t *d_seg_row,
+                          int32_t *d_flag, hipStream_t s)
+{
+    const int32_t ntiles = flat_tiles(nnz);
+    if (ntiles > 1)
+        hipLaunchKernelGGL(k_flat_has_carry, dim3((unsigned)ceil_div64(ntiles - 1, kBlock)), dim3(kBlock), 0, s,
+                           d_row_ptr, m, d_seg_row, ntiles, d_flag);
+    return check_launch();
+}
+
+template <typename T>
+int launch_spmv_flat(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, const int32_t *col,
+                     const T *val, const T *x, T beta, T *y, const int32_t *seg_row, T *carry,
+                     bool carry_pass, hipStream_t s)
+{
+    if (m <= 0) return ASX_STATUS_SUCCESS;
+    const int32_t ntiles = flat_tiles(nnz);
+    // the 16-byte loads need 16-byte aligned arrays (true for anything a device allocator returns;
+    // a caller may pass an offset view)
+    const bool aligned = ((uintptr_t)col % 16 == 0) && ((uintptr_t)val % 16 == 0);
+    const bool nt = use_nontemporal(nnz, sizeof(T));
+#define ASX_FLAT(VEC, NT)                                                                             \
+    hipLaunchKernelGGL((k_spmv_flat<T, VEC, NT>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, m, nnz, ntiles, \
+                       alpha, row_ptr, col, val, x, beta, y, seg_row, carry)
+    if (aligned && nt) ASX_FLAT(true, true);
+    else if (aligned) ASX_FLAT(true, false);
+    else if (nt) ASX_FLAT(false, true);
+    else ASX_FLAT(false, false);
+#undef ASX_FLAT
+    if (carry_pass)
+        hipLaunchKernelGGL((k_spmv_merge_fixup<T>), dim3((unsigned)ceil_div64(ntiles, kBlock / kWave)),
+                           dim3(kBlock), 0, s, m, ntiles, alpha, seg_row, carry, y);
+    return check_launch();
+}
+
 #define ASX_INST(T)                                                                                  \
     template int launch_spmv_vector<T>(int32_t, int32_t, T, const int32_t *, const int32_t *,        \
                                        const T *, const T *, T, T *, hipStream_t);                   \
@@ -490,7 +795,9 @@ int launch_spmv_merge(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, c
                                        const T *, const T *, T, T *, const int32_t *, hipStream_t);  \
     template int launch_spmv_merge<T>(int32_t, int32_t, T, const int32_t *, const int32_t *,         \
                                       const T *, const T *, T, T *, const int32_t *, const int32_t *, \
-                                      T *, hipStream_t);
+                                      T *, hipStream_t);                                             \
+    template int launch_spmv_flat<T>(int32_t, int32_t, T, const int32_t *, const int32_t *, const T *, \
+                                     const T *, T, T *, const int32_t *, T *, bool, hipStream_t);
 ASX_INST(float)
 ASX_INST(double)
 #undef ASX_INST

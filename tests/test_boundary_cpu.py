@@ -59,9 +59,11 @@ def test_alg_mapping_and_workspace(lib):
     # reference algorithm ids -> kernels (spdef.h:345-365)
     for alg in (5, 6, 10, 16):
         assert lib.asx_spmv_resolve_alg(alg, 100, 1000) == capi.SPMV_VECTOR
-    for alg in (2, 3, 8, 11, 12, 13, 14, 15, 18):
+    for alg in (2, 3, 8):
         assert lib.asx_spmv_resolve_alg(alg, 100, 1000) == capi.SPMV_STREAM
-    for alg in (0, 7, 9, 17):
+    for alg in (0, 11, 12, 13, 14, 15, 18):
+        assert lib.asx_spmv_resolve_alg(alg, 100, 1000) == capi.SPMV_FLAT
+    for alg in (7, 9, 17):
         assert lib.asx_spmv_resolve_alg(alg, 100, 1000) == capi.SPMV_MERGE
     for alg in (1, 4, 19, -1):
         assert lib.asx_spmv_resolve_alg(alg, 100, 1000) < 0
