@@ -430,3 +430,34 @@ def test_coo_sort_and_coo2csr(torch, capi, oracle):
             torch.cuda.synchronize()
             assert np.array_equal(r.cpu().numpy(), row_ind) and np.array_equal(c.cpu().numpy(), col)
             assert np.array_equal(v.cpu().numpy(), val.astype(dtype))
+
+
+# ------------------------------------------------------------------ randomised shapes, every SpMV kernel
+def test_spmv_random_shapes_all_kernels(torch, capi, oracle):
+    rng = np.random.default_rng(2024)
+    for case in range(60):
+        kind = case % 6
+        m = int(rng.integers(1, 4000))
+        if kind == 0:
+            lens = rng.integers(0, 12, m)
+        elif kind == 1:
+            lens = np.minimum(rng.zipf(1.5, m), 6000)
+        elif kind == 2:  # runs of empty rows between long rows
+            lens = np.where(rng.random(m) < 0.02, rng.integers(500, 5000, m), 0)
+        elif kind == 3:  # rows that end exactly on 4-, 1024- and 2048-element boundaries
+            lens = rng.choice([4, 8, 1020, 1024, 1028, 2044, 2048, 2052, 0, 1], m if m < 40 else 40)
+        elif kind == 4:
+            lens = np.r_[rng.integers(0, 3, m), int(rng.integers(3000, 30000)), rng.integers(0, 3, 5)]
+        else:
+            lens = rng.integers(30, 36, m)  # around the row-mode / walk-mode threshold of the flat kernel
+        ncols = int(max(np.max(lens), 8)) + int(rng.integers(1, 50))
+        dtype = np.float64 if case % 2 == 0 else np.float32
+        rp, col, val = csr_from_lengths(lens, ncols, 1000 + case, dtype)
+        x = rng.uniform(-1, 1, ncols).astype(dtype)
+        y0 = rng.uniform(-1, 1, rp.size - 1).astype(dtype)
+        alpha, beta = ((1.0, 0.0), (1.5, 0.5), (-2.0, 1.0))[case % 3]
+        ref = oracle.spmv(rp, col, val, x, alpha, beta, y0, 2)
+        scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
+        for alg in ALGS:
+            got = run_spmv(torch, capi, rp, col, val, x, y0, alpha, beta, alg_id(capi, alg), use_plan=(case % 4 < 2))
+            assert_close(got, ref, scale, dtype, f"case {case} kind {kind} {alg}")
