@@ -29,10 +29,10 @@ KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "
 # HBM traffic per call measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; see profiles/),
 # scaled by the same counters' reading for a plain copy of known size.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "powerlaw_f64": (2034745.4 * 2 + 34144.8) * 1024,    # profiles/spmv_merge_powerlaw_f64.md
-    "stencil5_f64": (694107.6 * 2 + 134039.3) * 1024,    # profiles/spmv_stream_stencil5_f64.md
-    "uniform16_f32": (220068.2 * 2 + 4096.1) * 1024,     # profiles/spmv_stream_uniform16_f32.md
-    "spmm_zipf_f32": (2319893.4 * 2 + 297719.3) * 1024,  # profiles/spmm_merge_spmm_zipf_f32.md
+    "powerlaw_f64": (2034538.2 * 2 + 34142.0) * 1024,    # profiles/spmv_merge_powerlaw_f64.md
+    "stencil5_f64": (675202.8 * 2 + 136963.3) * 1024,    # profiles/spmv_flat_stencil5_f64.md
+    "uniform16_f32": (213542.6 * 2 + 4702.8) * 1024,     # profiles/spmv_flat_uniform16_f32.md
+    "spmm_zipf_f32": (2319853.5 * 2 + 297720.7) * 1024,  # profiles/spmm_merge_spmm_zipf_f32.md
 }
 
 

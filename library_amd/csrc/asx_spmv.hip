@@ -437,11 +437,12 @@ __global__ __launch_bounds__(kBlock) void k_spmv_merge(int32_t m, int32_t nnz, i
     }
 }
 
-// Adds the carries to the rows that continue past a tile end.  One wave per tile; only the wave
-// of the first tile of a run of tiles that end inside the same row goes on: it finds the run
-// length with ballots over xs (64 tiles per step), sums the run's carries lane-parallel in a
-// fixed order and adds the total to y.  (A single thread walking the run pays one memory round
-// trip per tile: 100 round trips for a 200 000-element row.)
+// Adds the carries to the rows that continue past a tile end.  One thread per tile.  A tile
+// whose open row ends in the very next tile (the common case) is settled by its thread alone.
+// A run of several tiles that end inside the same row is settled by the whole wave of the run's
+// first tile: it finds the run length with ballots over xs (64 tiles per step), sums the run's
+// carries lane-parallel in a fixed order and adds the total to y.  (A single thread walking the
+// run pays one memory round trip per tile: 100 round trips for a 200 000-element row.)
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_spmv_merge_fixup(int32_t m, int32_t ntiles, T alpha,
                                                              const int32_t *__restrict__ xs,
@@ -449,24 +450,38 @@ __global__ __launch_bounds__(kBlock) void k_spmv_merge_fixup(int32_t m, int32_t 
                                                              T *__restrict__ y)
 {
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t b = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
-    if (b >= ntiles) return;  // wave-uniform from here on
-    const int32_t row = __builtin_amdgcn_readfirstlane(xs[b + 1]);
-    if (row >= m) return;
-    if (b > 0 && __builtin_amdgcn_readfirstlane(xs[b]) == row) return;  // not the first tile of its run
-    int64_t len = 1;
-    for (int64_t base = b + 1;; base += kWave) {
-        const int64_t j = base + lane;
-        const bool same = j < ntiles && xs[j + 1] == row;
-        const unsigned long long mask = __ballot(same);
-        const int n = mask == ~0ull ? kWave : __ffsll((unsigned long long)~mask) - 1;
-        len += n;
-        if (n < kWave) break;
+    const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    int32_t row = m;
+    bool first = false, run = false;
+    if (t < ntiles) {
+        row = xs[t + 1];
+        first = row < m && (t == 0 || xs[t] != row);
+        run = first && t + 1 < ntiles && xs[t + 2] == row;
     }
-    T part = T(0);
-    for (int64_t j = lane; j < len; j += kWave) part += carry[b + j];
-    const T sum = group_sum<kWave>(part);
-    if (lane == 0 && sum != T(0)) y[row] = fma_t<T>(alpha, sum, y[row]);
+    if (first && !run) {
+        const T c = carry[t];
+        if (c != T(0)) y[row] = fma_t<T>(alpha, c, y[row]);
+    }
+    unsigned long long todo = __ballot(run);
+    while (todo) {  // wave-uniform
+        const int src = __ffsll(todo) - 1;
+        todo &= todo - 1;
+        const int64_t b = t - lane + src;
+        const int32_t r = __shfl(row, src, kWave);
+        int64_t len = 1;
+        for (int64_t base = b + 1;; base += kWave) {
+            const int64_t j = base + lane;
+            const bool same = j < ntiles && xs[j + 1] == r;
+            const unsigned long long mask = __ballot(same);
+            const int n = mask == ~0ull ? kWave : __ffsll((unsigned long long)~mask) - 1;
+            len += n;
+            if (n < kWave) break;
+        }
+        T part = T(0);
+        for (int64_t j = lane; j < len; j += kWave) part += carry[b + j];
+        const T sum = group_sum<kWave>(part);
+        if (lane == 0 && sum != T(0)) y[r] = fma_t<T>(alpha, sum, y[r]);
+    }
 }
 
 template <typename T>
@@ -482,7 +497,7 @@ int launch_spmv_merge(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, c
     else
         hipLaunchKernelGGL((k_spmv_merge<T, false>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, m, nnz,
                            ntiles, alpha, row_ptr, col, val, x, beta, y, xs, ys, carry);
-    hipLaunchKernelGGL((k_spmv_merge_fixup<T>), dim3((unsigned)ceil_div64(ntiles, kBlock / kWave)),
+    hipLaunchKernelGGL((k_spmv_merge_fixup<T>), dim3((unsigned)ceil_div64(ntiles, kBlock)),
                        dim3(kBlock), 0, s, m, ntiles, alpha, xs, carry, y);
     return check_launch();
 }
@@ -502,6 +517,10 @@ int launch_spmv_merge(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, c
 constexpr int kFlatItemsPerThread = kFlatTile / kBlock;
 static_assert(kFlatItemsPerThread == 4, "the vector loads below read 4 elements per thread");
 constexpr int kFlatRowCap = 1024;  // rows of one tile kept in LDS
+#ifndef ASX_FLAT_TPG
+#define ASX_FLAT_TPG 1
+#endif
+constexpr int kFlatTilesPerGroup = ASX_FLAT_TPG;
 
 template <typename T>
 struct Vec4;
@@ -570,31 +589,14 @@ __device__ __forceinline__ void flat_reduce_rows(const T *s_prod, const int32_t 
 // row takes the register walk, whose cost does not depend on row lengths.
 constexpr int kFlatRowModeMaxLen = 32;
 
+// The 4 consecutive stored elements of thread `tid` in tile t.
 template <typename T, bool VEC, bool NT>
-__global__ __launch_bounds__(kBlock) void k_spmv_flat(int32_t m, int32_t nnz, int32_t ntiles, T alpha,
-                                                      const int32_t *__restrict__ row_ptr,
-                                                      const int32_t *__restrict__ col,
-                                                      const T *__restrict__ val,
-                                                      const T *__restrict__ x, T beta,
-                                                      T *__restrict__ y,
-                                                      const int32_t *__restrict__ seg_row,
-                                                      T *__restrict__ carry)
+__device__ __forceinline__ void flat_load(int t, int32_t nnz, const int32_t *__restrict__ col,
+                                          const T *__restrict__ val, int32_t c[4], T p[4])
 {
-    __shared__ int32_t s_rend[kFlatRowCap + 1];
-    __shared__ T s_out[kFlatRowCap + 1];
-    __shared__ T s_prod[kFlatTile + kFlatTile / 32];  // row mode (padded against bank conflicts)
-    __shared__ T s_wv[kBlock / kWave];
-    __shared__ int32_t s_wk[kBlock / kWave];
-
-    const int t = blockIdx.x;
-    const int tid = threadIdx.x;
     const int64_t base = (int64_t)t * kFlatTile;
     const int32_t n1 = nnz - base < kFlatTile ? (int32_t)(nnz - base) : kFlatTile;
-    const int32_t k0 = tid * 4;
-
-    // ---- this thread's 4 consecutive stored elements ----
-    int32_t c[4];
-    T p[4];
+    const int32_t k0 = threadIdx.x * 4;
     if (VEC && n1 == kFlatTile) {
         typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
         const i32x4 *cp = reinterpret_cast<const i32x4 *>(col + base + k0);
@@ -608,6 +610,33 @@ __global__ __launch_bounds__(kBlock) void k_spmv_flat(int32_t m, int32_t nnz, in
             p[j] = k0 + j < n1 ? val[base + k0 + j] : T(0);
         }
     }
+}
+
+template <typename T>
+struct FlatShared {
+    int32_t rend[kFlatRowCap + 1];
+    T out[kFlatRowCap + 1];
+    T prod[kFlatTile + kFlatTile / 32];  // row mode (padded against bank conflicts)
+    T wv[kBlock / kWave];
+    int32_t wk[kBlock / kWave];
+};
+
+// One tile: gathers, reduction, y and carry.  Every thread of the workgroup calls it.
+template <typename T, bool NT>
+__device__ __forceinline__ void flat_tile(FlatShared<T> &sh, int t, int32_t m, int32_t nnz, T alpha,
+                                          const int32_t *__restrict__ row_ptr, const int32_t c[4], T p[4],
+                                          const T *__restrict__ x, T beta, T *__restrict__ y,
+                                          const int32_t *__restrict__ seg_row, T *__restrict__ carry)
+{
+    int32_t *s_rend = sh.rend;
+    T *s_out = sh.out;
+    T *s_prod = sh.prod;
+    T *s_wv = sh.wv;
+    int32_t *s_wk = sh.wk;
+    const int tid = threadIdx.x;
+    const int64_t base = (int64_t)t * kFlatTile;
+    const int32_t n1 = nnz - base < kFlatTile ? (int32_t)(nnz - base) : kFlatTile;
+    const int32_t k0 = tid * 4;
     // ---- rows met by the tile: rs .. re; re (if < m) continues into the next tile ----
     const int32_t rs = t == 0 ? 0 : seg_row[t];
     const int32_t re = seg_row[t + 1];
@@ -734,6 +763,34 @@ __global__ __launch_bounds__(kBlock) void k_spmv_flat(int32_t m, int32_t nnz, in
     }
 }
 
+// kFlatTilesPerGroup consecutive tiles per workgroup: the loads of all of them are issued before
+// the first is reduced, so the reduction of one tile overlaps the memory latency of the next.
+template <typename T, bool VEC, bool NT, int TPG>
+__global__ __launch_bounds__(kBlock) void k_spmv_flat(int32_t m, int32_t nnz, int32_t ntiles, T alpha,
+                                                      const int32_t *__restrict__ row_ptr,
+                                                      const int32_t *__restrict__ col,
+                                                      const T *__restrict__ val,
+                                                      const T *__restrict__ x, T beta,
+                                                      T *__restrict__ y,
+                                                      const int32_t *__restrict__ seg_row,
+                                                      T *__restrict__ carry)
+{
+    __shared__ FlatShared<T> sh;
+    const int t0 = blockIdx.x * TPG;
+    int32_t c[TPG][4];
+    T p[TPG][4];
+#pragma unroll
+    for (int u = 0; u < TPG; ++u)
+        if (t0 + u < ntiles) flat_load<T, VEC, NT>(t0 + u, nnz, col, val, c[u], p[u]);
+#pragma unroll
+    for (int u = 0; u < TPG; ++u) {
+        if (t0 + u < ntiles) {  // uniform over the workgroup
+            if (u > 0) __syncthreads();  // the previous tile is done with the LDS buffers
+            flat_tile<T, NT>(sh, t0 + u, m, nnz, alpha, row_ptr, c[u], p[u], x, beta, y, seg_row, carry);
+        }
+    }
+}
+
 // seg_row[t] = row holding stored element t*kFlatTile for t < nt, seg_row[nt] = m,
 // nt = max(1, ceil(nnz / kFlatTile)): the reference's flat partition
 // (hip/kernel/level2/alphasparse_spmv_csr_flat.h:7-38) for 1024 elements per workgroup.
@@ -775,15 +832,16 @@ int launch_spmv_flat(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, co
     const bool aligned = ((uintptr_t)col % 16 == 0) && ((uintptr_t)val % 16 == 0);
     const bool nt = use_nontemporal(nnz, sizeof(T));
 #define ASX_FLAT(VEC, NT)                                                                             \
-    hipLaunchKernelGGL((k_spmv_flat<T, VEC, NT>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, m, nnz, ntiles, \
-                       alpha, row_ptr, col, val, x, beta, y, seg_row, carry)
+    hipLaunchKernelGGL((k_spmv_flat<T, VEC, NT, kFlatTilesPerGroup>),                                 \
+                       dim3((unsigned)ceil_div64(ntiles, kFlatTilesPerGroup)), dim3(kBlock), 0, s, m, nnz, \
+                       ntiles, alpha, row_ptr, col, val, x, beta, y, seg_row, carry)
     if (aligned && nt) ASX_FLAT(true, true);
     else if (aligned) ASX_FLAT(true, false);
     else if (nt) ASX_FLAT(false, true);
     else ASX_FLAT(false, false);
 #undef ASX_FLAT
     if (carry_pass)
-        hipLaunchKernelGGL((k_spmv_merge_fixup<T>), dim3((unsigned)ceil_div64(ntiles, kBlock / kWave)),
+        hipLaunchKernelGGL((k_spmv_merge_fixup<T>), dim3((unsigned)ceil_div64(ntiles, kBlock)),
                            dim3(kBlock), 0, s, m, ntiles, alpha, seg_row, carry, y);
     return check_launch();
 }
