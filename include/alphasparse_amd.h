@@ -128,6 +128,25 @@ int asx_coo2csr(const int32_t *d_row_ind, int32_t nnz, int32_t m, int32_t *d_row
 int asx_coo_sort(int value_type, int32_t *d_row_ind, int32_t *d_col_ind, void *d_val, int32_t nnz,
                  void *stream);
 
+/* A (m x n, CSR, idx_base 0 or 1) -> A^T (n x m) as zero-based CSR; the stored elements of each
+ * row of A^T come in ascending row of A, duplicates in their stored order.  What
+ * opA = TRANSPOSE runs on; device twin of transpose_csr, hip/format/transpose_csr.h:9-71 (host
+ * counting sort between two copies across PCIe, result written over the caller's arrays).
+ * d_row_ptr_t has n+1 entries, d_col_t and d_val_t nnz.  Allocates temporaries and synchronises
+ * `stream`. */
+int asx_csr_transpose(int value_type, int32_t m, int32_t n, int32_t nnz, int32_t idx_base,
+                      const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val,
+                      int32_t *d_row_ptr_t, int32_t *d_col_t, void *d_val_t, void *stream);
+/* Zero-based copies of one-based (idx_base = 1) row offsets and column indices.  The reference
+ * stores idx_base in the descriptor (hip/format/alphasparse_create_csr.h:44-47) and its CSR
+ * kernels index with the stored values unchanged. */
+int asx_csr_rebase(int32_t m, int32_t nnz, int32_t idx_base, const int32_t *d_row_ptr, const int32_t *d_col,
+                   int32_t *d_row_ptr_out, int32_t *d_col_out, void *stream);
+/* d_out[c*ld_out + r] = d_in[r*ld_in + c] for r < rows, c < cols: row-major <-> column-major
+ * copies of the dense operands of SpMM.  transpose_dn_mat, hip/format/transpose_dn_mat.h:4-35. */
+int asx_dense_transpose(int value_type, int64_t rows, int64_t cols, const void *d_in, int64_t ld_in,
+                        void *d_out, int64_t ld_out, void *stream);
+
 /* ------------------------------------------------------------------------------------
  * Plans: analysis results kept across calls (the reference recomputes them inside every
  * SpMV/SpMM call; its alphasparseSpMV_analysis is a stub, hip/kernel/level2/alphasparse_spmv.hip:

@@ -25,7 +25,8 @@ STATUS = {0: "SUCCESS", 1: "NOT_INITIALIZED", 2: "ALLOC_FAILED", 3: "INVALID_VAL
 EXPORTS = [
     "asx_version", "asx_device_info", "asx_row_length_histogram", "asx_partition_rows_by_nnz",
     "asx_nnz_split_rows", "asx_merge_path_search", "asx_loadbalance_nwarps",
-    "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_coo2csr", "asx_coo_sort", "asx_plan_create",
+    "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_coo2csr", "asx_coo_sort", "asx_csr_transpose", "asx_csr_rebase",
+    "asx_dense_transpose", "asx_plan_create",
     "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
     "asx_spmm_resolve_alg", "asx_spmm_workspace_bytes", "asx_spmm_csr_f32", "asx_spmm_csr_f64",
@@ -62,6 +63,9 @@ def lib():
     L.asx_csr_adaptive_row_blocks.argtypes = [vp, i32, vp, sz, C.POINTER(sz)]
     L.asx_coo2csr.argtypes = [vp, i32, i32, vp, vp]
     L.asx_coo_sort.argtypes = [C.c_int, vp, vp, vp, i32, vp]
+    L.asx_csr_transpose.argtypes = [C.c_int, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp]
+    L.asx_csr_rebase.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp]
+    L.asx_dense_transpose.argtypes = [C.c_int, C.c_int64, C.c_int64, vp, C.c_int64, vp, C.c_int64, vp]
     L.asx_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, C.c_int, i32, i32, i32, vp, i32, vp]
     L.asx_spmm_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, i32, i32, i32, vp, vp, vp, i32, vp]
     L.asx_plan_block_stats.argtypes = [vp, C.POINTER(i64), C.POINTER(C.c_double)]
@@ -165,6 +169,34 @@ def coo2csr(row_ind, m):
 def coo_sort(row_ind, col_ind, val):
     _check(lib().asx_coo_sort(value_type(val.dtype), _ptr(row_ind), _ptr(col_ind), _ptr(val), row_ind.numel(), _stream()),
            "asx_coo_sort")
+
+
+def csr_transpose(row_ptr, col, val, n, idx_base=0):
+    """A (m x n CSR, device tensors) -> (row_ptr_t, col_t, val_t) of A^T, zero-based."""
+    import torch
+    m = row_ptr.numel() - 1
+    nnz = col.numel()
+    rp = torch.empty(n + 1, dtype=torch.int32, device=row_ptr.device)
+    ct = torch.empty(nnz, dtype=torch.int32, device=row_ptr.device)
+    vt = torch.empty(nnz, dtype=val.dtype, device=row_ptr.device)
+    _check(lib().asx_csr_transpose(value_type(val.dtype), m, n, nnz, idx_base, _ptr(row_ptr), _ptr(col), _ptr(val),
+                                   _ptr(rp), _ptr(ct), _ptr(vt), _stream()), "asx_csr_transpose")
+    return rp, ct, vt
+
+
+def csr_rebase(row_ptr, col, idx_base):
+    import torch
+    rp = torch.empty_like(row_ptr)
+    c = torch.empty_like(col)
+    _check(lib().asx_csr_rebase(row_ptr.numel() - 1, col.numel(), idx_base, _ptr(row_ptr), _ptr(col), _ptr(rp), _ptr(c),
+                                _stream()), "asx_csr_rebase")
+    return rp, c
+
+
+def dense_transpose(a, rows, cols, ld_in, out, ld_out):
+    """out[c*ld_out + r] = a[r*ld_in + c] on flat device tensors."""
+    _check(lib().asx_dense_transpose(value_type(a.dtype), rows, cols, _ptr(a), ld_in, _ptr(out), ld_out, _stream()),
+           "asx_dense_transpose")
 
 
 def csr_adaptive_row_blocks(row_ptr_host):

@@ -11,7 +11,12 @@
 // unsupported type / format / operation / order combinations return NOT_SUPPORTED (the
 // reference returns SUCCESS, alphasparse_spmv.hip:213-226); alphasparseSpMV_analysis and
 // alphasparseSpMV_clear do something (stubs in the reference, alphasparse_spmv.hip:229-256);
-// kernels run on handle->stream.
+// kernels run on handle->stream; opA = TRANSPOSE runs on a device-built transposed copy and
+// leaves the caller's arrays alone (the reference transposes on the host, writes the result
+// over the caller's arrays and so toggles A between calls, hip/format/transpose_csr.h:9-71);
+// one-based CSR is honoured (the reference's CSR kernels ignore idx_base); column-major B / C
+// and opB go through a tiled device transpose into the call's workspace (the reference
+// transposes B and C in place and rewrites their descriptors, alphasparse_spmm.hip:186-216).
 #include <cstddef>
 #include <cstdlib>
 #include <new>
@@ -60,8 +65,20 @@ struct KeptPlan {
     int ncols;
     asx_plan *plan;
 };
+// A zero-based and/or transposed device copy of a caller's CSR matrix.
+struct DerivedCsr {
+    const int *src_row;
+    const int *src_col;
+    const void *src_val;
+    int64_t rows, cols, nnz;
+    int value_type, base;
+    bool transposed;
+    int *row_ptr, *col;
+    void *val;  // owned only when transposed (otherwise the caller's values)
+};
 struct HandlePlans {
     std::vector<KeptPlan> plans;
+    std::vector<DerivedCsr> derived;  // kept by alphasparseSpMV_analysis / alphasparseSpMM_preprocess
 };
 HandlePlans *plans_of(alphasparseHandle_t h, bool create)
 {
@@ -80,6 +97,7 @@ const asx_plan *find_plan(alphasparseHandle_t h, bool spmm, int alg, const _alph
             return k.plan;
     return nullptr;
 }
+void free_derived(DerivedCsr &d);
 void drop_plans(alphasparseHandle_t h, bool spmm, int alg, bool all)
 {
     HandlePlans *hp = plans_of(h, false);
@@ -92,6 +110,150 @@ void drop_plans(alphasparseHandle_t h, bool spmm, int alg, bool all)
             keep.push_back(k);
     }
     hp->plans.swap(keep);
+    if (all) {
+        for (DerivedCsr &d : hp->derived) free_derived(d);
+        hp->derived.clear();
+    }
+}
+
+bool is_transpose(alphasparseOperation_t op)
+{
+    // real value types only: the conjugate transpose is the transpose
+    return op == ALPHA_SPARSE_OPERATION_TRANSPOSE || op == ALPHA_SPARSE_OPERATION_CONJUGATE_TRANSPOSE;
+}
+
+void free_derived(DerivedCsr &d)
+{
+    if (d.row_ptr) (void)hipFree(d.row_ptr);
+    if (d.col) (void)hipFree(d.col);
+    if (d.transposed && d.val) (void)hipFree(d.val);
+    d.row_ptr = d.col = nullptr;
+    d.val = nullptr;
+}
+
+bool same_source(const DerivedCsr &d, const _alphasparseSpMatDescr *A, bool transposed)
+{
+    return d.src_row == A->row_data && d.src_col == A->col_data && d.src_val == A->val_data &&
+           d.rows == A->rows && d.cols == A->cols && d.nnz == A->nnz && d.value_type == (int)A->data_type &&
+           d.base == (int)A->idx_base && d.transposed == transposed;
+}
+
+// Builds the zero-based (and, if asked, transposed) device copy of A.
+alphasparseStatus_t build_derived(alphasparseHandle_t h, const _alphasparseSpMatDescr *A, bool transposed,
+                                  DerivedCsr *out)
+{
+    DerivedCsr d{};
+    d.src_row = A->row_data;
+    d.src_col = A->col_data;
+    d.src_val = A->val_data;
+    d.rows = A->rows;
+    d.cols = A->cols;
+    d.nnz = A->nnz;
+    d.value_type = (int)A->data_type;
+    d.base = (int)A->idx_base;
+    d.transposed = transposed;
+    const size_t sv = A->data_type == ALPHA_R_64F ? 8 : 4;
+    const size_t nrow = (size_t)(transposed ? A->cols : A->rows) + 1;
+    const size_t nnz1 = A->nnz > 0 ? (size_t)A->nnz : 1;
+    hipError_t e = hipMalloc((void **)&d.row_ptr, nrow * sizeof(int));
+    if (e == hipSuccess) e = hipMalloc((void **)&d.col, nnz1 * sizeof(int));
+    if (e == hipSuccess && transposed) e = hipMalloc(&d.val, nnz1 * sv);
+    if (e != hipSuccess) {
+        free_derived(d);
+        return from_hip(e);
+    }
+    int rc;
+    if (transposed) {
+        rc = asx_csr_transpose((int)A->data_type, (int32_t)A->rows, (int32_t)A->cols, (int32_t)A->nnz,
+                               (int32_t)A->idx_base, A->row_data, A->col_data, A->val_data, d.row_ptr, d.col,
+                               d.val, (void *)h->stream);
+    } else {
+        d.val = A->val_data;
+        rc = asx_csr_rebase((int32_t)A->rows, (int32_t)A->nnz, (int32_t)A->idx_base, A->row_data, A->col_data,
+                            d.row_ptr, d.col, (void *)h->stream);
+    }
+    if (rc) {
+        free_derived(d);
+        return st(rc);
+    }
+    *out = d;
+    return ALPHA_SPARSE_STATUS_SUCCESS;
+}
+
+// The matrix the kernels run on for (A, opA): A itself, a kept derived copy, or a copy made for
+// this call alone (`temporary`, released by release_effective once the call's work is queued).
+struct Effective {
+    _alphasparseSpMatDescr d;
+    DerivedCsr temp;
+    bool temporary;
+};
+alphasparseStatus_t make_effective(alphasparseHandle_t h, const _alphasparseSpMatDescr *A,
+                                   alphasparseOperation_t opA, Effective *e)
+{
+    e->d = *A;
+    e->temporary = false;
+    e->temp = DerivedCsr{};
+    const bool tr = is_transpose(opA);
+    if (!tr && A->idx_base == ALPHA_SPARSE_INDEX_BASE_ZERO) return ALPHA_SPARSE_STATUS_SUCCESS;
+    const DerivedCsr *use = nullptr;
+    if (HandlePlans *hp = plans_of(h, false))
+        for (const DerivedCsr &d : hp->derived)
+            if (same_source(d, A, tr)) use = &d;
+    if (!use) {
+        alphasparseStatus_t s = build_derived(h, A, tr, &e->temp);
+        if (s) return s;
+        e->temporary = true;
+        use = &e->temp;
+    }
+    e->d.row_data = use->row_ptr;
+    e->d.col_data = use->col;
+    e->d.val_data = use->val;
+    e->d.idx_base = ALPHA_SPARSE_INDEX_BASE_ZERO;
+    if (tr) {
+        e->d.rows = A->cols;
+        e->d.cols = A->rows;
+    }
+    return ALPHA_SPARSE_STATUS_SUCCESS;
+}
+void release_effective(alphasparseHandle_t h, Effective *e)
+{
+    if (!e->temporary) return;
+    (void)hipStreamSynchronize(h->stream);  // the call's kernels read the copy
+    free_derived(e->temp);
+    e->temporary = false;
+}
+
+// Makes (or remakes, picking up changed values or structure) the kept derived copy for (A, opA);
+// plans built on the copy it replaces are dropped.
+alphasparseStatus_t keep_derived(alphasparseHandle_t h, const _alphasparseSpMatDescr *A,
+                                 alphasparseOperation_t opA)
+{
+    const bool tr = is_transpose(opA);
+    if (!tr && A->idx_base == ALPHA_SPARSE_INDEX_BASE_ZERO) return ALPHA_SPARSE_STATUS_SUCCESS;
+    HandlePlans *hp = plans_of(h, true);
+    if (!hp) return ALPHA_SPARSE_STATUS_ALLOC_FAILED;
+    (void)hipStreamSynchronize(h->stream);
+    for (size_t i = 0; i < hp->derived.size();) {
+        if (!same_source(hp->derived[i], A, tr)) {
+            ++i;
+            continue;
+        }
+        std::vector<KeptPlan> keep;
+        for (KeptPlan &k : hp->plans) {
+            if (k.row_data == hp->derived[i].row_ptr)
+                asx_plan_destroy(k.plan);
+            else
+                keep.push_back(k);
+        }
+        hp->plans.swap(keep);
+        free_derived(hp->derived[i]);
+        hp->derived.erase(hp->derived.begin() + (long)i);
+    }
+    DerivedCsr d{};
+    alphasparseStatus_t s = build_derived(h, A, tr, &d);
+    if (s) return s;
+    hp->derived.push_back(d);
+    return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
 // Checks shared by SpMV and SpMM on the sparse operand.
@@ -99,8 +261,9 @@ alphasparseStatus_t check_csr(const _alphasparseSpMatDescr *A, alphasparseOperat
 {
     if (!A->init) return ALPHA_SPARSE_STATUS_NOT_INITIALIZED;
     if (A->format != ALPHA_SPARSE_FORMAT_CSR) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
-    if (opA != ALPHA_SPARSE_OPERATION_NON_TRANSPOSE) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
-    if (A->idx_base != ALPHA_SPARSE_INDEX_BASE_ZERO) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
+    if (opA != ALPHA_SPARSE_OPERATION_NON_TRANSPOSE && !is_transpose(opA)) return ALPHA_SPARSE_STATUS_INVALID_VALUE;
+    if (A->idx_base != ALPHA_SPARSE_INDEX_BASE_ZERO && A->idx_base != ALPHA_SPARSE_INDEX_BASE_ONE)
+        return ALPHA_SPARSE_STATUS_INVALID_VALUE;
     if (A->row_type != ALPHA_SPARSE_INDEXTYPE_I32 || A->col_type != ALPHA_SPARSE_INDEXTYPE_I32)
         return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
     if (A->data_type != ALPHA_R_32F && A->data_type != ALPHA_R_64F)
@@ -125,11 +288,30 @@ alphasparseStatus_t check_spmv(alphasparseHandle_t handle, alphasparseOperation_
     if (!X->init || !Y->init) return ALPHA_SPARSE_STATUS_NOT_INITIALIZED;
     if (X->data_type != A->data_type || Y->data_type != A->data_type || computeType != A->data_type)
         return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
-    if (X->size < A->cols || Y->size < A->rows) return ALPHA_SPARSE_STATUS_INVALID_SIZE;
-    if ((A->rows > 0 && !Y->values) || (A->nnz > 0 && !X->values))
+    const int64_t out_len = is_transpose(opA) ? A->cols : A->rows;
+    const int64_t in_len = is_transpose(opA) ? A->rows : A->cols;
+    if (X->size < in_len || Y->size < out_len) return ALPHA_SPARSE_STATUS_INVALID_SIZE;
+    if ((out_len > 0 && !Y->values) || (A->nnz > 0 && !X->values))
         return ALPHA_SPARSE_STATUS_INVALID_POINTER;
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
+
+// How a dense SpMM operand reaches the kernels, which take row-major k x N (B) and m x N (C).
+// A column-major matrix is a row-major matrix of the transposed shape in memory, and op = T
+// swaps the two readings, so each operand is either usable in place or needs one transpose.
+struct DenseUse {
+    int64_t rows, cols;  // of op(matrix)
+    bool direct;         // memory already is row-major rows x cols with stride ld
+};
+DenseUse dense_use(const _alphasparse_dnmat_descr *M, bool transposed)
+{
+    DenseUse u;
+    u.rows = transposed ? M->cols : M->rows;
+    u.cols = transposed ? M->rows : M->cols;
+    u.direct = (M->order == ALPHASPARSE_ORDER_ROW) != transposed;
+    return u;
+}
+size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 alphasparseStatus_t check_spmm(alphasparseHandle_t handle, alphasparseOperation_t opA,
                                alphasparseOperation_t opB, const void *alpha,
@@ -140,18 +322,34 @@ alphasparseStatus_t check_spmm(alphasparseHandle_t handle, alphasparseOperation_
     if (!alpha || !beta || !A || !B || !Cm) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
     alphasparseStatus_t s = check_csr(A, opA);
     if (s) return s;
-    if (opB != ALPHA_SPARSE_OPERATION_NON_TRANSPOSE) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
+    if (opB != ALPHA_SPARSE_OPERATION_NON_TRANSPOSE && !is_transpose(opB)) return ALPHA_SPARSE_STATUS_INVALID_VALUE;
     if (!B->init || !Cm->init) return ALPHA_SPARSE_STATUS_NOT_INITIALIZED;
-    if (B->order != ALPHASPARSE_ORDER_ROW || Cm->order != ALPHASPARSE_ORDER_ROW)
-        return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
+    if ((B->order != ALPHASPARSE_ORDER_ROW && B->order != ALPHASPARSE_ORDER_COL) ||
+        (Cm->order != ALPHASPARSE_ORDER_ROW && Cm->order != ALPHASPARSE_ORDER_COL))
+        return ALPHA_SPARSE_STATUS_INVALID_VALUE;
     if (B->data_type != A->data_type || Cm->data_type != A->data_type || computeType != A->data_type)
         return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
-    if (B->rows < A->cols || Cm->rows < A->rows || B->cols != Cm->cols)
-        return ALPHA_SPARSE_STATUS_INVALID_SIZE;
-    if (B->ld < B->cols || Cm->ld < Cm->cols || Cm->cols > INT32_MAX)
+    const int64_t m = is_transpose(opA) ? A->cols : A->rows, k = is_transpose(opA) ? A->rows : A->cols;
+    const DenseUse ub = dense_use(B, is_transpose(opB)), uc = dense_use(Cm, false);
+    if (ub.rows < k || uc.rows < m || ub.cols != uc.cols) return ALPHA_SPARSE_STATUS_INVALID_SIZE;
+    // the leading dimension spans a row of the row-major reading of the memory
+    if (B->ld < (ub.direct ? ub.cols : ub.rows) || Cm->ld < (uc.direct ? uc.cols : uc.rows) ||
+        uc.cols > INT32_MAX)
         return ALPHA_SPARSE_STATUS_INVALID_SIZE;
     if (!B->values || !Cm->values) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
     return ALPHA_SPARSE_STATUS_SUCCESS;
+}
+
+// Bytes of the row-major copies a call needs after its kernel workspace.
+void spmm_copy_bytes(const _alphasparseSpMatDescr *A, alphasparseOperation_t opA,
+                     const _alphasparse_dnmat_descr *B, alphasparseOperation_t opB,
+                     const _alphasparse_dnmat_descr *Cm, size_t *b_bytes, size_t *c_bytes)
+{
+    const size_t sv = A->data_type == ALPHA_R_64F ? 8 : 4;
+    const int64_t m = is_transpose(opA) ? A->cols : A->rows, k = is_transpose(opA) ? A->rows : A->cols;
+    const int64_t N = Cm->cols;
+    *b_bytes = dense_use(B, is_transpose(opB)).direct ? 0 : align256((size_t)k * (size_t)N * sv);
+    *c_bytes = dense_use(Cm, false).direct ? 0 : align256((size_t)m * (size_t)N * sv);
 }
 
 // Picks the workspace for a call: the caller's buffer, or the handle's own scratch when the
@@ -342,11 +540,11 @@ alphasparseStatus_t alphasparseSpMV_bufferSize(alphasparseHandle_t handle, alpha
     if (!bufferSize) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
     alphasparseStatus_t s = check_spmv(handle, opA, alpha, matA, vecX, beta, vecY, computeType);
     if (s) return s;
-    if (asx_spmv_resolve_alg((int)alg, (int32_t)matA->rows, (int32_t)matA->nnz) < 0)
+    const int32_t m_eff = (int32_t)(is_transpose(opA) ? matA->cols : matA->rows);
+    if (asx_spmv_resolve_alg((int)alg, m_eff, (int32_t)matA->nnz) < 0)
         return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
     // sized for a call without kept analysis; a call with kept analysis needs no more than this
-    *bufferSize = asx_spmv_workspace_bytes((int)alg, (int)matA->data_type, (int32_t)matA->rows,
-                                           (int32_t)matA->nnz);
+    *bufferSize = asx_spmv_workspace_bytes((int)alg, (int)matA->data_type, m_eff, (int32_t)matA->nnz);
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
@@ -357,16 +555,22 @@ alphasparseStatus_t alphasparseSpMV_analysis(alphasparseHandle_t handle, alphasp
     if (!matA) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
     alphasparseStatus_t s = check_csr(matA, opA);
     if (s) return s;
-    if (find_plan(handle, false, (int)alg, matA, 1)) return ALPHA_SPARSE_STATUS_SUCCESS;
+    // for opA = TRANSPOSE or one-based A this (re)builds the kept device copy the kernels run on:
+    // call again after changing A's values or structure
+    s = keep_derived(handle, matA, opA);
+    if (s) return s;
+    Effective eff;
+    s = make_effective(handle, matA, opA, &eff);
+    if (s) return s;
+    const _alphasparseSpMatDescr *A = &eff.d;
+    if (find_plan(handle, false, (int)alg, A, 1)) return ALPHA_SPARSE_STATUS_SUCCESS;
     HandlePlans *hp = plans_of(handle, true);
     if (!hp) return ALPHA_SPARSE_STATUS_ALLOC_FAILED;
     asx_plan *plan = nullptr;
-    int rc = asx_plan_create(&plan, 0, (int)alg, (int)matA->data_type, (int32_t)matA->rows,
-                             (int32_t)matA->cols, (int32_t)matA->nnz, matA->row_data, 1,
-                             (void *)handle->stream);
+    int rc = asx_plan_create(&plan, 0, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
+                             (int32_t)A->nnz, A->row_data, 1, (void *)handle->stream);
     if (rc) return st(rc);
-    hp->plans.push_back(KeptPlan{false, (int)alg, matA->row_data, matA->rows, matA->nnz,
-                                 (int)matA->data_type, 1, plan});
+    hp->plans.push_back(KeptPlan{false, (int)alg, A->row_data, A->rows, A->nnz, (int)A->data_type, 1, plan});
     matA->analysed = true;
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
@@ -386,28 +590,39 @@ alphasparseStatus_t alphasparseSpMV(alphasparseHandle_t handle, alphasparseOpera
 {
     alphasparseStatus_t s = check_spmv(handle, opA, alpha, matA, vecX, beta, vecY, computeType);
     if (s) return s;
-    const int32_t m = (int32_t)matA->rows, n = (int32_t)matA->cols, nnz = (int32_t)matA->nnz;
-    if (asx_spmv_resolve_alg((int)alg, m, nnz) < 0) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
-    const asx_plan *plan = find_plan(handle, false, (int)alg, matA, 1);
+    const int32_t m_eff = (int32_t)(is_transpose(opA) ? matA->cols : matA->rows);
+    if (asx_spmv_resolve_alg((int)alg, m_eff, (int32_t)matA->nnz) < 0) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
+    // without a copy kept by alphasparseSpMV_analysis, opA = TRANSPOSE and one-based A build their
+    // device copy for this call alone (from the values A holds now, as the reference does)
+    Effective eff;
+    s = make_effective(handle, matA, opA, &eff);
+    if (s) return s;
+    const _alphasparseSpMatDescr *A = &eff.d;
+    const int32_t m = (int32_t)A->rows, n = (int32_t)A->cols, nnz = (int32_t)A->nnz;
+    const asx_plan *plan = find_plan(handle, false, (int)alg, A, 1);
     const size_t need = plan ? asx_plan_workspace_bytes(plan)
-                             : asx_spmv_workspace_bytes((int)alg, (int)matA->data_type, m, nnz);
+                             : asx_spmv_workspace_bytes((int)alg, (int)A->data_type, m, nnz);
     bool ok;
     void *ws = pick_workspace(handle, externalBuffer, need, &ok);
-    if (!ok) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+    if (!ok) {
+        release_effective(handle, &eff);
+        return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+    }
     // the size of a caller's buffer is not part of the signature: it is trusted to be what
     // alphasparseSpMV_bufferSize reported
     const size_t ws_bytes = need;
     int rc;
-    if (matA->data_type == ALPHA_R_64F)
-        rc = asx_spmv_csr_f64(plan, (int)alg, m, n, nnz, *(const double *)alpha, matA->row_data,
-                              matA->col_data, (const double *)matA->val_data,
-                              (const double *)vecX->values, *(const double *)beta,
-                              (double *)vecY->values, ws, ws_bytes, (void *)handle->stream);
+    if (A->data_type == ALPHA_R_64F)
+        rc = asx_spmv_csr_f64(plan, (int)alg, m, n, nnz, *(const double *)alpha, A->row_data, A->col_data,
+                              (const double *)A->val_data, (const double *)vecX->values,
+                              *(const double *)beta, (double *)vecY->values, ws, ws_bytes,
+                              (void *)handle->stream);
     else
-        rc = asx_spmv_csr_f32(plan, (int)alg, m, n, nnz, *(const float *)alpha, matA->row_data,
-                              matA->col_data, (const float *)matA->val_data,
-                              (const float *)vecX->values, *(const float *)beta,
-                              (float *)vecY->values, ws, ws_bytes, (void *)handle->stream);
+        rc = asx_spmv_csr_f32(plan, (int)alg, m, n, nnz, *(const float *)alpha, A->row_data, A->col_data,
+                              (const float *)A->val_data, (const float *)vecX->values,
+                              *(const float *)beta, (float *)vecY->values, ws, ws_bytes,
+                              (void *)handle->stream);
+    release_effective(handle, &eff);
     return st(rc);
 }
 
@@ -445,10 +660,14 @@ alphasparseStatus_t alphasparseSpMM_bufferSize(alphasparseHandle_t handle, alpha
     if (!bufferSize) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
     alphasparseStatus_t s = check_spmm(handle, opA, opB, alpha, matA, matB, beta, matC, computeType);
     if (s) return s;
-    if (asx_spmm_resolve_alg((int)alg, (int32_t)matA->rows, (int32_t)matA->nnz, (int32_t)matC->cols) < 0)
+    const int32_t m_eff = (int32_t)(is_transpose(opA) ? matA->cols : matA->rows);
+    if (asx_spmm_resolve_alg((int)alg, m_eff, (int32_t)matA->nnz, (int32_t)matC->cols) < 0)
         return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
-    *bufferSize = asx_spmm_workspace_bytes((int)alg, (int)matA->data_type, (int32_t)matA->rows,
-                                           (int32_t)matA->nnz, (int32_t)matC->cols);
+    size_t b_bytes, c_bytes;
+    spmm_copy_bytes(matA, opA, matB, opB, matC, &b_bytes, &c_bytes);
+    *bufferSize = align256(asx_spmm_workspace_bytes((int)alg, (int)matA->data_type, m_eff, (int32_t)matA->nnz,
+                                                    (int32_t)matC->cols)) +
+                  b_bytes + c_bytes;
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
@@ -468,23 +687,33 @@ alphasparseStatus_t alphasparseSpMM_preprocess(alphasparseHandle_t handle, alpha
     alphasparseStatus_t s = check_spmm(handle, opA, opB, alpha, matA, matB, beta, matC, computeType);
     if (s) return s;
     const int ncols = (int)matC->cols;
-    if (asx_spmm_resolve_alg((int)alg, (int32_t)matA->rows, (int32_t)matA->nnz, ncols) < 0)
+    const int32_t m_eff = (int32_t)(is_transpose(opA) ? matA->cols : matA->rows);
+    if (asx_spmm_resolve_alg((int)alg, m_eff, (int32_t)matA->nnz, ncols) < 0)
         return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
-    const asx_plan *have = find_plan(handle, true, (int)alg, matA, ncols);
+    s = keep_derived(handle, matA, opA);  // (re)builds the kept copy for opA = T / one-based A
+    if (s) return s;
+    Effective eff;
+    s = make_effective(handle, matA, opA, &eff);
+    if (s) return s;
+    const _alphasparseSpMatDescr *A = &eff.d;
+    const asx_plan *have = find_plan(handle, true, (int)alg, A, ncols);
     if (!have) {
         HandlePlans *hp = plans_of(handle, true);
         if (!hp) return ALPHA_SPARSE_STATUS_ALLOC_FAILED;
         asx_plan *plan = nullptr;
-        int rc = asx_spmm_plan_create(&plan, (int)alg, (int)matA->data_type, (int32_t)matA->rows,
-                                      (int32_t)matA->cols, (int32_t)matA->nnz, matA->row_data,
-                                      matA->col_data, matA->val_data, ncols, (void *)handle->stream);
+        int rc = asx_spmm_plan_create(&plan, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
+                                      (int32_t)A->nnz, A->row_data, A->col_data, A->val_data, ncols,
+                                      (void *)handle->stream);
         if (rc) return st(rc);
-        hp->plans.push_back(KeptPlan{true, (int)alg, matA->row_data, matA->rows, matA->nnz,
-                                     (int)matA->data_type, ncols, plan});
+        hp->plans.push_back(KeptPlan{true, (int)alg, A->row_data, A->rows, A->nnz, (int)A->data_type, ncols, plan});
         have = plan;
         matA->analysed = true;
     }
-    if (bufferSize) *bufferSize = asx_plan_workspace_bytes(have);
+    if (bufferSize) {
+        size_t b_bytes, c_bytes;
+        spmm_copy_bytes(matA, opA, matB, opB, matC, &b_bytes, &c_bytes);
+        *bufferSize = align256(asx_plan_workspace_bytes(have)) + b_bytes + c_bytes;
+    }
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
@@ -497,25 +726,57 @@ alphasparseStatus_t alphasparseSpMM(alphasparseHandle_t handle, alphasparseOpera
 {
     alphasparseStatus_t s = check_spmm(handle, opA, opB, alpha, matA, matB, beta, matC, computeType);
     if (s) return s;
-    const int32_t m = (int32_t)matA->rows, k = (int32_t)matA->cols, nnz = (int32_t)matA->nnz;
     const int32_t ncols = (int32_t)matC->cols;
-    if (asx_spmm_resolve_alg((int)alg, m, nnz, ncols) < 0) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
-    const asx_plan *plan = find_plan(handle, true, (int)alg, matA, ncols);
-    const size_t need = plan ? asx_plan_workspace_bytes(plan)
-                             : asx_spmm_workspace_bytes((int)alg, (int)matA->data_type, m, nnz, ncols);
+    const int32_t m_eff = (int32_t)(is_transpose(opA) ? matA->cols : matA->rows);
+    if (asx_spmm_resolve_alg((int)alg, m_eff, (int32_t)matA->nnz, ncols) < 0) return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
+    Effective eff;
+    s = make_effective(handle, matA, opA, &eff);
+    if (s) return s;
+    const _alphasparseSpMatDescr *A = &eff.d;
+    const int32_t m = (int32_t)A->rows, k = (int32_t)A->cols, nnz = (int32_t)A->nnz;
+    const int vt = (int)A->data_type;
+    const asx_plan *plan = find_plan(handle, true, (int)alg, A, ncols);
+    const size_t kernel_need =
+        plan ? asx_plan_workspace_bytes(plan) : asx_spmm_workspace_bytes((int)alg, vt, m, nnz, ncols);
+    size_t b_bytes, c_bytes;
+    spmm_copy_bytes(matA, opA, matB, opB, matC, &b_bytes, &c_bytes);
+    const size_t need = b_bytes + c_bytes ? align256(kernel_need) + b_bytes + c_bytes : kernel_need;
     bool ok;
     void *ws = pick_workspace(handle, externalBuffer, need, &ok);
-    if (!ok) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
-    int rc;
-    if (matA->data_type == ALPHA_R_64F)
-        rc = asx_spmm_csr_f64(plan, (int)alg, m, k, nnz, ncols, *(const double *)alpha, matA->row_data,
-                              matA->col_data, (const double *)matA->val_data,
-                              (const double *)matB->values, matB->ld, *(const double *)beta,
-                              (double *)matC->values, matC->ld, ws, need, (void *)handle->stream);
-    else
-        rc = asx_spmm_csr_f32(plan, (int)alg, m, k, nnz, ncols, *(const float *)alpha, matA->row_data,
-                              matA->col_data, (const float *)matA->val_data,
-                              (const float *)matB->values, matB->ld, *(const float *)beta,
-                              (float *)matC->values, matC->ld, ws, need, (void *)handle->stream);
+    if (!ok) {
+        release_effective(handle, &eff);
+        return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+    }
+    void *stream = (void *)handle->stream;
+    const bool beta_zero = vt == ALPHA_R_64F ? *(const double *)beta == 0.0 : *(const float *)beta == 0.0f;
+    // row-major views of B and C: the caller's memory, or copies behind the kernel workspace
+    const void *Bv = matB->values;
+    int64_t ldb = matB->ld;
+    void *Cv = matC->values;
+    int64_t ldc = matC->ld;
+    int rc = 0;
+    if (b_bytes) {
+        void *Bc = (char *)ws + align256(kernel_need);
+        rc = asx_dense_transpose(vt, ncols, k, matB->values, matB->ld, Bc, ncols, stream);
+        Bv = Bc;
+        ldb = ncols;
+    }
+    if (!rc && c_bytes) {
+        Cv = (char *)ws + align256(kernel_need) + b_bytes;
+        ldc = ncols;
+        if (!beta_zero) rc = asx_dense_transpose(vt, ncols, m, matC->values, matC->ld, Cv, ncols, stream);
+    }
+    if (!rc) {
+        if (vt == ALPHA_R_64F)
+            rc = asx_spmm_csr_f64(plan, (int)alg, m, k, nnz, ncols, *(const double *)alpha, A->row_data,
+                                  A->col_data, (const double *)A->val_data, (const double *)Bv, ldb,
+                                  *(const double *)beta, (double *)Cv, ldc, ws, kernel_need, stream);
+        else
+            rc = asx_spmm_csr_f32(plan, (int)alg, m, k, nnz, ncols, *(const float *)alpha, A->row_data,
+                                  A->col_data, (const float *)A->val_data, (const float *)Bv, ldb,
+                                  *(const float *)beta, (float *)Cv, ldc, ws, kernel_need, stream);
+    }
+    if (!rc && c_bytes) rc = asx_dense_transpose(vt, m, ncols, Cv, ncols, matC->values, matC->ld, stream);
+    release_effective(handle, &eff);
     return st(rc);
 }

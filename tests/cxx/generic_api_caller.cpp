@@ -53,16 +53,24 @@ static T *to_device(const std::vector<T> &h)
     return d;
 }
 
+// Operand variants of a case: opA / opB = TRANSPOSE, one-based indices, column-major B / C.
+struct Variant {
+    int trans_a = 0, base = 0, col_major_b = 0, col_major_c = 0, trans_b = 0;
+};
+
 template <typename T>
 static int run_case(const std::string &dir, const char *op, long m, long n, long nnz, long ncols, int alg,
-                    double alpha_d, double beta_d, int analysis, alphasparseDataType dt)
+                    double alpha_d, double beta_d, int analysis, alphasparseDataType dt, const Variant &v)
 {
     auto rp = read_bin<int>(dir + "/row_ptr.bin", m + 1);
     auto col = read_bin<int>(dir + "/col.bin", nnz);
     auto val = read_bin<T>(dir + "/val.bin", nnz);
     const bool mm = std::strcmp(op, "spmm") == 0;
-    auto xin = read_bin<T>(dir + "/x.bin", mm ? n * ncols : n);
-    auto yin = read_bin<T>(dir + "/y.bin", mm ? m * ncols : m);
+    const long in_len = v.trans_a ? m : n, out_len = v.trans_a ? n : m;  // of op(A)
+    auto xin = read_bin<T>(dir + "/x.bin", mm ? in_len * ncols : in_len);
+    auto yin = read_bin<T>(dir + "/y.bin", mm ? out_len * ncols : out_len);
+    const auto opA = v.trans_a ? ALPHA_SPARSE_OPERATION_TRANSPOSE : ALPHA_SPARSE_OPERATION_NON_TRANSPOSE;
+    const auto opB = v.trans_b ? ALPHA_SPARSE_OPERATION_TRANSPOSE : ALPHA_SPARSE_OPERATION_NON_TRANSPOSE;
     int *d_rp = to_device(rp), *d_col = to_device(col);
     T *d_val = to_device(val), *d_x = to_device(xin), *d_y = to_device(yin);
     const T alpha = (T)alpha_d, beta = (T)beta_d;
@@ -71,26 +79,26 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
     if (alphasparseGetHandle(&handle) != ALPHA_SPARSE_STATUS_SUCCESS) return 4;
     alphasparseSpMatDescr_t A;
     if (alphasparseCreateCsr(&A, (int)m, (int)n, (int)nnz, d_rp, d_col, d_val, ALPHA_SPARSE_INDEXTYPE_I32,
-                             ALPHA_SPARSE_INDEXTYPE_I32, ALPHA_SPARSE_INDEX_BASE_ZERO, dt))
+                             ALPHA_SPARSE_INDEXTYPE_I32,
+                             v.base ? ALPHA_SPARSE_INDEX_BASE_ONE : ALPHA_SPARSE_INDEX_BASE_ZERO, dt))
         return 5;
     size_t bytes = 0;
     void *buffer = nullptr;
     alphasparseStatus_t s;
     if (!mm) {
         alphasparseDnVecDescr_t X, Y;
-        if (alphasparseCreateDnVec(&X, n, d_x, dt) || alphasparseCreateDnVec(&Y, m, d_y, dt)) return 6;
-        s = alphasparseSpMV_bufferSize(handle, ALPHA_SPARSE_OPERATION_NON_TRANSPOSE, &alpha, A, X, &beta, Y, dt,
+        if (alphasparseCreateDnVec(&X, in_len, d_x, dt) || alphasparseCreateDnVec(&Y, out_len, d_y, dt)) return 6;
+        s = alphasparseSpMV_bufferSize(handle, opA, &alpha, A, X, &beta, Y, dt,
                                        (alphasparseSpMVAlg_t)alg, &bytes);
         if (s) return 10 + (int)s;
         HIP_OK(hipMalloc(&buffer, bytes ? bytes : 1));
         if (analysis) {
-            s = alphasparseSpMV_analysis(handle, ALPHA_SPARSE_OPERATION_NON_TRANSPOSE, A, (alphasparseSpMVAlg_t)alg);
+            s = alphasparseSpMV_analysis(handle, opA, A, (alphasparseSpMVAlg_t)alg);
             if (s) return 30 + (int)s;
         }
         for (int rep = 0; rep < 2; ++rep) {  // twice: the second call must not depend on the first
             HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
-            s = alphasparseSpMV(handle, ALPHA_SPARSE_OPERATION_NON_TRANSPOSE, &alpha, A, X, &beta, Y, dt,
-                                (alphasparseSpMVAlg_t)alg, buffer);
+            s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
         }
         if (analysis && alphasparseSpMV_clear(handle, (alphasparseSpMVAlg_t)alg)) return 7;
@@ -98,22 +106,26 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
         alphasparseDestroyDnVec(Y);
     } else {
         alphasparseDnMatDescr_t B, C;
-        if (alphasparseCreateDnMat(&B, n, ncols, ncols, d_x, dt, ALPHASPARSE_ORDER_ROW) ||
-            alphasparseCreateDnMat(&C, m, ncols, ncols, d_y, dt, ALPHASPARSE_ORDER_ROW))
+        // the arrays are packed: the leading dimension is the length of a row (row-major) or of a
+        // column (column-major) of the matrix the descriptor describes
+        const long b_rows = v.trans_b ? ncols : in_len, b_cols = v.trans_b ? in_len : ncols;
+        if (alphasparseCreateDnMat(&B, b_rows, b_cols, v.col_major_b ? b_rows : b_cols, d_x, dt,
+                                   v.col_major_b ? ALPHASPARSE_ORDER_COL : ALPHASPARSE_ORDER_ROW) ||
+            alphasparseCreateDnMat(&C, out_len, ncols, v.col_major_c ? out_len : ncols, d_y, dt,
+                                   v.col_major_c ? ALPHASPARSE_ORDER_COL : ALPHASPARSE_ORDER_ROW))
             return 6;
-        const auto N = ALPHA_SPARSE_OPERATION_NON_TRANSPOSE;
-        s = alphasparseSpMM_bufferSize(handle, N, N, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, &bytes);
+        s = alphasparseSpMM_bufferSize(handle, opA, opB, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, &bytes);
         if (s) return 10 + (int)s;
         HIP_OK(hipMalloc(&buffer, bytes ? bytes : 1));
         if (analysis) {
             size_t b2 = 0;
-            s = alphasparseSpMM_preprocess(handle, N, N, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, &b2);
+            s = alphasparseSpMM_preprocess(handle, opA, opB, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, &b2);
             if (s) return 30 + (int)s;
             if (b2 > bytes) return 8;
         }
         for (int rep = 0; rep < 2; ++rep) {
             HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
-            s = alphasparseSpMM(handle, N, N, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, buffer);
+            s = alphasparseSpMM(handle, opA, opB, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
         }
         alphasparseDestroyDnMat(B);
@@ -155,9 +167,25 @@ static int selftest()
     HIP_OK(hipDeviceSynchronize());
     HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
     EXPECT(y[0] == 2.0 * 21.0 + 50.0 && y[1] == 2.0 * 30.0 + 50.0);
+    // opA = TRANSPOSE computes with A^T = [[1,0],[2,3]] and leaves the caller's arrays as they were
+    HIP_OK(hipMemcpy(d_y, x.data(), sizeof(double) * 2, hipMemcpyHostToDevice));
+    for (int rep = 0; rep < 2; ++rep) {
+        HIP_OK(hipMemcpy(d_y, x.data(), sizeof(double) * 2, hipMemcpyHostToDevice));
+        EXPECT(alphasparseSpMV(h, ALPHA_SPARSE_OPERATION_TRANSPOSE, &alpha, A, X, &beta, Y, ALPHA_R_64F,
+                               ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) == 0);
+        HIP_OK(hipDeviceSynchronize());
+        HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
+        EXPECT(y[0] == 2.0 * 1.0 + 0.5 && y[1] == 2.0 * 32.0 + 5.0);
+    }
+    {
+        std::vector<int> rp2(3), col2(3);
+        std::vector<double> val2(3);
+        HIP_OK(hipMemcpy(rp2.data(), d_rp, sizeof(int) * 3, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(col2.data(), d_col, sizeof(int) * 3, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(val2.data(), d_val, sizeof(double) * 3, hipMemcpyDeviceToHost));
+        EXPECT(rp2 == rp && col2 == col && val2 == val);
+    }
     // what is not supported says so
-    EXPECT(alphasparseSpMV(h, ALPHA_SPARSE_OPERATION_TRANSPOSE, &alpha, A, X, &beta, Y, ALPHA_R_64F,
-                           ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) == ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
     EXPECT(alphasparseSpMV(h, N, &alpha, A, Xf, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) ==
            ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
     EXPECT(alphasparseSpMV(h, N, &alpha, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_COO, nullptr) ==
@@ -170,10 +198,41 @@ static int selftest()
            bytes == 0);
     EXPECT(alphasparseSpMV_bufferSize(h, N, &alpha, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_MERGE, &bytes) == 0 &&
            bytes > 0);
-    A->idx_base = ALPHA_SPARSE_INDEX_BASE_ONE;
-    EXPECT(alphasparseSpMV(h, N, &alpha, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) ==
-           ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
-    A->idx_base = ALPHA_SPARSE_INDEX_BASE_ZERO;
+    // one-based indices
+    {
+        std::vector<int> rp1 = {1, 3, 4}, col1 = {1, 2, 2};
+        int *d_rp1 = to_device(rp1), *d_col1 = to_device(col1);
+        alphasparseSpMatDescr_t A1;
+        EXPECT(alphasparseCreateCsr(&A1, 2, 2, 3, d_rp1, d_col1, d_val, ALPHA_SPARSE_INDEXTYPE_I32,
+                                    ALPHA_SPARSE_INDEXTYPE_I32, ALPHA_SPARSE_INDEX_BASE_ONE, ALPHA_R_64F) == 0);
+        HIP_OK(hipMemcpy(d_y, x.data(), sizeof(double) * 2, hipMemcpyHostToDevice));
+        EXPECT(alphasparseSpMV(h, N, &alpha, A1, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) == 0);
+        HIP_OK(hipDeviceSynchronize());
+        HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
+        EXPECT(y[0] == 42.5 && y[1] == 65.0);
+        // kept copy: analysis, two calls, clear
+        EXPECT(alphasparseSpMV_analysis(h, ALPHA_SPARSE_OPERATION_TRANSPOSE, A1, ALPHA_SPARSE_SPMV_ALG_MERGE) == 0);
+        size_t nb = 0;
+        EXPECT(alphasparseSpMV_bufferSize(h, ALPHA_SPARSE_OPERATION_TRANSPOSE, &alpha, A1, X, &beta, Y, ALPHA_R_64F,
+                                          ALPHA_SPARSE_SPMV_ALG_MERGE, &nb) == 0);
+        void *tb = nullptr;
+        HIP_OK(hipMalloc(&tb, nb ? nb : 1));
+        for (int rep = 0; rep < 2; ++rep) {
+            HIP_OK(hipMemcpy(d_y, x.data(), sizeof(double) * 2, hipMemcpyHostToDevice));
+            EXPECT(alphasparseSpMV(h, ALPHA_SPARSE_OPERATION_TRANSPOSE, &alpha, A1, X, &beta, Y, ALPHA_R_64F,
+                                   ALPHA_SPARSE_SPMV_ALG_MERGE, tb) == 0);
+            HIP_OK(hipDeviceSynchronize());
+            HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
+            EXPECT(y[0] == 2.5 && y[1] == 69.0);
+        }
+        EXPECT(alphasparseSpMV_clear(h, ALPHA_SPARSE_SPMV_ALG_MERGE) == 0);
+        alphasparseDestroySpMat(A1);
+        (void)hipFree(tb);
+        (void)hipFree(d_rp1);
+        (void)hipFree(d_col1);
+    }
+    EXPECT(alphasparseSpMV(h, (alphasparseOperation_t)7, &alpha, A, X, &beta, Y, ALPHA_R_64F,
+                           ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) == ALPHA_SPARSE_STATUS_INVALID_VALUE);
     // analysis is kept on the handle, found again, and cleared
     EXPECT(alphasparseSpMV_analysis(h, N, A, ALPHA_SPARSE_SPMV_ALG_DEFAULT) == 0 && A->analysed);
     EXPECT(alphasparseSpMV_analysis(h, N, A, ALPHA_SPARSE_SPMV_ALG_DEFAULT) == 0);
@@ -213,13 +272,27 @@ static int selftest()
         (void)hipFree(d_ri);
         (void)hipFree(d_out);
     }
-    // SpMM: column-major operands are refused, row-major run
-    alphasparseDnMatDescr_t B, C, Bc;
+    // SpMM: row-major and column-major operands; a leading dimension shorter than a column is refused
+    alphasparseDnMatDescr_t B, C, Bc, Bbad;
     EXPECT(alphasparseCreateDnMat(&B, 2, 1, 1, d_x, ALPHA_R_64F, ALPHASPARSE_ORDER_ROW) == 0);
     EXPECT(alphasparseCreateDnMat(&C, 2, 1, 1, d_y, ALPHA_R_64F, ALPHASPARSE_ORDER_ROW) == 0);
     EXPECT(alphasparseCreateDnMat(&Bc, 2, 1, 2, d_x, ALPHA_R_64F, ALPHASPARSE_ORDER_COL) == 0);
-    EXPECT(alphasparseSpMM(h, N, N, &alpha, A, Bc, &beta, C, ALPHA_R_64F, ALPHASPARSE_SPMM_ALG_DEFAULT, nullptr) ==
-           ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
+    EXPECT(alphasparseCreateDnMat(&Bbad, 2, 1, 1, d_x, ALPHA_R_64F, ALPHASPARSE_ORDER_COL) == 0);
+    EXPECT(alphasparseSpMM(h, N, N, &alpha, A, Bbad, &beta, C, ALPHA_R_64F, ALPHASPARSE_SPMM_ALG_DEFAULT, nullptr) ==
+           ALPHA_SPARSE_STATUS_INVALID_SIZE);
+    {
+        size_t nb = 0;
+        EXPECT(alphasparseSpMM_bufferSize(h, N, N, &alpha, A, Bc, &beta, C, ALPHA_R_64F, ALPHASPARSE_SPMM_ALG_DEFAULT,
+                                          &nb) == 0 && nb > 0);
+        void *tb = nullptr;
+        HIP_OK(hipMalloc(&tb, nb));
+        HIP_OK(hipMemcpy(d_y, x.data(), sizeof(double) * 2, hipMemcpyHostToDevice));
+        EXPECT(alphasparseSpMM(h, N, N, &alpha, A, Bc, &beta, C, ALPHA_R_64F, ALPHASPARSE_SPMM_ALG_DEFAULT, tb) == 0);
+        HIP_OK(hipDeviceSynchronize());
+        HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
+        EXPECT(y[0] == 42.5 && y[1] == 65.0);
+        (void)hipFree(tb);
+    }
     EXPECT(alphasparseSpMM(h, N, N, &alpha, A, B, &beta, C, ALPHA_R_64F, ALPHASPARSE_SPMM_COO_ALG1, nullptr) ==
            ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
     HIP_OK(hipMemcpy(d_y, x.data(), sizeof(double) * 2, hipMemcpyHostToDevice));
@@ -249,10 +322,12 @@ int main(int argc, char **argv)
     if (std::fscanf(f, "%15s %15s %ld %ld %ld %ld %d %lf %lf %d", op, dtype, &m, &n, &nnz, &ncols, &alg, &alpha, &beta,
                     &analysis) != 10)
         return 1;
+    Variant v;  // optional: trans_a base col_major_b col_major_c trans_b
+    if (std::fscanf(f, "%d %d %d %d %d", &v.trans_a, &v.base, &v.col_major_b, &v.col_major_c, &v.trans_b) < 0) v = Variant();
     std::fclose(f);
     int rc = std::strcmp(dtype, "f64") == 0
-                 ? run_case<double>(dir, op, m, n, nnz, ncols, alg, alpha, beta, analysis, ALPHA_R_64F)
-                 : run_case<float>(dir, op, m, n, nnz, ncols, alg, alpha, beta, analysis, ALPHA_R_32F);
+                 ? run_case<double>(dir, op, m, n, nnz, ncols, alg, alpha, beta, analysis, ALPHA_R_64F, v)
+                 : run_case<float>(dir, op, m, n, nnz, ncols, alg, alpha, beta, analysis, ALPHA_R_32F, v);
     std::printf("rc %d\n", rc);
     return rc;
 }

@@ -14,14 +14,18 @@ pytestmark = pytest.mark.gpu
 EXE = os.path.join(ROOT, "tests", "cxx", "generic_api_caller")
 
 
-def _run_case(tmp_path, op, dtype, rp, col, val, x, y, ncols, alg, alpha, beta, analysis):
-    d = tmp_path / f"{op}_{np.dtype(dtype).name}_{alg}_{analysis}"
+def _run_case(tmp_path, op, dtype, rp, col, val, x, y, ncols, alg, alpha, beta, analysis, variant=(0, 0, 0, 0, 0),
+              n=None):
+    """variant = (trans_a, idx_base, col_major_b, col_major_c, trans_b); n = columns of A."""
+    d = tmp_path / f"{op}_{np.dtype(dtype).name}_{alg}_{analysis}_{''.join(map(str, variant))}"
     d.mkdir()
     for name, a in (("row_ptr", rp), ("col", col), ("val", val), ("x", x), ("y", y)):
         np.ascontiguousarray(a).tofile(d / f"{name}.bin")
     tag = "f64" if np.dtype(dtype) == np.float64 else "f32"
-    n = x.size // ncols
-    (d / "meta.txt").write_text(f"{op} {tag} {rp.size - 1} {n} {col.size} {ncols} {alg} {alpha!r} {beta!r} {analysis}\n")
+    if n is None:
+        n = x.size // ncols
+    (d / "meta.txt").write_text(f"{op} {tag} {rp.size - 1} {n} {col.size} {ncols} {alg} {alpha!r} {beta!r} {analysis}\n"
+                                + " ".join(map(str, variant)) + "\n")
     r = subprocess.run([EXE, str(d)], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
     return np.fromfile(d / "out.bin", dtype=dtype)
@@ -62,3 +66,83 @@ def test_spmm_through_generic_api(tmp_path, oracle):
     for alg, analysis in ((0, 0), (0, 1), (5, 0), (6, 0), (7, 1), (8, 0), (9, 0), (10, 1)):
         got = _run_case(tmp_path, "spmm", np.float32, rp, col, val, B, C0, n, alg, alpha, beta, analysis)
         assert_close(got, ref, scale, np.float32, f"spmm alg {alg} analysis {analysis}")
+
+
+def _transpose_csr(rp, col, val, n):
+    """A^T with the stored elements of each row in ascending row of A, duplicates in stored order."""
+    rows = np.repeat(np.arange(rp.size - 1, dtype=np.int32), np.diff(rp))
+    order = np.argsort(col, kind="stable")
+    rp_t = np.zeros(n + 1, dtype=np.int32)
+    np.cumsum(np.bincount(col, minlength=n), out=rp_t[1:])
+    return rp_t, rows[order].astype(np.int32), val[order]
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_spmv_transpose_and_one_based(tmp_path, oracle, dtype):
+    """opA = TRANSPOSE and idx_base = ONE against the oracle run on the explicitly transposed /
+    rebased matrix (a rectangular one, so a mix-up of rows and columns cannot pass)."""
+    rng = np.random.default_rng(51)
+    lens = np.r_[np.minimum(rng.zipf(1.7, 9000), 3000), 12000, np.zeros(25, int)]
+    m, n = lens.size, 15000
+    rp, col, val = csr_from_lengths(lens, n, 52, dtype)
+    alpha, beta = 2.1, 3.2
+    x_n = rng.uniform(-1, 1, n).astype(dtype)
+    y_m = rng.uniform(-1, 1, m).astype(dtype)
+    x_m = rng.uniform(-1, 1, m).astype(dtype)
+    y_n = rng.uniform(-1, 1, n).astype(dtype)
+    ref_n = oracle.spmv(rp, col, val, x_n, dtype(alpha), dtype(beta), y_m, 4)
+    rp_t, col_t, val_t = _transpose_csr(rp, col, val, n)
+    ref_t = oracle.spmv(rp_t, col_t, val_t, x_m, dtype(alpha), dtype(beta), y_n, 4)
+    scale_n = spmv_scale(rp, col, val, x_n, alpha, beta, y_m)
+    scale_t = spmv_scale(rp_t, col_t, val_t, x_m, alpha, beta, y_n)
+    for alg, analysis in ((0, 0), (0, 1), (9, 1), (6, 0), (3, 1)):
+        for base in (0, 1):
+            if base:
+                got = _run_case(tmp_path, "spmv", dtype, rp + 1, col + 1, val, x_n, y_m, 1, alg, alpha, beta, analysis,
+                                (0, 1, 0, 0, 0), n=n)
+                assert_close(got, ref_n, scale_n, dtype, f"one-based alg {alg} analysis {analysis}")
+            got = _run_case(tmp_path, "spmv", dtype, rp + base, col + base, val, x_m, y_n, 1, alg, alpha, beta, analysis,
+                            (1, base, 0, 0, 0), n=n)
+            assert_close(got, ref_t, scale_t, dtype, f"transpose base {base} alg {alg} analysis {analysis}")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_spmm_layouts_and_ops(tmp_path, oracle, dtype):
+    """Column-major B / C, opB = TRANSPOSE, opA = TRANSPOSE and one-based A: every variant must give
+    the row-major, non-transposed result of the same product."""
+    rng = np.random.default_rng(53)
+    lens = np.r_[np.minimum(rng.zipf(2.0, 1500) * 2, 700), 2000, np.zeros(9, int)]
+    m, k, ncols = lens.size, 2100, 40
+    rp, col, val = csr_from_lengths(lens, k, 54, dtype)
+    alpha, beta = 2.0, 3.0
+    B = rng.uniform(-1, 1, (k, ncols)).astype(dtype)
+    C0 = rng.uniform(-1, 1, (m, ncols)).astype(dtype)
+    ref = oracle.spmm(rp, col, val, B.ravel(), ncols, alpha, beta, C0.ravel(), 4).reshape(m, ncols)
+    scale = spmm_scale(rp, col, val, B.ravel(), ncols, alpha, beta, C0.ravel()).reshape(m, ncols)
+    for alg, analysis, (cb, cc, tb) in ((0, 0, (1, 0, 0)), (0, 1, (0, 1, 0)), (7, 0, (1, 1, 0)), (5, 0, (0, 0, 1)),
+                                        (0, 1, (1, 1, 1)), (10, 1, (1, 1, 0))):
+        # memory of B: op(B) = B.  Row-major without opB and column-major with opB hold B itself
+        b_mem = B if cb == tb else B.T
+        c_mem = C0.T if cc else C0
+        got = _run_case(tmp_path, "spmm", dtype, rp, col, val, np.ascontiguousarray(b_mem).ravel(),
+                        np.ascontiguousarray(c_mem).ravel(), ncols, alg, alpha, beta, analysis, (0, 0, cb, cc, tb), n=k)
+        got = got.reshape(ncols, m).T if cc else got.reshape(m, ncols)
+        assert_close(got.ravel(), ref.ravel(), scale.ravel(), dtype, f"alg {alg} analysis {analysis} cb{cb} cc{cc} tb{tb}")
+    # beta = 0 with a column-major C full of NaN: C must not be read
+    nanC = np.full((ncols, m), np.nan, dtype=dtype)
+    ref0 = oracle.spmm(rp, col, val, B.ravel(), ncols, alpha, 0.0, np.zeros(m * ncols, dtype), 4)
+    got = _run_case(tmp_path, "spmm", dtype, rp, col, val, B.ravel(), nanC.ravel(), ncols, 0, alpha, 0.0, 0,
+                    (0, 0, 0, 1, 0), n=k)
+    assert_close(got.reshape(ncols, m).T.ravel(), ref0, scale.ravel(), dtype, "beta 0, column-major C")
+    # opA = TRANSPOSE (one-based): C (k x ncols) = alpha * A^T * Bm (m x ncols) + beta * C
+    rp_t, col_t, val_t = _transpose_csr(rp, col, val, k)
+    Bm = rng.uniform(-1, 1, (m, ncols)).astype(dtype)
+    Ck = rng.uniform(-1, 1, (k, ncols)).astype(dtype)
+    ref_t = oracle.spmm(rp_t, col_t, val_t, Bm.ravel(), ncols, alpha, beta, Ck.ravel(), 4)
+    scale_t = spmm_scale(rp_t, col_t, val_t, Bm.ravel(), ncols, alpha, beta, Ck.ravel())
+    for alg, analysis, cc in ((0, 0, 0), (0, 1, 1), (5, 1, 0)):
+        c_mem = Ck.T if cc else Ck
+        got = _run_case(tmp_path, "spmm", dtype, rp + 1, col + 1, val, Bm.ravel(), np.ascontiguousarray(c_mem).ravel(),
+                        ncols, alg, alpha, beta, analysis, (1, 1, 0, cc, 0), n=k)
+        got = got.reshape(ncols, k).T if cc else got.reshape(k, ncols)
+        assert_close(got.ravel(), ref_t, scale_t, dtype, f"opA=T alg {alg} analysis {analysis} cc{cc}")

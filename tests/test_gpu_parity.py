@@ -432,6 +432,53 @@ def test_coo_sort_and_coo2csr(torch, capi, oracle):
             assert np.array_equal(v.cpu().numpy(), val.astype(dtype))
 
 
+# ------------------------------------------------------------------ operand conversions, bit exact
+def test_csr_transpose_rebase_dense_transpose(torch, capi):
+    """The transposed copy must equal a stable counting transpose (each row of A^T in ascending row
+    of A, duplicate entries in stored order): checked against numpy's stable argsort, with the
+    transpose of the transpose giving A back, for both index bases."""
+    rng = np.random.default_rng(81)
+    for name, lens in analysis_shapes().items():
+        n = int(max(np.max(lens), 64)) + 5
+        rp, col, val = csr_from_lengths(lens, n, 12, np.float64)
+        if col.size:  # duplicate entries: repeat some columns inside their rows
+            dup = rng.integers(0, col.size, max(col.size // 20, 1))
+            dup = dup[dup + 1 < col.size]
+            rows = np.repeat(np.arange(rp.size - 1), np.diff(rp))
+            keep = rows[dup] == rows[dup + 1]
+            col[dup[keep] + 1] = col[dup[keep]]
+        m = rp.size - 1
+        rows = np.repeat(np.arange(m, dtype=np.int32), np.diff(rp))
+        order = np.argsort(col, kind="stable")
+        rp_t = np.zeros(n + 1, dtype=np.int32)
+        np.cumsum(np.bincount(col, minlength=n), out=rp_t[1:])
+        for dtype in (np.float64, np.float32):
+            v = val.astype(dtype)
+            for base in (0, 1):
+                got = capi.csr_transpose(dev(torch, rp + base), dev(torch, col + base), dev(torch, v), n, idx_base=base)
+                torch.cuda.synchronize()
+                assert np.array_equal(got[0].cpu().numpy(), rp_t), (name, base)
+                assert np.array_equal(got[1].cpu().numpy(), rows[order]), (name, base)
+                assert np.array_equal(got[2].cpu().numpy(), v[order]), (name, base)
+            back = capi.csr_transpose(got[0], got[1], got[2], m)
+            torch.cuda.synchronize()
+            assert np.array_equal(back[0].cpu().numpy(), rp)
+            assert np.array_equal(back[1].cpu().numpy(), col) and np.array_equal(back[2].cpu().numpy(), v)
+        r0, c0 = capi.csr_rebase(dev(torch, rp + 1), dev(torch, col + 1), 1)
+        torch.cuda.synchronize()
+        assert np.array_equal(r0.cpu().numpy(), rp) and np.array_equal(c0.cpu().numpy(), col)
+    for dtype in (np.float32, np.float64):
+        for rows_, cols_, ld_in, ld_out in ((1, 1, 1, 1), (64, 64, 64, 64), (65, 63, 70, 67), (300, 7, 7, 300), (3, 1000, 1001, 5)):
+            a = rng.uniform(-1, 1, rows_ * ld_in).astype(dtype)
+            out = np.full(cols_ * ld_out, 7.0, dtype=dtype)
+            d_out = dev(torch, out)
+            capi.dense_transpose(dev(torch, a), rows_, cols_, ld_in, d_out, ld_out)
+            torch.cuda.synchronize()
+            want = out.reshape(cols_, ld_out).copy()
+            want[:, :rows_] = a.reshape(rows_, ld_in)[:, :cols_].T
+            assert np.array_equal(d_out.cpu().numpy().reshape(cols_, ld_out), want), (rows_, cols_)
+
+
 # ------------------------------------------------------------------ randomised shapes, every SpMV kernel
 def test_spmv_random_shapes_all_kernels(torch, capi, oracle):
     rng = np.random.default_rng(2024)
