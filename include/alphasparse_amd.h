@@ -147,6 +147,15 @@ int asx_csr_rebase(int32_t m, int32_t nnz, int32_t idx_base, const int32_t *d_ro
 int asx_dense_transpose(int value_type, int64_t rows, int64_t cols, const void *d_in, int64_t ld_in,
                         void *d_out, int64_t ld_out, void *stream);
 
+/* Reads a MatrixMarket coordinate file into HOST COO arrays (zero-based, file order; symmetric,
+ * Hermitian and skew-symmetric files expanded by following every off-diagonal entry with its
+ * mirror image carrying the same value; pattern entries are 1; the real part of complex entries).
+ * alpha_read_coo, hip/test/io.hip:100-330.  The arrays are malloc'ed: release with
+ * asx_host_free.  value_type selects float or double values. */
+int asx_mtx_read(const char *path, int value_type, int32_t *m, int32_t *n, int32_t *nnz, int32_t **h_row,
+                 int32_t **h_col, void **h_val);
+void asx_host_free(void *p);
+
 /* ------------------------------------------------------------------------------------
  * Plans: analysis results kept across calls (the reference recomputes them inside every
  * SpMV/SpMM call; its alphasparseSpMV_analysis is a stub, hip/kernel/level2/alphasparse_spmv.hip:

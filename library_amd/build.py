@@ -17,7 +17,7 @@ WORKLOADS = os.path.join(HERE, "libasx_workloads.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 HIP_SOURCES = ["asx_analysis.hip", "asx_spmv.hip", "asx_spmm.hip", "asx_capi.hip", "asx_probes.hip", "asx_blocked.hip", "asx_coo.hip", "asx_convert.hip"]
-CXX_SOURCES = ["asx_rowblocks.cpp", "alphasparse_generic.cpp"]
+CXX_SOURCES = ["asx_rowblocks.cpp", "alphasparse_generic.cpp", "asx_mtx.cpp"]
 
 # packed-fp32 code generation is switched off for all device code
 HIP_FLAGS = ["--offload-arch=gfx950", "-std=c++17", "-O3", "-fPIC", "-Wall", "-Wno-unused-function",
@@ -86,9 +86,23 @@ def build_cxx_example():
     return exe
 
 
+def build_cli():
+    """The command-line driver (MatrixMarket file -> SpMV / SpMM timings), library_amd/bin/."""
+    src = os.path.join(HERE, "cli", "alphasparse_amd_cli.cpp")
+    bindir = os.path.join(HERE, "bin")
+    os.makedirs(bindir, exist_ok=True)
+    exe = os.path.join(bindir, "alphasparse_amd_cli")
+    _run([HIPCC, "-x", "hip", "--offload-arch=gfx950", "-std=c++17", "-O2", "-Wall",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          "-I" + os.path.join(ROOT, "include"), src, "-o", exe,
+          "-L" + HERE, "-lalphasparse_amd", "-Wl,-rpath," + HERE, "-Wl,-rpath,$ORIGIN/.."])
+    return exe
+
+
 def build_all():
     build_workloads()
     build_library()
+    build_cli()
     build_oracle()
 
 

@@ -26,7 +26,7 @@ EXPORTS = [
     "asx_version", "asx_device_info", "asx_row_length_histogram", "asx_partition_rows_by_nnz",
     "asx_nnz_split_rows", "asx_merge_path_search", "asx_loadbalance_nwarps",
     "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_coo2csr", "asx_coo_sort", "asx_csr_transpose", "asx_csr_rebase",
-    "asx_dense_transpose", "asx_plan_create",
+    "asx_dense_transpose", "asx_mtx_read", "asx_host_free", "asx_plan_create",
     "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
     "asx_spmm_resolve_alg", "asx_spmm_workspace_bytes", "asx_spmm_csr_f32", "asx_spmm_csr_f64",
@@ -66,6 +66,9 @@ def lib():
     L.asx_csr_transpose.argtypes = [C.c_int, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp]
     L.asx_csr_rebase.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp]
     L.asx_dense_transpose.argtypes = [C.c_int, C.c_int64, C.c_int64, vp, C.c_int64, vp, C.c_int64, vp]
+    L.asx_mtx_read.argtypes = [C.c_char_p, C.c_int] + [C.POINTER(i32)] * 3 + [C.POINTER(vp)] * 3
+    L.asx_host_free.argtypes = [vp]
+    L.asx_host_free.restype = None
     L.asx_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, C.c_int, i32, i32, i32, vp, i32, vp]
     L.asx_spmm_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, i32, i32, i32, vp, vp, vp, i32, vp]
     L.asx_plan_block_stats.argtypes = [vp, C.POINTER(i64), C.POINTER(C.c_double)]
@@ -197,6 +200,26 @@ def dense_transpose(a, rows, cols, ld_in, out, ld_out):
     """out[c*ld_out + r] = a[r*ld_in + c] on flat device tensors."""
     _check(lib().asx_dense_transpose(value_type(a.dtype), rows, cols, _ptr(a), ld_in, _ptr(out), ld_out, _stream()),
            "asx_dense_transpose")
+
+
+def mtx_read(path, dtype):
+    """MatrixMarket coordinate file -> (m, n, row, col, val) as numpy arrays (host; no GPU needed)."""
+    import numpy as np
+    dtype = np.dtype(dtype)
+    m, n, nnz = C.c_int32(), C.c_int32(), C.c_int32()
+    row, col, val = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    _check(lib().asx_mtx_read(str(path).encode(), R_64F if dtype == np.float64 else R_32F, C.byref(m), C.byref(n),
+                              C.byref(nnz), C.byref(row), C.byref(col), C.byref(val)), "asx_mtx_read")
+    try:
+        k = nnz.value
+        r = np.ctypeslib.as_array(C.cast(row, C.POINTER(C.c_int32)), (k,)).copy() if k else np.empty(0, np.int32)
+        c = np.ctypeslib.as_array(C.cast(col, C.POINTER(C.c_int32)), (k,)).copy() if k else np.empty(0, np.int32)
+        ct = C.c_double if dtype == np.float64 else C.c_float
+        v = np.ctypeslib.as_array(C.cast(val, C.POINTER(ct)), (k,)).copy() if k else np.empty(0, dtype)
+    finally:
+        for p in (row, col, val):
+            lib().asx_host_free(p)
+    return m.value, n.value, r, c, v
 
 
 def csr_adaptive_row_blocks(row_ptr_host):

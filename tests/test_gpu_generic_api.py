@@ -146,3 +146,38 @@ def test_spmm_layouts_and_ops(tmp_path, oracle, dtype):
                         ncols, alg, alpha, beta, analysis, (1, 1, 0, cc, 0), n=k)
         got = got.reshape(ncols, k).T if cc else got.reshape(k, ncols)
         assert_close(got.ravel(), ref_t, scale_t, dtype, f"opA=T alg {alg} analysis {analysis} cc{cc}")
+
+
+CLI = os.path.join(ROOT, "library_amd", "bin", "alphasparse_amd_cli")
+
+
+def test_cli_on_matrixmarket_files(tmp_path):
+    """The command-line driver end to end: MatrixMarket file -> device sort -> CSR -> generic API,
+    with its own --check (double-precision host loop) for SpMV and SpMM variants."""
+    import scipy.io
+    import scipy.sparse as sp
+    assert os.path.exists(CLI), "build step did not produce the command-line driver"
+    A = sp.random(3000, 2500, density=0.004, random_state=3, format="coo", dtype=np.float64)
+    gen = tmp_path / "general.mtx"
+    scipy.io.mmwrite(str(gen), A, precision=17)
+    S = sp.random(1500, 1500, density=0.01, random_state=4, format="coo", dtype=np.float64)
+    sym = tmp_path / "sym.mtx"
+    scipy.io.mmwrite(str(sym), sp.tril(S) + sp.tril(S, -1).T, symmetry="symmetric", precision=17)
+    metrics = tmp_path / "metrics.csv"
+    runs = [
+        [f"--data-file={gen}", "--data-type=D", "--check", "--iter=3", "--warmup=1", f"--metrics-file={metrics}"],
+        [f"--data-file={gen}", "--data-type=S", "--check", "--iter=2", "--warmup=1", "--alg_num=9", "--analysis"],
+        [f"--data-file={gen}", "--data-type=D", "--check", "--iter=2", "--warmup=1", "--transA=T", "--alg_num=0"],
+        [f"--data-file={sym}", "--op=spmm", "--data-type=S", "--check", "--iter=2", "--warmup=1", "--cols=40"],
+        [f"--data-file={gen}", "--op=spmm", "--data-type=D", "--check", "--iter=2", "--warmup=1", "--cols=9",
+         "--layout=C", "--transA=T", "--alg_num=0", "--analysis"],
+    ]
+    for args in runs:
+        r = subprocess.run([CLI, *args], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0, (args, r.returncode, r.stdout[-2000:], r.stderr[-2000:])
+        assert "correct: require" in r.stdout and "error: require" not in r.stdout, r.stdout
+        assert "alphasparse alg" in r.stdout
+    lines = metrics.read_text().strip().splitlines()
+    assert len(lines) == 8 and all(len(l.split(",")) == 11 for l in lines)  # DEFAULT + the reference's 7 ids
+    r = subprocess.run([CLI, f"--data-file={tmp_path / 'none.mtx'}"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 4
