@@ -54,8 +54,8 @@ FlatLayout spmv_flat_layout(int32_t nnz, size_t sv, bool with_split)
     return L;
 }
 
-struct SpmmLayout {  // [xs | ys | carry_row | carry]
-    size_t xs_off, ys_off, crow_off, carry_off, bytes;
+struct SpmmLayout {  // [raw xs | raw ys | xs | ys | carry_row | carry]
+    size_t raw_xs_off, raw_ys_off, xs_off, ys_off, crow_off, carry_off, bytes;
 };
 SpmmLayout spmm_merge_layout(int32_t m, int32_t nnz, int32_t ncols, size_t sv, bool with_split)
 {
@@ -63,10 +63,10 @@ SpmmLayout spmm_merge_layout(int32_t m, int32_t nnz, int32_t ncols, size_t sv, b
     const size_t ns = (size_t)spmm_segments(m, nnz);
     size_t off = 0;
     if (with_split) {
-        L.xs_off = off;
-        off = align_up(off + (ns + 1) * 4, kAlign);
-        L.ys_off = off;
-        off = align_up(off + (ns + 1) * 4, kAlign);
+        for (size_t *o : {&L.raw_xs_off, &L.raw_ys_off, &L.xs_off, &L.ys_off}) {
+            *o = off;
+            off = align_up(off + (ns + 1) * 4, kAlign);
+        }
     }
     L.crow_off = off;
     off = align_up(off + std::max<size_t>(ns, 1) * 4, kAlign);
@@ -76,14 +76,19 @@ SpmmLayout spmm_merge_layout(int32_t m, int32_t nnz, int32_t ncols, size_t sv, b
     return L;
 }
 
+constexpr int32_t kSmallNnz = 1 << 18;
+constexpr int64_t kSmallMaxRow = 2048;
+
 // DEFAULT with a plan: the flat kernel, except for matrices with very long rows, where the
 // merge-path kernel measured about 1 % faster (power-law: 569 vs 576 us).  Elsewhere flat is the
 // fastest of the four or within 1 % of it (5-point stencil 300 us vs stream 305; uniform 16/row
 // 95 vs stream 96), and it has no bad case: work per tile is bounded whatever the row lengths.
+// Matrices small enough to be bound by launch overhead take the vector kernel, the only one that
+// is a single launch with no metadata (1280 x 1280 banded: 13.4 us against 16.2 us).
 int choose_spmv_from_stats(const int64_t stats[4], int32_t m, int32_t nnz)
 {
     (void)m;
-    (void)nnz;
+    if (nnz <= kSmallNnz && stats[0] <= kSmallMaxRow) return ASX_SPMV_VECTOR;
     return stats[0] > kLongRow ? ASX_SPMV_MERGE : ASX_SPMV_FLAT;
 }
 
@@ -195,8 +200,12 @@ int spmm_impl(const asx_plan *plan, int alg, int32_t m, int32_t k, int32_t nnz, 
             xs = plan->d_meta;
             ys = plan->d_meta + (ns + 1);
         } else {
-            int st = launch_merge_path_search(row_ptr, m, nnz, kSpmmSegment, (int32_t *)(w + L.xs_off),
-                                              (int32_t *)(w + L.ys_off), s);
+            int st = launch_merge_path_search(row_ptr, m, nnz, kSpmmSegment, (int32_t *)(w + L.raw_xs_off),
+                                              (int32_t *)(w + L.raw_ys_off), s);
+            if (!st)
+                st = launch_spmm_snap_splits(m, nnz, row_ptr, (const int32_t *)(w + L.raw_xs_off),
+                                             (const int32_t *)(w + L.raw_ys_off), (int32_t *)(w + L.xs_off),
+                                             (int32_t *)(w + L.ys_off), s);
             if (st) return st;
             xs = (const int32_t *)(w + L.xs_off);
             ys = (const int32_t *)(w + L.ys_off);
@@ -395,10 +404,15 @@ int asx_plan_create(asx_plan **out, int is_spmm, int alg, int value_type, int32_
             const size_t ns = (size_t)spmm_segments(m, nnz);
             p->nunits = (int32_t)ns;
             p->meta_bytes = 2 * (ns + 1) * 4;
+            int32_t *raw = nullptr;  // the merge-path points, then snapped to short-row ends
             st = status_of(hipMalloc((void **)&p->d_meta, p->meta_bytes));
+            if (!st) st = status_of(hipMalloc((void **)&raw, p->meta_bytes));
+            if (!st) st = launch_merge_path_search(d_row_ptr, m, nnz, kSpmmSegment, raw, raw + (ns + 1), s);
             if (!st)
-                st = launch_merge_path_search(d_row_ptr, m, nnz, kSpmmSegment, p->d_meta,
-                                              p->d_meta + (ns + 1), s);
+                st = launch_spmm_snap_splits(m, nnz, d_row_ptr, raw, raw + (ns + 1), p->d_meta,
+                                             p->d_meta + (ns + 1), s);
+            if (!st) st = status_of(hipStreamSynchronize(s));
+            if (raw) (void)hipFree(raw);
             p->workspace_bytes = spmm_merge_layout(m, nnz, ncols_dense, sv, false).bytes;
         } else {
             p->workspace_bytes = 0;

@@ -82,6 +82,10 @@ int launch_spmm_merge(int32_t m, int32_t nnz, int32_t ncols, T alpha, const int3
                       int64_t ldc, const int32_t *xs, const int32_t *ys, T *carry, int32_t *carry_row,
                       hipStream_t s);
 
+// merge-path split points of SpMM moved to the ends of the short rows they cut (out of place)
+int launch_spmm_snap_splits(int32_t m, int32_t nnz, const int32_t *row_ptr, const int32_t *xs, const int32_t *ys,
+                            int32_t *xs_out, int32_t *ys_out, hipStream_t s);
+
 // ---- blocked (MFMA) SpMM (asx_blocked.hip) ----
 struct BlockedMatrix {
     int32_t nbrows;     // ceil(m / 16)

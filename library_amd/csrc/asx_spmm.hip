@@ -9,9 +9,9 @@
 //   row   : one wave per (row, column tile).  Simple; long rows serialise.
 //   merge : one wave per kSpmmSegment consecutive items of the merge path over
 //           (row ends, stored elements): bounded work per wave whatever the row lengths.
-//           Rows that end inside a segment are written by that segment; the part of a row
-//           that runs past a segment end is kept as a carry row and added by an ordered
-//           pass afterwards.  No atomics (the reference's default SpMM,
+//           Rows that end inside a segment are written by that segment, and so is a row
+//           that starts in it and ends in the next; of a longer row the part that runs past
+//           a segment end is kept as a carry row and added by an ordered pass afterwards.  No atomics (the reference's default SpMM,
 //           hip/kernel/level3/alphasparse_spmm_csr_nnz_split.h:283-409, scales C in a
 //           separate pass and joins segments with atomicAdd).
 #include "asx_internal.hpp"
@@ -114,6 +114,42 @@ int launch_spmm_row(int32_t m, int32_t ncols, T alpha, const int32_t *row_ptr, c
 // ===========================================================================================
 // merge: one wave per kSpmmSegment merge items
 // ===========================================================================================
+// Boundary g of the merge path lies between segments g-1 and g, at row xs[g], element ys[g].
+// The row cut by a boundary is SHORT there if it starts inside segment g-1 and ends inside
+// segment g: then the boundary moves to the end of that row, so segment g-1 takes the whole row
+// (running up to kSpmmSegment items past its nominal end) and segment g starts after it.  Only
+// rows long enough to cover a whole segment are still cut and leave carries.
+__global__ __launch_bounds__(kBlock) void k_spmm_snap_splits(int32_t m, int32_t nseg,
+                                                             const int32_t *__restrict__ row_ptr,
+                                                             const int32_t *__restrict__ xs,
+                                                             const int32_t *__restrict__ ys,
+                                                             int32_t *__restrict__ xs_out,
+                                                             int32_t *__restrict__ ys_out)
+{
+    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g > nseg) return;
+    int32_t x = xs[g], y = ys[g];
+    if (g > 0 && g < nseg && x < m) {
+        const int32_t b = row_ptr[x], e = row_ptr[x + 1];
+        if (b < y && b >= ys[g - 1] && e <= ys[g + 1] && x < xs[g + 1]) {
+            x += 1;
+            y = e;
+        }
+    }
+    xs_out[g] = x;
+    ys_out[g] = y;
+}
+
+int launch_spmm_snap_splits(int32_t m, int32_t nnz, const int32_t *row_ptr, const int32_t *xs, const int32_t *ys,
+                            int32_t *xs_out, int32_t *ys_out, hipStream_t s)
+{
+    const int32_t nseg = spmm_segments(m, nnz);
+    hipLaunchKernelGGL(k_spmm_snap_splits, dim3((unsigned)ceil_div64((int64_t)nseg + 1, kBlock)), dim3(kBlock), 0, s, m,
+                       nseg, row_ptr, xs, ys, xs_out, ys_out);
+    return check_launch();
+}
+
+// xs, ys: the snapped split points
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_spmm_merge(int32_t m, int32_t nnz, int32_t nseg,
                                                        int32_t ncols, T alpha,
@@ -139,7 +175,7 @@ __global__ __launch_bounds__(kBlock) void k_spmm_merge(int32_t m, int32_t nnz, i
 
     int32_t k = y0;
     T acc = T(0);
-    for (int32_t row = x0; row < x1; ++row) {  // rows whose end lies inside this segment
+    for (int32_t row = x0; row < x1; ++row) {  // rows this segment finishes
         const int32_t e = __builtin_amdgcn_readfirstlane(row_ptr[row + 1]);
         acc = spmm_accumulate<T>(acc, k, e, lane, col_ok, c, col, val, B, ldb);
         k = e;
@@ -158,10 +194,11 @@ __global__ __launch_bounds__(kBlock) void k_spmm_merge(int32_t m, int32_t nnz, i
     if (lane == 0 && blockIdx.y == 0) carry_row[seg] = has_tail ? x1 : -1;
 }
 
-// One wave per segment that opens a run of segments ending inside the same row: finds the
-// length of the run (64 segments per step, one ballot each), then sums the run's carry rows in
-// segment order with a counted, unrolled loop (many independent loads in flight; a loop that
-// tests carry_row before every add would pay one memory round trip per segment).
+// One thread per segment looks for the first segment of a run of segments that left carries for
+// the same row; each such run is then summed by the whole wave (lanes = columns): the run length
+// comes from ballots over carry_row (64 segments per step), the carry rows are added in segment
+// order with a counted, unrolled loop (many independent loads in flight; a loop that tests
+// carry_row before every add would pay one memory round trip per segment).
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_spmm_merge_fixup(int32_t m, int32_t nseg, int32_t ncols,
                                                              T alpha, const T *__restrict__ carry,
@@ -169,35 +206,44 @@ __global__ __launch_bounds__(kBlock) void k_spmm_merge_fixup(int32_t m, int32_t 
                                                              T *__restrict__ C, int64_t ldc)
 {
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t seg = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
-    if (seg >= nseg) return;  // wave-uniform from here on
-    const int32_t row = __builtin_amdgcn_readfirstlane(carry_row[seg]);
-    if (row < 0 || row >= m) return;
-    if (seg > 0 && __builtin_amdgcn_readfirstlane(carry_row[seg - 1]) == row) return;
-    int64_t len = 1;
-    for (int64_t base = seg + 1;; base += kWave) {
-        const int64_t idx = base + lane;
-        const bool same = idx < nseg && carry_row[idx] == row;
-        const unsigned long long mask = __ballot(same);
-        const int n = mask == ~0ull ? kWave : __ffsll((unsigned long long)~mask) - 1;
-        len += n;
-        if (n < kWave) break;
+    const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    int32_t my_row = -1;
+    bool head = false;
+    if (t < nseg) {
+        my_row = carry_row[t];
+        head = my_row >= 0 && my_row < m && (t == 0 || carry_row[t - 1] != my_row);
     }
-    const int64_t c = (int64_t)blockIdx.y * kWave + lane;
-    if (c >= ncols) return;
-    const T *p = carry + seg * ncols + c;
-    T sum = T(0);
-    int64_t j = 0;
-    for (; j + 16 <= len; j += 16) {
-        T v[16];
+    unsigned long long todo = __ballot(head);
+    while (todo) {  // wave-uniform
+        const int src = __ffsll(todo) - 1;
+        todo &= todo - 1;
+        const int64_t seg = t - lane + src;
+        const int32_t row = __shfl(my_row, src, kWave);
+        int64_t len = 1;
+        for (int64_t base = seg + 1;; base += kWave) {
+            const int64_t idx = base + lane;
+            const bool same = idx < nseg && carry_row[idx] == row;
+            const unsigned long long mask = __ballot(same);
+            const int n = mask == ~0ull ? kWave : __ffsll((unsigned long long)~mask) - 1;
+            len += n;
+            if (n < kWave) break;
+        }
+        for (int64_t c = lane; c < ncols; c += kWave) {
+            const T *p = carry + seg * ncols + c;
+            T sum = T(0);
+            int64_t j = 0;
+            for (; j + 16 <= len; j += 16) {
+                T v[16];
 #pragma unroll
-        for (int u = 0; u < 16; ++u) v[u] = p[(j + u) * ncols];
+                for (int u = 0; u < 16; ++u) v[u] = p[(j + u) * ncols];
 #pragma unroll
-        for (int u = 0; u < 16; ++u) sum += v[u];
+                for (int u = 0; u < 16; ++u) sum += v[u];
+            }
+            for (; j < len; ++j) sum += p[j * ncols];
+            const int64_t idx = (int64_t)row * ldc + c;
+            C[idx] = fma_t<T>(alpha, sum, C[idx]);
+        }
     }
-    for (; j < len; ++j) sum += p[j * ncols];
-    const int64_t idx = (int64_t)row * ldc + c;
-    C[idx] = fma_t<T>(alpha, sum, C[idx]);
 }
 
 template <typename T>
@@ -211,8 +257,8 @@ int launch_spmm_merge(int32_t m, int32_t nnz, int32_t ncols, T alpha, const int3
     dim3 grid((unsigned)ceil_div64(nseg, kBlock / kWave), (unsigned)ceil_div64(ncols, kWave));
     hipLaunchKernelGGL((k_spmm_merge<T>), grid, dim3(kBlock), 0, s, m, nnz, nseg, ncols, alpha, row_ptr,
                        col, val, B, ldb, beta, C, ldc, xs, ys, carry, carry_row);
-    hipLaunchKernelGGL((k_spmm_merge_fixup<T>), grid, dim3(kBlock), 0, s, m, nseg, ncols, alpha, carry,
-                       carry_row, C, ldc);
+    hipLaunchKernelGGL((k_spmm_merge_fixup<T>), dim3((unsigned)ceil_div64(nseg, kBlock)), dim3(kBlock), 0, s, m,
+                       nseg, ncols, alpha, carry, carry_row, C, ldc);
     return check_launch();
 }
 

@@ -234,11 +234,15 @@ def test_spmv_errors_and_empty(torch, capi):
 
 def test_default_plan_and_histogram(torch, capi):
     from library_amd import workloads as W
-    rp, col, val = W.csr_stencil5(128, 128)
+    rp, col, val = W.csr_stencil5(128, 128)  # launch-bound size: the single-launch kernel
     p = capi.Plan(False, capi.SPMV_DEFAULT, np.dtype(np.float64), rp.size - 1, rp.size - 1, col.size, dev(torch, rp))
-    assert p.alg == capi.SPMV_FLAT
+    assert p.alg == capi.SPMV_VECTOR
     hist, stats = p.histogram()
     assert stats[0] == 5 and hist.sum() == rp.size - 1
+    p.destroy()
+    rp, col, val = W.csr_stencil5(512, 512)
+    p = capi.Plan(False, capi.SPMV_DEFAULT, np.dtype(np.float64), rp.size - 1, rp.size - 1, col.size, dev(torch, rp))
+    assert p.alg == capi.SPMV_FLAT
     p.destroy()
     rp = row_ptr_from_lengths(np.r_[np.full(1000, 3), 50000])
     p = capi.Plan(False, capi.SPMV_DEFAULT, np.dtype(np.float64), rp.size - 1, 60000, int(rp[-1]), dev(torch, rp))
