@@ -259,6 +259,62 @@ static int selftest()
                                 ALPHA_SPARSE_DCU_SPMV_ALG_DEFAULT, &need, nullptr) == ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
         (void)hipFree(tb);
     }
+    // HIP graph: with kept analysis and a caller's buffer a call is kernels only (no allocation, no
+    // copy, no synchronisation), so it can be captured once and replayed; every replay must give
+    // the eager result bit for bit
+    {
+        const int gm = 6000, per = 7;
+        std::vector<int> grp(gm + 1), gcol((size_t)gm * per);
+        std::vector<double> gval(gcol.size()), gx(gm), gy0(gm), eager(gm), replay(gm);
+        for (int i = 0; i <= gm; ++i) grp[i] = i * per;
+        for (int i = 0; i < gm; ++i)
+            for (int j = 0; j < per; ++j) {
+                gcol[(size_t)i * per + j] = (int)(((long)i * 31 + (long)j * 977) % gm);
+                gval[(size_t)i * per + j] = 0.25 + 0.001 * ((i + 3 * j) % 17);
+            }
+        for (int i = 0; i < gm; ++i) gx[i] = 1.0 + 0.01 * (i % 13), gy0[i] = 0.5 - 0.002 * (i % 7);
+        int *g_rp = to_device(grp), *g_col = to_device(gcol);
+        double *g_val = to_device(gval), *g_x = to_device(gx), *g_y = to_device(gy0);
+        alphasparseSpMatDescr_t GA;
+        alphasparseDnVecDescr_t GX, GY;
+        EXPECT(alphasparseCreateCsr(&GA, gm, gm, gm * per, g_rp, g_col, g_val, ALPHA_SPARSE_INDEXTYPE_I32,
+                                    ALPHA_SPARSE_INDEXTYPE_I32, ALPHA_SPARSE_INDEX_BASE_ZERO, ALPHA_R_64F) == 0);
+        EXPECT(alphasparseCreateDnVec(&GX, gm, g_x, ALPHA_R_64F) == 0 && alphasparseCreateDnVec(&GY, gm, g_y, ALPHA_R_64F) == 0);
+        h->stream = h->streams[0];  // capture needs a stream of its own, not the null stream
+        for (alphasparseSpMVAlg_t galg : {ALPHA_SPARSE_SPMV_ALG_MERGE, ALPHA_SPARSE_SPMV_ALG_FLAT8}) {
+            size_t nb = 0;
+            EXPECT(alphasparseSpMV_bufferSize(h, N, &alpha, GA, GX, &beta, GY, ALPHA_R_64F, galg, &nb) == 0);
+            void *gb = nullptr;
+            HIP_OK(hipMalloc(&gb, nb ? nb : 1));
+            EXPECT(alphasparseSpMV_analysis(h, N, GA, galg) == 0);
+            EXPECT(alphasparseSpMV(h, N, &alpha, GA, GX, &beta, GY, ALPHA_R_64F, galg, gb) == 0);
+            HIP_OK(hipStreamSynchronize(h->stream));
+            HIP_OK(hipMemcpy(eager.data(), g_y, sizeof(double) * gm, hipMemcpyDeviceToHost));
+            hipGraph_t graph;
+            hipGraphExec_t exec;
+            HIP_OK(hipStreamBeginCapture(h->stream, hipStreamCaptureModeGlobal));
+            EXPECT(alphasparseSpMV(h, N, &alpha, GA, GX, &beta, GY, ALPHA_R_64F, galg, gb) == 0);
+            HIP_OK(hipStreamEndCapture(h->stream, &graph));
+            HIP_OK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+            for (int rep = 0; rep < 3; ++rep) {
+                HIP_OK(hipMemcpy(g_y, gy0.data(), sizeof(double) * gm, hipMemcpyHostToDevice));
+                HIP_OK(hipGraphLaunch(exec, h->stream));
+                HIP_OK(hipStreamSynchronize(h->stream));
+                HIP_OK(hipMemcpy(replay.data(), g_y, sizeof(double) * gm, hipMemcpyDeviceToHost));
+                EXPECT(replay == eager);
+            }
+            HIP_OK(hipGraphExecDestroy(exec));
+            HIP_OK(hipGraphDestroy(graph));
+            EXPECT(alphasparseSpMV_clear(h, galg) == 0);
+            (void)hipFree(gb);
+            HIP_OK(hipMemcpy(g_y, gy0.data(), sizeof(double) * gm, hipMemcpyHostToDevice));
+        }
+        h->stream = nullptr;
+        alphasparseDestroySpMat(GA);
+        alphasparseDestroyDnVec(GX);
+        alphasparseDestroyDnVec(GY);
+        for (void *p : {(void *)g_rp, (void *)g_col, (void *)g_val, (void *)g_x, (void *)g_y}) (void)hipFree(p);
+    }
     // COO -> CSR through the reference's name
     {
         std::vector<int> ri = {0, 0, 1};
