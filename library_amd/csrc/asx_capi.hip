@@ -85,11 +85,14 @@ constexpr int64_t kSmallMaxRow = 2048;
 // 95 vs stream 96), and it has no bad case: work per tile is bounded whatever the row lengths.
 // Matrices small enough to be bound by launch overhead take the vector kernel, the only one that
 // is a single launch with no metadata (1280 x 1280 banded: 13.4 us against 16.2 us).
-int choose_spmv_from_stats(const int64_t stats[4], int32_t m, int32_t nnz)
+// Mostly-empty matrices (more than half of the rows hold nothing) take the merge-path kernel,
+// which counts row ends as work: a flat tile next to a long run of empty rows has to write all
+// of them itself.
+int choose_spmv_from_stats(const int64_t hist[33], const int64_t stats[4], int32_t m, int32_t nnz)
 {
-    (void)m;
-    if (nnz <= kSmallNnz && stats[0] <= kSmallMaxRow) return ASX_SPMV_VECTOR;
-    return stats[0] > kLongRow ? ASX_SPMV_MERGE : ASX_SPMV_FLAT;
+    if (nnz <= kSmallNnz && stats[0] <= kSmallMaxRow && m <= kSmallNnz) return ASX_SPMV_VECTOR;
+    if (stats[0] > kLongRow || hist[0] > (int64_t)m / 2) return ASX_SPMV_MERGE;
+    return ASX_SPMV_FLAT;
 }
 
 template <typename T>
@@ -341,7 +344,7 @@ int asx_plan_create(asx_plan **out, int is_spmm, int alg, int value_type, int32_
     if (!is_spmm) {
         int kernel = alg;
         if (alg == ASX_SPMV_DEFAULT)
-            kernel = choose_spmv_from_stats(p->stats, m, nnz);
+            kernel = choose_spmv_from_stats(p->hist, p->stats, m, nnz);
         else
             kernel = asx_spmv_resolve_alg(alg, m, nnz);
         if (kernel < 0) {

@@ -43,10 +43,6 @@ public:
         if (rows_in_block > 1 && n_ >= 2 && n_ - 2 < cap_)
             out_[n_ - 2] |= largest_pow2_not_above((uint32_t)(kWorkgroup / rows_in_block));
     }
-    uint64_t last_row(uint64_t fallback) const
-    {
-        return (n_ >= 1 && n_ - 1 < cap_) ? (out_[n_ - 1] >> 32) : fallback;
-    }
     size_t count() const { return n_; }
 
 private:

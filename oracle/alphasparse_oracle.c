@@ -90,13 +90,7 @@ static inline float row_dot_f32(const int32_t *col, const float *val, const floa
     return sum;
 }
 
-static int clamp_threads(int nthreads, int32_t m)
-{
-    if (nthreads < 1)
-        nthreads = 1;
-    (void)m;
-    return nthreads;
-}
+static int at_least_one(int nthreads) { return nthreads < 1 ? 1 : nthreads; }
 
 /* ---- gemv_csr.hpp:48-78 : rows are dealt to threads by orc_partition_rows_by_nnz ---- */
 void orc_spmv_csr_f64(int32_t m, const int32_t *row_ptr, const int32_t *col, const double *val,
@@ -104,7 +98,7 @@ void orc_spmv_csr_f64(int32_t m, const int32_t *row_ptr, const int32_t *col, con
 {
     if (m <= 0)
         return;
-    nthreads = clamp_threads(nthreads, m);
+    nthreads = at_least_one(nthreads);
     int32_t *part = (int32_t *)malloc(sizeof(int32_t) * (size_t)(nthreads + 1));
     orc_partition_rows_by_nnz(row_ptr + 1, m, nthreads, part);
 #pragma omp parallel num_threads(nthreads)
@@ -135,7 +129,7 @@ void orc_spmv_csr_f32(int32_t m, const int32_t *row_ptr, const int32_t *col, con
 {
     if (m <= 0)
         return;
-    nthreads = clamp_threads(nthreads, m);
+    nthreads = at_least_one(nthreads);
     int32_t *part = (int32_t *)malloc(sizeof(int32_t) * (size_t)(nthreads + 1));
     orc_partition_rows_by_nnz(row_ptr + 1, m, nthreads, part);
 #pragma omp parallel num_threads(nthreads)
@@ -175,7 +169,7 @@ void orc_spmm_csr_row_f32(int32_t m, const int32_t *row_ptr, const int32_t *col,
 {
     if (m <= 0)
         return;
-    nthreads = clamp_threads(nthreads, m);
+    nthreads = at_least_one(nthreads);
 #pragma omp parallel for num_threads(nthreads) schedule(dynamic, 64)
     for (int32_t r = 0; r < m; ++r) {
         float *c = C + (size_t)r * (size_t)ldc;
@@ -196,7 +190,7 @@ void orc_spmm_csr_row_f64(int32_t m, const int32_t *row_ptr, const int32_t *col,
 {
     if (m <= 0)
         return;
-    nthreads = clamp_threads(nthreads, m);
+    nthreads = at_least_one(nthreads);
 #pragma omp parallel for num_threads(nthreads) schedule(dynamic, 64)
     for (int32_t r = 0; r < m; ++r) {
         double *c = C + (size_t)r * (size_t)ldc;

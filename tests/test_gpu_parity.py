@@ -248,6 +248,12 @@ def test_default_plan_and_histogram(torch, capi):
     p = capi.Plan(False, capi.SPMV_DEFAULT, np.dtype(np.float64), rp.size - 1, 60000, int(rp[-1]), dev(torch, rp))
     assert p.alg == capi.SPMV_MERGE
     p.destroy()
+    lens = np.zeros(600000, dtype=np.int64)  # mostly empty rows: row ends must count as work
+    lens[::7] = 5
+    rp = row_ptr_from_lengths(lens)
+    p = capi.Plan(False, capi.SPMV_DEFAULT, np.dtype(np.float64), rp.size - 1, 1000, int(rp[-1]), dev(torch, rp))
+    assert p.alg == capi.SPMV_MERGE
+    p.destroy()
 
 
 # ------------------------------------------------------------------ SpMM
