@@ -23,7 +23,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 ORDER = ["banded_f64", "uniform16_f32", "powerlaw_f64", "stencil5_f64", "spmm_zipf_f32"]
 EXTRA = ["spmm_banded_f32"]  # not a BASELINE configuration: dense-block matrix for the MFMA SpMM variant
-KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "k_spmv_flat", 5: "k_spmm_row", 7: "k_spmm_merge",
+KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "k_spmv_flat", 100: "k_spmv_panel", 5: "k_spmm_row", 7: "k_spmm_merge",
                 10: "k_spmm_blocked"}
 
 # HBM traffic per call measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; see profiles/),

@@ -49,7 +49,9 @@ enum {
     ASX_SPMV_VECTOR = 6,  /* wave64 sub-groups, one group per row */
     ASX_SPMV_STREAM = 3,  /* LDS-staged row blocks, segmented reduction */
     ASX_SPMV_MERGE = 9,   /* merge-path tiles + ordered carry fix-up */
-    ASX_SPMV_FLAT = 15    /* tiles of 1024 stored elements, register walk + ordered carry fix-up */
+    ASX_SPMV_FLAT = 15,   /* tiles of 1024 stored elements, register walk + ordered carry fix-up */
+    ASX_SPMV_PANEL = 100  /* not a reference id: the flat kernel over 8 column panels, one per XCD
+                             (needs a plan from asx_spmv_plan_create) */
 };
 
 /* SpMM kernels (alphasparseSpMMAlg_t values, include/alphasparse/spdef.h:390-402) */
@@ -179,6 +181,19 @@ int asx_plan_create(asx_plan **plan, int is_spmm, int alg, int value_type, int32
 int asx_spmm_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, int32_t k, int32_t nnz,
                          const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, int32_t ncols,
                          void *stream);
+/* SpMV plan that may look at A's columns and values.  alg = ASX_SPMV_PANEL regroups the stored
+ * elements into 8 column panels, one per XCD, so that each XCD's L2 holds the slice of x its
+ * workgroups gather from (for matrices whose x is 1.5 to 8 L2s large and whose columns are
+ * scattered; the plan then holds a COPY of the values: rebuild it when they change; calls need
+ * 8*m values of workspace for the per-panel partial results).  alg = ASX_SPMV_DEFAULT on such a
+ * matrix builds the panels, times the panel kernel against the kernel the histogram picks (three
+ * runs each on scratch vectors) and keeps the faster.  Otherwise as asx_plan_create.  No
+ * counterpart in the reference (its alphasparseSpMV_analysis is a stub).  Synchronises `stream`. */
+int asx_spmv_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
+                         const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, void *stream);
+/* Upper bound of the workspace a panel plan for (m, n, nnz) needs; 0 when the matrix is not a
+ * candidate for panels.  For sizing a buffer before the plan exists. */
+size_t asx_spmv_panel_workspace_bytes(int value_type, int32_t m, int32_t n, int32_t nnz);
 /* Number of 16x4 blocks and their fill of a blocked plan. */
 int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill);
 int asx_plan_destroy(asx_plan *plan);

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libalphasparse_amd.so")
 
 R_32F, R_64F = 0, 1
-SPMV_DEFAULT, SPMV_STREAM, SPMV_VECTOR, SPMV_MERGE, SPMV_FLAT = 0, 3, 6, 9, 15
+SPMV_DEFAULT, SPMV_STREAM, SPMV_VECTOR, SPMV_MERGE, SPMV_FLAT, SPMV_PANEL = 0, 3, 6, 9, 15, 100
 SPMM_DEFAULT, SPMM_ROW, SPMM_MERGE, SPMM_BLOCKED = 0, 5, 7, 10
 
 STATUS = {0: "SUCCESS", 1: "NOT_INITIALIZED", 2: "ALLOC_FAILED", 3: "INVALID_VALUE",
@@ -26,7 +26,8 @@ EXPORTS = [
     "asx_version", "asx_device_info", "asx_row_length_histogram", "asx_partition_rows_by_nnz",
     "asx_nnz_split_rows", "asx_merge_path_search", "asx_loadbalance_nwarps",
     "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_coo2csr", "asx_coo_sort", "asx_csr_transpose", "asx_csr_rebase",
-    "asx_dense_transpose", "asx_mtx_read", "asx_host_free", "asx_plan_create",
+    "asx_dense_transpose", "asx_mtx_read", "asx_host_free", "asx_spmv_plan_create",
+    "asx_spmv_panel_workspace_bytes", "asx_plan_create",
     "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
     "asx_spmm_resolve_alg", "asx_spmm_workspace_bytes", "asx_spmm_csr_f32", "asx_spmm_csr_f64",
@@ -71,6 +72,9 @@ def lib():
     L.asx_host_free.restype = None
     L.asx_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, C.c_int, i32, i32, i32, vp, i32, vp]
     L.asx_spmm_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, i32, i32, i32, vp, vp, vp, i32, vp]
+    L.asx_spmv_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, i32, i32, i32, vp, vp, vp, vp]
+    L.asx_spmv_panel_workspace_bytes.argtypes = [C.c_int, i32, i32, i32]
+    L.asx_spmv_panel_workspace_bytes.restype = sz
     L.asx_plan_block_stats.argtypes = [vp, C.POINTER(i64), C.POINTER(C.c_double)]
     L.asx_plan_destroy.argtypes = [vp]
     L.asx_plan_alg.argtypes = [vp]
@@ -242,6 +246,9 @@ class Plan:
         if is_spmm and col is not None and val is not None:
             _check(lib().asx_spmm_plan_create(C.byref(h), alg, value_type(dtype), m, n, nnz, _ptr(row_ptr), _ptr(col),
                                               _ptr(val), ncols, _stream()), "asx_spmm_plan_create")
+        elif not is_spmm and col is not None and val is not None:
+            _check(lib().asx_spmv_plan_create(C.byref(h), alg, value_type(dtype), m, n, nnz, _ptr(row_ptr), _ptr(col),
+                                              _ptr(val), _stream()), "asx_spmv_plan_create")
         else:
             _check(lib().asx_plan_create(C.byref(h), int(is_spmm), alg, value_type(dtype), m, n, nnz, _ptr(row_ptr),
                                          ncols, _stream()), "asx_plan_create")

@@ -544,7 +544,14 @@ alphasparseStatus_t alphasparseSpMV_bufferSize(alphasparseHandle_t handle, alpha
     if (asx_spmv_resolve_alg((int)alg, m_eff, (int32_t)matA->nnz) < 0)
         return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
     // sized for a call without kept analysis; a call with kept analysis needs no more than this
-    *bufferSize = asx_spmv_workspace_bytes((int)alg, (int)matA->data_type, m_eff, (int32_t)matA->nnz);
+    // (DEFAULT: including the column-panel kernel the analysis may pick for this matrix)
+    size_t need = asx_spmv_workspace_bytes((int)alg, (int)matA->data_type, m_eff, (int32_t)matA->nnz);
+    if (alg == ALPHA_SPARSE_SPMV_ALG_DEFAULT) {
+        const int32_t n_eff = (int32_t)(is_transpose(opA) ? matA->rows : matA->cols);
+        const size_t panel = asx_spmv_panel_workspace_bytes((int)matA->data_type, m_eff, n_eff, (int32_t)matA->nnz);
+        if (panel > need) need = panel;
+    }
+    *bufferSize = need;
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
@@ -567,8 +574,10 @@ alphasparseStatus_t alphasparseSpMV_analysis(alphasparseHandle_t handle, alphasp
     HandlePlans *hp = plans_of(handle, true);
     if (!hp) return ALPHA_SPARSE_STATUS_ALLOC_FAILED;
     asx_plan *plan = nullptr;
-    int rc = asx_plan_create(&plan, 0, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
-                             (int32_t)A->nnz, A->row_data, 1, (void *)handle->stream);
+    // may keep a regrouped copy of A's columns and values (column panels): call again after
+    // changing them
+    int rc = asx_spmv_plan_create(&plan, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
+                                  (int32_t)A->nnz, A->row_data, A->col_data, A->val_data, (void *)handle->stream);
     if (rc) return st(rc);
     hp->plans.push_back(KeptPlan{false, (int)alg, A->row_data, A->rows, A->nnz, (int)A->data_type, 1, plan});
     matA->analysed = true;

@@ -76,6 +76,26 @@ SpmmLayout spmm_merge_layout(int32_t m, int32_t nnz, int32_t ncols, size_t sv, b
     return L;
 }
 
+struct PanelLayout {  // [partial | carry]
+    size_t partial_off, carry_off, bytes;
+};
+PanelLayout spmv_panel_layout(int32_t m, size_t total_tiles, size_t sv)
+{
+    PanelLayout L{};
+    L.partial_off = 0;
+    L.carry_off = align_up((size_t)kPanels * (size_t)m * sv, kAlign);
+    L.bytes = L.carry_off + align_up(std::max<size_t>(total_tiles, 1) * sv, kAlign);
+    return L;
+}
+
+// Panels pay when x is too large for one 4 MiB L2 but each of kPanels slices fits one.
+constexpr size_t kL2Bytes = (size_t)4 << 20;
+bool panel_candidate(int32_t m, int32_t n, int32_t nnz, size_t sv)
+{
+    const size_t xbytes = (size_t)n * sv;
+    return m > 0 && nnz >= (1 << 22) && xbytes > kL2Bytes + kL2Bytes / 2 && xbytes <= kPanels * kL2Bytes;
+}
+
 constexpr int32_t kSmallNnz = 1 << 18;
 constexpr int64_t kSmallMaxRow = 2048;
 
@@ -164,6 +184,15 @@ int spmv_impl(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, 
         }
         return launch_spmv_flat<T>(m, nnz, alpha, row_ptr, col, val, x, beta, y, seg, (T *)(w + L.carry_off),
                                    plan ? plan->carry_pass != 0 : true, s);
+    }
+    case ASX_SPMV_PANEL: {
+        // the panels hold a copy of A's columns and values and are built by asx_spmv_plan_create
+        if (!plan || !plan->panel.col) return ASX_STATUS_NOT_INITIALIZED;
+        const PanelLayout L = spmv_panel_layout(m, (size_t)plan->panel.tile_off[kPanels], sizeof(T));
+        if (!ws) return ASX_STATUS_INVALID_POINTER;
+        if (ws_bytes < L.bytes) return ASX_STATUS_INVALID_SIZE;
+        return launch_spmv_panel<T>(m, alpha, &plan->panel, x, beta, y, (T *)(w + L.partial_off),
+                                    (T *)(w + L.carry_off), s);
     }
     default: return ASX_STATUS_NOT_SUPPORTED;
     }
@@ -437,6 +466,7 @@ int asx_plan_destroy(asx_plan *plan)
     int st = ASX_STATUS_SUCCESS;
     if (plan->d_meta) st = status_of(hipFree(plan->d_meta));
     free_blocked(&plan->blocked);
+    free_panels(&plan->panel);
     delete plan;
     return st;
 }
@@ -491,6 +521,130 @@ int asx_spmm_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     p->workspace_bytes = 0;
     *out = p;
     return ASX_STATUS_SUCCESS;
+}
+
+}  // extern "C"
+
+// Average time of one call through `plan` on scratch vectors (x = 0), in milliseconds; < 0 on error.
+template <typename T>
+static float time_plan(const asx_plan *plan, const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val,
+                       const T *d_x, T *d_y, void *d_ws, size_t ws_bytes, hipStream_t s)
+{
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess) return -1.0f;
+    if (hipEventCreate(&e1) != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return -1.0f;
+    }
+    float ms = -1.0f;
+    int st = spmv_impl<T>(plan, plan->alg, plan->m, plan->n, plan->nnz, T(1), d_row_ptr, d_col, d_val, d_x, T(0), d_y,
+                          d_ws, ws_bytes, s);  // warm-up
+    if (!st) st = status_of(hipEventRecord(e0, s));
+    for (int i = 0; i < 3 && !st; ++i)
+        st = spmv_impl<T>(plan, plan->alg, plan->m, plan->n, plan->nnz, T(1), d_row_ptr, d_col, d_val, d_x, T(0), d_y,
+                          d_ws, ws_bytes, s);
+    if (!st) st = status_of(hipEventRecord(e1, s));
+    if (!st) st = status_of(hipEventSynchronize(e1));
+    if (!st && hipEventElapsedTime(&ms, e0, e1) == hipSuccess)
+        ms /= 3.0f;
+    else
+        ms = -1.0f;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return ms;
+}
+
+template <typename T>
+static int spmv_plan_with_panels(asx_plan **out, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
+                                 const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, hipStream_t s)
+{
+    // the plan the histogram picks: the fallback, and for DEFAULT the opponent of the timing
+    asx_plan *base = nullptr;
+    int st = asx_plan_create(&base, 0, alg == ASX_SPMV_PANEL ? ASX_SPMV_DEFAULT : alg, value_type, m, n, nnz, d_row_ptr,
+                             1, (void *)s);
+    if (st) return st;
+    asx_plan *pp = new (std::nothrow) asx_plan();
+    if (!pp) {
+        asx_plan_destroy(base);
+        return ASX_STATUS_ALLOC_FAILED;
+    }
+    *pp = *base;  // histogram, sizes
+    pp->d_meta = nullptr;
+    pp->meta_bytes = 0;
+    pp->alg = ASX_SPMV_PANEL;
+    pp->panel = PanelMatrix{};
+    st = build_panels<T>(m, n, nnz, d_row_ptr, d_col, d_val, &pp->panel, s);
+    if (st) {
+        delete pp;
+        if (alg == ASX_SPMV_PANEL) {
+            asx_plan_destroy(base);
+            return st;
+        }
+        *out = base;  // DEFAULT: no panels (out of memory, ...) is not an error
+        return ASX_STATUS_SUCCESS;
+    }
+    pp->nunits = pp->panel.tile_off[kPanels];
+    pp->carry_pass = pp->panel.carry_pass;
+    pp->workspace_bytes = spmv_panel_layout(m, (size_t)pp->panel.tile_off[kPanels], sizeof(T)).bytes;
+    if (alg == ASX_SPMV_PANEL) {
+        asx_plan_destroy(base);
+        *out = pp;
+        return ASX_STATUS_SUCCESS;
+    }
+    // DEFAULT: keep the faster of the two on this matrix
+    const size_t ws_bytes = std::max(pp->workspace_bytes, base->workspace_bytes);
+    T *d_x = nullptr, *d_y = nullptr;
+    void *d_ws = nullptr;
+    bool panel_wins = false;
+    if (hipMalloc((void **)&d_x, sizeof(T) * (size_t)n) == hipSuccess &&
+        hipMalloc((void **)&d_y, sizeof(T) * (size_t)m) == hipSuccess &&
+        hipMalloc(&d_ws, ws_bytes ? ws_bytes : 1) == hipSuccess &&
+        hipMemsetAsync(d_x, 0, sizeof(T) * (size_t)n, s) == hipSuccess) {
+        const float t_base = time_plan<T>(base, d_row_ptr, d_col, d_val, d_x, d_y, d_ws, ws_bytes, s);
+        const float t_panel = time_plan<T>(pp, d_row_ptr, d_col, d_val, d_x, d_y, d_ws, ws_bytes, s);
+        panel_wins = t_base > 0 && t_panel > 0 && t_panel < 0.9f * t_base;
+    }
+    (void)hipStreamSynchronize(s);
+    for (void *q : {(void *)d_x, (void *)d_y, d_ws})
+        if (q) (void)hipFree(q);
+    if (panel_wins) {
+        asx_plan_destroy(base);
+        *out = pp;
+    } else {
+        asx_plan_destroy(pp);
+        *out = base;
+    }
+    return ASX_STATUS_SUCCESS;
+}
+
+extern "C" {
+
+int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
+                         const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, void *stream)
+{
+    if (!out) return ASX_STATUS_INVALID_POINTER;
+    *out = nullptr;
+    if (m < 0 || n < 0 || nnz < 0) return ASX_STATUS_INVALID_SIZE;
+    if (value_type != ASX_R_32F && value_type != ASX_R_64F) return ASX_STATUS_NOT_SUPPORTED;
+    const bool want = alg == ASX_SPMV_PANEL;
+    const bool candidate = d_col && d_val && panel_candidate(m, n, nnz, vsize(value_type));
+    if (want && (m == 0 || nnz == 0 || n < kPanels)) return ASX_STATUS_INVALID_SIZE;
+    if (want && (!d_row_ptr || !d_col || !d_val)) return ASX_STATUS_INVALID_POINTER;
+    if (!want && !(alg == ASX_SPMV_DEFAULT && candidate))
+        return asx_plan_create(out, 0, alg, value_type, m, n, nnz, d_row_ptr, 1, stream);
+    if (value_type == ASX_R_64F)
+        return spmv_plan_with_panels<double>(out, alg, value_type, m, n, nnz, d_row_ptr, d_col, (const double *)d_val,
+                                             (hipStream_t)stream);
+    return spmv_plan_with_panels<float>(out, alg, value_type, m, n, nnz, d_row_ptr, d_col, (const float *)d_val,
+                                        (hipStream_t)stream);
+}
+
+size_t asx_spmv_panel_workspace_bytes(int value_type, int32_t m, int32_t n, int32_t nnz)
+{
+    if (m <= 0 || n <= 0 || nnz <= 0) return 0;
+    const size_t sv = vsize(value_type);
+    if (!panel_candidate(m, n, nnz, sv)) return 0;
+    return spmv_panel_layout(m, (size_t)ceil_div64(nnz, kFlatTile) + kPanels, sv).bytes;
 }
 
 int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill)

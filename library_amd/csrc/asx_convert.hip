@@ -69,6 +69,13 @@ __global__ __launch_bounds__(kBlock) void k_offsets_from_sorted(const int32_t *_
     row_ptr_t[r] = lo;
 }
 
+int launch_offsets_from_sorted(const int32_t *sorted, int32_t count, int32_t n, int32_t *out, hipStream_t s)
+{
+    hipLaunchKernelGGL(k_offsets_from_sorted, dim3((unsigned)ceil_div64((int64_t)n + 1, kBlock)), dim3(kBlock), 0, s,
+                       sorted, count, n, out);
+    return check_launch();
+}
+
 static int bits_for(int64_t v)
 {
     int b = 1;

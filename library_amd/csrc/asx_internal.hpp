@@ -102,6 +102,33 @@ template <typename T>
 int launch_spmm_blocked(int32_t m, int32_t k, int32_t ncols, T alpha, const BlockedMatrix *bm, const T *B,
                         int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t s);
 
+// ---- column-panel SpMV (asx_panel.hip builds, asx_spmv.hip runs) ----
+// The stored elements regrouped into kPanels column panels (panel = col / width), each panel a
+// CSR matrix of its own over all m rows.  Workgroup b works on panel b % kPanels: consecutive
+// workgroups go to consecutive XCDs, so each XCD's L2 only ever sees one panel's slice of x.
+constexpr int kPanels = 8;
+struct PanelMatrix {
+    int32_t width;                  // columns per panel
+    int32_t count[kPanels];         // stored elements per panel
+    int64_t elem_off[kPanels + 1];  // start of each panel in col / val (multiples of 4 elements)
+    int32_t tile_off[kPanels + 1];  // start of each panel's tiles in the carry array
+    int32_t max_tiles;
+    int32_t *col;      // device
+    void *val;         // device, a copy of A's values in panel order
+    int32_t *row_ptr;  // device, kPanels x (m + 1)
+    int32_t *seg_row;  // device, panel j at tile_off[j] + j, tiles_j + 1 entries
+    int carry_pass;
+};
+template <typename T>
+int build_panels(int32_t m, int32_t n, int32_t nnz, const int32_t *row_ptr, const int32_t *col, const T *val,
+                 PanelMatrix *out, hipStream_t s);
+void free_panels(PanelMatrix *p);
+template <typename T>
+int launch_spmv_panel(int32_t m, T alpha, const PanelMatrix *pm, const T *x, T beta, T *y, T *partial, T *carry,
+                      hipStream_t s);
+// out[r] = first i with sorted[i] >= r, r in [0, n]
+int launch_offsets_from_sorted(const int32_t *sorted, int32_t count, int32_t n, int32_t *out, hipStream_t s);
+
 inline int32_t merge_tiles(int32_t m, int32_t nnz) { return (int32_t)ceil_div64((int64_t)m + nnz, kMergeTile); }
 inline int32_t flat_tiles(int32_t nnz) { int32_t t = (int32_t)ceil_div64(nnz, kFlatTile); return t < 1 ? 1 : t; }
 inline int32_t stream_blocks(int32_t nnz) { return (int32_t)ceil_div64(nnz, kStreamTile); }
@@ -124,4 +151,5 @@ struct asx_plan {
     int64_t stats[4];
     size_t workspace_bytes;
     asx::BlockedMatrix blocked;  // only for ASX_SPMM_BLOCKED plans
+    asx::PanelMatrix panel;      // only for ASX_SPMV_PANEL plans
 };

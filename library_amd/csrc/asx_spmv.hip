@@ -444,13 +444,11 @@ __global__ __launch_bounds__(kBlock) void k_spmv_merge(int32_t m, int32_t nnz, i
 // carries lane-parallel in a fixed order and adds the total to y.  (A single thread walking the
 // run pays one memory round trip per tile: 100 round trips for a 200 000-element row.)
 template <typename T>
-__global__ __launch_bounds__(kBlock) void k_spmv_merge_fixup(int32_t m, int32_t ntiles, T alpha,
-                                                             const int32_t *__restrict__ xs,
-                                                             const T *__restrict__ carry,
-                                                             T *__restrict__ y)
+__device__ __forceinline__ void fixup_tiles(int64_t t, int32_t m, int32_t ntiles, T alpha,
+                                            const int32_t *__restrict__ xs, const T *__restrict__ carry,
+                                            T *__restrict__ y)
 {
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     int32_t row = m;
     bool first = false, run = false;
     if (t < ntiles) {
@@ -482,6 +480,15 @@ __global__ __launch_bounds__(kBlock) void k_spmv_merge_fixup(int32_t m, int32_t 
         const T sum = group_sum<kWave>(part);
         if (lane == 0 && sum != T(0)) y[r] = fma_t<T>(alpha, sum, y[r]);
     }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_spmv_merge_fixup(int32_t m, int32_t ntiles, T alpha,
+                                                             const int32_t *__restrict__ xs,
+                                                             const T *__restrict__ carry,
+                                                             T *__restrict__ y)
+{
+    fixup_tiles<T>((int64_t)blockIdx.x * kBlock + threadIdx.x, m, ntiles, alpha, xs, carry, y);
 }
 
 template <typename T>
@@ -846,6 +853,99 @@ int launch_spmv_flat(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, co
     return check_launch();
 }
 
+// ===========================================================================================
+// panel: the flat kernel over kPanels column panels, one panel per XCD
+// ===========================================================================================
+// Random gathers that miss the 4 MiB L2 of an XCD cost a 128-byte fill each (60 G gathers/s
+// against 180 G/s for hits).  With the stored elements regrouped by column panel and workgroup b
+// working on panel b % kPanels, workgroups on one XCD (consecutive workgroups go to consecutive
+// XCDs) only gather from one slice of x, which then lives in that XCD's L2.  Each panel writes
+// its own partial result vector; an ordered pass adds the kPanels partial vectors into y.
+struct PanelView {
+    const int32_t *row_ptr, *col, *seg_row;
+    const void *val;
+    int64_t elem_off[kPanels];
+    int32_t count[kPanels];
+    int32_t tile_off[kPanels];
+};
+
+template <typename T, bool NT>
+__global__ __launch_bounds__(kBlock) void k_spmv_panel(PanelView v, int32_t m, const T *__restrict__ x,
+                                                       T *__restrict__ partial, T *__restrict__ carry)
+{
+    __shared__ FlatShared<T> sh;
+    const int j = blockIdx.x % kPanels;
+    const int t = blockIdx.x / kPanels;
+    const int32_t cnt = v.count[j];
+    if (cnt == 0 || t >= (cnt + kFlatTile - 1) / kFlatTile) return;  // uniform over the workgroup
+    const int32_t *col = v.col + v.elem_off[j];
+    const T *val = static_cast<const T *>(v.val) + v.elem_off[j];
+    int32_t c[4];
+    T p[4];
+    flat_load<T, true, NT>(t, cnt, col, val, c, p);
+    flat_tile<T, NT>(sh, t, m, cnt, T(1), v.row_ptr + (int64_t)j * (m + 1), c, p, x, T(0),
+                     partial + (int64_t)j * m, v.seg_row + v.tile_off[j] + j, carry + v.tile_off[j]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_spmv_panel_fixup(PanelView v, int32_t m, const T *__restrict__ carry,
+                                                             T *__restrict__ partial)
+{
+    const int j = blockIdx.y;
+    const int32_t cnt = v.count[j];
+    if (cnt == 0) return;
+    const int32_t ntiles = (cnt + kFlatTile - 1) / kFlatTile;
+    if ((int64_t)blockIdx.x * kBlock >= ntiles) return;
+    fixup_tiles<T>((int64_t)blockIdx.x * kBlock + threadIdx.x, m, ntiles, T(1), v.seg_row + v.tile_off[j] + j,
+                   carry + v.tile_off[j], partial + (int64_t)j * m);
+}
+
+// y = alpha * (partial_0 + partial_1 + ...) + beta * y, panels added in index order
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_spmv_panel_reduce(int32_t m, T alpha, T beta, unsigned mask,
+                                                              const T *__restrict__ partial, T *__restrict__ y)
+{
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r >= m) return;
+    T v[kPanels];
+#pragma unroll
+    for (int j = 0; j < kPanels; ++j)
+        v[j] = (mask >> j) & 1u ? __builtin_nontemporal_load(partial + (int64_t)j * m + r) : T(0);
+    T sum = T(0);
+#pragma unroll
+    for (int j = 0; j < kPanels; ++j) sum += v[j];
+    y[r] = axpby_out<T>(alpha, sum, beta, y, r);
+}
+
+template <typename T>
+int launch_spmv_panel(int32_t m, T alpha, const PanelMatrix *pm, const T *x, T beta, T *y, T *partial, T *carry,
+                      hipStream_t s)
+{
+    if (m <= 0) return ASX_STATUS_SUCCESS;
+    PanelView v{};
+    v.row_ptr = pm->row_ptr;
+    v.col = pm->col;
+    v.seg_row = pm->seg_row;
+    v.val = pm->val;
+    unsigned mask = 0;
+    for (int j = 0; j < kPanels; ++j) {
+        v.elem_off[j] = pm->elem_off[j];
+        v.count[j] = pm->count[j];
+        v.tile_off[j] = pm->tile_off[j];
+        if (pm->count[j] > 0) mask |= 1u << j;
+    }
+    if (pm->max_tiles > 0) {
+        hipLaunchKernelGGL((k_spmv_panel<T, true>), dim3((unsigned)pm->max_tiles * kPanels), dim3(kBlock), 0, s, v, m, x,
+                           partial, carry);
+        if (pm->carry_pass)
+            hipLaunchKernelGGL((k_spmv_panel_fixup<T>), dim3((unsigned)ceil_div64(pm->max_tiles, kBlock), kPanels),
+                               dim3(kBlock), 0, s, v, m, carry, partial);
+    }
+    hipLaunchKernelGGL((k_spmv_panel_reduce<T>), dim3((unsigned)ceil_div64(m, kBlock)), dim3(kBlock), 0, s, m, alpha,
+                       beta, mask, partial, y);
+    return check_launch();
+}
+
 #define ASX_INST(T)                                                                                  \
     template int launch_spmv_vector<T>(int32_t, int32_t, T, const int32_t *, const int32_t *,        \
                                        const T *, const T *, T, T *, hipStream_t);                   \
@@ -855,7 +955,8 @@ int launch_spmv_flat(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, co
                                       const T *, const T *, T, T *, const int32_t *, const int32_t *, \
                                       T *, hipStream_t);                                             \
     template int launch_spmv_flat<T>(int32_t, int32_t, T, const int32_t *, const int32_t *, const T *, \
-                                     const T *, T, T *, const int32_t *, T *, bool, hipStream_t);
+                                     const T *, T, T *, const int32_t *, T *, bool, hipStream_t);      \
+    template int launch_spmv_panel<T>(int32_t, T, const PanelMatrix *, const T *, T, T *, T *, T *, hipStream_t);
 ASX_INST(float)
 ASX_INST(double)
 #undef ASX_INST

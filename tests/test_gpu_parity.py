@@ -348,6 +348,22 @@ def test_benchmark_configs_full_size(torch, capi, oracle):
             torch.cuda.synchronize()
             assert_close(y.cpu().numpy(), ref, scale, w.dtype, f"{name} alg={alg}")
             plan.destroy()
+        if name == "powerlaw_f64":
+            # plans that may look at columns and values: the column-panel kernel, forced and as the
+            # winner of DEFAULT's timing on this matrix (x is 8 L2s large, columns are scattered)
+            for alg in (capi.SPMV_PANEL, capi.SPMV_DEFAULT):
+                plan = capi.Plan(False, alg, w.val.dtype, w.m, w.n, w.nnz, d[0], col=d[1], val=d[2])
+                assert plan.alg == capi.SPMV_PANEL
+                for rep in range(2):
+                    y = dev(torch, w.y)
+                    capi.spmv(d[0], d[1], d[2], d[3], y, w.alpha, w.beta, alg=alg, plan=plan)
+                    torch.cuda.synchronize()
+                    assert_close(y.cpu().numpy(), ref, scale, w.dtype, f"{name} panel alg={alg} rep={rep}")
+                plan.destroy()
+        else:  # not candidates for panels: DEFAULT with values behaves as without
+            plan = capi.Plan(False, capi.SPMV_DEFAULT, w.val.dtype, w.m, w.n, w.nnz, d[0], col=d[1], val=d[2])
+            assert plan.alg == capi.SPMV_FLAT
+            plan.destroy()
         del d
     w = W.spmm_zipf_f32()
     ref = oracle.spmm(w.row_ptr, w.col, w.val, w.x, w.ncols, w.alpha, w.beta, w.y, 16)
@@ -487,6 +503,52 @@ def test_csr_transpose_rebase_dense_transpose(torch, capi):
             want = out.reshape(cols_, ld_out).copy()
             want[:, :rows_] = a.reshape(rows_, ld_in)[:, :cols_].T
             assert np.array_equal(d_out.cpu().numpy().reshape(cols_, ld_out), want), (rows_, cols_)
+
+
+# ------------------------------------------------------------------ column-panel SpMV
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_spmv_panel_kernel_shapes(torch, capi, oracle, dtype):
+    """The panel kernel forced on small matrices of every awkward shape: panels without elements,
+    rows that span many tiles of one panel, runs of empty rows, a single column panel in use,
+    beta = 0 over NaN, and two calls through one plan."""
+    rng = np.random.default_rng(91)
+    cases = []
+    for name, lens in analysis_shapes().items():
+        if np.sum(lens) == 0:
+            continue
+        n = int(max(np.max(lens), 64)) + 29
+        cases.append((name, csr_from_lengths(lens, n, 6, dtype), n))
+    # every column in the first panel; columns in the last panel only; one dense-ish long row
+    lens = np.r_[rng.integers(0, 9, 3000), 20000]
+    rp, col, val = csr_from_lengths(lens, 30000, 8, dtype)
+    cases.append(("first_panel", (rp, (col % 100).astype(np.int32), val), 30000))
+    cases.append(("last_panel", (rp, (29999 - col % 50).astype(np.int32), val), 30000))
+    cases.append(("spread", (rp, col, val), 30000))
+    for name, (rp, col, val), n in cases:
+        m = rp.size - 1
+        x = rng.uniform(-1, 1, n).astype(dtype)
+        y0 = rng.uniform(-1, 1, m).astype(dtype)
+        d = [dev(torch, a) for a in (rp, col, val, x)]
+        plan = capi.Plan(False, capi.SPMV_PANEL, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
+        assert plan.alg == capi.SPMV_PANEL
+        for alpha, beta in ((1.5, 0.5), (1.0, 0.0), (-2.0, 1.0)):
+            ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 2)
+            scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
+            for rep in range(2):
+                y = dev(torch, y0 if beta else np.full(m, np.nan, dtype=dtype))
+                capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_PANEL, plan=plan)
+                torch.cuda.synchronize()
+                assert_close(y.cpu().numpy(), ref, scale, dtype, f"{name} a={alpha} b={beta} rep={rep}")
+        plan.destroy()
+    # the panel kernel needs its plan; a plan without columns and values cannot be a panel plan
+    L = capi.lib()
+    h = capi.C.c_void_p()
+    assert L.asx_plan_create(capi.C.byref(h), 0, capi.SPMV_PANEL, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), 1, None) == 6
+    assert L.asx_spmv_csr_f64(None, capi.SPMV_PANEL, 1, 1, 0, 1.0, capi._ptr(d[0]), None, None, None, 0.0,
+                              capi._ptr(d[3]), None, 0, None) == 6
+    assert L.asx_spmv_panel_workspace_bytes(capi.R_64F, 1 << 22, 1 << 22, 1 << 25) >= 8 * (1 << 22) * 8
+    assert L.asx_spmv_panel_workspace_bytes(capi.R_64F, 1 << 24, 1 << 24, 1 << 26) == 0  # x too large for 8 slices
+    assert L.asx_spmv_panel_workspace_bytes(capi.R_32F, 1 << 20, 1 << 20, 1 << 24) == 0  # x fits one L2
 
 
 # ------------------------------------------------------------------ randomised shapes, every SpMV kernel
