@@ -185,7 +185,7 @@ int asx_spmm_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, in
  * elements into 8 column panels, one per XCD, so that each XCD's L2 holds the slice of x its
  * workgroups gather from (for matrices whose x is 1.5 to 8 L2s large and whose columns are
  * scattered; the plan then holds a COPY of the values: rebuild it when they change; calls need
- * 8*m values of workspace for the per-panel partial results).  alg = ASX_SPMV_DEFAULT on such a
+ * up to min(nnz, 8*m) values of workspace for the per-panel partial sums).  alg = ASX_SPMV_DEFAULT on such a
  * matrix builds the panels, times the panel kernel against the kernel the histogram picks (three
  * runs each on scratch vectors) and keeps the faster.  Otherwise as asx_plan_create.  No
  * counterpart in the reference (its alphasparseSpMV_analysis is a stub).  Synchronises `stream`. */

@@ -79,11 +79,11 @@ SpmmLayout spmm_merge_layout(int32_t m, int32_t nnz, int32_t ncols, size_t sv, b
 struct PanelLayout {  // [partial | carry]
     size_t partial_off, carry_off, bytes;
 };
-PanelLayout spmv_panel_layout(int32_t m, size_t total_tiles, size_t sv)
+PanelLayout spmv_panel_layout(size_t partial_sums, size_t total_tiles, size_t sv)
 {
     PanelLayout L{};
     L.partial_off = 0;
-    L.carry_off = align_up((size_t)kPanels * (size_t)m * sv, kAlign);
+    L.carry_off = align_up(std::max<size_t>(partial_sums, 1) * sv, kAlign);
     L.bytes = L.carry_off + align_up(std::max<size_t>(total_tiles, 1) * sv, kAlign);
     return L;
 }
@@ -188,7 +188,7 @@ int spmv_impl(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, 
     case ASX_SPMV_PANEL: {
         // the panels hold a copy of A's columns and values and are built by asx_spmv_plan_create
         if (!plan || !plan->panel.col) return ASX_STATUS_NOT_INITIALIZED;
-        const PanelLayout L = spmv_panel_layout(m, (size_t)plan->panel.tile_off[kPanels], sizeof(T));
+        const PanelLayout L = spmv_panel_layout((size_t)plan->panel.kbase[kPanels], (size_t)plan->panel.tile_off[kPanels], sizeof(T));
         if (!ws) return ASX_STATUS_INVALID_POINTER;
         if (ws_bytes < L.bytes) return ASX_STATUS_INVALID_SIZE;
         return launch_spmv_panel<T>(m, alpha, &plan->panel, x, beta, y, (T *)(w + L.partial_off),
@@ -585,7 +585,8 @@ static int spmv_plan_with_panels(asx_plan **out, int alg, int value_type, int32_
     }
     pp->nunits = pp->panel.tile_off[kPanels];
     pp->carry_pass = pp->panel.carry_pass;
-    pp->workspace_bytes = spmv_panel_layout(m, (size_t)pp->panel.tile_off[kPanels], sizeof(T)).bytes;
+    pp->workspace_bytes =
+        spmv_panel_layout((size_t)pp->panel.kbase[kPanels], (size_t)pp->panel.tile_off[kPanels], sizeof(T)).bytes;
     if (alg == ASX_SPMV_PANEL) {
         asx_plan_destroy(base);
         *out = pp;
@@ -644,7 +645,9 @@ size_t asx_spmv_panel_workspace_bytes(int value_type, int32_t m, int32_t n, int3
     if (m <= 0 || n <= 0 || nnz <= 0) return 0;
     const size_t sv = vsize(value_type);
     if (!panel_candidate(m, n, nnz, sv)) return 0;
-    return spmv_panel_layout(m, (size_t)ceil_div64(nnz, kFlatTile) + kPanels, sv).bytes;
+    // a row leaves at most one partial sum per panel and no more than it has stored elements
+    const size_t partial_sums = std::min<size_t>((size_t)nnz, (size_t)kPanels * (size_t)m);
+    return spmv_panel_layout(partial_sums, (size_t)ceil_div64(nnz, kFlatTile) + kPanels, sv).bytes;
 }
 
 int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill)

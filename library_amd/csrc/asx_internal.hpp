@@ -103,20 +103,27 @@ int launch_spmm_blocked(int32_t m, int32_t k, int32_t ncols, T alpha, const Bloc
                         int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t s);
 
 // ---- column-panel SpMV (asx_panel.hip builds, asx_spmv.hip runs) ----
-// The stored elements regrouped into kPanels column panels (panel = col / width), each panel a
-// CSR matrix of its own over all m rows.  Workgroup b works on panel b % kPanels: consecutive
+// The stored elements regrouped into kPanels column panels (panel = col / width).  Each panel is
+// a CSR matrix over the rows that have elements in it (rows without any are left out: with short
+// rows most panels miss most rows).  Workgroup b works on panel b % kPanels: consecutive
 // workgroups go to consecutive XCDs, so each XCD's L2 only ever sees one panel's slice of x.
+// A panel writes one partial sum per row it holds; `prow_ptr` / `ppos` list, for every row of A,
+// where its partial sums are, in panel order.
 constexpr int kPanels = 8;
 struct PanelMatrix {
     int32_t width;                  // columns per panel
     int32_t count[kPanels];         // stored elements per panel
     int64_t elem_off[kPanels + 1];  // start of each panel in col / val (multiples of 4 elements)
     int32_t tile_off[kPanels + 1];  // start of each panel's tiles in the carry array
+    int32_t krows[kPanels];         // rows present in each panel
+    int32_t kbase[kPanels + 1];     // start of each panel in the partial-sum array
     int32_t max_tiles;
-    int32_t *col;      // device
-    void *val;         // device, a copy of A's values in panel order
-    int32_t *row_ptr;  // device, kPanels x (m + 1)
-    int32_t *seg_row;  // device, panel j at tile_off[j] + j, tiles_j + 1 entries
+    int32_t *col;       // device
+    void *val;          // device, a copy of A's values in panel order
+    int32_t *row_ptr;   // device, panel j at kbase[j] + j, krows[j] + 1 entries
+    int32_t *seg_row;   // device, panel j at tile_off[j] + j, tiles_j + 1 entries
+    int32_t *prow_ptr;  // device, m + 1
+    int32_t *ppos;      // device, kbase[kPanels]
     int carry_pass;
 };
 template <typename T>

@@ -1,7 +1,7 @@
 // Builds the column-panel copy of a CSR matrix for the panel SpMV kernel (device side, once per
-// plan): a stable radix sort of the stored elements by panel keeps CSR order inside each panel,
-// so every panel is itself a CSR matrix over all m rows; its row offsets come from binary
-// searches of the original row offsets in the sorted element positions.
+// plan).  A stable radix sort of the stored elements by panel keeps CSR order inside each panel;
+// the first element of every (panel, row) run opens a compact row of that panel; a second stable
+// sort of those run heads by row lists, for every row of A, its partial sums in panel order.
 #include <hipcub/hipcub.hpp>
 
 #include "asx_internal.hpp"
@@ -22,11 +22,13 @@ struct PanelOffsets {
     int64_t elem_off[kPanels + 1];
 };
 
+// Copies columns and values into panel order and finds the row of A of every element.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_panel_gather(const int32_t *__restrict__ keys, const int32_t *__restrict__ idx,
-                                                         int32_t nnz, PanelOffsets o, const int32_t *__restrict__ col,
+                                                         int32_t nnz, PanelOffsets o, const int32_t *__restrict__ row_ptr,
+                                                         int32_t m, const int32_t *__restrict__ col,
                                                          const T *__restrict__ val, int32_t *__restrict__ col_out,
-                                                         T *__restrict__ val_out)
+                                                         T *__restrict__ val_out, int32_t *__restrict__ srow)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= nnz) return;
@@ -35,35 +37,59 @@ __global__ __launch_bounds__(kBlock) void k_panel_gather(const int32_t *__restri
     const int32_t src = idx[i];
     col_out[dst] = col[src];
     val_out[dst] = val[src];
+    int32_t lo = 0, hi = m;  // largest r with row_ptr[r] <= src
+    while (lo < hi) {
+        const int32_t mid = lo + (hi - lo + 1) / 2;
+        if (row_ptr[mid] <= src)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    srow[i] = lo;
 }
 
-// row_ptr_out[j][r] = number of panel-j elements whose original position is below row_ptr[r]
-__global__ __launch_bounds__(kBlock) void k_panel_row_ptr(const int32_t *__restrict__ idx, PanelOffsets o,
-                                                          const int32_t *__restrict__ row_ptr, int32_t m,
-                                                          int32_t *__restrict__ row_ptr_out)
+// head[i] = 1 where element i opens a (panel, row) run
+__global__ __launch_bounds__(kBlock) void k_panel_heads(const int32_t *__restrict__ keys, const int32_t *__restrict__ srow,
+                                                        int32_t nnz, int32_t *__restrict__ head)
 {
-    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int j = blockIdx.y;
-    if (r > m) return;
-    const int32_t *p = idx + o.pstart[j];
-    const int32_t target = row_ptr[r];
-    int32_t lo = 0, hi = o.pstart[j + 1] - o.pstart[j];
-    while (lo < hi) {
-        const int32_t mid = (lo + hi) / 2;
-        if (p[mid] < target)
-            lo = mid + 1;
-        else
-            hi = mid;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nnz) return;
+    head[i] = i == 0 || keys[i] != keys[i - 1] || srow[i] != srow[i - 1];
+}
+
+// For every run head (its index among all heads is g = hscan - 1): where the run starts inside its
+// panel, which row of A it belongs to, and g itself as the payload of the sort by row.  The last
+// element of a panel also closes the panel's offsets.
+__global__ __launch_bounds__(kBlock) void k_panel_rows(const int32_t *__restrict__ keys, const int32_t *__restrict__ srow,
+                                                       const int32_t *__restrict__ head, const int32_t *__restrict__ hscan,
+                                                       int32_t nnz, PanelOffsets o, int32_t *__restrict__ crow_ptr,
+                                                       int32_t *__restrict__ hrow, int32_t *__restrict__ hpos)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nnz) return;
+    const int j = keys[i];
+    if (head[i]) {
+        const int32_t g = hscan[i] - 1;
+        crow_ptr[g + j] = (int32_t)(i - o.pstart[j]);
+        hrow[g] = srow[i];
+        hpos[g] = g;
     }
-    row_ptr_out[(int64_t)j * (m + 1) + r] = lo;
+    if (i + 1 == o.pstart[j + 1]) crow_ptr[hscan[i] + j] = o.pstart[j + 1] - o.pstart[j];
 }
 
 void free_panels(PanelMatrix *p)
 {
-    for (void *q : {(void *)p->col, p->val, (void *)p->row_ptr, (void *)p->seg_row})
+    for (void *q : {(void *)p->col, p->val, (void *)p->row_ptr, (void *)p->seg_row, (void *)p->prow_ptr, (void *)p->ppos})
         if (q) (void)hipFree(q);
-    p->col = p->row_ptr = p->seg_row = nullptr;
+    p->col = p->row_ptr = p->seg_row = p->prow_ptr = p->ppos = nullptr;
     p->val = nullptr;
+}
+
+static int bits_to_hold(int64_t v)
+{
+    int b = 1;
+    while (b < 31 && ((int64_t)1 << b) <= v) ++b;
+    return b;
 }
 
 template <typename T>
@@ -74,34 +100,38 @@ int build_panels(int32_t m, int32_t n, int32_t nnz, const int32_t *row_ptr, cons
     if (m <= 0 || nnz <= 0 || n < kPanels) return ASX_STATUS_INVALID_SIZE;
     pm.width = (int32_t)(ceil_div64(ceil_div64(n, kPanels), 32) * 32);
     int st = ASX_STATUS_SUCCESS;
-    int32_t *keys = nullptr, *keys2 = nullptr, *idx = nullptr, *idx2 = nullptr, *d_pstart = nullptr, *d_flag = nullptr;
+    // a..f: six nnz-sized scratch arrays reused through the stages
+    int32_t *a = nullptr, *b = nullptr, *c = nullptr, *d = nullptr, *e = nullptr, *f = nullptr, *d_small = nullptr;
     void *tmp = nullptr;
-    size_t tmp_bytes = 0;
+    size_t tmp_sort = 0, tmp_scan = 0, tmp_sort2 = 0, tmp_bytes = 0;
     PanelOffsets o{};
-    int32_t h_flag = 0;
+    int32_t h_flag = 0, ktotal = 0;
     const unsigned grid = (unsigned)ceil_div64(nnz, kBlock);
+    const size_t nb = sizeof(int32_t) * (size_t)nnz;
+    const int row_bits = bits_to_hold(m);
 #define ASX_TRY(expr)             \
     do {                          \
         st = status_of(expr);     \
         if (st) goto done;        \
     } while (0)
-#define ASX_TRY_ST(expr) \
-    do {                 \
-        st = (expr);     \
+#define ASX_TRY_ST(expr)   \
+    do {                   \
+        st = (expr);       \
         if (st) goto done; \
     } while (0)
-    ASX_TRY(hipMalloc((void **)&keys, sizeof(int32_t) * (size_t)nnz));
-    ASX_TRY(hipMalloc((void **)&keys2, sizeof(int32_t) * (size_t)nnz));
-    ASX_TRY(hipMalloc((void **)&idx, sizeof(int32_t) * (size_t)nnz));
-    ASX_TRY(hipMalloc((void **)&idx2, sizeof(int32_t) * (size_t)nnz));
-    ASX_TRY(hipMalloc((void **)&d_pstart, sizeof(int32_t) * (kPanels + 1)));
-    ASX_TRY(hipMalloc((void **)&d_flag, sizeof(int32_t)));
-    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, keys, keys2, idx, idx2, nnz, 0, 3, s));
+    for (int32_t **q : {&a, &b, &c, &d, &e, &f}) ASX_TRY(hipMalloc((void **)q, nb));
+    ASX_TRY(hipMalloc((void **)&d_small, sizeof(int32_t) * (kPanels + 2)));
+    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_sort, a, b, c, d, nnz, 0, 3, s));
+    ASX_TRY(hipcub::DeviceScan::InclusiveSum(nullptr, tmp_scan, a, b, nnz, s));
+    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_sort2, a, b, c, d, nnz, 0, row_bits, s));
+    tmp_bytes = std::max(tmp_sort, std::max(tmp_scan, tmp_sort2));
     ASX_TRY(hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1));
-    hipLaunchKernelGGL(k_panel_keys, dim3(grid), dim3(kBlock), 0, s, col, nnz, pm.width, keys, idx);
-    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, keys, keys2, idx, idx2, nnz, 0, 3, s));
-    ASX_TRY_ST(launch_offsets_from_sorted(keys2, nnz, kPanels, d_pstart, s));
-    ASX_TRY(hipMemcpyAsync(o.pstart, d_pstart, sizeof(o.pstart), hipMemcpyDeviceToHost, s));
+
+    // 1. elements by panel: b = panel of each sorted element, d = its position in A
+    hipLaunchKernelGGL(k_panel_keys, dim3(grid), dim3(kBlock), 0, s, col, nnz, pm.width, a, c);
+    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, a, b, c, d, nnz, 0, 3, s));
+    ASX_TRY_ST(launch_offsets_from_sorted(b, nnz, kPanels, d_small, s));
+    ASX_TRY(hipMemcpyAsync(o.pstart, d_small, sizeof(o.pstart), hipMemcpyDeviceToHost, s));
     ASX_TRY(hipStreamSynchronize(s));
     pm.max_tiles = 0;
     for (int j = 0; j < kPanels; ++j) {
@@ -115,27 +145,45 @@ int build_panels(int32_t m, int32_t n, int32_t nnz, const int32_t *row_ptr, cons
     o.elem_off[kPanels] = pm.elem_off[kPanels];
     ASX_TRY(hipMalloc((void **)&pm.col, sizeof(int32_t) * (size_t)(pm.elem_off[kPanels] + 4)));
     ASX_TRY(hipMalloc(&pm.val, sizeof(T) * (size_t)(pm.elem_off[kPanels] + 4)));
-    ASX_TRY(hipMalloc((void **)&pm.row_ptr, sizeof(int32_t) * (size_t)kPanels * ((size_t)m + 1)));
-    ASX_TRY(hipMalloc((void **)&pm.seg_row, sizeof(int32_t) * (size_t)(pm.tile_off[kPanels] + kPanels)));
-    hipLaunchKernelGGL((k_panel_gather<T>), dim3(grid), dim3(kBlock), 0, s, keys2, idx2, nnz, o, col, val, pm.col,
-                       (T *)pm.val);
-    hipLaunchKernelGGL(k_panel_row_ptr, dim3((unsigned)ceil_div64((int64_t)m + 1, kBlock), kPanels), dim3(kBlock), 0, s,
-                       idx2, o, row_ptr, m, pm.row_ptr);
-    ASX_TRY(hipGetLastError());
-    ASX_TRY(hipMemsetAsync(d_flag, 0, sizeof(int32_t), s));
-    for (int j = 0; j < kPanels; ++j) {
-        const int32_t *rp = pm.row_ptr + (int64_t)j * (m + 1);
-        int32_t *seg = pm.seg_row + pm.tile_off[j] + j;
-        ASX_TRY_ST(launch_nnz_split_rows_n(rp, m, flat_tiles(pm.count[j]), kFlatTile, seg, s));
-        if (pm.count[j] > 0) ASX_TRY_ST(launch_flat_has_carry(rp, m, pm.count[j], seg, d_flag, s));
+    // 2. columns and values in panel order; a = row of A of each sorted element
+    hipLaunchKernelGGL((k_panel_gather<T>), dim3(grid), dim3(kBlock), 0, s, b, d, nnz, o, row_ptr, m, col, val, pm.col,
+                       (T *)pm.val, a);
+    // 3. run heads: c = flags, e = their inclusive scan
+    hipLaunchKernelGGL(k_panel_heads, dim3(grid), dim3(kBlock), 0, s, b, a, nnz, c);
+    ASX_TRY(hipcub::DeviceScan::InclusiveSum(tmp, tmp_bytes, c, e, nnz, s));
+    ASX_TRY(hipMemcpyAsync(&ktotal, e + (nnz - 1), sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    for (int j = 1; j <= kPanels; ++j) {
+        if (o.pstart[j] > 0)
+            ASX_TRY(hipMemcpyAsync(&pm.kbase[j], e + (o.pstart[j] - 1), sizeof(int32_t), hipMemcpyDeviceToHost, s));
     }
-    ASX_TRY(hipMemcpyAsync(&h_flag, d_flag, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    ASX_TRY(hipStreamSynchronize(s));
+    for (int j = 0; j < kPanels; ++j) pm.krows[j] = pm.kbase[j + 1] - pm.kbase[j];
+    ASX_TRY(hipMalloc((void **)&pm.row_ptr, sizeof(int32_t) * ((size_t)ktotal + kPanels)));
+    ASX_TRY(hipMalloc((void **)&pm.seg_row, sizeof(int32_t) * (size_t)(pm.tile_off[kPanels] + kPanels)));
+    ASX_TRY(hipMalloc((void **)&pm.prow_ptr, sizeof(int32_t) * ((size_t)m + 1)));
+    ASX_TRY(hipMalloc((void **)&pm.ppos, sizeof(int32_t) * (size_t)ktotal));
+    // panels without elements still need their single offset
+    ASX_TRY(hipMemsetAsync(pm.row_ptr, 0, sizeof(int32_t) * ((size_t)ktotal + kPanels), s));
+    // 4. compact row offsets per panel; d = row of A of each head, f = index of each head
+    hipLaunchKernelGGL(k_panel_rows, dim3(grid), dim3(kBlock), 0, s, b, a, c, e, nnz, o, pm.row_ptr, d, f);
+    // 5. heads by row of A (stable: panel order inside a row): a = sorted rows, ppos = partial-sum index
+    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, d, a, f, pm.ppos, ktotal, 0, row_bits, s));
+    ASX_TRY_ST(launch_offsets_from_sorted(a, ktotal, m, pm.prow_ptr, s));
+    // 6. tiles of each panel
+    ASX_TRY(hipMemsetAsync(d_small, 0, sizeof(int32_t), s));
+    for (int j = 0; j < kPanels; ++j) {
+        const int32_t *rp = pm.row_ptr + pm.kbase[j] + j;
+        int32_t *seg = pm.seg_row + pm.tile_off[j] + j;
+        ASX_TRY_ST(launch_nnz_split_rows_n(rp, pm.krows[j], flat_tiles(pm.count[j]), kFlatTile, seg, s));
+        if (pm.count[j] > 0) ASX_TRY_ST(launch_flat_has_carry(rp, pm.krows[j], pm.count[j], seg, d_small, s));
+    }
+    ASX_TRY(hipMemcpyAsync(&h_flag, d_small, sizeof(int32_t), hipMemcpyDeviceToHost, s));
     ASX_TRY(hipStreamSynchronize(s));
     pm.carry_pass = h_flag != 0;
 #undef ASX_TRY
 #undef ASX_TRY_ST
 done:
-    for (void *p : {(void *)keys, (void *)keys2, (void *)idx, (void *)idx2, (void *)d_pstart, (void *)d_flag, tmp})
+    for (void *p : {(void *)a, (void *)b, (void *)c, (void *)d, (void *)e, (void *)f, (void *)d_small, tmp})
         if (p) (void)hipFree(p);
     if (st) {
         free_panels(&pm);

@@ -859,19 +859,22 @@ int launch_spmv_flat(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, co
 // Random gathers that miss the 4 MiB L2 of an XCD cost a 128-byte fill each (60 G gathers/s
 // against 180 G/s for hits).  With the stored elements regrouped by column panel and workgroup b
 // working on panel b % kPanels, workgroups on one XCD (consecutive workgroups go to consecutive
-// XCDs) only gather from one slice of x, which then lives in that XCD's L2.  Each panel writes
-// its own partial result vector; an ordered pass adds the kPanels partial vectors into y.
+// XCDs) only gather from one slice of x, which then lives in that XCD's L2.  A panel is a CSR
+// matrix over the rows present in it and writes one partial sum per such row; an ordered pass
+// then adds, for every row of A, its partial sums in panel order.
 struct PanelView {
     const int32_t *row_ptr, *col, *seg_row;
     const void *val;
     int64_t elem_off[kPanels];
     int32_t count[kPanels];
     int32_t tile_off[kPanels];
+    int32_t krows[kPanels];
+    int32_t kbase[kPanels];
 };
 
 template <typename T, bool NT>
-__global__ __launch_bounds__(kBlock) void k_spmv_panel(PanelView v, int32_t m, const T *__restrict__ x,
-                                                       T *__restrict__ partial, T *__restrict__ carry)
+__global__ __launch_bounds__(kBlock) void k_spmv_panel(PanelView v, const T *__restrict__ x, T *__restrict__ partial,
+                                                       T *__restrict__ carry)
 {
     __shared__ FlatShared<T> sh;
     const int j = blockIdx.x % kPanels;
@@ -883,12 +886,12 @@ __global__ __launch_bounds__(kBlock) void k_spmv_panel(PanelView v, int32_t m, c
     int32_t c[4];
     T p[4];
     flat_load<T, true, NT>(t, cnt, col, val, c, p);
-    flat_tile<T, NT>(sh, t, m, cnt, T(1), v.row_ptr + (int64_t)j * (m + 1), c, p, x, T(0),
-                     partial + (int64_t)j * m, v.seg_row + v.tile_off[j] + j, carry + v.tile_off[j]);
+    flat_tile<T, false>(sh, t, v.krows[j], cnt, T(1), v.row_ptr + v.kbase[j] + j, c, p, x, T(0), partial + v.kbase[j],
+                        v.seg_row + v.tile_off[j] + j, carry + v.tile_off[j]);
 }
 
 template <typename T>
-__global__ __launch_bounds__(kBlock) void k_spmv_panel_fixup(PanelView v, int32_t m, const T *__restrict__ carry,
+__global__ __launch_bounds__(kBlock) void k_spmv_panel_fixup(PanelView v, const T *__restrict__ carry,
                                                              T *__restrict__ partial)
 {
     const int j = blockIdx.y;
@@ -896,21 +899,23 @@ __global__ __launch_bounds__(kBlock) void k_spmv_panel_fixup(PanelView v, int32_
     if (cnt == 0) return;
     const int32_t ntiles = (cnt + kFlatTile - 1) / kFlatTile;
     if ((int64_t)blockIdx.x * kBlock >= ntiles) return;
-    fixup_tiles<T>((int64_t)blockIdx.x * kBlock + threadIdx.x, m, ntiles, T(1), v.seg_row + v.tile_off[j] + j,
-                   carry + v.tile_off[j], partial + (int64_t)j * m);
+    fixup_tiles<T>((int64_t)blockIdx.x * kBlock + threadIdx.x, v.krows[j], ntiles, T(1), v.seg_row + v.tile_off[j] + j,
+                   carry + v.tile_off[j], partial + v.kbase[j]);
 }
 
-// y = alpha * (partial_0 + partial_1 + ...) + beta * y, panels added in index order
+// y[r] = alpha * (sum of row r's partial sums, in panel order) + beta * y[r]
 template <typename T>
-__global__ __launch_bounds__(kBlock) void k_spmv_panel_reduce(int32_t m, T alpha, T beta, unsigned mask,
+__global__ __launch_bounds__(kBlock) void k_spmv_panel_reduce(int32_t m, T alpha, T beta,
+                                                              const int32_t *__restrict__ prow_ptr,
+                                                              const int32_t *__restrict__ ppos,
                                                               const T *__restrict__ partial, T *__restrict__ y)
 {
     const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (r >= m) return;
+    const int32_t s = prow_ptr[r], e = prow_ptr[r + 1];
     T v[kPanels];
 #pragma unroll
-    for (int j = 0; j < kPanels; ++j)
-        v[j] = (mask >> j) & 1u ? __builtin_nontemporal_load(partial + (int64_t)j * m + r) : T(0);
+    for (int j = 0; j < kPanels; ++j) v[j] = s + j < e ? partial[ppos[s + j]] : T(0);
     T sum = T(0);
 #pragma unroll
     for (int j = 0; j < kPanels; ++j) sum += v[j];
@@ -927,22 +932,22 @@ int launch_spmv_panel(int32_t m, T alpha, const PanelMatrix *pm, const T *x, T b
     v.col = pm->col;
     v.seg_row = pm->seg_row;
     v.val = pm->val;
-    unsigned mask = 0;
     for (int j = 0; j < kPanels; ++j) {
         v.elem_off[j] = pm->elem_off[j];
         v.count[j] = pm->count[j];
         v.tile_off[j] = pm->tile_off[j];
-        if (pm->count[j] > 0) mask |= 1u << j;
+        v.krows[j] = pm->krows[j];
+        v.kbase[j] = pm->kbase[j];
     }
     if (pm->max_tiles > 0) {
-        hipLaunchKernelGGL((k_spmv_panel<T, true>), dim3((unsigned)pm->max_tiles * kPanels), dim3(kBlock), 0, s, v, m, x,
+        hipLaunchKernelGGL((k_spmv_panel<T, true>), dim3((unsigned)pm->max_tiles * kPanels), dim3(kBlock), 0, s, v, x,
                            partial, carry);
         if (pm->carry_pass)
             hipLaunchKernelGGL((k_spmv_panel_fixup<T>), dim3((unsigned)ceil_div64(pm->max_tiles, kBlock), kPanels),
-                               dim3(kBlock), 0, s, v, m, carry, partial);
+                               dim3(kBlock), 0, s, v, carry, partial);
     }
     hipLaunchKernelGGL((k_spmv_panel_reduce<T>), dim3((unsigned)ceil_div64(m, kBlock)), dim3(kBlock), 0, s, m, alpha,
-                       beta, mask, partial, y);
+                       beta, pm->prow_ptr, pm->ppos, partial, y);
     return check_launch();
 }
 
