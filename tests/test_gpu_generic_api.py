@@ -181,3 +181,25 @@ def test_cli_on_matrixmarket_files(tmp_path):
     assert len(lines) == 8 and all(len(l.split(",")) == 11 for l in lines)  # DEFAULT + the reference's 7 ids
     r = subprocess.run([CLI, f"--data-file={tmp_path / 'none.mtx'}"], capture_output=True, text=True, timeout=60)
     assert r.returncode == 4
+
+
+def test_spmv_analysis_on_a_panel_candidate(tmp_path, oracle):
+    """A matrix whose x (8 MiB) is a candidate for the column-panel kernel: analysis with DEFAULT
+    builds the panels and times them; whichever kernel it keeps, the buffer alphasparseSpMV_bufferSize
+    reported must do and the result must match, also for opA = TRANSPOSE."""
+    from library_amd import workloads as W
+    rp, col, val = W.csr_zipf(1 << 20, 1 << 20, 20, 1.0, 5000, 0.01, np.float64, 3)
+    n = 1 << 20
+    assert col.size >= 1 << 22
+    rng = np.random.default_rng(61)
+    x = rng.uniform(-1, 1, n)
+    y0 = rng.uniform(-1, 1, rp.size - 1)
+    alpha, beta = 2.1, 3.2
+    ref = oracle.spmv(rp, col, val, x, alpha, beta, y0, 8)
+    scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
+    got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, alpha, beta, 1)
+    assert_close(got, ref, scale, np.float64, "DEFAULT with analysis")
+    rp_t, col_t, val_t = _transpose_csr(rp, col, val, n)
+    ref_t = oracle.spmv(rp_t, col_t, val_t, y0, alpha, beta, x, 8)
+    got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, y0, x, 1, 0, alpha, beta, 1, (1, 0, 0, 0, 0), n=n)
+    assert_close(got, ref_t, spmv_scale(rp_t, col_t, val_t, y0, alpha, beta, x), np.float64, "transpose, DEFAULT with analysis")
