@@ -224,24 +224,33 @@ int launch_loadbalance_partition(const int32_t *d_row_ptr, int32_t m, int32_t nn
 }
 
 // -------------------------------------------------------------------------------------------
-// Calibration copy: 16 bytes per lane per iteration, grid-stride.
+// Calibration copy: four 16-byte non-temporal loads in flight per lane, then four non-temporal
+// stores, grid-stride.
 // -------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
-                                                size_t n16)
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void k_copy16(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, size_t n16)
 {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16;
-         i += (size_t)gridDim.x * blockDim.x)
-        dst[i] = src[i];
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        const u32x4 a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + stride),
+                    c = __builtin_nontemporal_load(src + i + 2 * stride),
+                    d = __builtin_nontemporal_load(src + i + 3 * stride);
+        __builtin_nontemporal_store(a, dst + i);
+        __builtin_nontemporal_store(b, dst + i + stride);
+        __builtin_nontemporal_store(c, dst + i + 2 * stride);
+        __builtin_nontemporal_store(d, dst + i + 3 * stride);
+    }
+    for (; i < n16; i += stride) dst[i] = src[i];
 }
 
 int launch_copy_bytes(const void *d_src, void *d_dst, size_t bytes, hipStream_t s)
 {
     size_t n16 = bytes / 16;
     if (n16 == 0) return ASX_STATUS_SUCCESS;
-    size_t grid = (n16 + 255) / 256;
-    if (grid > 256 * 32) grid = 256 * 32;
-    hipLaunchKernelGGL(k_copy16, dim3((unsigned)grid), dim3(256), 0, s, (const uint4 *)d_src,
-                       (uint4 *)d_dst, n16);
+    size_t grid = (n16 + 256 * 4 - 1) / (256 * 4);
+    if (grid > 256 * 64) grid = 256 * 64;
+    hipLaunchKernelGGL(k_copy16, dim3((unsigned)grid), dim3(256), 0, s, (const u32x4 *)d_src, (u32x4 *)d_dst, n16);
     return check_launch();
 }
 
