@@ -247,7 +247,7 @@ def main():
     a = parse()
     if a.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {a.gpus} is not supported "
-              "(the path has no multi-GPU part: rows shard by nnz with an all-gather of x, see DESIGN.md)",
+              "(the path has no multi-GPU part: rows shard by nnz with an all-gather of x)",
               file=sys.stderr)
         sys.exit(2)
     import torch
