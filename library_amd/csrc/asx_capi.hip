@@ -88,7 +88,7 @@ PanelLayout spmv_panel_layout(size_t partial_sums, size_t total_tiles, size_t sv
     return L;
 }
 
-// Panels pay when x is too large for one 4 MiB L2 but each of kPanels slices fits one.
+// Panels pay when x is too large for one 4 MiB L2 but each of the kPanels slices fits one.
 constexpr size_t kL2Bytes = (size_t)4 << 20;
 bool panel_candidate(int32_t m, int32_t n, int32_t nnz, size_t sv)
 {

@@ -105,11 +105,17 @@ int launch_spmm_blocked(int32_t m, int32_t k, int32_t ncols, T alpha, const Bloc
 // ---- column-panel SpMV (asx_panel.hip builds, asx_spmv.hip runs) ----
 // The stored elements regrouped into kPanels column panels (panel = col / width).  Each panel is
 // a CSR matrix over the rows that have elements in it (rows without any are left out: with short
-// rows most panels miss most rows).  Workgroup b works on panel b % kPanels: consecutive
-// workgroups go to consecutive XCDs, so each XCD's L2 only ever sees one panel's slice of x.
-// A panel writes one partial sum per row it holds; `prow_ptr` / `ppos` list, for every row of A,
-// where its partial sums are, in panel order.
-constexpr int kPanels = 8;
+// rows most panels miss most rows).  Workgroup b runs on XCD b % kXcds (consecutive workgroups
+// go to consecutive XCDs) and works on panel b % kXcds first and then, when that panel's tiles
+// are used up, on panel b % kXcds + kXcds, ...: at any time an XCD's L2 sees one panel's slice
+// of x (workgroups are dispatched in order, so the phases of one XCD barely overlap).
+// A panel writes one partial sum per row it holds.  `rowid` names the row of A of every partial
+// sum; `blk_lo` says, for every block of kPanelRowBlock rows of A, where in each panel's partial
+// sums the block's rows start, so the reduction reads contiguous ranges.
+constexpr int kXcds = 8;
+constexpr int kPanelPhases = 2;
+constexpr int kPanels = kXcds * kPanelPhases;
+constexpr int kPanelRowBlock = 1024;  // rows of A per workgroup of the reduction
 struct PanelMatrix {
     int32_t width;                  // columns per panel
     int32_t count[kPanels];         // stored elements per panel
@@ -117,13 +123,13 @@ struct PanelMatrix {
     int32_t tile_off[kPanels + 1];  // start of each panel's tiles in the carry array
     int32_t krows[kPanels];         // rows present in each panel
     int32_t kbase[kPanels + 1];     // start of each panel in the partial-sum array
-    int32_t max_tiles;
+    int32_t max_tiles;              // largest number of tiles one XCD works through
     int32_t *col;       // device
     void *val;          // device, a copy of A's values in panel order
     int32_t *row_ptr;   // device, panel j at kbase[j] + j, krows[j] + 1 entries
     int32_t *seg_row;   // device, panel j at tile_off[j] + j, tiles_j + 1 entries
-    int32_t *prow_ptr;  // device, m + 1
-    int32_t *ppos;      // device, kbase[kPanels]
+    int32_t *rowid;     // device, kbase[kPanels]: row of A of each partial sum
+    int32_t *blk_lo;    // device, (ceil(m / kPanelRowBlock) + 1) x kPanels
     int carry_pass;
 };
 template <typename T>

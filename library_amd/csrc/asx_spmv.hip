@@ -857,9 +857,10 @@ int launch_spmv_flat(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, co
 // panel: the flat kernel over kPanels column panels, one panel per XCD
 // ===========================================================================================
 // Random gathers that miss the 4 MiB L2 of an XCD cost a 128-byte fill each (60 G gathers/s
-// against 180 G/s for hits).  With the stored elements regrouped by column panel and workgroup b
-// working on panel b % kPanels, workgroups on one XCD (consecutive workgroups go to consecutive
-// XCDs) only gather from one slice of x, which then lives in that XCD's L2.  A panel is a CSR
+// against 180 G/s for hits).  With the stored elements regrouped by column panel and the
+// workgroups of one XCD (consecutive workgroups go to consecutive XCDs) working through that
+// XCD's panels one after the other, an XCD gathers from one slice of x at a time, which then
+// lives in its L2.  A panel is a CSR
 // matrix over the rows present in it and writes one partial sum per such row; an ordered pass
 // then adds, for every row of A, its partial sums in panel order.
 struct PanelView {
@@ -877,10 +878,16 @@ __global__ __launch_bounds__(kBlock) void k_spmv_panel(PanelView v, const T *__r
                                                        T *__restrict__ carry)
 {
     __shared__ FlatShared<T> sh;
-    const int j = blockIdx.x % kPanels;
-    const int t = blockIdx.x / kPanels;
-    const int32_t cnt = v.count[j];
-    if (cnt == 0 || t >= (cnt + kFlatTile - 1) / kFlatTile) return;  // uniform over the workgroup
+    int j = blockIdx.x % kXcds;
+    int t = blockIdx.x / kXcds;
+    int32_t cnt = 0;
+    for (; j < kPanels; j += kXcds) {  // the panel of this XCD that tile t falls into
+        cnt = v.count[j];
+        const int tiles = (cnt + kFlatTile - 1) / kFlatTile;
+        if (t < tiles) break;
+        t -= tiles;
+    }
+    if (j >= kPanels) return;  // uniform over the workgroup
     const int32_t *col = v.col + v.elem_off[j];
     const T *val = static_cast<const T *>(v.val) + v.elem_off[j];
     int32_t c[4];
@@ -903,23 +910,50 @@ __global__ __launch_bounds__(kBlock) void k_spmv_panel_fixup(PanelView v, const 
                    carry + v.tile_off[j], partial + v.kbase[j]);
 }
 
-// y[r] = alpha * (sum of row r's partial sums, in panel order) + beta * y[r]
+// y[r] = alpha * (sum of row r's partial sums, in panel order) + beta * y[r].  One workgroup per
+// block of kPanelRowBlock rows of A: the partial sums of those rows are one contiguous range of
+// every panel (blk_lo), so all loads are contiguous; they are added into an LDS accumulator per
+// row, one panel after the other (a row appears at most once in a panel, so the adds of one
+// panel never collide).
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_spmv_panel_reduce(int32_t m, T alpha, T beta,
-                                                              const int32_t *__restrict__ prow_ptr,
-                                                              const int32_t *__restrict__ ppos,
+                                                              const int32_t *__restrict__ blk_lo,
+                                                              const int32_t *__restrict__ rowid,
                                                               const T *__restrict__ partial, T *__restrict__ y)
 {
-    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (r >= m) return;
-    const int32_t s = prow_ptr[r], e = prow_ptr[r + 1];
+    __shared__ T acc[kPanelRowBlock];
+    __shared__ int32_t s_lo[kPanels], s_hi[kPanels];
+    const int tid = threadIdx.x;
+    const int64_t b = blockIdx.x;
+    const int32_t r0 = (int32_t)(b * kPanelRowBlock);
+    if (tid < kPanels) {
+        s_lo[tid] = blk_lo[b * kPanels + tid];
+        s_hi[tid] = blk_lo[(b + 1) * kPanels + tid];
+    }
+#pragma unroll
+    for (int i = tid; i < kPanelRowBlock; i += kBlock) acc[i] = T(0);
+    __syncthreads();
+    // first kBlock entries of every panel's range: all loads issued before the first add
     T v[kPanels];
+    int32_t rid[kPanels];
 #pragma unroll
-    for (int j = 0; j < kPanels; ++j) v[j] = s + j < e ? partial[ppos[s + j]] : T(0);
-    T sum = T(0);
+    for (int j = 0; j < kPanels; ++j) {
+        const int32_t k = s_lo[j] + tid;
+        const bool ok = k < s_hi[j];
+        rid[j] = ok ? rowid[k] - r0 : -1;
+        v[j] = ok ? partial[k] : T(0);
+    }
 #pragma unroll
-    for (int j = 0; j < kPanels; ++j) sum += v[j];
-    y[r] = axpby_out<T>(alpha, sum, beta, y, r);
+    for (int j = 0; j < kPanels; ++j) {
+        if (rid[j] >= 0) acc[rid[j]] += v[j];
+        for (int32_t k = s_lo[j] + kBlock + tid; k < s_hi[j]; k += kBlock) acc[rowid[k] - r0] += partial[k];
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = tid; i < kPanelRowBlock; i += kBlock) {
+        const int64_t r = (int64_t)r0 + i;
+        if (r < m) y[r] = axpby_out<T>(alpha, acc[i], beta, y, r);
+    }
 }
 
 template <typename T>
@@ -940,14 +974,14 @@ int launch_spmv_panel(int32_t m, T alpha, const PanelMatrix *pm, const T *x, T b
         v.kbase[j] = pm->kbase[j];
     }
     if (pm->max_tiles > 0) {
-        hipLaunchKernelGGL((k_spmv_panel<T, true>), dim3((unsigned)pm->max_tiles * kPanels), dim3(kBlock), 0, s, v, x,
+        hipLaunchKernelGGL((k_spmv_panel<T, true>), dim3((unsigned)pm->max_tiles * kXcds), dim3(kBlock), 0, s, v, x,
                            partial, carry);
         if (pm->carry_pass)
             hipLaunchKernelGGL((k_spmv_panel_fixup<T>), dim3((unsigned)ceil_div64(pm->max_tiles, kBlock), kPanels),
                                dim3(kBlock), 0, s, v, carry, partial);
     }
-    hipLaunchKernelGGL((k_spmv_panel_reduce<T>), dim3((unsigned)ceil_div64(m, kBlock)), dim3(kBlock), 0, s, m, alpha,
-                       beta, pm->prow_ptr, pm->ppos, partial, y);
+    hipLaunchKernelGGL((k_spmv_panel_reduce<T>), dim3((unsigned)ceil_div64(m, kPanelRowBlock)), dim3(kBlock), 0, s, m,
+                       alpha, beta, pm->blk_lo, pm->rowid, partial, y);
     return check_launch();
 }
 
