@@ -29,7 +29,7 @@ KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "
 # HBM traffic per call measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; see profiles/),
 # scaled by the same counters' reading for a plain copy of known size.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "powerlaw_f64": (508087.2 * 2 + 98787.4) * 1024,     # profiles/spmv_panel_powerlaw_f64.md
+    "powerlaw_f64": (305282.3 * 2 + 111347.2) * 1024,     # profiles/spmv_panel_powerlaw_f64.md
     "stencil5_f64": (679827.7 * 2 + 138992.2) * 1024,    # profiles/spmv_flat_stencil5_f64.md
     "uniform16_f32": (213635.9 * 2 + 4707.5) * 1024,     # profiles/spmv_flat_uniform16_f32.md
     "spmm_zipf_f32": (2324920.8 * 2 + 278612.4) * 1024,  # profiles/spmm_merge_spmm_zipf_f32.md

@@ -50,7 +50,7 @@ enum {
     ASX_SPMV_STREAM = 3,  /* LDS-staged row blocks, segmented reduction */
     ASX_SPMV_MERGE = 9,   /* merge-path tiles + ordered carry fix-up */
     ASX_SPMV_FLAT = 15,   /* tiles of 1024 stored elements, register walk + ordered carry fix-up */
-    ASX_SPMV_PANEL = 100  /* not a reference id: the flat kernel over 8 column panels, one per XCD
+    ASX_SPMV_PANEL = 100  /* not a reference id: the flat kernel over 16 column panels, two per XCD
                              (needs a plan from asx_spmv_plan_create) */
 };
 
@@ -182,10 +182,11 @@ int asx_spmm_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, in
                          const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, int32_t ncols,
                          void *stream);
 /* SpMV plan that may look at A's columns and values.  alg = ASX_SPMV_PANEL regroups the stored
- * elements into 8 column panels, one per XCD, so that each XCD's L2 holds the slice of x its
- * workgroups gather from (for matrices whose x is 1.5 to 8 L2s large and whose columns are
- * scattered; the plan then holds a COPY of the values: rebuild it when they change; calls need
- * up to min(nnz, 8*m) values of workspace for the per-panel partial sums).  alg = ASX_SPMV_DEFAULT on such a
+ * elements into 16 column panels, two per XCD, worked through one after the other, so that each
+ * XCD's L2 holds the slice of x its workgroups gather from (for matrices whose x is 1.5 to 16
+ * L2s large and whose columns are scattered; the plan then holds a COPY of the values: rebuild
+ * it when they change; calls need up to min(nnz, 16*m) values of workspace for the per-panel
+ * partial sums).  alg = ASX_SPMV_DEFAULT on such a
  * matrix builds the panels, times the panel kernel against the kernel the histogram picks (three
  * runs each on scratch vectors) and keeps the faster.  Otherwise as asx_plan_create.  No
  * counterpart in the reference (its alphasparseSpMV_analysis is a stub).  Synchronises `stream`. */
