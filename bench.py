@@ -228,7 +228,7 @@ def cpu_baseline(w, budget_s):
     call()  # warm-up (first touch, thread pool)
     warm = time.perf_counter() - t_start
     reps = 0
-    while reps < 20 and (time.perf_counter() - t_start) < budget_s and (reps < 3 or warm * (reps + 2) < budget_s):
+    while reps < 1000 and (time.perf_counter() - t_start) < budget_s and (reps < 3 or warm * (reps + 2) < budget_s):
         t0 = time.perf_counter()
         call()
         times.append(time.perf_counter() - t0)
