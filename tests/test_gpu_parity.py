@@ -554,7 +554,7 @@ def test_spmv_panel_kernel_shapes(torch, capi, oracle, dtype):
 # ------------------------------------------------------------------ randomised shapes, every SpMV kernel
 def test_spmv_random_shapes_all_kernels(torch, capi, oracle):
     rng = np.random.default_rng(2024)
-    for case in range(60):
+    for case in range(90):
         kind = case % 6
         m = int(rng.integers(1, 4000))
         if kind == 0:
@@ -580,3 +580,11 @@ def test_spmv_random_shapes_all_kernels(torch, capi, oracle):
         for alg in ALGS:
             got = run_spmv(torch, capi, rp, col, val, x, y0, alpha, beta, alg_id(capi, alg), use_plan=(case % 4 < 2))
             assert_close(got, ref, scale, dtype, f"case {case} kind {kind} {alg}")
+        if col.size:  # the panel kernel needs its plan
+            d = [dev(torch, a) for a in (rp, col, val, x)]
+            y = dev(torch, y0)
+            plan = capi.Plan(False, capi.SPMV_PANEL, np.dtype(dtype), rp.size - 1, ncols, col.size, d[0], col=d[1], val=d[2])
+            capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_PANEL, plan=plan)
+            torch.cuda.synchronize()
+            assert_close(y.cpu().numpy(), ref, scale, dtype, f"case {case} kind {kind} panel")
+            plan.destroy()
