@@ -649,7 +649,7 @@ __device__ __forceinline__ void flat_tile(FlatShared<T> &sh, int t, int32_t m, i
     const int32_t re = seg_row[t + 1];
     const int32_t nwritten = re - rs;                   // rows that end inside this tile
     const int32_t rcount = nwritten + (re < m ? 1 : 0);  // plus the one left open
-    const bool fits = rcount <= kFlatRowCap;
+    const bool fits = rcount <= kFlatRowCap + 1;  // 1024 one-element rows plus the open row still fit
     int has_long = 0;
     if (fits) {
         for (int i = tid; i < rcount; i += kBlock) {
