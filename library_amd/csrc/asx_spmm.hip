@@ -33,6 +33,11 @@ __device__ __forceinline__ double readlane_t<double>(double v, int l)
     return __hiloint2double(hi, lo);
 }
 
+#ifndef ASX_SPMM_IN_FLIGHT
+#define ASX_SPMM_IN_FLIGHT 8
+#endif
+constexpr int kSpmmInFlight = ASX_SPMM_IN_FLIGHT;  // rows of B a wave has in flight
+
 // acc += sum over stored elements [k_begin, k_end) of one row: a * B[col, c]
 template <typename T>
 __device__ __forceinline__ T spmm_accumulate(T acc, int32_t k_begin, int32_t k_end, int lane, bool col_ok,
@@ -45,28 +50,28 @@ __device__ __forceinline__ T spmm_accumulate(T acc, int32_t k_begin, int32_t k_e
         const int32_t cl = kk < k_end ? col[kk] : 0;
         const T vl = kk < k_end ? val[kk] : T(0);
         const int cnt = k_end - k0 < kWave ? k_end - k0 : kWave;
+        // kSpmmInFlight rows of B at a time
         int j = 0;
-        for (; j + 4 <= cnt; j += 4) {
-            const int32_t c0 = __builtin_amdgcn_readlane(cl, j);
-            const int32_t c1 = __builtin_amdgcn_readlane(cl, j + 1);
-            const int32_t c2 = __builtin_amdgcn_readlane(cl, j + 2);
-            const int32_t c3 = __builtin_amdgcn_readlane(cl, j + 3);
-            T b0 = T(0), b1 = T(0), b2 = T(0), b3 = T(0);
-            if (col_ok) {
-                b0 = B[(int64_t)c0 * ldb + c];
-                b1 = B[(int64_t)c1 * ldb + c];
-                b2 = B[(int64_t)c2 * ldb + c];
-                b3 = B[(int64_t)c3 * ldb + c];
-            }
-            acc = fma_t<T>(readlane_t<T>(vl, j), b0, acc);
-            acc = fma_t<T>(readlane_t<T>(vl, j + 1), b1, acc);
-            acc = fma_t<T>(readlane_t<T>(vl, j + 2), b2, acc);
-            acc = fma_t<T>(readlane_t<T>(vl, j + 3), b3, acc);
+        for (; j + kSpmmInFlight <= cnt; j += kSpmmInFlight) {
+            int32_t cc[kSpmmInFlight];
+            T b[kSpmmInFlight];
+#pragma unroll
+            for (int u = 0; u < kSpmmInFlight; ++u) cc[u] = __builtin_amdgcn_readlane(cl, j + u);
+#pragma unroll
+            for (int u = 0; u < kSpmmInFlight; ++u) b[u] = col_ok ? B[(int64_t)cc[u] * ldb + c] : T(0);
+#pragma unroll
+            for (int u = 0; u < kSpmmInFlight; ++u) acc = fma_t<T>(readlane_t<T>(vl, j + u), b[u], acc);
         }
-        for (; j < cnt; ++j) {
-            const int32_t c0 = __builtin_amdgcn_readlane(cl, j);
-            T b0 = col_ok ? B[(int64_t)c0 * ldb + c] : T(0);
-            acc = fma_t<T>(readlane_t<T>(vl, j), b0, acc);
+        if (j < cnt) {  // the last, partial batch: all its loads are issued before the first use
+            int32_t cc[kSpmmInFlight];
+            T b[kSpmmInFlight];
+#pragma unroll
+            for (int u = 0; u < kSpmmInFlight; ++u) cc[u] = __builtin_amdgcn_readlane(cl, (j + u) & (kWave - 1));
+#pragma unroll
+            for (int u = 0; u < kSpmmInFlight; ++u) b[u] = (col_ok && j + u < cnt) ? B[(int64_t)cc[u] * ldb + c] : T(0);
+#pragma unroll
+            for (int u = 0; u < kSpmmInFlight; ++u)
+                if (j + u < cnt) acc = fma_t<T>(readlane_t<T>(vl, (j + u) & (kWave - 1)), b[u], acc);
         }
     }
     return acc;
