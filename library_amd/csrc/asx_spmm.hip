@@ -154,7 +154,54 @@ int launch_spmm_snap_splits(int32_t m, int32_t nnz, const int32_t *row_ptr, cons
     return check_launch();
 }
 
-// xs, ys: the snapped split points
+// A segment's stored elements and row ends, staged in LDS by the wave that owns the segment.
+// After snapping a segment holds at most 2 * kSpmmSegment elements and kSpmmSegment + 1 row ends.
+constexpr int kSegElems = 2 * kSpmmSegment;
+constexpr int kSegRows = kSpmmSegment + kWave;
+
+// acc += sum over staged elements [i0, i1) (positions relative to the segment start): a * B[col, c].
+// The LDS reads are broadcasts (every lane reads the same address).
+template <typename T>
+__device__ __forceinline__ T spmm_accumulate_staged(T acc, int32_t i0, int32_t i1, bool col_ok, int64_t c,
+                                                    const int32_t *s_col, const T *s_val,
+                                                    const T *__restrict__ B, int64_t ldb)
+{
+    int32_t i = i0;
+    for (; i + kSpmmInFlight <= i1; i += kSpmmInFlight) {
+        int32_t cc[kSpmmInFlight];
+        T a[kSpmmInFlight], b[kSpmmInFlight];
+#pragma unroll
+        for (int u = 0; u < kSpmmInFlight; ++u) {
+            cc[u] = __builtin_amdgcn_readfirstlane(s_col[i + u]);
+            a[u] = s_val[i + u];
+        }
+#pragma unroll
+        for (int u = 0; u < kSpmmInFlight; ++u) b[u] = col_ok ? B[(int64_t)cc[u] * ldb + c] : T(0);
+#pragma unroll
+        for (int u = 0; u < kSpmmInFlight; ++u) acc = fma_t<T>(a[u], b[u], acc);
+    }
+    if (i < i1) {  // the last, partial batch: all its loads are issued before the first use
+        int32_t cc[kSpmmInFlight];
+        T a[kSpmmInFlight], b[kSpmmInFlight];
+#pragma unroll
+        for (int u = 0; u < kSpmmInFlight; ++u) {
+            const int32_t iu = i + u < i1 ? i + u : i1 - 1;
+            cc[u] = __builtin_amdgcn_readfirstlane(s_col[iu]);
+            a[u] = s_val[iu];
+        }
+#pragma unroll
+        for (int u = 0; u < kSpmmInFlight; ++u) b[u] = (col_ok && i + u < i1) ? B[(int64_t)cc[u] * ldb + c] : T(0);
+#pragma unroll
+        for (int u = 0; u < kSpmmInFlight; ++u)
+            if (i + u < i1) acc = fma_t<T>(a[u], b[u], acc);
+    }
+    return acc;
+}
+
+// xs, ys: the snapped split points.  The wave first stages the segment's column indices, values
+// and row ends in LDS (one round trip for all of them), so that the loads of B of one row after
+// the other follow without waiting on row offsets or stored elements in between; the old value
+// of a row of C (beta != 0) is requested before the row's loads of B.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_spmm_merge(int32_t m, int32_t nnz, int32_t nseg,
                                                        int32_t ncols, T alpha,
@@ -168,8 +215,12 @@ __global__ __launch_bounds__(kBlock) void k_spmm_merge(int32_t m, int32_t nnz, i
                                                        T *__restrict__ carry,
                                                        int32_t *__restrict__ carry_row)
 {
+    __shared__ int32_t s_col_all[kBlock / kWave][kSegElems];
+    __shared__ T s_val_all[kBlock / kWave][kSegElems];
+    __shared__ int32_t s_end_all[kBlock / kWave][kSegRows];
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t seg = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    const int w = threadIdx.x / kWave;
+    const int64_t seg = (int64_t)blockIdx.x * (kBlock / kWave) + w;
     if (seg >= nseg) return;  // wave-uniform
     const int64_t c = (int64_t)blockIdx.y * kWave + lane;
     const bool col_ok = c < ncols;
@@ -177,10 +228,48 @@ __global__ __launch_bounds__(kBlock) void k_spmm_merge(int32_t m, int32_t nnz, i
     const int32_t y0 = __builtin_amdgcn_readfirstlane(ys[seg]);
     const int32_t x1 = __builtin_amdgcn_readfirstlane(xs[seg + 1]);
     const int32_t y1 = __builtin_amdgcn_readfirstlane(ys[seg + 1]);
+    const int32_t nel = y1 - y0, nrow = x1 - x0;
 
+    if (nel <= kSegElems && nrow <= kSegRows) {
+        int32_t *s_col = s_col_all[w];
+        T *s_val = s_val_all[w];
+        int32_t *s_end = s_end_all[w];
+#pragma unroll
+        for (int i = lane; i < kSegElems; i += kWave) {
+            if (i < nel) {
+                s_col[i] = col[y0 + i];
+                s_val[i] = val[y0 + i];
+            }
+        }
+#pragma unroll
+        for (int i = lane; i < kSegRows; i += kWave)
+            if (i < nrow) s_end[i] = row_ptr[x0 + 1 + i] - y0;
+        // the staged data is private to this wave: order its LDS writes before its LDS reads
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        int32_t k = 0;
+        for (int32_t r = 0; r < nrow; ++r) {  // rows this segment finishes
+            const int32_t e = __builtin_amdgcn_readfirstlane(s_end[r]);
+            const int64_t idx = (int64_t)(x0 + r) * ldc + c;
+            const T c_old = (beta != T(0) && col_ok) ? C[idx] : T(0);
+            const T acc = spmm_accumulate_staged<T>(T(0), k, e, col_ok, c, s_col, s_val, B, ldb);
+            k = e;
+            if (col_ok) C[idx] = beta == T(0) ? alpha * acc : fma_t<T>(alpha, acc, beta * c_old);
+        }
+        const bool has_tail = nel > k;  // row x1 continues past the segment end
+        if (has_tail) {
+            const T acc = spmm_accumulate_staged<T>(T(0), k, nel, col_ok, c, s_col, s_val, B, ldb);
+            if (col_ok) carry[seg * ncols + c] = acc;
+        }
+        if (lane == 0 && blockIdx.y == 0) carry_row[seg] = has_tail ? x1 : -1;
+        return;
+    }
+
+    // a segment too large to stage (cannot happen with snapped merge-path points; kept for safety)
     int32_t k = y0;
     T acc = T(0);
-    for (int32_t row = x0; row < x1; ++row) {  // rows this segment finishes
+    for (int32_t row = x0; row < x1; ++row) {
         const int32_t e = __builtin_amdgcn_readfirstlane(row_ptr[row + 1]);
         acc = spmm_accumulate<T>(acc, k, e, lane, col_ok, c, col, val, B, ldb);
         k = e;
@@ -190,7 +279,6 @@ __global__ __launch_bounds__(kBlock) void k_spmm_merge(int32_t m, int32_t nnz, i
         }
         acc = T(0);
     }
-    // row x1 continues past the segment end: keep what this segment saw of it
     const bool has_tail = y1 > k;
     if (has_tail) {
         acc = spmm_accumulate<T>(T(0), k, y1, lane, col_ok, c, col, val, B, ldb);
