@@ -31,8 +31,8 @@ KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "
 MEASURED_TRAFFIC_BYTES = {
     "powerlaw_f64": (305282.3 * 2 + 111347.2) * 1024,     # profiles/spmv_panel_powerlaw_f64.md
     "stencil5_f64": (679827.7 * 2 + 138992.2) * 1024,    # profiles/spmv_flat_stencil5_f64.md
-    "uniform16_f32": (213635.9 * 2 + 4707.5) * 1024,     # profiles/spmv_flat_uniform16_f32.md
-    "spmm_zipf_f32": (2324920.8 * 2 + 278612.4) * 1024,  # profiles/spmm_merge_spmm_zipf_f32.md
+    "uniform16_f32": (215067.3 * 2 + 4699.0) * 1024,     # profiles/spmv_flat_uniform16_f32.md
+    "spmm_zipf_f32": (2284685.2 * 2 + 278616.5) * 1024,  # profiles/spmm_merge_spmm_zipf_f32.md
 }
 
 
