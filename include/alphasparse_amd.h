@@ -50,7 +50,7 @@ enum {
     ASX_SPMV_STREAM = 3,  /* LDS-staged row blocks, segmented reduction */
     ASX_SPMV_MERGE = 9,   /* merge-path tiles + ordered carry fix-up */
     ASX_SPMV_FLAT = 15,   /* tiles of 1024 stored elements, register walk + ordered carry fix-up */
-    ASX_SPMV_PANEL = 100  /* not a reference id: the flat kernel over 16 column panels, two per XCD
+    ASX_SPMV_PANEL = 100  /* not a reference id: the flat kernel over 16 or 32 column panels, 2 or 4 per XCD
                              (needs a plan from asx_spmv_plan_create) */
 };
 
@@ -182,14 +182,16 @@ int asx_spmm_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, in
                          const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, int32_t ncols,
                          void *stream);
 /* SpMV plan that may look at A's columns and values.  alg = ASX_SPMV_PANEL regroups the stored
- * elements into 16 column panels, two per XCD, worked through one after the other, so that each
- * XCD's L2 holds the slice of x its workgroups gather from (for matrices whose x is 1.5 to 16
- * L2s large and whose columns are scattered; the plan then holds a COPY of the values: rebuild
- * it when they change; calls need up to min(nnz, 16*m) values of workspace for the per-panel
- * partial sums).  alg = ASX_SPMV_DEFAULT on such a
- * matrix builds the panels, times the panel kernel against the kernel the histogram picks (three
- * runs each on scratch vectors) and keeps the faster.  Otherwise as asx_plan_create.  No
- * counterpart in the reference (its alphasparseSpMV_analysis is a stub).  Synchronises `stream`. */
+ * elements into 16 (x up to 64 MiB) or 32 column panels, 2 or 4 per XCD, worked through one after
+ * the other, so that each XCD's L2 holds the slice of x its workgroups gather from.  The plan
+ * then holds a COPY of the values: rebuild it when they change; calls need up to
+ * min(nnz, 32*m) values of workspace for the per-panel partial sums.  alg = ASX_SPMV_DEFAULT
+ * considers panels when x is 6 to 256 MiB large, nnz >= 2^22 and the columns are scattered (a
+ * sample of 64 tiles of 1024 stored elements touches on average more than 512 distinct 128-byte
+ * lines of x per tile): it builds the panels, times the panel kernel against the kernel the
+ * histogram picks (three runs each on scratch vectors) and keeps the faster.  Otherwise as
+ * asx_plan_create.  No counterpart in the reference (its alphasparseSpMV_analysis is a stub).
+ * Synchronises `stream`. */
 int asx_spmv_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
                          const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, void *stream);
 /* Upper bound of the workspace a panel plan for (m, n, nnz) needs; 0 when the matrix is not a

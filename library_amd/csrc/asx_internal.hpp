@@ -113,10 +113,11 @@ int launch_spmm_blocked(int32_t m, int32_t k, int32_t ncols, T alpha, const Bloc
 // sum; `blk_lo` says, for every block of kPanelRowBlock rows of A, where in each panel's partial
 // sums the block's rows start, so the reduction reads contiguous ranges.
 constexpr int kXcds = 8;
-constexpr int kPanelPhases = 2;
+constexpr int kPanelPhases = 4;  // at most; a matrix uses 2 phases while its slices of x stay small
 constexpr int kPanels = kXcds * kPanelPhases;
 constexpr int kPanelRowBlock = 1024;  // rows of A per workgroup of the reduction
 struct PanelMatrix {
+    int32_t npanels;                // panels in use (a multiple of kXcds, <= kPanels); the rest are empty
     int32_t width;                  // columns per panel
     int32_t count[kPanels];         // stored elements per panel
     int64_t elem_off[kPanels + 1];  // start of each panel in col / val (multiples of 4 elements)
@@ -133,8 +134,8 @@ struct PanelMatrix {
     int carry_pass;
 };
 template <typename T>
-int build_panels(int32_t m, int32_t n, int32_t nnz, const int32_t *row_ptr, const int32_t *col, const T *val,
-                 PanelMatrix *out, hipStream_t s);
+int build_panels(int32_t m, int32_t n, int32_t nnz, int32_t npanels, const int32_t *row_ptr, const int32_t *col,
+                 const T *val, PanelMatrix *out, hipStream_t s);
 void free_panels(PanelMatrix *p);
 template <typename T>
 int launch_spmv_panel(int32_t m, T alpha, const PanelMatrix *pm, const T *x, T beta, T *y, T *partial, T *carry,

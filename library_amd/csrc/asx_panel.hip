@@ -109,12 +109,14 @@ constexpr int kPanelBits = 5;  // radix bits that hold a panel index
 static_assert(kPanels <= (1 << kPanelBits), "panel index must fit the sort key bits");
 
 template <typename T>
-int build_panels(int32_t m, int32_t n, int32_t nnz, const int32_t *row_ptr, const int32_t *col, const T *val,
-                 PanelMatrix *out, hipStream_t s)
+int build_panels(int32_t m, int32_t n, int32_t nnz, int32_t npanels, const int32_t *row_ptr, const int32_t *col,
+                 const T *val, PanelMatrix *out, hipStream_t s)
 {
     PanelMatrix pm{};
-    if (m <= 0 || nnz <= 0 || n < kPanels) return ASX_STATUS_INVALID_SIZE;
-    pm.width = (int32_t)(ceil_div64(ceil_div64(n, kPanels), 32) * 32);
+    if (m <= 0 || nnz <= 0 || n <= 0) return ASX_STATUS_INVALID_SIZE;
+    if (npanels < kXcds || npanels > kPanels || npanels % kXcds) return ASX_STATUS_INVALID_VALUE;
+    pm.npanels = npanels;
+    pm.width = (int32_t)(ceil_div64(ceil_div64(n, npanels), 32) * 32);
     int st = ASX_STATUS_SUCCESS;
     // a..e: five nnz-sized scratch arrays reused through the stages
     int32_t *a = nullptr, *b = nullptr, *c = nullptr, *d = nullptr, *e = nullptr, *d_small = nullptr;
@@ -213,9 +215,9 @@ done:
     return ASX_STATUS_SUCCESS;
 }
 
-template int build_panels<float>(int32_t, int32_t, int32_t, const int32_t *, const int32_t *, const float *,
+template int build_panels<float>(int32_t, int32_t, int32_t, int32_t, const int32_t *, const int32_t *, const float *,
                                  PanelMatrix *, hipStream_t);
-template int build_panels<double>(int32_t, int32_t, int32_t, const int32_t *, const int32_t *, const double *,
-                                  PanelMatrix *, hipStream_t);
+template int build_panels<double>(int32_t, int32_t, int32_t, int32_t, const int32_t *, const int32_t *,
+                                  const double *, PanelMatrix *, hipStream_t);
 
 }  // namespace asx

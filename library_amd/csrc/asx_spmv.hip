@@ -916,7 +916,7 @@ __global__ __launch_bounds__(kBlock) void k_spmv_panel_fixup(PanelView v, const 
 // row, one panel after the other (a row appears at most once in a panel, so the adds of one
 // panel never collide).
 template <typename T>
-__global__ __launch_bounds__(kBlock) void k_spmv_panel_reduce(int32_t m, T alpha, T beta,
+__global__ __launch_bounds__(kBlock) void k_spmv_panel_reduce(int32_t m, int32_t npanels, T alpha, T beta,
                                                               const int32_t *__restrict__ blk_lo,
                                                               const int32_t *__restrict__ rowid,
                                                               const T *__restrict__ partial, T *__restrict__ y)
@@ -933,21 +933,24 @@ __global__ __launch_bounds__(kBlock) void k_spmv_panel_reduce(int32_t m, T alpha
 #pragma unroll
     for (int i = tid; i < kPanelRowBlock; i += kBlock) acc[i] = T(0);
     __syncthreads();
-    // first kBlock entries of every panel's range: all loads issued before the first add
-    T v[kPanels];
-    int32_t rid[kPanels];
+    constexpr int kChunk = 16;  // panels whose loads are in flight together
+    for (int j0 = 0; j0 < npanels; j0 += kChunk) {
+        // first kBlock entries of every panel's range: all loads issued before the first add
+        T v[kChunk];
+        int32_t rid[kChunk];
 #pragma unroll
-    for (int j = 0; j < kPanels; ++j) {
-        const int32_t k = s_lo[j] + tid;
-        const bool ok = k < s_hi[j];
-        rid[j] = ok ? rowid[k] - r0 : -1;
-        v[j] = ok ? partial[k] : T(0);
-    }
+        for (int j = 0; j < kChunk; ++j) {
+            const int32_t k = s_lo[j0 + j] + tid;
+            const bool ok = k < s_hi[j0 + j];
+            rid[j] = ok ? rowid[k] - r0 : -1;
+            v[j] = ok ? partial[k] : T(0);
+        }
 #pragma unroll
-    for (int j = 0; j < kPanels; ++j) {
-        if (rid[j] >= 0) acc[rid[j]] += v[j];
-        for (int32_t k = s_lo[j] + kBlock + tid; k < s_hi[j]; k += kBlock) acc[rowid[k] - r0] += partial[k];
-        __syncthreads();
+        for (int j = 0; j < kChunk; ++j) {
+            if (rid[j] >= 0) acc[rid[j]] += v[j];
+            for (int32_t k = s_lo[j0 + j] + kBlock + tid; k < s_hi[j0 + j]; k += kBlock) acc[rowid[k] - r0] += partial[k];
+            __syncthreads();
+        }
     }
 #pragma unroll
     for (int i = tid; i < kPanelRowBlock; i += kBlock) {
@@ -977,11 +980,11 @@ int launch_spmv_panel(int32_t m, T alpha, const PanelMatrix *pm, const T *x, T b
         hipLaunchKernelGGL((k_spmv_panel<T, true>), dim3((unsigned)pm->max_tiles * kXcds), dim3(kBlock), 0, s, v, x,
                            partial, carry);
         if (pm->carry_pass)
-            hipLaunchKernelGGL((k_spmv_panel_fixup<T>), dim3((unsigned)ceil_div64(pm->max_tiles, kBlock), kPanels),
+            hipLaunchKernelGGL((k_spmv_panel_fixup<T>), dim3((unsigned)ceil_div64(pm->max_tiles, kBlock), (unsigned)pm->npanels),
                                dim3(kBlock), 0, s, v, carry, partial);
     }
     hipLaunchKernelGGL((k_spmv_panel_reduce<T>), dim3((unsigned)ceil_div64(m, kPanelRowBlock)), dim3(kBlock), 0, s, m,
-                       alpha, beta, pm->blk_lo, pm->rowid, partial, y);
+                       pm->npanels, alpha, beta, pm->blk_lo, pm->rowid, partial, y);
     return check_launch();
 }
 

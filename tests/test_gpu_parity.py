@@ -547,7 +547,7 @@ def test_spmv_panel_kernel_shapes(torch, capi, oracle, dtype):
     assert L.asx_spmv_csr_f64(None, capi.SPMV_PANEL, 1, 1, 0, 1.0, capi._ptr(d[0]), None, None, None, 0.0,
                               capi._ptr(d[3]), None, 0, None) == 6
     assert L.asx_spmv_panel_workspace_bytes(capi.R_64F, 1 << 22, 1 << 22, 1 << 25) >= 8 * (1 << 22) * 8
-    assert L.asx_spmv_panel_workspace_bytes(capi.R_64F, 1 << 24, 1 << 24, 1 << 26) == 0  # x too large for 8 slices
+    assert L.asx_spmv_panel_workspace_bytes(capi.R_64F, 1 << 26, 1 << 26, 1 << 27) == 0  # x (512 MiB) too large
     assert L.asx_spmv_panel_workspace_bytes(capi.R_32F, 1 << 20, 1 << 20, 1 << 24) == 0  # x fits one L2
 
 
