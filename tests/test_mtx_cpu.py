@@ -88,3 +88,18 @@ def test_errors(tmp_path):
     _write(p, "%%MatrixMarket matrix coordinate real general", "4 6 0", [])
     m, n, r, c, v = capi.mtx_read(p, np.float32)
     assert (m, n, r.size) == (4, 6, 0)
+
+
+def test_reference_sample_file():
+    """tests/golden/reference_test_matrix.mtx is the reference's own matrix_test/test.mtx (a data
+    file): declared complex Hermitian, but with one value per entry and both triangles stored.  The
+    reference's reader (hip/test/io.hip:180-250) takes the first value and mirrors every
+    off-diagonal entry right after it, whatever else the file holds: 16 entries from 8 lines."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_test_matrix.mtx")
+    m, n, r, c, v = capi.mtx_read(path, np.float32)
+    assert (m, n) == (4, 4)
+    lines = [(1, 3, 1), (1, 4, 2), (2, 3, 3), (2, 4, 4), (3, 1, 5), (3, 2, 6), (4, 1, 7), (4, 2, 8)]
+    want = []
+    for i, j, a in lines:
+        want += [(i - 1, j - 1, float(a)), (j - 1, i - 1, float(a))]
+    assert list(zip(r.tolist(), c.tolist(), v.tolist())) == want
