@@ -203,3 +203,17 @@ def test_spmv_analysis_on_a_panel_candidate(tmp_path, oracle):
     ref_t = oracle.spmv(rp_t, col_t, val_t, y0, alpha, beta, x, 8)
     got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, y0, x, 1, 0, alpha, beta, 1, (1, 0, 0, 0, 0), n=n)
     assert_close(got, ref_t, spmv_scale(rp_t, col_t, val_t, y0, alpha, beta, x), np.float64, "transpose, DEFAULT with analysis")
+
+
+def test_cli_on_the_reference_matrix():
+    """matrix_test/mhd1280b.mtx of the reference (kept as tests/golden/mhd1280b.mtx), run the way the
+    reference's drivers are run: every listed algorithm, with --check, in both precisions."""
+    mtx = os.path.join(ROOT, "tests", "golden", "mhd1280b.mtx")
+    for args in (["--data-type=D", "--check", "--iter=5", "--warmup=2"],
+                 ["--data-type=S", "--check", "--iter=5", "--warmup=2", "--analysis"],
+                 ["--op=spmm", "--data-type=S", "--check", "--iter=3", "--warmup=1", "--cols=64"],
+                 ["--op=spmm", "--data-type=D", "--check", "--iter=3", "--warmup=1", "--cols=17", "--layout=C"]):
+        r = subprocess.run([CLI, f"--data-file={mtx}", *args], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0, (args, r.returncode, r.stdout[-2000:], r.stderr[-2000:])
+        assert "Dimensions: 1280 x 1280, NNZ: 22778" in r.stdout
+        assert "correct: require" in r.stdout and "error: require" not in r.stdout, r.stdout

@@ -103,3 +103,14 @@ def test_reference_sample_file():
     for i, j, a in lines:
         want += [(i - 1, j - 1, float(a)), (j - 1, i - 1, float(a))]
     assert list(zip(r.tolist(), c.tolist(), v.tolist())) == want
+
+
+def test_mhd1280b_matches_scipy():
+    """The SuiteSparse matrix the reference ships (matrix_test/mhd1280b.mtx, complex Hermitian):
+    real parts, Hermitian expansion, against scipy.io.mmread."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mhd1280b.mtx")
+    m, n, r, c, v = capi.mtx_read(path, np.float64)
+    A = scipy.io.mmread(path).tocsr()
+    assert (m, n) == A.shape == (1280, 1280) and r.size == 22778
+    B = sp.coo_matrix((v, (r, c)), shape=(m, n)).tocsr()
+    assert abs(B - A.real).max() == 0.0
