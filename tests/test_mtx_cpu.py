@@ -114,3 +114,27 @@ def test_mhd1280b_matches_scipy():
     assert (m, n) == A.shape == (1280, 1280) and r.size == 22778
     B = sp.coo_matrix((v, (r, c)), shape=(m, n)).tocsr()
     assert abs(B - A.real).max() == 0.0
+
+
+def test_reader_survives_garbage(tmp_path):
+    """Truncations and byte flips of a valid file must end in an error status or a consistent
+    result, never in a crash or an index outside the matrix."""
+    rng = np.random.default_rng(9)
+    good = ("%%MatrixMarket matrix coordinate real symmetric\n% c\n6 6 7\n"
+            "1 1 1.5\n2 1 -2\n3 3 4e0\n4 2 .5\n5 5 1\n6 1 2\n6 6 3\n").encode()
+    p = tmp_path / "f.mtx"
+    for case in range(300):
+        b = bytearray(good)
+        if case % 3 == 0:
+            b = b[:int(rng.integers(0, len(b)))]
+        else:
+            for _ in range(int(rng.integers(1, 6))):
+                b[int(rng.integers(0, len(b)))] = int(rng.integers(0, 256))
+        p.write_bytes(bytes(b))
+        try:
+            m, n, r, c, v = capi.mtx_read(p, np.float64)
+        except RuntimeError:
+            continue
+        assert r.size == c.size == v.size
+        if r.size:
+            assert 0 <= r.min() and r.max() < m and 0 <= c.min() and c.max() < n
