@@ -546,6 +546,14 @@ def test_spmv_panel_kernel_shapes(torch, capi, oracle, dtype):
     assert L.asx_plan_create(capi.C.byref(h), 0, capi.SPMV_PANEL, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), 1, None) == 6
     assert L.asx_spmv_csr_f64(None, capi.SPMV_PANEL, 1, 1, 0, 1.0, capi._ptr(d[0]), None, None, None, 0.0,
                               capi._ptr(d[3]), None, 0, None) == 6
+    # argument errors of the plan constructor that takes columns and values
+    for args, want in (((None, capi.SPMV_PANEL, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 7),
+                       ((capi.C.byref(h), capi.SPMV_PANEL, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), None, capi._ptr(d[2]), None), 7),
+                       ((capi.C.byref(h), capi.SPMV_PANEL, capi.R_64F, -1, 10, 10, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 10),
+                       ((capi.C.byref(h), capi.SPMV_PANEL, capi.R_64F, 10, 10, 0, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 10),
+                       ((capi.C.byref(h), capi.SPMV_PANEL, 7, 10, 10, 10, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 6),
+                       ((capi.C.byref(h), 1, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 6)):
+        assert L.asx_spmv_plan_create(*args) == want, args
     assert L.asx_spmv_panel_workspace_bytes(capi.R_64F, 1 << 22, 1 << 22, 1 << 25) >= 8 * (1 << 22) * 8
     assert L.asx_spmv_panel_workspace_bytes(capi.R_64F, 1 << 26, 1 << 26, 1 << 27) == 0  # x (512 MiB) too large
     assert L.asx_spmv_panel_workspace_bytes(capi.R_32F, 1 << 20, 1 << 20, 1 << 24) == 0  # x fits one L2
