@@ -32,6 +32,7 @@ MEASURED_TRAFFIC_BYTES = {
     "powerlaw_f64": (305282.3 * 2 + 111347.2) * 1024,     # profiles/spmv_panel_powerlaw_f64.md
     "stencil5_f64": (679827.7 * 2 + 138992.2) * 1024,    # profiles/spmv_flat_stencil5_f64.md
     "uniform16_f32": (215067.3 * 2 + 4699.0) * 1024,     # profiles/spmv_flat_uniform16_f32.md
+    "spmm_banded_f32": (741844.7 * 2 + 340585.3) * 1024,  # profiles/spmm_blocked_spmm_banded_f32.md
     "spmm_zipf_f32": (2284685.2 * 2 + 278616.5) * 1024,  # profiles/spmm_merge_spmm_zipf_f32.md
 }
 
