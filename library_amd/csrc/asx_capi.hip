@@ -707,7 +707,7 @@ int asx_plan_histogram(const asx_plan *plan, int64_t h_hist[33], int64_t h_stats
 }
 
 // ---------------------------------------------------------------- SpMV
-// Reference algorithm ids (include/alphasparse/spdef.h:345-365) onto the three kernels here:
+// Reference algorithm ids (include/alphasparse/spdef.h:345-365) onto the four plan-less kernels here:
 // the reference's scalar/vector/line-enhance families are one-row-per-lane-group kernels, its
 // adaptive/stream families stage row blocks through LDS, its flat/acc families cut the stored
 // elements into equal tiles of 1024, its merge/row-partition/load-balance families split work

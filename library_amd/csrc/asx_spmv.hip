@@ -14,6 +14,9 @@
 //            items; partial rows are joined by a segmented scan inside the workgroup and by
 //            an ordered carry pass between workgroups.  No atomics: results do not depend on
 //            scheduling.
+//   panel  : the flat kernel's tile code over column panels of a regrouped copy of A, the
+//            panels dealt to the XCDs so that each XCD's L2 holds the slice of x it gathers
+//            from; per-panel partial sums are added in panel order by a last pass.
 //
 // The reference's kernels for the same job (hip/kernel/level2/alphasparse_spmv_csr_vector.h,
 // _flat.h, _merge_ginkgo.h, _adaptive.h) join partial rows with floating-point atomicAdd and
