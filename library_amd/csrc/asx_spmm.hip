@@ -325,12 +325,19 @@ __global__ __launch_bounds__(kBlock) void k_spmm_merge_fixup(int32_t m, int32_t 
             const T *p = carry + seg * ncols + c;
             T sum = T(0);
             int64_t j = 0;
-            for (; j + 16 <= len; j += 16) {
-                T v[16];
+            for (; j + 64 <= len; j += 64) {  // a 50 000-element row leaves 390 carry rows
+                T v[64];
 #pragma unroll
-                for (int u = 0; u < 16; ++u) v[u] = p[(j + u) * ncols];
+                for (int u = 0; u < 64; ++u) v[u] = p[(j + u) * ncols];
 #pragma unroll
-                for (int u = 0; u < 16; ++u) sum += v[u];
+                for (int u = 0; u < 64; ++u) sum += v[u];
+            }
+            for (; j + 8 <= len; j += 8) {
+                T v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = p[(j + u) * ncols];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) sum += v[u];
             }
             for (; j < len; ++j) sum += p[j * ncols];
             const int64_t idx = (int64_t)row * ldc + c;
