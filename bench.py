@@ -177,9 +177,14 @@ def probe(w, steps):
     vt = capi.value_type(w.val.dtype)
     stream = torch.cuda.current_stream().cuda_stream
     out = {"workload": w.name, "nnz": w.nnz, "stream_bytes": w.nnz * (w.dtype.itemsize + 4)}
-    for mode, key in ((0, "stream"), (1, "stream_gather")):
-        call = lambda: capi.lib().asx_probe_stream_gather(vt, mode, w.nnz, d_col.data_ptr(), d_val.data_ptr(),
-                                                          d_x.data_ptr(), sink.data_ptr(), stream)
+    for mode, key in ((0, "stream"), (1, "stream_gather"), (10, "gather_slice_per_xcd"), (11, "gather_16_slices_2_phases"),
+                      (12, "gather_slices_mixed_over_xcds")):
+        if mode < 10:
+            call = lambda: capi.lib().asx_probe_stream_gather(vt, mode, w.nnz, d_col.data_ptr(), d_val.data_ptr(),
+                                                              d_x.data_ptr(), sink.data_ptr(), stream)
+        else:
+            call = lambda: capi.lib().asx_probe_sliced_gather(vt, mode - 10, w.nnz, w.n, d_col.data_ptr(),
+                                                              d_val.data_ptr(), d_x.data_ptr(), sink.data_ptr(), stream)
         for _ in range(3):
             call()
         torch.cuda.synchronize()

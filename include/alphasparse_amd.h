@@ -258,6 +258,12 @@ int asx_copy_bytes(const void *d_src, void *d_dst, size_t bytes, void *stream);
  * column pattern.  d_sink: one value of the value type (never written in practice). */
 int asx_probe_stream_gather(int value_type, int mode, int64_t nnz, const int32_t *d_col,
                             const void *d_val, const void *d_x, void *d_sink, void *stream);
+/* As mode 1, with the gathers of every workgroup folded into one slice of d_x (n entries) chosen
+ * from the workgroup id: slicing 0 = 8 slices, slice = workgroup id mod 8 (one slice per XCD);
+ * 1 = 16 slices in two phases; 2 = 8 slices changing every 8 workgroups (control: every XCD sees
+ * every slice).  Measures what a column-panel layout can gain. */
+int asx_probe_sliced_gather(int value_type, int slicing, int64_t nnz, int32_t n, const int32_t *d_col,
+                            const void *d_val, const void *d_x, void *d_sink, void *stream);
 
 #ifdef __cplusplus
 }

@@ -31,7 +31,7 @@ EXPORTS = [
     "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
     "asx_spmm_resolve_alg", "asx_spmm_workspace_bytes", "asx_spmm_csr_f32", "asx_spmm_csr_f64",
-    "asx_copy_bytes", "asx_probe_stream_gather",
+    "asx_copy_bytes", "asx_probe_stream_gather", "asx_probe_sliced_gather",
 ]
 
 
@@ -93,6 +93,7 @@ def lib():
     L.asx_spmm_csr_f64.argtypes = [vp, C.c_int, i32, i32, i32, i32, C.c_double, vp, vp, vp, vp, i64, C.c_double, vp, i64, vp, sz, vp]
     L.asx_copy_bytes.argtypes = [vp, vp, sz, vp]
     L.asx_probe_stream_gather.argtypes = [C.c_int, C.c_int, i64, vp, vp, vp, vp, vp]
+    L.asx_probe_sliced_gather.argtypes = [C.c_int, C.c_int, i64, i32, vp, vp, vp, vp, vp]
     _lib = L
     return L
 
