@@ -596,3 +596,32 @@ def test_spmv_random_shapes_all_kernels(torch, capi, oracle):
             torch.cuda.synchronize()
             assert_close(y.cpu().numpy(), ref, scale, dtype, f"case {case} kind {kind} panel")
             plan.destroy()
+
+
+# ------------------------------------------------------------------ measurement helpers
+def test_probes_and_copy_run(torch, capi):
+    """The measurement entry points launch, finish and write nothing but the copy's destination."""
+    L = capi.lib()
+    rng = np.random.default_rng(5)
+    n, nnz = 5000, 70001
+    col = dev(torch, rng.integers(0, n, nnz).astype(np.int32))
+    stream = capi._stream()
+    for dtype, vt in ((np.float64, capi.R_64F), (np.float32, capi.R_32F)):
+        val = dev(torch, rng.uniform(-1, 1, nnz).astype(dtype))
+        x = dev(torch, rng.uniform(-1, 1, n).astype(dtype))
+        sink = torch.zeros(4, dtype=val.dtype, device="cuda")
+        for mode in (0, 1):
+            assert L.asx_probe_stream_gather(vt, mode, nnz, capi._ptr(col), capi._ptr(val), capi._ptr(x), capi._ptr(sink), stream) == 0
+        for slicing in (0, 1, 2):
+            assert L.asx_probe_sliced_gather(vt, slicing, nnz, n, capi._ptr(col), capi._ptr(val), capi._ptr(x), capi._ptr(sink), stream) == 0
+        torch.cuda.synchronize()
+        assert sink.cpu().numpy().tolist() == [0, 0, 0, 0]
+    assert L.asx_probe_stream_gather(capi.R_64F, 5, nnz, capi._ptr(col), capi._ptr(val), capi._ptr(x), capi._ptr(sink), stream) == 3
+    assert L.asx_probe_sliced_gather(capi.R_64F, 3, nnz, n, capi._ptr(col), capi._ptr(val), capi._ptr(x), capi._ptr(sink), stream) == 3
+    assert L.asx_probe_sliced_gather(capi.R_64F, 0, nnz, 8, capi._ptr(col), capi._ptr(val), capi._ptr(x), capi._ptr(sink), stream) == 10
+    src = dev(torch, rng.integers(0, 255, 1 << 20).astype(np.uint8))
+    dst = torch.zeros_like(src)
+    assert L.asx_copy_bytes(capi._ptr(src), capi._ptr(dst), src.numel(), stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(src, dst)
+    assert L.asx_copy_bytes(capi._ptr(src), capi._ptr(dst), 17, stream) == 10
