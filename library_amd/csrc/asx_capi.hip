@@ -520,7 +520,11 @@ int asx_spmm_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     const int kernel = asx_spmm_resolve_alg(alg, m, nnz, ncols);
     if (kernel < 0) return ASX_STATUS_NOT_SUPPORTED;
     const bool want_blocked = kernel == ASX_SPMM_BLOCKED;
-    const bool probe_blocked = alg == ASX_SPMM_DEFAULT && nnz > 0 && nnz <= kBlockedProbeMaxNnz;
+    // scattered columns (a sample of tiles of 1024 stored elements touches mostly distinct
+    // 128-byte lines) cannot fill 16x4 blocks: the blocks are not even built then
+    const bool probe_blocked = alg == ASX_SPMM_DEFAULT && nnz > 0 && nnz <= kBlockedProbeMaxNnz && d_col &&
+                               (value_type == ASX_R_32F || value_type == ASX_R_64F) &&
+                               sampled_line_spread(d_col, nnz, vsize(value_type), (hipStream_t)stream) < kPanelMinSpread;
     if (!want_blocked && !probe_blocked)
         return asx_plan_create(out, 1, alg, value_type, m, k, nnz, d_row_ptr, ncols, stream);
     if (m < 0 || k < 0 || nnz < 0 || ncols < 1) return ASX_STATUS_INVALID_SIZE;
