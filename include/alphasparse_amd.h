@@ -50,7 +50,10 @@ enum {
     ASX_SPMV_STREAM = 3,  /* LDS-staged row blocks, segmented reduction */
     ASX_SPMV_MERGE = 9,   /* merge-path tiles + ordered carry fix-up */
     ASX_SPMV_FLAT = 15,   /* tiles of 1024 stored elements, register walk + ordered carry fix-up */
-    ASX_SPMV_PANEL = 100  /* not a reference id: the flat kernel over 16 or 32 column panels, 2 or 4 per XCD
+    ASX_SPMV_PANEL = 100, /* not a reference id: the flat kernel over 16 or 32 column panels, 2 or 4 per XCD
+                             (needs a plan from asx_spmv_plan_create) */
+    ASX_SPMV_SLICED = 101 /* not a reference id: stored elements regrouped by column slice, each slice of x
+                             held in LDS; one partial sum per (row, slice), added per row by a second pass
                              (needs a plan from asx_spmv_plan_create) */
 };
 

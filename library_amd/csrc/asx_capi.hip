@@ -3,6 +3,7 @@
 // point launches HIP kernels or returns an error status.
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -228,6 +229,15 @@ int spmv_impl(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, 
         if (ws_bytes < L.bytes) return ASX_STATUS_INVALID_SIZE;
         return launch_spmv_panel<T>(m, alpha, &plan->panel, x, beta, y, (T *)(w + L.partial_off),
                                     (T *)(w + L.carry_off), s);
+    }
+    case ASX_SPMV_SLICED: {
+        // the slices hold a copy of A's columns and values and are built by asx_spmv_plan_create
+        if (!plan || !plan->sliced.cf) return ASX_STATUS_NOT_INITIALIZED;
+        if (plan->n != n) return ASX_STATUS_INVALID_VALUE;
+        const size_t need = align_up(((size_t)plan->sliced.npartials + kWave) * sizeof(T), kAlign);
+        if (!ws) return ASX_STATUS_INVALID_POINTER;
+        if (ws_bytes < need) return ASX_STATUS_INVALID_SIZE;
+        return launch_spmv_sliced<T>(m, n, alpha, &plan->sliced, x, beta, y, (T *)w, s);
     }
     default: return ASX_STATUS_NOT_SUPPORTED;
     }
@@ -502,6 +512,7 @@ int asx_plan_destroy(asx_plan *plan)
     if (plan->d_meta) st = status_of(hipFree(plan->d_meta));
     free_blocked(&plan->blocked);
     free_panels(&plan->panel);
+    free_sliced(&plan->sliced);
     delete plan;
     return st;
 }
@@ -657,6 +668,48 @@ static int spmv_plan_with_panels(asx_plan **out, int alg, int value_type, int32_
     return ASX_STATUS_SUCCESS;
 }
 
+// Slice width: 128 KiB of x per slice (one workgroup of 16 waves per compute unit).
+template <typename T>
+static int spmv_plan_sliced(asx_plan **out, int value_type, int32_t m, int32_t n, int32_t nnz,
+                            const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, hipStream_t s)
+{
+    asx_plan *base = nullptr;  // histogram and sizes
+    int st = asx_plan_create(&base, 0, ASX_SPMV_VECTOR, value_type, m, n, nnz, d_row_ptr, 1, (void *)s);
+    if (st) return st;
+    asx_plan *p = new (std::nothrow) asx_plan();
+    if (!p) {
+        asx_plan_destroy(base);
+        return ASX_STATUS_ALLOC_FAILED;
+    }
+    *p = *base;
+    asx_plan_destroy(base);
+    p->d_meta = nullptr;
+    p->meta_bytes = 0;
+    p->alg = ASX_SPMV_SLICED;
+    p->sliced = SlicedMatrix{};
+    int cus = 256;
+    (void)asx_device_info(&cus, nullptr);
+    int32_t slice_bytes = 131072;
+    if (const char *e = std::getenv("ASX_SLICE_BYTES")) slice_bytes = std::atoi(e);
+    int32_t target = cus * (131072 / slice_bytes);
+    if (const char *e = std::getenv("ASX_SLICE_WGS")) target = std::atoi(e);
+    // pass 2: one wave per block of rows; at least 8 waves per compute unit where m allows, at most
+    // 16 KiB of accumulators per wave
+    int32_t rpw = 256;
+    while (rpw < (int32_t)(16384 / sizeof(T)) && (int64_t)rpw * cus * 8 < m) rpw *= 2;
+    if (const char *e = std::getenv("ASX_SLICE_RPW")) rpw = std::atoi(e);
+    st = build_sliced<T>(m, n, nnz, (int32_t)(slice_bytes / sizeof(T)), rpw, target, d_row_ptr, d_col, d_val,
+                         &p->sliced, s);
+    if (st) {
+        delete p;
+        return st;
+    }
+    p->nunits = p->sliced.ntiles;
+    p->workspace_bytes = align_up(((size_t)p->sliced.npartials + kWave) * sizeof(T), kAlign);
+    *out = p;
+    return ASX_STATUS_SUCCESS;
+}
+
 extern "C" {
 
 int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
@@ -666,6 +719,15 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     *out = nullptr;
     if (m < 0 || n < 0 || nnz < 0) return ASX_STATUS_INVALID_SIZE;
     if (value_type != ASX_R_32F && value_type != ASX_R_64F) return ASX_STATUS_NOT_SUPPORTED;
+    if (alg == ASX_SPMV_SLICED) {
+        if (m == 0 || nnz == 0 || n == 0) return ASX_STATUS_INVALID_SIZE;
+        if (!d_row_ptr || !d_col || !d_val) return ASX_STATUS_INVALID_POINTER;
+        if (value_type == ASX_R_64F)
+            return spmv_plan_sliced<double>(out, value_type, m, n, nnz, d_row_ptr, d_col, (const double *)d_val,
+                                            (hipStream_t)stream);
+        return spmv_plan_sliced<float>(out, value_type, m, n, nnz, d_row_ptr, d_col, (const float *)d_val,
+                                       (hipStream_t)stream);
+    }
     const bool want = alg == ASX_SPMV_PANEL;
     const bool candidate = alg == ASX_SPMV_DEFAULT && d_col && d_val &&
                            panel_candidate(m, n, nnz, vsize(value_type)) &&

@@ -74,6 +74,57 @@ __device__ __forceinline__ T wave_segscan_incl(int key, T v)
     return v;
 }
 
+// ---- segmented inclusive sum over a wave, DPP only (no LDS traffic) ---------------------------
+// Lanes whose `closed` is set start a new segment (their v already is the sum from the segment's
+// start inside the lane); lane 0 must be closed.  Returns, per lane, the sum of v from the nearest
+// closed lane at or below it up to itself.  Hillis-Steele over rows of 16 lanes (row_shr), then
+// row_bcast15 / row_bcast31 across rows; stops as soon as every lane has a segment start in reach
+// (after one step when nearly every lane is closed).  Lanes a move does not reach receive 0.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp0_i32(int v)
+{
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xF, false);
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp0(float v)
+{
+    return __int_as_float(dpp0_i32<CTRL, ROW_MASK>(__float_as_int(v)));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp0(double v)
+{
+    const int lo = dpp0_i32<CTRL, ROW_MASK>(__double2loint(v));
+    const int hi = dpp0_i32<CTRL, ROW_MASK>(__double2hiint(v));
+    return __hiloint2double(hi, lo);
+}
+template <typename T>
+__device__ __forceinline__ T wave_segsum_dpp(T v, bool closed)
+{
+    int f = closed ? 1 : 0;
+#define ASX_SEG_STEP(CTRL, ROW_MASK)                        \
+    {                                                       \
+        if (__ballot(f == 0) == 0) return v;                \
+        const T v2 = dpp0<CTRL, ROW_MASK>(v);               \
+        const int f2 = dpp0_i32<CTRL, ROW_MASK>(f);         \
+        v = f ? v : v + v2;                                 \
+        f |= f2;                                            \
+    }
+    ASX_SEG_STEP(0x111, 0xF)  // row_shr:1
+    ASX_SEG_STEP(0x112, 0xF)  // row_shr:2
+    ASX_SEG_STEP(0x114, 0xF)  // row_shr:4
+    ASX_SEG_STEP(0x118, 0xF)  // row_shr:8
+    ASX_SEG_STEP(0x142, 0xA)  // row_bcast15 into rows 1 and 3
+    ASX_SEG_STEP(0x143, 0xC)  // row_bcast31 into rows 2 and 3
+#undef ASX_SEG_STEP
+    return v;
+}
+// value of the lane below (lane 0 receives 0): wave_shr:1
+template <typename T>
+__device__ __forceinline__ T wave_shift_up1(T v)
+{
+    return dpp0<0x138, 0xF>(v);
+}
+
 template <typename T>
 __device__ __forceinline__ T fma_t(T a, T b, T c);
 template <>

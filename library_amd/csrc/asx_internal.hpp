@@ -143,6 +143,42 @@ int launch_spmv_panel(int32_t m, T alpha, const PanelMatrix *pm, const T *x, T b
 // out[r] = first i with sorted[i] >= r, r in [0, n]
 int launch_offsets_from_sorted(const int32_t *sorted, int32_t count, int32_t n, int32_t *out, hipStream_t s);
 
+// ---- column-sliced SpMV (asx_sliced.hip) ----
+// The stored elements regrouped by column slice (slice = col / width), a slice of x being small
+// enough to sit in the LDS of one compute unit, so that the gathers of x never reach the L2.
+// Pass 1: one workgroup per (slice, range of tiles) loads the slice of x into LDS and streams
+// the slice's stored elements, kSlicedTile per wave and step, in row order; it writes one partial
+// sum per run of elements of the same row (a run is also cut at every tile start, so tiles are
+// independent).  Pass 2: one wave per block of `rows_per_wave` rows of A adds the partial sums of
+// its rows, slice after slice, into LDS accumulators and writes y.  The partial sums of one row
+// block inside one slice are a contiguous range (`chunk_lo`).
+constexpr int kSlicedTile = 256;  // stored elements per wave and step: 4 per lane
+struct SlicedMatrix {
+    int32_t width;          // columns per slice
+    int32_t nslices;
+    int32_t ntiles;         // all slices; every slice starts a new tile and is padded to whole tiles
+    int32_t npartials;      // partial sums written per call
+    int32_t nwg;            // workgroups of pass 1
+    int32_t rows_per_wave;  // pass 2
+    int32_t nrb;            // ceil(m / rows_per_wave)
+    void *val;              // ntiles * kSlicedTile values (a copy of A's, in slice order; pads are 0)
+    uint16_t *cf;           // ntiles * kSlicedTile: column inside the slice, bit 15 = first element of a run
+    int32_t *perm;          // where each stored copy comes from in A's val (-1 for pads)
+    int32_t *tile_base;     // ntiles + 1: index of the first partial sum of each tile
+    int32_t *wg_tab;        // nwg x 4: slice, first tile, end tile, 0
+    uint16_t *prow;         // npartials: row of each partial sum inside its row block
+    int32_t *chunk_lo;      // (nrb + 1) x nslices: first partial sum of row block b in slice s
+};
+template <typename T>
+int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_per_wave, int32_t target_wgs,
+                 const int32_t *row_ptr, const int32_t *col, const T *val, SlicedMatrix *out, hipStream_t s);
+void free_sliced(SlicedMatrix *p);
+template <typename T>
+int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s);
+template <typename T>
+int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, T *partial,
+                       hipStream_t s);
+
 inline int32_t merge_tiles(int32_t m, int32_t nnz) { return (int32_t)ceil_div64((int64_t)m + nnz, kMergeTile); }
 inline int32_t flat_tiles(int32_t nnz) { int32_t t = (int32_t)ceil_div64(nnz, kFlatTile); return t < 1 ? 1 : t; }
 inline int32_t stream_blocks(int32_t nnz) { return (int32_t)ceil_div64(nnz, kStreamTile); }
@@ -166,4 +202,5 @@ struct asx_plan {
     size_t workspace_bytes;
     asx::BlockedMatrix blocked;  // only for ASX_SPMM_BLOCKED plans
     asx::PanelMatrix panel;      // only for ASX_SPMV_PANEL plans
+    asx::SlicedMatrix sliced;    // only for ASX_SPMV_SLICED plans
 };

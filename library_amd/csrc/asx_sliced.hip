@@ -1,0 +1,662 @@
+// Column-sliced CSR SpMV for matrices whose columns are scattered over a large x.
+//
+// A random gather of x that is served by an L2 costs one 128-byte L2 request per stored element,
+// and that request rate, not HBM, bounds the row-ordered kernels on such matrices.  Here the
+// stored elements are regrouped once (plan build) by column slice, a slice of x being at most
+// 128 KiB, and each workgroup of pass 1 copies its slice of x into LDS before it streams the
+// slice's stored elements: every gather is an LDS read.  What crosses slices is one partial sum
+// per (row, slice) pair with at least one stored element, written by pass 1 in slice order and
+// added up per row by pass 2.
+//
+//   pass 1  k_sliced_products : workgroup = (slice, range of tiles); wave = one tile of 256 stored
+//           elements per step (4 consecutive elements per lane, row order inside the slice).
+//           16-bit column-in-slice + "first element of a run" flag per element, values in the
+//           order the 16-byte loads deliver them.  In-lane running sums, one segmented wave scan,
+//           partial sums stored at tile_base[tile] + rank of the run.  A run is cut at every tile
+//           start, so a tile needs nothing from its neighbours (a row with 1000 elements in one
+//           slice leaves 4 or 5 partial sums there instead of 1).
+//   pass 2  k_sliced_reduce   : wave = block of rows_per_wave rows of A with an accumulator per row
+//           in LDS.  The partial sums of the block inside slice s are the contiguous range
+//           chunk_lo[b][s] .. chunk_lo[b+1][s]; the wave walks the slices in order and adds each
+//           range with LDS adds (only this wave touches its accumulators and a wave's LDS
+//           operations execute in order, so the order of additions is fixed), then writes
+//           y = alpha * acc + beta * y.
+//
+// No global atomics; results are bit-reproducible.  The reference has no counterpart (its CSR
+// kernels gather x from global memory: hip/kernel/level2/alphasparse_spmv_csr_vector.h:99-126).
+#include <hipcub/hipcub.hpp>
+
+#include <algorithm>
+#include <cstdlib>
+#include <vector>
+
+#include "asx_internal.hpp"
+
+namespace asx {
+
+namespace {
+
+constexpr int32_t kPadRow = 0x7fffffff;
+
+// Position of logical element e (= 4*lane + j) of a tile in the tile's value storage: the order
+// in which 16-byte loads at consecutive lanes deliver 4 consecutive elements to each lane.
+template <typename T>
+__host__ __device__ __forceinline__ int sliced_val_pos(int e)
+{
+    if (sizeof(T) == 8) {  // two loads of 2 doubles: [half][lane][2]
+        const int lane = e >> 2, j = e & 3;
+        return (j >> 1) * 128 + lane * 2 + (j & 1);
+    }
+    return e;  // one load of 4 floats
+}
+
+__global__ __launch_bounds__(kBlock) void k_sliced_keys(const int32_t *__restrict__ col, int32_t nnz, int32_t width,
+                                                        int32_t *__restrict__ keys, int32_t *__restrict__ idx)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nnz) return;
+    keys[i] = col[i] / width;
+    idx[i] = (int32_t)i;
+}
+
+// srow[p] = row of A that holds stored element sidx[p]
+__global__ __launch_bounds__(kBlock) void k_sliced_rows(const int32_t *__restrict__ sidx, int32_t nnz,
+                                                        const int32_t *__restrict__ row_ptr, int32_t m,
+                                                        int32_t *__restrict__ srow)
+{
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= nnz) return;
+    const int32_t src = sidx[p];
+    int32_t lo = 0, hi = m;  // largest r with row_ptr[r] <= src
+    while (lo < hi) {
+        const int32_t mid = lo + (hi - lo + 1) / 2;
+        if (row_ptr[mid] <= src)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    srow[p] = lo;
+}
+
+// Every slot of the padded element space starts as a pad: a run of its own with value 0 whose
+// partial sum no row block reads.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_sliced_fill_pads(int64_t slots, int32_t *__restrict__ lrow,
+                                                             int32_t *__restrict__ lhead, uint16_t *__restrict__ cf,
+                                                             T *__restrict__ val, int32_t *__restrict__ perm)
+{
+    const int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (d >= slots) return;
+    lrow[d] = kPadRow;
+    lhead[d] = 1;
+    cf[d] = 0x8000u;
+    val[d] = T(0);
+    perm[d] = -1;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_sliced_place(const int32_t *__restrict__ skey, const int32_t *__restrict__ sidx,
+                                                         const int32_t *__restrict__ srow, int32_t nnz, int32_t width,
+                                                         const int32_t *__restrict__ pstart,
+                                                         const int32_t *__restrict__ tile_off,
+                                                         const int32_t *__restrict__ col, const T *__restrict__ val,
+                                                         int32_t *__restrict__ lrow, int32_t *__restrict__ lhead,
+                                                         uint16_t *__restrict__ cf, T *__restrict__ val_out,
+                                                         int32_t *__restrict__ perm)
+{
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= nnz) return;
+    const int32_t sl = skey[p];
+    const int32_t q = (int32_t)(p - pstart[sl]);
+    const int64_t d = (int64_t)tile_off[sl] * kSlicedTile + q;
+    const int32_t src = sidx[p];
+    const int32_t row = srow[p];
+    const bool head = (q % kSlicedTile) == 0 || srow[p - 1] != row;
+    lrow[d] = row;
+    lhead[d] = head ? 1 : 0;
+    cf[d] = (uint16_t)((col[src] - sl * width) | (head ? 0x8000 : 0));
+    const int64_t t = d / kSlicedTile;
+    const int64_t phys = t * kSlicedTile + sliced_val_pos<T>((int)(d % kSlicedTile));
+    val_out[phys] = val[src];
+    perm[phys] = src;
+}
+
+__global__ __launch_bounds__(kBlock) void k_sliced_tile_base(const int32_t *__restrict__ hscan, int32_t ntiles,
+                                                             int32_t *__restrict__ tile_base)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t > ntiles) return;
+    tile_base[t] = t < ntiles ? hscan[t * kSlicedTile] - 1 : hscan[(int64_t)ntiles * kSlicedTile - 1];
+}
+
+__global__ __launch_bounds__(kBlock) void k_sliced_partial_rows(const int32_t *__restrict__ lrow,
+                                                                const int32_t *__restrict__ lhead,
+                                                                const int32_t *__restrict__ hscan, int64_t slots,
+                                                                int32_t rows_per_wave, int32_t *__restrict__ prow_full,
+                                                                uint16_t *__restrict__ prow)
+{
+    const int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (d >= slots || !lhead[d]) return;
+    const int32_t id = hscan[d] - 1;
+    const int32_t r = lrow[d];
+    prow_full[id] = r;
+    // bit 15: this partial sum may belong to the same row as the one before it (a run cut at a tile
+    // start); pass 2 must not add the two with one read-modify-write
+    const bool cont = d > 0 && d % kSlicedTile == 0 && lrow[d - 1] == r;
+    prow[id] = (uint16_t)((r % rows_per_wave) | (cont ? 0x8000 : 0));
+}
+
+// chunk_lo[b * nslices + s] = first partial sum of slice s whose row is >= b * rows_per_wave
+__global__ __launch_bounds__(kBlock) void k_sliced_chunks(const int32_t *__restrict__ prow_full,
+                                                          const int32_t *__restrict__ tile_base,
+                                                          const int32_t *__restrict__ tile_off, int32_t nslices,
+                                                          int32_t nrb, int32_t rows_per_wave,
+                                                          int32_t *__restrict__ chunk_lo)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= ((int64_t)nrb + 1) * nslices) return;
+    const int32_t b = (int32_t)(i / nslices), sl = (int32_t)(i % nslices);
+    const int64_t target = (int64_t)b * rows_per_wave;
+    int32_t lo = tile_base[tile_off[sl]], hi = tile_base[tile_off[sl + 1]];
+    while (lo < hi) {
+        const int32_t mid = lo + (hi - lo) / 2;
+        if ((int64_t)prow_full[mid] < target)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    chunk_lo[i] = lo;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_sliced_regather(const int32_t *__restrict__ perm, int64_t slots,
+                                                            const T *__restrict__ val, T *__restrict__ val_out)
+{
+    const int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (d >= slots) return;
+    const int32_t src = perm[d];
+    val_out[d] = src >= 0 ? val[src] : T(0);
+}
+
+// ---- pass 1 ------------------------------------------------------------------------------
+template <typename T>
+struct SlicedTileLoad;
+template <>
+struct SlicedTileLoad<double> {
+    static __device__ __forceinline__ void load(const double *tile, int lane, double v[4])
+    {
+        typedef double f64x2 __attribute__((ext_vector_type(2)));
+        const f64x2 *q = reinterpret_cast<const f64x2 *>(tile);
+        const f64x2 a = __builtin_nontemporal_load(q + lane);
+        const f64x2 b = __builtin_nontemporal_load(q + 64 + lane);
+        v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
+    }
+};
+template <>
+struct SlicedTileLoad<float> {
+    static __device__ __forceinline__ void load(const float *tile, int lane, float v[4])
+    {
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(tile) + lane);
+        v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w;
+    }
+};
+
+__device__ __forceinline__ int lanes_below(unsigned long long mask)
+{
+    return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0));
+}
+
+// One tile's stored elements as the loads deliver them.
+template <typename T>
+struct SlicedTile {
+    uint32_t c01, c23;  // 4 x (column in slice | run start << 15)
+    T v[4];
+    int32_t base;  // index of the tile's first partial sum
+};
+template <typename T>
+__device__ __forceinline__ void sliced_tile_load(SlicedTile<T> &tl, int32_t t, int lane, const uint16_t *__restrict__ cf,
+                                                 const T *__restrict__ val, const int32_t *__restrict__ tile_base)
+{
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 cw = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(cf + (int64_t)t * kSlicedTile) + lane);
+    tl.c01 = cw.x;
+    tl.c23 = cw.y;
+    SlicedTileLoad<T>::load(val + (int64_t)t * kSlicedTile, lane, tl.v);
+    tl.base = tile_base[t];
+}
+
+// Products, running sums, wave scan and the stores of one tile.
+template <typename T>
+__device__ __forceinline__ void sliced_tile_reduce(const SlicedTile<T> &tl, int lane, const T *xs, T *__restrict__ partial)
+{
+    const bool f0 = (tl.c01 >> 15) & 1, f1 = tl.c01 >> 31, f2 = (tl.c23 >> 15) & 1, f3 = tl.c23 >> 31;
+    const T p0 = tl.v[0] * xs[tl.c01 & 0x7fff], p1 = tl.v[1] * xs[(tl.c01 >> 16) & 0x7fff];
+    const T p2 = tl.v[2] * xs[tl.c23 & 0x7fff], p3 = tl.v[3] * xs[(tl.c23 >> 16) & 0x7fff];
+    // running sums that restart at every run start
+    const T r0 = p0;
+    const T r1 = f1 ? p1 : r0 + p1;
+    const T r2 = f2 ? p2 : r1 + p2;
+    const T r3 = f3 ? p3 : r2 + p3;
+    const int nh = (int)f0 + (int)f1 + (int)f2 + (int)f3;
+    const unsigned long long m0 = __ballot(f0), m1 = __ballot(f1), m2 = __ballot(f2), m3 = __ballot(f3);
+    const int before = lanes_below(m0) + lanes_below(m1) + lanes_below(m2) + lanes_below(m3);
+    const int total = __popcll(m0) + __popcll(m1) + __popcll(m2) + __popcll(m3);
+    // sum of the run that is open at the end of each lane, over the lanes it spans
+    const T open = wave_segsum_dpp<T>(r3, nh != 0);
+    const T cin = wave_shift_up1<T>(open);  // what earlier lanes hold of the run open at this lane's start
+    // a run start closes the run before it
+    T *out = partial + tl.base;
+    int hb = before;
+    if (f0 && hb > 0) out[hb - 1] = cin;
+    hb += f0;
+    if (f1) out[hb - 1] = f0 ? r0 : cin + r0;
+    hb += f1;
+    if (f2) out[hb - 1] = (f0 | f1) ? r1 : cin + r1;
+    hb += f2;
+    if (f3) out[hb - 1] = (f0 | f1 | f2) ? r2 : cin + r2;
+    if (lane == kWave - 1) out[total - 1] = open;
+}
+
+template <typename T, int WIDTH, int NW, int D>
+__global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const int4 *__restrict__ wg_tab,
+                                                               const uint16_t *__restrict__ cf,
+                                                               const T *__restrict__ val,
+                                                               const int32_t *__restrict__ tile_base,
+                                                               const T *__restrict__ x, T *__restrict__ partial)
+{
+    __shared__ T xs[WIDTH];
+    const int4 wg = wg_tab[blockIdx.x];
+    const int64_t c0 = (int64_t)wg.x * WIDTH;
+    const int32_t cnt = n - c0 < WIDTH ? (int32_t)(n - c0) : WIDTH;
+    {
+        // the slice of x: every load issued before the first LDS write (one memory round trip)
+        constexpr int V = 16 / sizeof(T);                 // values per 16-byte load
+        constexpr int PER = WIDTH / (NW * kWave * V);     // loads per thread
+        static_assert(PER * NW * kWave * V == WIDTH, "slice width must be a multiple of the workgroup's loads");
+        typedef T vec_t __attribute__((ext_vector_type(V)));
+        vec_t buf[PER];
+        const bool whole = cnt == WIDTH && ((uintptr_t)(x + c0) % 16) == 0;
+        if (whole) {
+#pragma unroll
+            for (int k = 0; k < PER; ++k)
+                buf[k] = reinterpret_cast<const vec_t *>(x + c0)[k * NW * kWave + threadIdx.x];
+        } else {
+#pragma unroll
+            for (int k = 0; k < PER; ++k) {
+                const int i0 = (k * NW * kWave + (int)threadIdx.x) * V;
+#pragma unroll
+                for (int e = 0; e < V; ++e) buf[k][e] = i0 + e < cnt ? x[c0 + i0 + e] : T(0);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < PER; ++k) reinterpret_cast<vec_t *>(xs)[k * NW * kWave + threadIdx.x] = buf[k];
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    // D tiles in turn; a tile's loads are issued D steps ahead, right after the stores of the tile
+    // that used the buffer before it.  The loads are unconditional (past the end they re-read the
+    // last tile), so that the number of memory operations issued after them is known and a step
+    // waits for its own loads only.
+    const int32_t last = wg.z - 1;
+    SlicedTile<T> tl[D];
+    int32_t t = wg.y + wave;
+#pragma unroll
+    for (int d = 0; d < D; ++d) sliced_tile_load<T>(tl[d], t + d * NW < last ? t + d * NW : last, lane, cf, val, tile_base);
+    while (t < wg.z) {  // uniform over the wave
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            if (t + d * NW < wg.z) sliced_tile_reduce<T>(tl[d], lane, xs, partial);
+            sliced_tile_load<T>(tl[d], t + (D + d) * NW < last ? t + (D + d) * NW : last, lane, cf, val, tile_base);
+        }
+        t += D * NW;
+    }
+}
+
+// ---- pass 2 ------------------------------------------------------------------------------
+// acc[id & 0x7fff] += v for the lanes that are `on`.  MODE 0: LDS atomic adds.  MODE 1: plain
+// read-add-write for entries whose row differs from the entry before them (sorted rows: no two
+// such lanes share an address), atomic adds afterwards for the marked rest (rare).  The wave owns
+// its accumulators and its LDS operations execute in order, so either way the sums are added in
+// a fixed order.
+template <int MODE, typename T>
+__device__ __forceinline__ void lds_add(T *acc, uint16_t id, T v, bool on)
+{
+    T *p = acc + (id & 0x7fff);
+    if (MODE == 0) {
+        if (on) __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);  // ds_add_f32 / _f64
+    } else {
+        const bool cont = (id & 0x8000) != 0;
+        if (on && !cont) *p += v;
+        if (__ballot(on && cont) != 0) {
+            if (on && cont) __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    }
+}
+
+// Walks the ranges of one row block, 64 entries per step.
+struct RangeWalk {
+    int32_t lo_v, len_v;  // per lane: start and length of range `lane` of the current 64 slices
+    int32_t ns;           // ranges in the current group
+    int32_t j, k0;        // current range and offset inside it
+    int32_t a, len;       // start and length of the current range (uniform)
+    __device__ __forceinline__ void fetch()
+    {
+        a = __builtin_amdgcn_readlane(lo_v, j & (kWave - 1));
+        len = j < ns ? __builtin_amdgcn_readlane(len_v, j & (kWave - 1)) : 0;
+    }
+    // start (an index that is safe to load from for 64 lanes) and count of the next step
+    __device__ __forceinline__ void next(int32_t &start, int32_t &count)
+    {
+        const int32_t left = len - k0;
+        count = left < kWave ? (left > 0 ? left : 0) : kWave;
+        start = j < ns ? a + k0 : 0;
+        k0 += kWave;
+        if (k0 >= len && j < ns) {
+            ++j;
+            k0 = 0;
+            fetch();
+        }
+    }
+};
+
+template <typename T, int NW, int MODE>
+__global__ __launch_bounds__(NW *kWave) void k_sliced_reduce(int32_t m, int32_t nrb, int32_t rw, int32_t nslices, T alpha,
+                                                             T beta, const int32_t *__restrict__ chunk_lo,
+                                                             const uint16_t *__restrict__ prow,
+                                                             const T *__restrict__ partial, T *__restrict__ y)
+{
+    extern __shared__ __align__(16) unsigned char sliced_lds[];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    // neighbouring row blocks share the cache lines at the ends of their ranges: keep them on one XCD
+    // (the grid is a multiple of kXcds workgroups, dealt to the XCDs round-robin)
+    const int32_t per_xcd = (int32_t)gridDim.x / kXcds;
+    const int32_t wg = ((int32_t)blockIdx.x % kXcds) * per_xcd + (int32_t)blockIdx.x / kXcds;
+    const int64_t b = (int64_t)wg * NW + wave;
+    if (b >= nrb) return;  // whole waves leave; no workgroup barrier below
+    T *acc = reinterpret_cast<T *>(sliced_lds) + (size_t)wave * rw;
+    for (int i = lane; i < rw; i += kWave) acc[i] = T(0);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    const int32_t *lo_row = chunk_lo + b * nslices;
+    const int32_t *hi_row = lo_row + nslices;
+    // Steps of 64 (row, partial sum) pairs, U steps per batch, two batches in turn: a batch's loads
+    // are issued before the other batch is added.  Loads are unconditional (prow and partial are
+    // readable for 64 entries past the last partial sum; a step past the end reads entry 0 on);
+    // entries past a range's end are dropped at the add.
+    constexpr int U = 16;
+    for (int32_t s0 = 0; s0 < nslices; s0 += kWave) {
+        const int32_t ns = nslices - s0 < kWave ? nslices - s0 : kWave;
+        const int32_t lo_v = lane < ns ? lo_row[s0 + lane] : 0;
+        const int32_t len_v = lane < ns ? hi_row[s0 + lane] - lo_v : 0;
+        uint16_t ida[U], idb[U];
+        T pa[U], pb[U];
+#define ASX_ADD(ID, PV, N)                        \
+    _Pragma("unroll") for (int u = 0; u < U; ++u) \
+    {                                             \
+        lds_add<MODE, T>(acc, ID[u], PV[u], lane < N[u]); \
+    }
+        if (__ballot(len_v > kWave) == 0) {
+            // every range fits one step: range j is step j
+#define ASX_LOAD(ID, PV, J)                                         \
+    _Pragma("unroll") for (int u = 0; u < U; ++u)                   \
+    {                                                               \
+        const int32_t a = __builtin_amdgcn_readlane(lo_v, (J) + u); \
+        ID[u] = prow[a + lane];                                     \
+        PV[u] = partial[a + lane];                                  \
+    }
+#define ASX_ADDJ(ID, PV, J)                       \
+    _Pragma("unroll") for (int u = 0; u < U; ++u) \
+    {                                             \
+        lds_add<MODE, T>(acc, ID[u], PV[u], lane < __builtin_amdgcn_readlane(len_v, (J) + u)); \
+    }
+            ASX_LOAD(ida, pa, 0)
+            if (ns > U) ASX_LOAD(idb, pb, U)
+            ASX_ADDJ(ida, pa, 0)
+            if (ns > 2 * U) ASX_LOAD(ida, pa, 2 * U)
+            if (ns > U) ASX_ADDJ(idb, pb, U)
+            if (ns > 3 * U) ASX_LOAD(idb, pb, 3 * U)
+            if (ns > 2 * U) ASX_ADDJ(ida, pa, 2 * U)
+            if (ns > 3 * U) ASX_ADDJ(idb, pb, 3 * U)
+#undef ASX_LOAD
+#undef ASX_ADDJ
+        } else {
+            RangeWalk w;
+            w.ns = ns;
+            w.lo_v = lo_v;
+            w.len_v = len_v;
+            w.j = 0;
+            w.k0 = 0;
+            w.fetch();
+            int32_t na[U], nb[U];
+#define ASX_LOAD(ID, PV, N)                       \
+    _Pragma("unroll") for (int u = 0; u < U; ++u) \
+    {                                             \
+        int32_t start;                            \
+        w.next(start, N[u]);                      \
+        ID[u] = prow[start + lane];               \
+        PV[u] = partial[start + lane];            \
+    }
+            ASX_LOAD(ida, pa, na)
+            ASX_LOAD(idb, pb, nb)
+            while (true) {  // uniform over the wave
+                ASX_ADD(ida, pa, na)
+                const bool more_a = w.j < w.ns;
+                ASX_LOAD(ida, pa, na)
+                ASX_ADD(idb, pb, nb)
+                if (!more_a) break;  // nothing was left when batch a was reloaded: a and b are spent
+                ASX_LOAD(idb, pb, nb)
+            }
+#undef ASX_LOAD
+        }
+#undef ASX_ADD
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int64_t r0 = b * rw;
+    for (int i = lane; i < rw; i += kWave) {
+        const int64_t r = r0 + i;
+        if (r < m) y[r] = beta == T(0) ? alpha * acc[i] : fma_t<T>(alpha, acc[i], beta * y[r]);
+    }
+}
+
+}  // namespace
+
+void free_sliced(SlicedMatrix *p)
+{
+    for (void *q : {p->val, (void *)p->cf, (void *)p->perm, (void *)p->tile_base, (void *)p->wg_tab, (void *)p->prow,
+                    (void *)p->chunk_lo})
+        if (q) (void)hipFree(q);
+    p->val = nullptr;
+    p->cf = p->prow = nullptr;
+    p->perm = p->tile_base = p->wg_tab = p->chunk_lo = nullptr;
+}
+
+template <typename T>
+int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_per_wave, int32_t target_wgs,
+                 const int32_t *row_ptr, const int32_t *col, const T *val, SlicedMatrix *out, hipStream_t s)
+{
+    SlicedMatrix sm{};
+    if (m <= 0 || nnz <= 0 || n <= 0) return ASX_STATUS_INVALID_SIZE;
+    if (width < 1 || width > 32768 || rows_per_wave < 1 || rows_per_wave > 65536 || target_wgs < 1)
+        return ASX_STATUS_INVALID_VALUE;
+    sm.width = width;
+    sm.nslices = (int32_t)ceil_div64(n, width);
+    sm.rows_per_wave = rows_per_wave;
+    sm.nrb = (int32_t)ceil_div64(m, rows_per_wave);
+    int key_bits = 1;
+    while ((1 << key_bits) < sm.nslices) ++key_bits;
+
+    int st = ASX_STATUS_SUCCESS;
+    int32_t *a = nullptr, *b = nullptr, *c = nullptr, *d = nullptr;  // nnz-sized scratch
+    int32_t *lrow = nullptr, *lhead = nullptr, *hscan = nullptr, *prow_full = nullptr;
+    int32_t *d_pstart = nullptr, *d_tile_off = nullptr;
+    void *tmp = nullptr;
+    size_t tmp_sort = 0, tmp_scan = 0, tmp_bytes = 0;
+    std::vector<int32_t> pstart((size_t)sm.nslices + 1), tile_off((size_t)sm.nslices + 1, 0);
+    std::vector<int32_t> tab;
+    int64_t slots = 0;
+    const unsigned grid = (unsigned)ceil_div64(nnz, kBlock);
+    const size_t nb = sizeof(int32_t) * (size_t)nnz;
+#define ASX_TRY(expr)         \
+    do {                      \
+        st = status_of(expr); \
+        if (st) goto done;    \
+    } while (0)
+#define ASX_TRY_ST(expr)   \
+    do {                   \
+        st = (expr);       \
+        if (st) goto done; \
+    } while (0)
+    for (int32_t **q : {&a, &b, &c, &d}) ASX_TRY(hipMalloc((void **)q, nb));
+    ASX_TRY(hipMalloc((void **)&d_pstart, sizeof(int32_t) * ((size_t)sm.nslices + 1)));
+    ASX_TRY(hipMalloc((void **)&d_tile_off, sizeof(int32_t) * ((size_t)sm.nslices + 1)));
+
+    // 1. stored elements by slice (stable: row order, then column order, survives inside a slice)
+    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_sort, a, b, c, d, nnz, 0, key_bits, s));
+    ASX_TRY(hipMalloc(&tmp, tmp_sort ? tmp_sort : 1));
+    hipLaunchKernelGGL(k_sliced_keys, dim3(grid), dim3(kBlock), 0, s, col, nnz, width, a, c);
+    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_sort, a, b, c, d, nnz, 0, key_bits, s));
+    // b = slice of each sorted element, d = its position in A; a = its row
+    hipLaunchKernelGGL(k_sliced_rows, dim3(grid), dim3(kBlock), 0, s, d, nnz, row_ptr, m, a);
+    ASX_TRY_ST(launch_offsets_from_sorted(b, nnz, sm.nslices, d_pstart, s));
+    ASX_TRY(hipMemcpyAsync(pstart.data(), d_pstart, sizeof(int32_t) * pstart.size(), hipMemcpyDeviceToHost, s));
+    ASX_TRY(hipStreamSynchronize(s));
+    (void)hipFree(tmp);
+    tmp = nullptr;
+
+    // 2. tiles: every slice starts a new tile
+    for (int32_t sl = 0; sl < sm.nslices; ++sl)
+        tile_off[sl + 1] = tile_off[sl] + (int32_t)ceil_div64(pstart[sl + 1] - pstart[sl], kSlicedTile);
+    sm.ntiles = tile_off[sm.nslices];
+    slots = (int64_t)sm.ntiles * kSlicedTile;
+    if (slots > 0x7fffffff) {
+        st = ASX_STATUS_INVALID_SIZE;
+        goto done;
+    }
+    ASX_TRY(hipMemcpyAsync(d_tile_off, tile_off.data(), sizeof(int32_t) * tile_off.size(), hipMemcpyHostToDevice, s));
+    ASX_TRY(hipMalloc(&sm.val, sizeof(T) * (size_t)slots));
+    ASX_TRY(hipMalloc((void **)&sm.cf, sizeof(uint16_t) * (size_t)slots));
+    ASX_TRY(hipMalloc((void **)&sm.perm, sizeof(int32_t) * (size_t)slots));
+    ASX_TRY(hipMalloc((void **)&lrow, sizeof(int32_t) * (size_t)slots));
+    ASX_TRY(hipMalloc((void **)&lhead, sizeof(int32_t) * (size_t)slots));
+    ASX_TRY(hipMalloc((void **)&hscan, sizeof(int32_t) * (size_t)slots));
+    {
+        const unsigned sgrid = (unsigned)ceil_div64(slots, kBlock);
+        hipLaunchKernelGGL((k_sliced_fill_pads<T>), dim3(sgrid), dim3(kBlock), 0, s, slots, lrow, lhead, sm.cf,
+                           (T *)sm.val, sm.perm);
+        hipLaunchKernelGGL((k_sliced_place<T>), dim3(grid), dim3(kBlock), 0, s, b, d, a, nnz, width, d_pstart, d_tile_off,
+                           col, val, lrow, lhead, sm.cf, (T *)sm.val, sm.perm);
+        // 3. partial sums: one per run start
+        ASX_TRY(hipcub::DeviceScan::InclusiveSum(nullptr, tmp_scan, lhead, hscan, (int)slots, s));
+        tmp_bytes = tmp_scan;
+        ASX_TRY(hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1));
+        ASX_TRY(hipcub::DeviceScan::InclusiveSum(tmp, tmp_bytes, lhead, hscan, (int)slots, s));
+        ASX_TRY(hipMemcpyAsync(&sm.npartials, hscan + (slots - 1), sizeof(int32_t), hipMemcpyDeviceToHost, s));
+        ASX_TRY(hipStreamSynchronize(s));
+        ASX_TRY(hipMalloc((void **)&sm.tile_base, sizeof(int32_t) * ((size_t)sm.ntiles + 1)));
+        ASX_TRY(hipMalloc((void **)&sm.prow, sizeof(uint16_t) * ((size_t)sm.npartials + kWave)));
+        ASX_TRY(hipMemsetAsync(sm.prow, 0, sizeof(uint16_t) * ((size_t)sm.npartials + kWave), s));
+        ASX_TRY(hipMalloc((void **)&prow_full, sizeof(int32_t) * (size_t)sm.npartials));
+        ASX_TRY(hipMalloc((void **)&sm.chunk_lo, sizeof(int32_t) * ((size_t)sm.nrb + 1) * (size_t)sm.nslices));
+        hipLaunchKernelGGL(k_sliced_tile_base, dim3((unsigned)ceil_div64((int64_t)sm.ntiles + 1, kBlock)), dim3(kBlock),
+                           0, s, hscan, sm.ntiles, sm.tile_base);
+        hipLaunchKernelGGL(k_sliced_partial_rows, dim3(sgrid), dim3(kBlock), 0, s, lrow, lhead, hscan, slots,
+                           rows_per_wave, prow_full, sm.prow);
+        // 4. where each row block starts inside each slice's partial sums
+        const int64_t nchunks = ((int64_t)sm.nrb + 1) * sm.nslices;
+        hipLaunchKernelGGL(k_sliced_chunks, dim3((unsigned)ceil_div64(nchunks, kBlock)), dim3(kBlock), 0, s, prow_full,
+                           sm.tile_base, d_tile_off, sm.nslices, sm.nrb, rows_per_wave, sm.chunk_lo);
+    }
+    // 5. workgroups of pass 1: every slice gets its share of about `target_wgs` workgroups (at
+    //    least one, and no workgroup smaller than 32 tiles unless the slice is), its tiles in equal
+    //    pieces
+    {
+        for (int32_t sl = 0; sl < sm.nslices; ++sl) {
+            const int32_t tiles = tile_off[sl + 1] - tile_off[sl];
+            if (tiles == 0) continue;
+            int32_t pieces = (int32_t)(((int64_t)tiles * target_wgs + sm.ntiles / 2) / sm.ntiles);
+            pieces = std::min<int32_t>(pieces, tiles / 32);
+            pieces = std::max<int32_t>(pieces, 1);
+            for (int32_t k = 0; k < pieces; ++k) {
+                tab.push_back(sl);
+                tab.push_back(tile_off[sl] + (int32_t)((int64_t)tiles * k / pieces));
+                tab.push_back(tile_off[sl] + (int32_t)((int64_t)tiles * (k + 1) / pieces));
+                tab.push_back(0);
+            }
+        }
+        sm.nwg = (int32_t)(tab.size() / 4);
+        ASX_TRY(hipMalloc((void **)&sm.wg_tab, sizeof(int32_t) * std::max<size_t>(tab.size(), 4)));
+        ASX_TRY(hipMemcpyAsync(sm.wg_tab, tab.data(), sizeof(int32_t) * tab.size(), hipMemcpyHostToDevice, s));
+    }
+    ASX_TRY(hipStreamSynchronize(s));
+    ASX_TRY(hipGetLastError());
+#undef ASX_TRY
+#undef ASX_TRY_ST
+done:
+    for (void *p : {(void *)a, (void *)b, (void *)c, (void *)d, (void *)lrow, (void *)lhead, (void *)hscan,
+                    (void *)prow_full, (void *)d_pstart, (void *)d_tile_off, tmp})
+        if (p) (void)hipFree(p);
+    if (st) {
+        free_sliced(&sm);
+        return st;
+    }
+    *out = sm;
+    return ASX_STATUS_SUCCESS;
+}
+
+template <typename T>
+int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s)
+{
+    const int64_t slots = (int64_t)sm->ntiles * kSlicedTile;
+    if (slots == 0) return ASX_STATUS_SUCCESS;
+    hipLaunchKernelGGL((k_sliced_regather<T>), dim3((unsigned)ceil_div64(slots, kBlock)), dim3(kBlock), 0, s, sm->perm,
+                       slots, val, (T *)sm->val);
+    return check_launch();
+}
+
+template <typename T>
+int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, T *partial,
+                       hipStream_t s)
+{
+    if (m <= 0) return ASX_STATUS_SUCCESS;
+    constexpr int kSmall = 65536 / sizeof(T), kLarge = 131072 / sizeof(T);
+    const int4 *tab = reinterpret_cast<const int4 *>(sm->wg_tab);
+    static const int depth = std::getenv("ASX_P1_DEPTH") ? std::atoi(std::getenv("ASX_P1_DEPTH")) : 4;
+#define ASX_PROD(W, NW, D)                                                                                          \
+    hipLaunchKernelGGL((k_sliced_products<T, W, NW, D>), dim3((unsigned)sm->nwg), dim3(NW * kWave), 0, s, n, tab, \
+                       sm->cf, (const T *)sm->val, sm->tile_base, x, partial)
+    if (sm->nwg > 0) {
+        if (sm->width == kLarge) {
+            if (depth == 2) ASX_PROD(kLarge, 16, 2); else if (depth == 8) ASX_PROD(kLarge, 16, 8); else ASX_PROD(kLarge, 16, 4);
+        } else if (sm->width == kSmall) {
+            if (depth == 2) ASX_PROD(kSmall, 16, 2); else if (depth == 8) ASX_PROD(kSmall, 16, 8); else ASX_PROD(kSmall, 16, 4);
+        } else
+            return ASX_STATUS_INVALID_VALUE;
+    }
+#undef ASX_PROD
+    constexpr int kWaves = 4;
+    if (sm->rows_per_wave < 1 || (size_t)sm->rows_per_wave * sizeof(T) > 16384) return ASX_STATUS_INVALID_VALUE;
+    const unsigned rgrid = (unsigned)(ceil_div64(ceil_div64(sm->nrb, kWaves), kXcds) * kXcds);
+    const size_t lds = (size_t)kWaves * sm->rows_per_wave * sizeof(T);
+    static const int mode_env = std::getenv("ASX_P2_MODE") ? std::atoi(std::getenv("ASX_P2_MODE")) : -1;
+    const int mode = mode_env >= 0 ? mode_env : (sizeof(T) == 4 ? 1 : 0);
+#define ASX_RED(MODE)                                                                                              \
+    hipLaunchKernelGGL((k_sliced_reduce<T, kWaves, MODE>), dim3(rgrid), dim3(kWaves * kWave), lds, s, m, sm->nrb,  \
+                       sm->rows_per_wave, sm->nslices, alpha, beta, sm->chunk_lo, sm->prow, partial, y)
+    if (mode == 1)
+        ASX_RED(1);
+    else
+        ASX_RED(0);
+#undef ASX_RED
+    return check_launch();
+}
+
+#define ASX_INST(T)                                                                                              \
+    template int build_sliced<T>(int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, const int32_t *,          \
+                                 const int32_t *, const T *, SlicedMatrix *, hipStream_t);                       \
+    template int sliced_update_values<T>(const SlicedMatrix *, const T *, hipStream_t);                          \
+    template int launch_spmv_sliced<T>(int32_t, int32_t, T, const SlicedMatrix *, const T *, T, T *, T *, hipStream_t);
+ASX_INST(float)
+ASX_INST(double)
+#undef ASX_INST
+
+}  // namespace asx
