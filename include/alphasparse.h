@@ -169,7 +169,7 @@ typedef struct alphasparse_handle_s {
     double *done;
     bool check_flag;
     int *process;
-    void *pflat_analysis_data;  // analysis results kept by alphasparseSpMV_analysis / SpMM_preprocess
+    void *pflat_analysis_data;  // here: the matrices that hold analysis results made through this handle
 
     alphasparse_handle_s()
         : device(0), wavefront_size(0), asic_rev(0), properties(), stream(nullptr), streams(),
@@ -181,11 +181,90 @@ typedef struct alphasparse_handle_s {
 } alphasparse_handle;
 typedef alphasparse_handle *alphasparseHandle_t;
 
-// ---- descriptors -----------------------------------------------------------------------------
-struct _alphasparse_mat_info;  // opaque here
+// ---- analysis info (include/alphasparse/handle.h:147-198, 216-248) ----------------------------
+// The reference's home for what an analysis call learns about a matrix.  Nothing on the
+// reference's generic SpMV / SpMM path fills it; here alphasparseSpMV_analysis and
+// alphasparseSpMM_preprocess hang their results on the matrix through it (matA->info->csrmv_info,
+// whose verification fields m, n, nnz, trans, csr_row_ptr, csr_col_ind are filled as the struct
+// intends; the kernels' own metadata lives in an extension behind the same allocation).
+struct alpha_matrix_descr {  // include/alphasparse/spdef.h:288-296
+    alphasparse_matrix_type_t type;
+    alphasparse_fill_mode_t mode;
+    alphasparse_diag_type_t diag;
+    alphasparseIndexBase_t base;
+};
+enum csrgemv_algo {  // handle.h:147-156
+    ALPHA_CSRMV_AUTO,
+    ALPHA_CSRMV_SCALAR,
+    ALPHA_CSRMV_VECTOR,
+    ALPHA_CSRMV_ROW_PARTITION,
+    ALPHA_CSRMV_ADAPTIVE,
+    ALPHA_CSRMV_MERGE,
+    ALPHA_CSRMV_XXX
+};
+struct _alphasparse_csrmv_info {  // handle.h:158-198
+    bool algo_tuning;
+    csrgemv_algo algo;
+    int iter;
+    size_t size;
+    unsigned long long *row_blocks;
+    bool csr_adaptive_has_tuned;
+    int32_t stream_num;
+    int32_t vector_num;
+    int32_t vectorL_num;
+    int *partition;
+    bool csr_rowpartition_has_tuned;
+    void *coordinate;
+    void *reduc_val;
+    void *reduc_row;
+    int num_merge_tiles;
+    bool csr_merge_has_tuned;
+    int *r_csr_row_ptr;
+    int *r_csr_col_ind;
+    int *r_row_indx;
+    void *r_csr_val;
+    alphasparseOperation_t trans;
+    int m;
+    int n;
+    int nnz;
+    const struct alpha_matrix_descr *descr;
+    const void *csr_row_ptr;
+    const void *csr_col_ind;
+};
+struct _alphasparse_trm_info;      // triangular-solve analysis: not on this path
+struct _alphasparse_csrgemm_info;  // SpGEMM analysis: not on this path
+typedef struct _alphasparse_trm_info *alphasparse_trm_info_t;
+typedef struct _alphasparse_csrmv_info *alphasparse_csrmv_info_t;
+typedef struct _alphasparse_csrgemm_info *alphasparse_csrgemm_info_t;
+struct _alphasparse_mat_info {  // handle.h:216-248
+    alphasparse_trm_info_t bsrsv_upper_info;
+    alphasparse_trm_info_t bsrsv_lower_info;
+    alphasparse_trm_info_t bsrsvt_upper_info;
+    alphasparse_trm_info_t bsrsvt_lower_info;
+    alphasparse_trm_info_t bsric0_info;
+    alphasparse_trm_info_t bsrilu0_info;
+    alphasparse_csrmv_info_t csrmv_info;
+    alphasparse_trm_info_t csric0_info;
+    alphasparse_trm_info_t csrilu0_info;
+    alphasparse_trm_info_t csrsv_upper_info;
+    alphasparse_trm_info_t csrsv_lower_info;
+    alphasparse_trm_info_t csrsvt_upper_info;
+    alphasparse_trm_info_t csrsvt_lower_info;
+    alphasparse_trm_info_t csrsm_upper_info;
+    alphasparse_trm_info_t csrsm_lower_info;
+    alphasparse_trm_info_t csrsmt_upper_info;
+    alphasparse_trm_info_t csrsmt_lower_info;
+    alphasparse_csrgemm_info_t csrgemm_info;
+    int *zero_pivot;
+    int boost_enable;
+    int use_double_prec_tol;
+    const void *boost_tol;
+    const void *boost_val;
+};
 typedef struct _alphasparse_mat_info *alphasparse_mat_info_t;
 
-struct _alphasparse_mat_descr {  // handle.h:329-352 (fields used on this path first)
+// ---- descriptors -----------------------------------------------------------------------------
+struct _alphasparse_mat_descr {  // handle.h:329-358
     alphasparse_matrix_type_t type = ALPHA_SPARSE_MATRIX_TYPE_GENERAL;
     alphasparse_fill_mode_t fill_mode = ALPHA_SPARSE_FILL_MODE_LOWER;
     alphasparse_diag_type_t diag_type = ALPHA_SPARSE_DIAG_NON_UNIT;
@@ -201,6 +280,11 @@ struct _alphasparse_mat_descr {  // handle.h:329-352 (fields used on this path f
     void *d_level_ptr = {};
     void *h_chain_ptr = {};
     int64_t h_level_size = 0;
+    int64_t h_chain_size = 0;
+    void *in_degree = {};
+    void *csr_row_idx = {};
+    void *csr_rdiag = {};
+    void *rcsr_rdiag = {};
 };
 typedef struct _alphasparse_mat_descr *alphasparse_mat_descr_t;
 typedef struct _alphasparse_mat_descr *alphasparseMatDescr_t;

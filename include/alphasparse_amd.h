@@ -50,8 +50,6 @@ enum {
     ASX_SPMV_STREAM = 3,  /* LDS-staged row blocks, segmented reduction */
     ASX_SPMV_MERGE = 9,   /* merge-path tiles + ordered carry fix-up */
     ASX_SPMV_FLAT = 15,   /* tiles of 1024 stored elements, register walk + ordered carry fix-up */
-    ASX_SPMV_PANEL = 100, /* not a reference id: the flat kernel over 16 or 32 column panels, 2 or 4 per XCD
-                             (needs a plan from asx_spmv_plan_create) */
     ASX_SPMV_SLICED = 101 /* not a reference id: stored elements regrouped by column slice, each slice of x
                              held in LDS; one partial sum per (row, slice), added per row by a second pass
                              (needs a plan from asx_spmv_plan_create) */
@@ -166,7 +164,7 @@ void asx_host_free(void *p);
  * SpMV/SpMM call; its alphasparseSpMV_analysis is a stub, hip/kernel/level2/alphasparse_spmv.hip:
  * 229-247, and _alphasparse_csrmv_info, include/alphasparse/handle.h:147-198, is never filled).
  * A plan owns device memory (allocated at creation, freed at destruction) and is bound to the
- * row_ptr contents it was built from.
+ * sparsity pattern it was built from.
  * ---------------------------------------------------------------------------------- */
 typedef struct asx_plan asx_plan;
 
@@ -178,28 +176,31 @@ int asx_plan_create(asx_plan **plan, int is_spmm, int alg, int value_type, int32
 /* SpMM plan that may look at A's columns and values.  alg = ASX_SPMM_BLOCKED re-tiles A into
  * zero-filled 16x4 blocks for the MFMA kernel (tc_preprocess,
  * hip/kernel/level3/alphasparse_spmm_tc4csr.h:38-153; the plan then holds a COPY of the values:
- * rebuild it when they change).  alg = ASX_SPMM_DEFAULT measures the block fill
- * nnz / (64 * blocks) and picks the blocked kernel when it is at least 1/8, else the merge
- * kernel.  Other algorithms behave as asx_plan_create.  Synchronises `stream`. */
+ * asx_plan_update_values after changing them; repeated (row, column) entries are summed; B must
+ * be finite, see below).  alg = ASX_SPMM_DEFAULT measures the block fill nnz / (64 * blocks) and
+ * picks the blocked kernel when it is at least 1/8, else the merge kernel.  Other algorithms
+ * behave as asx_plan_create.  Synchronises `stream`. */
 int asx_spmm_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, int32_t k, int32_t nnz,
                          const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, int32_t ncols,
                          void *stream);
-/* SpMV plan that may look at A's columns and values.  alg = ASX_SPMV_PANEL regroups the stored
- * elements into 16 (x up to 64 MiB) or 32 column panels, 2 or 4 per XCD, worked through one after
- * the other, so that each XCD's L2 holds the slice of x its workgroups gather from.  The plan
- * then holds a COPY of the values: rebuild it when they change; calls need up to
- * min(nnz, 32*m) values of workspace for the per-panel partial sums.  alg = ASX_SPMV_DEFAULT
- * considers panels when x is 6 to 256 MiB large, nnz >= 2^22 and the columns are scattered (a
- * sample of 64 tiles of 1024 stored elements touches on average more than 512 distinct 128-byte
- * lines of x per tile): it builds the panels, times the panel kernel against the kernel the
- * histogram picks (three runs each on scratch vectors) and keeps the faster.  Otherwise as
- * asx_plan_create.  No counterpart in the reference (its alphasparseSpMV_analysis is a stub).
- * Synchronises `stream`. */
+/* SpMV plan that may look at A's columns and values.  alg = ASX_SPMV_SLICED regroups the stored
+ * elements by column slice (128 KiB of x per slice) for the kernel that holds its slice of x in
+ * LDS.  The plan then holds a COPY of the columns and values (asx_plan_update_values after
+ * changing the values) and the buffer for the partial sums of a call: calls through one plan
+ * must not overlap.  alg = ASX_SPMV_DEFAULT picks that kernel when nnz >= 2^21, the columns are
+ * scattered (a sample of 64 tiles of 1024 stored elements touches on average more than 512
+ * distinct 128-byte lines of x per tile) and a cost model over the row-length histogram and the
+ * sizes puts it at least 10 % ahead of the row-ordered kernels; the choice depends on the matrix
+ * alone, not on timings.  Otherwise as asx_plan_create.  No counterpart in the reference (its
+ * alphasparseSpMV_analysis is a stub).  Synchronises `stream`. */
 int asx_spmv_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
                          const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, void *stream);
-/* Upper bound of the workspace a panel plan for (m, n, nnz) needs; 0 when the matrix is not a
- * candidate for panels.  For sizing a buffer before the plan exists. */
-size_t asx_spmv_panel_workspace_bytes(int value_type, int32_t m, int32_t n, int32_t nnz);
+/* Brings a plan that holds a copy of A's values (ASX_SPMV_SLICED, ASX_SPMM_BLOCKED) up to date
+ * with d_val (same sparsity pattern as when the plan was built); asynchronous on `stream`.  For
+ * the other kernels, which read the caller's values in every call, it does nothing.
+ * asx_plan_holds_values tells the two kinds apart.  No counterpart in the reference. */
+int asx_plan_update_values(asx_plan *plan, const void *d_val, void *stream);
+int asx_plan_holds_values(const asx_plan *plan);
 /* Number of 16x4 blocks and their fill of a blocked plan. */
 int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill);
 int asx_plan_destroy(asx_plan *plan);
@@ -250,23 +251,6 @@ int asx_spmm_csr_f64(const asx_plan *plan, int alg, int32_t m, int32_t k, int32_
                      double alpha, const int32_t *d_row_ptr, const int32_t *d_col, const double *d_val,
                      const double *d_B, int64_t ldb, double beta, double *d_C, int64_t ldc,
                      void *d_workspace, size_t workspace_bytes, void *stream);
-
-/* ------------------------------------------------------------------------------------
- * Measurement helpers (used by the benchmark; plain HIP underneath)
- * ---------------------------------------------------------------------------------- */
-/* A coalesced copy kernel of `bytes` bytes (multiple of 16): calibration for bandwidth counters. */
-int asx_copy_bytes(const void *d_src, void *d_dst, size_t bytes, void *stream);
-/* The memory side of a CSR SpMV without reduction and without output: mode 0 streams d_col and
- * d_val only, mode 1 also gathers d_x[col].  Gives the rates the chip sustains for a given
- * column pattern.  d_sink: one value of the value type (never written in practice). */
-int asx_probe_stream_gather(int value_type, int mode, int64_t nnz, const int32_t *d_col,
-                            const void *d_val, const void *d_x, void *d_sink, void *stream);
-/* As mode 1, with the gathers of every workgroup folded into one slice of d_x (n entries) chosen
- * from the workgroup id: slicing 0 = 8 slices, slice = workgroup id mod 8 (one slice per XCD);
- * 1 = 16 slices in two phases; 2 = 8 slices changing every 8 workgroups (control: every XCD sees
- * every slice).  Measures what a column-panel layout can gain. */
-int asx_probe_sliced_gather(int value_type, int slicing, int64_t nnz, int32_t n, const int32_t *d_col,
-                            const void *d_val, const void *d_x, void *d_sink, void *stream);
 
 #ifdef __cplusplus
 }

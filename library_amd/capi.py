@@ -14,24 +14,24 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libalphasparse_amd.so")
 
 R_32F, R_64F = 0, 1
-SPMV_DEFAULT, SPMV_STREAM, SPMV_VECTOR, SPMV_MERGE, SPMV_FLAT, SPMV_PANEL, SPMV_SLICED = 0, 3, 6, 9, 15, 100, 101
+SPMV_DEFAULT, SPMV_STREAM, SPMV_VECTOR, SPMV_MERGE, SPMV_FLAT, SPMV_SLICED = 0, 3, 6, 9, 15, 101
 SPMM_DEFAULT, SPMM_ROW, SPMM_MERGE, SPMM_BLOCKED = 0, 5, 7, 10
 
 STATUS = {0: "SUCCESS", 1: "NOT_INITIALIZED", 2: "ALLOC_FAILED", 3: "INVALID_VALUE",
           4: "EXECUTION_FAILED", 5: "INTERNAL_ERROR", 6: "NOT_SUPPORTED", 7: "INVALID_POINTER",
           8: "INVALID_HANDLE", 9: "INVALID_KERNEL_PARAM", 10: "INVALID_SIZE"}
 
-# every symbol include/alphasparse_amd.h declares
+# every symbol include/alphasparse_amd.h (and, last, include/alphasparse_amd_bench.h) declares
 EXPORTS = [
     "asx_version", "asx_device_info", "asx_row_length_histogram", "asx_partition_rows_by_nnz",
     "asx_nnz_split_rows", "asx_merge_path_search", "asx_loadbalance_nwarps",
     "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_coo2csr", "asx_coo_sort", "asx_csr_transpose", "asx_csr_rebase",
     "asx_dense_transpose", "asx_mtx_read", "asx_host_free", "asx_spmv_plan_create",
-    "asx_spmv_panel_workspace_bytes", "asx_plan_create",
+    "asx_plan_update_values", "asx_plan_holds_values", "asx_plan_create",
     "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
     "asx_spmm_resolve_alg", "asx_spmm_workspace_bytes", "asx_spmm_csr_f32", "asx_spmm_csr_f64",
-    "asx_copy_bytes", "asx_probe_stream_gather", "asx_probe_sliced_gather",
+    "asx_copy_bytes",
 ]
 
 
@@ -73,8 +73,8 @@ def lib():
     L.asx_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, C.c_int, i32, i32, i32, vp, i32, vp]
     L.asx_spmm_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, i32, i32, i32, vp, vp, vp, i32, vp]
     L.asx_spmv_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, i32, i32, i32, vp, vp, vp, vp]
-    L.asx_spmv_panel_workspace_bytes.argtypes = [C.c_int, i32, i32, i32]
-    L.asx_spmv_panel_workspace_bytes.restype = sz
+    L.asx_plan_update_values.argtypes = [vp, vp, vp]
+    L.asx_plan_holds_values.argtypes = [vp]
     L.asx_plan_block_stats.argtypes = [vp, C.POINTER(i64), C.POINTER(C.c_double)]
     L.asx_plan_destroy.argtypes = [vp]
     L.asx_plan_alg.argtypes = [vp]
@@ -92,8 +92,6 @@ def lib():
     L.asx_spmm_csr_f32.argtypes = [vp, C.c_int, i32, i32, i32, i32, C.c_float, vp, vp, vp, vp, i64, C.c_float, vp, i64, vp, sz, vp]
     L.asx_spmm_csr_f64.argtypes = [vp, C.c_int, i32, i32, i32, i32, C.c_double, vp, vp, vp, vp, i64, C.c_double, vp, i64, vp, sz, vp]
     L.asx_copy_bytes.argtypes = [vp, vp, sz, vp]
-    L.asx_probe_stream_gather.argtypes = [C.c_int, C.c_int, i64, vp, vp, vp, vp, vp]
-    L.asx_probe_sliced_gather.argtypes = [C.c_int, C.c_int, i64, i32, vp, vp, vp, vp, vp]
     _lib = L
     return L
 
@@ -274,6 +272,14 @@ class Plan:
         stats = np.zeros(4, dtype=np.int64)
         _check(lib().asx_plan_histogram(self.h, hist.ctypes.data_as(C.c_void_p), stats.ctypes.data_as(C.c_void_p)), "asx_plan_histogram")
         return hist, stats
+
+    def update_values(self, val):
+        _check(lib().asx_plan_update_values(self.h, _ptr(val), _stream()), "asx_plan_update_values")
+        self._keep = (self._keep[0], self._keep[1], val)
+
+    @property
+    def holds_values(self):
+        return bool(lib().asx_plan_holds_values(self.h))
 
     def destroy(self):
         if self.h:

@@ -24,19 +24,61 @@
 
 #include "../../include/alphasparse.h"
 
-// Layout checks against the reference headers compiled with the same ROCm headers.
-static_assert(offsetof(_alphasparseSpMatDescr, rows) == 8, "SpMat layout");
-static_assert(offsetof(_alphasparseSpMatDescr, row_data) == 40, "SpMat layout");
-static_assert(offsetof(_alphasparseSpMatDescr, col_data) == 48, "SpMat layout");
-static_assert(offsetof(_alphasparseSpMatDescr, val_data) == 64, "SpMat layout");
-static_assert(offsetof(_alphasparseSpMatDescr, row_type) == 104, "SpMat layout");
-static_assert(offsetof(_alphasparseSpMatDescr, data_type) == 112, "SpMat layout");
-static_assert(offsetof(_alphasparseSpMatDescr, idx_base) == 116, "SpMat layout");
-static_assert(offsetof(_alphasparseSpMatDescr, format) == 120, "SpMat layout");
-static_assert(offsetof(_alphasparseSpMatDescr, descr) == 128, "SpMat layout");
+// Layout checks.  The numbers are those of the reference's own headers compiled with the same
+// ROCm headers (tests/golden/layout.json, written by tests/golden/make_layout.py).
+#define ASX_OFF(T, f, v) static_assert(offsetof(T, f) == (v), #T "::" #f " moved")
+static_assert(sizeof(alphasparse_handle_s) == 1608, "handle layout");
+ASX_OFF(alphasparse_handle_s, properties, 16);
+ASX_OFF(alphasparse_handle_s, stream, 1488);
+ASX_OFF(alphasparse_handle_s, streams, 1496);
+ASX_OFF(alphasparse_handle_s, pointer_mode, 1544);
+ASX_OFF(alphasparse_handle_s, layer_mode, 1548);
+ASX_OFF(alphasparse_handle_s, buffer_size, 1552);
+ASX_OFF(alphasparse_handle_s, buffer, 1560);
+ASX_OFF(alphasparse_handle_s, sone, 1568);
+ASX_OFF(alphasparse_handle_s, done, 1576);
+ASX_OFF(alphasparse_handle_s, check_flag, 1584);
+ASX_OFF(alphasparse_handle_s, process, 1592);
+ASX_OFF(alphasparse_handle_s, pflat_analysis_data, 1600);
 static_assert(sizeof(_alphasparseSpMatDescr) == 208, "SpMat layout");
+ASX_OFF(_alphasparseSpMatDescr, rows, 8);
+ASX_OFF(_alphasparseSpMatDescr, row_data, 40);
+ASX_OFF(_alphasparseSpMatDescr, col_data, 48);
+ASX_OFF(_alphasparseSpMatDescr, val_data, 64);
+ASX_OFF(_alphasparseSpMatDescr, const_row_data, 72);
+ASX_OFF(_alphasparseSpMatDescr, row_type, 104);
+ASX_OFF(_alphasparseSpMatDescr, data_type, 112);
+ASX_OFF(_alphasparseSpMatDescr, idx_base, 116);
+ASX_OFF(_alphasparseSpMatDescr, format, 120);
+ASX_OFF(_alphasparseSpMatDescr, descr, 128);
+ASX_OFF(_alphasparseSpMatDescr, info, 136);
+ASX_OFF(_alphasparseSpMatDescr, batch_count, 176);
+static_assert(sizeof(_alphasparse_mat_descr) == 144, "mat_descr layout");
+ASX_OFF(_alphasparse_mat_descr, base, 12);
+ASX_OFF(_alphasparse_mat_descr, max_nnz_per_row, 16);
+ASX_OFF(_alphasparse_mat_descr, row_map, 32);
+ASX_OFF(_alphasparse_mat_descr, h_level_size, 96);
+ASX_OFF(_alphasparse_mat_descr, h_chain_size, 104);
+ASX_OFF(_alphasparse_mat_descr, csr_rdiag, 128);
+ASX_OFF(_alphasparse_mat_descr, rcsr_rdiag, 136);
 static_assert(sizeof(_alphasparse_dnvec_descr) == 32, "DnVec layout");
+ASX_OFF(_alphasparse_dnvec_descr, values, 16);
+ASX_OFF(_alphasparse_dnvec_descr, data_type, 24);
 static_assert(sizeof(_alphasparse_dnmat_descr) == 48, "DnMat layout");
+ASX_OFF(_alphasparse_dnmat_descr, ld, 24);
+ASX_OFF(_alphasparse_dnmat_descr, values, 32);
+ASX_OFF(_alphasparse_dnmat_descr, order, 44);
+static_assert(sizeof(_alphasparse_csrmv_info) == 168, "csrmv_info layout");
+ASX_OFF(_alphasparse_csrmv_info, row_blocks, 24);
+ASX_OFF(_alphasparse_csrmv_info, partition, 48);
+ASX_OFF(_alphasparse_csrmv_info, coordinate, 64);
+ASX_OFF(_alphasparse_csrmv_info, trans, 128);
+ASX_OFF(_alphasparse_csrmv_info, csr_row_ptr, 152);
+static_assert(sizeof(_alphasparse_mat_info) == 176, "mat_info layout");
+ASX_OFF(_alphasparse_mat_info, csrmv_info, 48);
+ASX_OFF(_alphasparse_mat_info, csrgemm_info, 136);
+ASX_OFF(_alphasparse_mat_info, boost_val, 168);
+#undef ASX_OFF
 
 namespace {
 
@@ -55,12 +97,20 @@ alphasparseStatus_t from_hip(hipError_t e)  // hip/util/handle.hip:19-51
     }
 }
 
-// Analysis results kept on the handle (its pflat_analysis_data slot).
+// What analysis keeps, per matrix.  The object sits behind matA->info: its first member is the
+// reference's _alphasparse_mat_info (include/alphasparse/handle.h:216-248), whose csrmv_info
+// points at the second (handle.h:158-198); the kernels' plans follow.  The matrix owns it
+// (alphasparseDestroySpMat releases it); the handle that made it lists it, so that
+// alphasparseSpMV_clear and the handle's destruction can release the device memory of callers
+// who, like the reference's, never destroy a descriptor.
 struct KeptPlan {
     bool spmm;
     int requested_alg;
+    // the arrays the plan was built from (the caller's, or a kept zero-based / transposed copy)
     const int *row_data;
-    int64_t rows, nnz;
+    const int *col_data;
+    const void *val_data;
+    int64_t rows, cols, nnz;
     int value_type;
     int ncols;
     asx_plan *plan;
@@ -76,44 +126,89 @@ struct DerivedCsr {
     int *row_ptr, *col;
     void *val;  // owned only when transposed (otherwise the caller's values)
 };
-struct HandlePlans {
+constexpr uint64_t kInfoMagic = 0x415358494e464f31ull;  // "ASXINFO1"
+struct MatInfoExt {
+    _alphasparse_mat_info info;
+    _alphasparse_csrmv_info csrmv;
+    uint64_t magic;
+    alphasparseHandle_t owner;  // null once that handle is gone
     std::vector<KeptPlan> plans;
     std::vector<DerivedCsr> derived;  // kept by alphasparseSpMV_analysis / alphasparseSpMM_preprocess
 };
-HandlePlans *plans_of(alphasparseHandle_t h, bool create)
+struct HandleRegistry {
+    std::vector<MatInfoExt *> mats;
+};
+HandleRegistry *registry_of(alphasparseHandle_t h, bool create)
 {
-    if (!h->pflat_analysis_data && create) h->pflat_analysis_data = new (std::nothrow) HandlePlans();
-    return (HandlePlans *)h->pflat_analysis_data;
+    if (!h->pflat_analysis_data && create) h->pflat_analysis_data = new (std::nothrow) HandleRegistry();
+    return (HandleRegistry *)h->pflat_analysis_data;
 }
-const asx_plan *find_plan(alphasparseHandle_t h, bool spmm, int alg, const _alphasparseSpMatDescr *A,
-                          int ncols)
+MatInfoExt *ext_of(const _alphasparseSpMatDescr *A)
 {
-    HandlePlans *hp = plans_of(h, false);
-    if (!hp) return nullptr;
-    for (const KeptPlan &k : hp->plans)
-        if (k.spmm == spmm && k.requested_alg == alg && k.row_data == A->row_data &&
-            k.rows == A->rows && k.nnz == A->nnz && k.value_type == (int)A->data_type &&
-            k.ncols == ncols)
-            return k.plan;
-    return nullptr;
+    MatInfoExt *e = (MatInfoExt *)A->info;
+    return e && e->magic == kInfoMagic ? e : nullptr;
+}
+// The matrix's store, made on first use (a foreign object already behind matA->info is left alone:
+// analysis then reports NOT_SUPPORTED).
+MatInfoExt *ext_create(alphasparseHandle_t h, _alphasparseSpMatDescr *A)
+{
+    if (MatInfoExt *e = ext_of(A)) {
+        if (!e->owner) {  // the handle that made it is gone: this one takes it over
+            HandleRegistry *reg = registry_of(h, true);
+            if (!reg) return nullptr;
+            reg->mats.push_back(e);
+            e->owner = h;
+        }
+        return e;
+    }
+    if (A->info) return nullptr;
+    HandleRegistry *reg = registry_of(h, true);
+    if (!reg) return nullptr;
+    MatInfoExt *e = new (std::nothrow) MatInfoExt();
+    if (!e) return nullptr;
+    e->info = _alphasparse_mat_info{};
+    e->csrmv = _alphasparse_csrmv_info{};
+    e->info.csrmv_info = &e->csrmv;
+    e->magic = kInfoMagic;
+    e->owner = h;
+    reg->mats.push_back(e);
+    A->info = &e->info;
+    return e;
 }
 void free_derived(DerivedCsr &d);
-void drop_plans(alphasparseHandle_t h, bool spmm, int alg, bool all)
+// Releases plans: those of one (kind, algorithm), or everything the matrix keeps.
+void ext_drop(MatInfoExt *e, bool spmm, int alg, bool all)
 {
-    HandlePlans *hp = plans_of(h, false);
-    if (!hp) return;
     std::vector<KeptPlan> keep;
-    for (KeptPlan &k : hp->plans) {
+    for (KeptPlan &k : e->plans) {
         if (all || (k.spmm == spmm && k.requested_alg == alg))
             asx_plan_destroy(k.plan);
         else
             keep.push_back(k);
     }
-    hp->plans.swap(keep);
+    e->plans.swap(keep);
     if (all) {
-        for (DerivedCsr &d : hp->derived) free_derived(d);
-        hp->derived.clear();
+        for (DerivedCsr &d : e->derived) free_derived(d);
+        e->derived.clear();
     }
+}
+asx_plan *find_plan(const _alphasparseSpMatDescr *owner, bool spmm, int alg, const _alphasparseSpMatDescr *A,
+                    int ncols)
+{
+    MatInfoExt *e = ext_of(owner);
+    if (!e) return nullptr;
+    for (const KeptPlan &k : e->plans)
+        if (k.spmm == spmm && k.requested_alg == alg && k.row_data == A->row_data && k.col_data == A->col_data &&
+            k.val_data == A->val_data && k.rows == A->rows && k.cols == A->cols && k.nnz == A->nnz &&
+            k.value_type == (int)A->data_type && k.ncols == ncols)
+            return k.plan;
+    return nullptr;
+}
+void drop_plans(alphasparseHandle_t h, bool spmm, int alg, bool all)
+{
+    HandleRegistry *reg = registry_of(h, false);
+    if (!reg) return;
+    for (MatInfoExt *e : reg->mats) ext_drop(e, spmm, alg, all);
 }
 
 bool is_transpose(alphasparseOperation_t op)
@@ -196,8 +291,8 @@ alphasparseStatus_t make_effective(alphasparseHandle_t h, const _alphasparseSpMa
     const bool tr = is_transpose(opA);
     if (!tr && A->idx_base == ALPHA_SPARSE_INDEX_BASE_ZERO) return ALPHA_SPARSE_STATUS_SUCCESS;
     const DerivedCsr *use = nullptr;
-    if (HandlePlans *hp = plans_of(h, false))
-        for (const DerivedCsr &d : hp->derived)
+    if (MatInfoExt *x = ext_of(A))
+        for (const DerivedCsr &d : x->derived)
             if (same_source(d, A, tr)) use = &d;
     if (!use) {
         alphasparseStatus_t s = build_derived(h, A, tr, &e->temp);
@@ -225,34 +320,33 @@ void release_effective(alphasparseHandle_t h, Effective *e)
 
 // Makes (or remakes, picking up changed values or structure) the kept derived copy for (A, opA);
 // plans built on the copy it replaces are dropped.
-alphasparseStatus_t keep_derived(alphasparseHandle_t h, const _alphasparseSpMatDescr *A,
-                                 alphasparseOperation_t opA)
+alphasparseStatus_t keep_derived(alphasparseHandle_t h, _alphasparseSpMatDescr *A, alphasparseOperation_t opA)
 {
     const bool tr = is_transpose(opA);
     if (!tr && A->idx_base == ALPHA_SPARSE_INDEX_BASE_ZERO) return ALPHA_SPARSE_STATUS_SUCCESS;
-    HandlePlans *hp = plans_of(h, true);
-    if (!hp) return ALPHA_SPARSE_STATUS_ALLOC_FAILED;
+    MatInfoExt *x = ext_create(h, A);
+    if (!x) return A->info ? ALPHA_SPARSE_STATUS_NOT_SUPPORTED : ALPHA_SPARSE_STATUS_ALLOC_FAILED;
     (void)hipStreamSynchronize(h->stream);
-    for (size_t i = 0; i < hp->derived.size();) {
-        if (!same_source(hp->derived[i], A, tr)) {
+    for (size_t i = 0; i < x->derived.size();) {
+        if (!same_source(x->derived[i], A, tr)) {
             ++i;
             continue;
         }
         std::vector<KeptPlan> keep;
-        for (KeptPlan &k : hp->plans) {
-            if (k.row_data == hp->derived[i].row_ptr)
+        for (KeptPlan &k : x->plans) {
+            if (k.row_data == x->derived[i].row_ptr)
                 asx_plan_destroy(k.plan);
             else
                 keep.push_back(k);
         }
-        hp->plans.swap(keep);
-        free_derived(hp->derived[i]);
-        hp->derived.erase(hp->derived.begin() + (long)i);
+        x->plans.swap(keep);
+        free_derived(x->derived[i]);
+        x->derived.erase(x->derived.begin() + (long)i);
     }
     DerivedCsr d{};
     alphasparseStatus_t s = build_derived(h, A, tr, &d);
     if (s) return s;
-    hp->derived.push_back(d);
+    x->derived.push_back(d);
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
@@ -423,8 +517,13 @@ alphasparseStatus_t alphasparseGetHandle(alphasparseHandle_t *handle)
 alphasparseStatus_t alphasparse_destory_handle(alphasparseHandle_t handle)
 {
     if (!handle) return ALPHA_SPARSE_STATUS_INVALID_HANDLE;
+    // the device memory of everything analysed through this handle goes with it; the (small)
+    // host objects stay with their matrices
     drop_plans(handle, false, 0, true);
-    delete (HandlePlans *)handle->pflat_analysis_data;
+    if (HandleRegistry *reg = registry_of(handle, false)) {
+        for (MatInfoExt *e : reg->mats) e->owner = nullptr;
+        delete reg;
+    }
     handle->pflat_analysis_data = nullptr;
     if (handle->buffer) (void)hipFree(handle->buffer);
     if (handle->sone) (void)hipFree(handle->sone);
@@ -512,6 +611,19 @@ alphasparseStatus_t alphasparseCreateCsrUntyped(alphasparseSpMatDescr_t *spMatDe
 alphasparseStatus_t alphasparseDestroySpMat(alphasparseSpMatDescr_t descr)
 {
     if (!descr) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+    if (MatInfoExt *e = ext_of(descr)) {
+        ext_drop(e, false, 0, true);
+        if (e->owner)
+            if (HandleRegistry *reg = registry_of(e->owner, false))
+                for (size_t i = 0; i < reg->mats.size(); ++i)
+                    if (reg->mats[i] == e) {
+                        reg->mats.erase(reg->mats.begin() + (long)i);
+                        break;
+                    }
+        e->magic = 0;
+        delete e;
+        descr->info = nullptr;
+    }
     delete descr->descr;
     delete descr;
     return ALPHA_SPARSE_STATUS_SUCCESS;
@@ -543,14 +655,9 @@ alphasparseStatus_t alphasparseSpMV_bufferSize(alphasparseHandle_t handle, alpha
     const int32_t m_eff = (int32_t)(is_transpose(opA) ? matA->cols : matA->rows);
     if (asx_spmv_resolve_alg((int)alg, m_eff, (int32_t)matA->nnz) < 0)
         return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
-    // sized for a call without kept analysis; a call with kept analysis needs no more than this
-    // (DEFAULT: including the column-panel kernel the analysis may pick for this matrix)
-    size_t need = asx_spmv_workspace_bytes((int)alg, (int)matA->data_type, m_eff, (int32_t)matA->nnz);
-    if (alg == ALPHA_SPARSE_SPMV_ALG_DEFAULT) {
-        const int32_t n_eff = (int32_t)(is_transpose(opA) ? matA->rows : matA->cols);
-        const size_t panel = asx_spmv_panel_workspace_bytes((int)matA->data_type, m_eff, n_eff, (int32_t)matA->nnz);
-        if (panel > need) need = panel;
-    }
+    // sized for a call without kept analysis, and for DEFAULT for every kernel a later
+    // alphasparseSpMV_analysis may settle on: a call with kept analysis needs no more than this
+    const size_t need = asx_spmv_workspace_bytes((int)alg, (int)matA->data_type, m_eff, (int32_t)matA->nnz);
     *bufferSize = need;
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
@@ -570,16 +677,28 @@ alphasparseStatus_t alphasparseSpMV_analysis(alphasparseHandle_t handle, alphasp
     s = make_effective(handle, matA, opA, &eff);
     if (s) return s;
     const _alphasparseSpMatDescr *A = &eff.d;
-    if (find_plan(handle, false, (int)alg, A, 1)) return ALPHA_SPARSE_STATUS_SUCCESS;
-    HandlePlans *hp = plans_of(handle, true);
-    if (!hp) return ALPHA_SPARSE_STATUS_ALLOC_FAILED;
+    if (asx_plan *have = find_plan(matA, false, (int)alg, A, 1)) {
+        // analysed before: the sparsity pattern is taken to be the same (alphasparseSpMV_clear first
+        // if it is not); a plan that holds a copy of the values picks up the current ones
+        return st(asx_plan_update_values(have, A->val_data, (void *)handle->stream));
+    }
+    MatInfoExt *x = ext_create(handle, matA);
+    if (!x) return matA->info ? ALPHA_SPARSE_STATUS_NOT_SUPPORTED : ALPHA_SPARSE_STATUS_ALLOC_FAILED;
     asx_plan *plan = nullptr;
-    // may keep a regrouped copy of A's columns and values (column panels): call again after
-    // changing them
+    // may keep a regrouped copy of A's columns and values (column slices): call again after
+    // changing the values
     int rc = asx_spmv_plan_create(&plan, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
                                   (int32_t)A->nnz, A->row_data, A->col_data, A->val_data, (void *)handle->stream);
     if (rc) return st(rc);
-    hp->plans.push_back(KeptPlan{false, (int)alg, A->row_data, A->rows, A->nnz, (int)A->data_type, 1, plan});
+    x->plans.push_back(KeptPlan{false, (int)alg, A->row_data, A->col_data, A->val_data, A->rows, A->cols, A->nnz,
+                                (int)A->data_type, 1, plan});
+    // the reference's own record of what was analysed (include/alphasparse/handle.h:190-197)
+    x->csrmv.trans = opA;
+    x->csrmv.m = (int)matA->rows;
+    x->csrmv.n = (int)matA->cols;
+    x->csrmv.nnz = (int)matA->nnz;
+    x->csrmv.csr_row_ptr = matA->row_data;
+    x->csrmv.csr_col_ind = matA->col_data;
     matA->analysed = true;
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
@@ -608,7 +727,7 @@ alphasparseStatus_t alphasparseSpMV(alphasparseHandle_t handle, alphasparseOpera
     if (s) return s;
     const _alphasparseSpMatDescr *A = &eff.d;
     const int32_t m = (int32_t)A->rows, n = (int32_t)A->cols, nnz = (int32_t)A->nnz;
-    const asx_plan *plan = find_plan(handle, false, (int)alg, A, 1);
+    const asx_plan *plan = find_plan(matA, false, (int)alg, A, 1);
     const size_t need = plan ? asx_plan_workspace_bytes(plan)
                              : asx_spmv_workspace_bytes((int)alg, (int)A->data_type, m, nnz);
     bool ok;
@@ -705,16 +824,21 @@ alphasparseStatus_t alphasparseSpMM_preprocess(alphasparseHandle_t handle, alpha
     s = make_effective(handle, matA, opA, &eff);
     if (s) return s;
     const _alphasparseSpMatDescr *A = &eff.d;
-    const asx_plan *have = find_plan(handle, true, (int)alg, A, ncols);
-    if (!have) {
-        HandlePlans *hp = plans_of(handle, true);
-        if (!hp) return ALPHA_SPARSE_STATUS_ALLOC_FAILED;
+    asx_plan *have = find_plan(matA, true, (int)alg, A, ncols);
+    if (have) {
+        // preprocessed before: a plan that holds a copy of A's values picks up the current ones
+        int rc = asx_plan_update_values(have, A->val_data, (void *)handle->stream);
+        if (rc) return st(rc);
+    } else {
+        MatInfoExt *x = ext_create(handle, matA);
+        if (!x) return matA->info ? ALPHA_SPARSE_STATUS_NOT_SUPPORTED : ALPHA_SPARSE_STATUS_ALLOC_FAILED;
         asx_plan *plan = nullptr;
         int rc = asx_spmm_plan_create(&plan, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
                                       (int32_t)A->nnz, A->row_data, A->col_data, A->val_data, ncols,
                                       (void *)handle->stream);
         if (rc) return st(rc);
-        hp->plans.push_back(KeptPlan{true, (int)alg, A->row_data, A->rows, A->nnz, (int)A->data_type, ncols, plan});
+        x->plans.push_back(KeptPlan{true, (int)alg, A->row_data, A->col_data, A->val_data, A->rows, A->cols, A->nnz,
+                                    (int)A->data_type, ncols, plan});
         have = plan;
         matA->analysed = true;
     }
@@ -744,7 +868,7 @@ alphasparseStatus_t alphasparseSpMM(alphasparseHandle_t handle, alphasparseOpera
     const _alphasparseSpMatDescr *A = &eff.d;
     const int32_t m = (int32_t)A->rows, k = (int32_t)A->cols, nnz = (int32_t)A->nnz;
     const int vt = (int)A->data_type;
-    const asx_plan *plan = find_plan(handle, true, (int)alg, A, ncols);
+    const asx_plan *plan = find_plan(matA, true, (int)alg, A, ncols);
     const size_t kernel_need =
         plan ? asx_plan_workspace_bytes(plan) : asx_spmm_workspace_bytes((int)alg, vt, m, nnz, ncols);
     size_t b_bytes, c_bytes;

@@ -11,6 +11,10 @@
 // blocks on the host through a dense ceil(M/16) x ceil(K/4) bitmap, keeps them in a global, and
 // multiplies with Hygon `mmac` builtins.  Here the blocks are built on the device by sorting
 // (block row, column quad) keys; they live in the plan.
+//
+// The zero fill of a block is multiplied with real rows of B: a non-finite value in a row of B
+// that some row of the block does not reference reaches that row of C as NaN (0 * Inf), where a
+// row-wise kernel would not have read it.  As for any padded block format, B must be finite.
 #include <hipcub/hipcub.hpp>
 
 #include "asx_internal.hpp"
@@ -49,12 +53,15 @@ __global__ __launch_bounds__(kBlock) void k_block_heads(const uint64_t *__restri
     head[i] = (i == 0 || (keys[i] >> 6) != (keys[i - 1] >> 6)) ? 1 : 0;
 }
 
-template <typename T>
-__global__ __launch_bounds__(kBlock) void k_block_fill(const uint64_t *__restrict__ keys,
-                                                       const int32_t *__restrict__ idx,
-                                                       const int32_t *__restrict__ block_of,
-                                                       const T *__restrict__ val, int32_t nnz,
-                                                       uint64_t *__restrict__ bkey, T *__restrict__ bval)
+// Where every stored element goes: upd_src[i] = its position in A's arrays, upd_dst[i] = its slot
+// in bval (lane order of the MFMA A operand), sign bit set when the element repeats the (row,
+// column) of the element before it (CSR may hold duplicates; they are summed, as every other
+// kernel here and the reference do).
+__global__ __launch_bounds__(kBlock) void k_block_slots(const uint64_t *__restrict__ keys,
+                                                        const int32_t *__restrict__ idx,
+                                                        const int32_t *__restrict__ block_of, int32_t nnz,
+                                                        uint64_t *__restrict__ bkey, int32_t *__restrict__ upd_src,
+                                                        int64_t *__restrict__ upd_dst)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= nnz) return;
@@ -62,7 +69,24 @@ __global__ __launch_bounds__(kBlock) void k_block_fill(const uint64_t *__restric
     const int64_t b = block_of[i] - 1;  // inclusive scan of the head flags
     if (i == 0 || (key >> 6) != (keys[i - 1] >> 6)) bkey[b] = key >> 6;
     const int r16 = (int)((key >> 2) & 15), c4 = (int)(key & 3);
-    bval[b * 64 + c4 * 16 + r16] = val[idx[i]];  // lane order of the MFMA A operand
+    const bool repeat = i > 0 && keys[i - 1] == key;
+    upd_src[i] = idx[i];
+    upd_dst[i] = (b * 64 + c4 * 16 + r16) | (repeat ? (int64_t)1 << 63 : 0);
+}
+
+// bval[slot] = sum of the values stored for that (row, column), in stored order
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_block_values(const int32_t *__restrict__ upd_src,
+                                                         const int64_t *__restrict__ upd_dst, int32_t nnz,
+                                                         const T *__restrict__ val, T *__restrict__ bval)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nnz) return;
+    const int64_t dst = upd_dst[i];
+    if (dst < 0) return;  // summed by the first element of its run
+    T sum = val[upd_src[i]];
+    for (int64_t j = i + 1; j < nnz && upd_dst[j] < 0; ++j) sum += val[upd_src[j]];
+    bval[dst] = sum;
 }
 
 __global__ __launch_bounds__(kBlock) void k_block_rows(const uint64_t *__restrict__ bkey, int32_t nblocks,
@@ -118,6 +142,9 @@ int build_blocked(int32_t m, int32_t k, int32_t nnz, const int32_t *row_ptr, con
     out->brow_ptr = nullptr;
     out->bcol = nullptr;
     out->bval = nullptr;
+    out->upd_src = nullptr;
+    out->upd_dst = nullptr;
+    out->nnz = nnz;
     const unsigned g_nnz = (unsigned)ceil_div64(nnz > 0 ? nnz : 1, kBlock);
     if (nnz > 0) {
         ASX_TRY(hipMalloc((void **)&keys, sizeof(uint64_t) * (size_t)nnz));
@@ -143,9 +170,13 @@ int build_blocked(int32_t m, int32_t k, int32_t nnz, const int32_t *row_ptr, con
     ASX_TRY(hipMalloc((void **)&out->bval, sizeof(T) * 64 * (size_t)(nblocks > 0 ? nblocks : 1)));
     ASX_TRY(hipMalloc((void **)&bkey, sizeof(uint64_t) * (size_t)(nblocks > 0 ? nblocks : 1)));
     if (nblocks > 0) {
+        ASX_TRY(hipMalloc((void **)&out->upd_src, sizeof(int32_t) * (size_t)nnz));
+        ASX_TRY(hipMalloc((void **)&out->upd_dst, sizeof(int64_t) * (size_t)nnz));
         hipLaunchKernelGGL((k_fill_zero<T>), dim3(4096), dim3(kBlock), 0, s, (T *)out->bval, (int64_t)nblocks * 64);
-        hipLaunchKernelGGL((k_block_fill<T>), dim3(g_nnz), dim3(kBlock), 0, s, keys2, idx2, block_of, val, nnz,
-                           bkey, (T *)out->bval);
+        hipLaunchKernelGGL(k_block_slots, dim3(g_nnz), dim3(kBlock), 0, s, keys2, idx2, block_of, nnz, bkey,
+                           out->upd_src, out->upd_dst);
+        hipLaunchKernelGGL((k_block_values<T>), dim3(g_nnz), dim3(kBlock), 0, s, out->upd_src, out->upd_dst, nnz, val,
+                           (T *)out->bval);
     }
     {
         const int64_t span = (int64_t)(nblocks > nbrows + 1 ? nblocks : nbrows + 1);
@@ -168,9 +199,23 @@ void free_blocked(BlockedMatrix *b)
     if (b->brow_ptr) (void)hipFree(b->brow_ptr);
     if (b->bcol) (void)hipFree(b->bcol);
     if (b->bval) (void)hipFree(b->bval);
+    if (b->upd_src) (void)hipFree(b->upd_src);
+    if (b->upd_dst) (void)hipFree(b->upd_dst);
     b->brow_ptr = nullptr;
     b->bcol = nullptr;
     b->bval = nullptr;
+    b->upd_src = nullptr;
+    b->upd_dst = nullptr;
+}
+
+// Refreshes the blocks' values from A's (same sparsity pattern); the zero fill is untouched.
+template <typename T>
+int blocked_update_values(const BlockedMatrix *bm, const T *val, hipStream_t s)
+{
+    if (bm->nblocks <= 0 || bm->nnz <= 0) return ASX_STATUS_SUCCESS;
+    hipLaunchKernelGGL((k_block_values<T>), dim3((unsigned)ceil_div64(bm->nnz, kBlock)), dim3(kBlock), 0, s, bm->upd_src,
+                       bm->upd_dst, bm->nnz, val, (T *)bm->bval);
+    return check_launch();
 }
 
 // ---- MFMA wrappers: A 16x4 (lane l: row l%16, k l/16), B 4x16 (lane l: k l/16, col l%16),
@@ -258,6 +303,8 @@ template int build_blocked<float>(int32_t, int32_t, int32_t, const int32_t *, co
                                   BlockedMatrix *, hipStream_t);
 template int build_blocked<double>(int32_t, int32_t, int32_t, const int32_t *, const int32_t *, const double *,
                                    BlockedMatrix *, hipStream_t);
+template int blocked_update_values<float>(const BlockedMatrix *, const float *, hipStream_t);
+template int blocked_update_values<double>(const BlockedMatrix *, const double *, hipStream_t);
 template int launch_spmm_blocked<float>(int32_t, int32_t, int32_t, float, const BlockedMatrix *, const float *,
                                         int64_t, float, float *, int64_t, hipStream_t);
 template int launch_spmm_blocked<double>(int32_t, int32_t, int32_t, double, const BlockedMatrix *, const double *,

@@ -3,11 +3,11 @@
 // point launches HIP kernels or returns an error status.
 #include <algorithm>
 #include <cmath>
-#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <vector>
 
+#include "../../include/alphasparse_amd_bench.h"
 #include "asx_internal.hpp"
 
 using namespace asx;
@@ -78,36 +78,10 @@ SpmmLayout spmm_merge_layout(int32_t m, int32_t nnz, int32_t ncols, size_t sv, b
     return L;
 }
 
-struct PanelLayout {  // [partial | carry]
-    size_t partial_off, carry_off, bytes;
-};
-PanelLayout spmv_panel_layout(size_t partial_sums, size_t total_tiles, size_t sv)
-{
-    PanelLayout L{};
-    L.partial_off = 0;
-    L.carry_off = align_up(std::max<size_t>(partial_sums, 1) * sv, kAlign);
-    L.bytes = L.carry_off + align_up(std::max<size_t>(total_tiles, 1) * sv, kAlign);
-    return L;
-}
-
-// Panels can pay when x is too large for one 4 MiB L2 and its slices are at most two L2s large
-// (x of 128 MiB in 32 slices of 4 MiB still measured 1.5x faster than the flat kernel).
-constexpr size_t kL2Bytes = (size_t)4 << 20;
-bool panel_candidate(int32_t m, int32_t n, int32_t nnz, size_t sv)
-{
-    const size_t xbytes = (size_t)n * sv;
-    return m > 0 && nnz >= (1 << 22) && xbytes > kL2Bytes + kL2Bytes / 2 && xbytes <= 2 * kPanels * kL2Bytes;
-}
-// 16 panels while that keeps the slices within one L2 (fewer partial sums per row), else 32.
-int32_t panels_for(int32_t n, size_t sv)
-{
-    return (size_t)n * sv <= 16 * kL2Bytes ? 16 : kPanels;
-}
-
 // How scattered the columns are: the number of distinct 128-byte lines of x that the columns of a
 // tile of 1024 consecutive stored elements touch, divided by 1024, averaged over up to 64 tiles
 // spread over the matrix (copied to the host; 256 KiB).  Random columns give about 1, a 5-point
-// stencil 0.04, a band matrix 0.01.  Panels are only worth building for scattered columns.
+// stencil 0.04, a band matrix 0.01.  Regrouping by column slice only pays for scattered columns.
 double sampled_line_spread(const int32_t *d_col, int32_t nnz, size_t sv, hipStream_t s)
 {
     const int64_t tiles = nnz / kFlatTile;
@@ -130,7 +104,7 @@ double sampled_line_spread(const int32_t *d_col, int32_t nnz, size_t sv, hipStre
     }
     return (double)distinct / ((double)samples * kFlatTile);
 }
-constexpr double kPanelMinSpread = 0.5;
+constexpr double kScatteredMinSpread = 0.5;
 
 constexpr int32_t kSmallNnz = 1 << 18;
 constexpr int64_t kSmallMaxRow = 2048;
@@ -221,24 +195,12 @@ int spmv_impl(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, 
         return launch_spmv_flat<T>(m, nnz, alpha, row_ptr, col, val, x, beta, y, seg, (T *)(w + L.carry_off),
                                    plan ? plan->carry_pass != 0 : true, s);
     }
-    case ASX_SPMV_PANEL: {
-        // the panels hold a copy of A's columns and values and are built by asx_spmv_plan_create
-        if (!plan || !plan->panel.col) return ASX_STATUS_NOT_INITIALIZED;
-        const PanelLayout L = spmv_panel_layout((size_t)plan->panel.kbase[kPanels], (size_t)plan->panel.tile_off[kPanels], sizeof(T));
-        if (!ws) return ASX_STATUS_INVALID_POINTER;
-        if (ws_bytes < L.bytes) return ASX_STATUS_INVALID_SIZE;
-        return launch_spmv_panel<T>(m, alpha, &plan->panel, x, beta, y, (T *)(w + L.partial_off),
-                                    (T *)(w + L.carry_off), s);
-    }
-    case ASX_SPMV_SLICED: {
-        // the slices hold a copy of A's columns and values and are built by asx_spmv_plan_create
+    case ASX_SPMV_SLICED:
+        // the slices hold a copy of A's columns and values (and the partial sums of a call) and are
+        // built by asx_spmv_plan_create; no workspace
         if (!plan || !plan->sliced.cf) return ASX_STATUS_NOT_INITIALIZED;
         if (plan->n != n) return ASX_STATUS_INVALID_VALUE;
-        const size_t need = align_up(((size_t)plan->sliced.npartials + kWave) * sizeof(T), kAlign);
-        if (!ws) return ASX_STATUS_INVALID_POINTER;
-        if (ws_bytes < need) return ASX_STATUS_INVALID_SIZE;
-        return launch_spmv_sliced<T>(m, n, alpha, &plan->sliced, x, beta, y, (T *)w, s);
-    }
+        return launch_spmv_sliced<T>(m, n, alpha, &plan->sliced, x, beta, y, s);
     default: return ASX_STATUS_NOT_SUPPORTED;
     }
 }
@@ -511,7 +473,6 @@ int asx_plan_destroy(asx_plan *plan)
     int st = ASX_STATUS_SUCCESS;
     if (plan->d_meta) st = status_of(hipFree(plan->d_meta));
     free_blocked(&plan->blocked);
-    free_panels(&plan->panel);
     free_sliced(&plan->sliced);
     delete plan;
     return st;
@@ -535,7 +496,7 @@ int asx_spmm_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     // 128-byte lines) cannot fill 16x4 blocks: the blocks are not even built then
     const bool probe_blocked = alg == ASX_SPMM_DEFAULT && nnz > 0 && nnz <= kBlockedProbeMaxNnz && d_col &&
                                (value_type == ASX_R_32F || value_type == ASX_R_64F) &&
-                               sampled_line_spread(d_col, nnz, vsize(value_type), (hipStream_t)stream) < kPanelMinSpread;
+                               sampled_line_spread(d_col, nnz, vsize(value_type), (hipStream_t)stream) < kScatteredMinSpread;
     if (!want_blocked && !probe_blocked)
         return asx_plan_create(out, 1, alg, value_type, m, k, nnz, d_row_ptr, ncols, stream);
     if (m < 0 || k < 0 || nnz < 0 || ncols < 1) return ASX_STATUS_INVALID_SIZE;
@@ -575,138 +536,69 @@ int asx_spmm_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
 
 }  // extern "C"
 
-// Average time of one call through `plan` on scratch vectors (x = 0), in milliseconds; < 0 on error.
-template <typename T>
-static float time_plan(const asx_plan *plan, const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val,
-                       const T *d_x, T *d_y, void *d_ws, size_t ws_bytes, hipStream_t s)
+// ---- the column-sliced kernel as DEFAULT's choice ------------------------------------------
+// Decided from figures that do not change from one plan build to the next: the row-length
+// histogram, the sizes, and the column sample.  Model (fitted to measurements on MI355X):
+//   row-ordered kernels   t = nnz / g(x bytes), g = 180 G gathers/s while x fits an L2 (<= 3 MiB),
+//                         62 G/s once it does not (>= 6 MiB), linear in between, and never less
+//                         than their bytes at 5 TB/s;
+//   column-sliced kernel  t = 12 us + bytes / 4.7 TB/s with
+//                         bytes = nnz (sv + 2) + P (2 sv + 2) + n sv + 2 m sv,
+//                         P = expected number of (row, slice) pairs = sum over rows of
+//                         S (1 - (1 - 1/S)^len), S = number of slices, from the histogram.
+// Sliced is chosen when its estimate is at least 10 % lower.
+constexpr int32_t kSlicedMinNnz = 1 << 21;
+constexpr int32_t kSliceBytes = 131072;  // of x per slice: one workgroup of 16 waves per compute unit
+double sliced_expected_partials(const int64_t hist[33], int32_t nslices)
 {
-    hipEvent_t e0, e1;
-    if (hipEventCreate(&e0) != hipSuccess) return -1.0f;
-    if (hipEventCreate(&e1) != hipSuccess) {
-        (void)hipEventDestroy(e0);
-        return -1.0f;
+    double p = 0.0;
+    const double q = nslices > 1 ? std::log1p(-1.0 / (double)nslices) : 0.0;
+    for (int b = 1; b <= 32; ++b) {
+        if (!hist[b]) continue;
+        const double len = b == 1 ? 1.0 : 0.75 * std::ldexp(1.0, b);  // middle of [2^(b-1), 2^b)
+        p += (double)hist[b] * (nslices > 1 ? (double)nslices * -std::expm1(len * q) : 1.0);
     }
-    float ms = -1.0f;
-    int st = spmv_impl<T>(plan, plan->alg, plan->m, plan->n, plan->nnz, T(1), d_row_ptr, d_col, d_val, d_x, T(0), d_y,
-                          d_ws, ws_bytes, s);  // warm-up
-    if (!st) st = status_of(hipEventRecord(e0, s));
-    for (int i = 0; i < 3 && !st; ++i)
-        st = spmv_impl<T>(plan, plan->alg, plan->m, plan->n, plan->nnz, T(1), d_row_ptr, d_col, d_val, d_x, T(0), d_y,
-                          d_ws, ws_bytes, s);
-    if (!st) st = status_of(hipEventRecord(e1, s));
-    if (!st) st = status_of(hipEventSynchronize(e1));
-    if (!st && hipEventElapsedTime(&ms, e0, e1) == hipSuccess)
-        ms /= 3.0f;
-    else
-        ms = -1.0f;
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
-    return ms;
+    return p;
+}
+bool sliced_pays(const int64_t hist[33], int32_t m, int32_t n, int32_t nnz, size_t sv)
+{
+    if (nnz < kSlicedMinNnz || m <= 0 || n <= 0) return false;
+    const double xbytes = (double)n * (double)sv;
+    const double lo = 3.0 * 1048576.0, hi = 6.0 * 1048576.0;
+    const double f = xbytes <= lo ? 0.0 : xbytes >= hi ? 1.0 : (xbytes - lo) / (hi - lo);
+    const double gather_rate = 180e9 + f * (62e9 - 180e9);
+    const double row_bytes = (double)nnz * (sv + 4) + (double)n * sv + (double)m * (sv + 4);
+    const double t_rows = std::max((double)nnz / gather_rate, row_bytes / 5e12);
+    const int32_t nslices = (int32_t)ceil_div64((int64_t)n * (int64_t)sv, kSliceBytes);
+    const double partials = sliced_expected_partials(hist, nslices);
+    const double sl_bytes = (double)nnz * (sv + 2) + partials * (2.0 * sv + 2) + (double)n * sv + 2.0 * (double)m * sv;
+    const double t_sliced = 12e-6 + sl_bytes / 4.7e12;
+    return t_sliced < 0.9 * t_rows;
 }
 
+// Builds the sliced copy onto a plan that already holds the histogram (`p` takes the slices over;
+// its own split points are dropped).
 template <typename T>
-static int spmv_plan_with_panels(asx_plan **out, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
-                                 const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, hipStream_t s)
+int plan_add_slices(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, hipStream_t s)
 {
-    // the plan the histogram picks: the fallback, and for DEFAULT the opponent of the timing
-    asx_plan *base = nullptr;
-    int st = asx_plan_create(&base, 0, alg == ASX_SPMV_PANEL ? ASX_SPMV_DEFAULT : alg, value_type, m, n, nnz, d_row_ptr,
-                             1, (void *)s);
-    if (st) return st;
-    asx_plan *pp = new (std::nothrow) asx_plan();
-    if (!pp) {
-        asx_plan_destroy(base);
-        return ASX_STATUS_ALLOC_FAILED;
-    }
-    *pp = *base;  // histogram, sizes
-    pp->d_meta = nullptr;
-    pp->meta_bytes = 0;
-    pp->alg = ASX_SPMV_PANEL;
-    pp->panel = PanelMatrix{};
-    st = build_panels<T>(m, n, nnz, panels_for(n, sizeof(T)), d_row_ptr, d_col, d_val, &pp->panel, s);
-    if (st) {
-        delete pp;
-        if (alg == ASX_SPMV_PANEL) {
-            asx_plan_destroy(base);
-            return st;
-        }
-        *out = base;  // DEFAULT: no panels (out of memory, ...) is not an error
-        return ASX_STATUS_SUCCESS;
-    }
-    pp->nunits = pp->panel.tile_off[kPanels];
-    pp->carry_pass = pp->panel.carry_pass;
-    pp->workspace_bytes =
-        spmv_panel_layout((size_t)pp->panel.kbase[kPanels], (size_t)pp->panel.tile_off[kPanels], sizeof(T)).bytes;
-    if (alg == ASX_SPMV_PANEL) {
-        asx_plan_destroy(base);
-        *out = pp;
-        return ASX_STATUS_SUCCESS;
-    }
-    // DEFAULT: keep the faster of the two on this matrix
-    const size_t ws_bytes = std::max(pp->workspace_bytes, base->workspace_bytes);
-    T *d_x = nullptr, *d_y = nullptr;
-    void *d_ws = nullptr;
-    bool panel_wins = false;
-    if (hipMalloc((void **)&d_x, sizeof(T) * (size_t)n) == hipSuccess &&
-        hipMalloc((void **)&d_y, sizeof(T) * (size_t)m) == hipSuccess &&
-        hipMalloc(&d_ws, ws_bytes ? ws_bytes : 1) == hipSuccess &&
-        hipMemsetAsync(d_x, 0, sizeof(T) * (size_t)n, s) == hipSuccess) {
-        const float t_base = time_plan<T>(base, d_row_ptr, d_col, d_val, d_x, d_y, d_ws, ws_bytes, s);
-        const float t_panel = time_plan<T>(pp, d_row_ptr, d_col, d_val, d_x, d_y, d_ws, ws_bytes, s);
-        panel_wins = t_base > 0 && t_panel > 0 && t_panel < 0.9f * t_base;
-    }
-    (void)hipStreamSynchronize(s);
-    for (void *q : {(void *)d_x, (void *)d_y, d_ws})
-        if (q) (void)hipFree(q);
-    if (panel_wins) {
-        asx_plan_destroy(base);
-        *out = pp;
-    } else {
-        asx_plan_destroy(pp);
-        *out = base;
-    }
-    return ASX_STATUS_SUCCESS;
-}
-
-// Slice width: 128 KiB of x per slice (one workgroup of 16 waves per compute unit).
-template <typename T>
-static int spmv_plan_sliced(asx_plan **out, int value_type, int32_t m, int32_t n, int32_t nnz,
-                            const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, hipStream_t s)
-{
-    asx_plan *base = nullptr;  // histogram and sizes
-    int st = asx_plan_create(&base, 0, ASX_SPMV_VECTOR, value_type, m, n, nnz, d_row_ptr, 1, (void *)s);
-    if (st) return st;
-    asx_plan *p = new (std::nothrow) asx_plan();
-    if (!p) {
-        asx_plan_destroy(base);
-        return ASX_STATUS_ALLOC_FAILED;
-    }
-    *p = *base;
-    asx_plan_destroy(base);
-    p->d_meta = nullptr;
-    p->meta_bytes = 0;
-    p->alg = ASX_SPMV_SLICED;
-    p->sliced = SlicedMatrix{};
     int cus = 256;
     (void)asx_device_info(&cus, nullptr);
-    int32_t slice_bytes = 131072;
-    if (const char *e = std::getenv("ASX_SLICE_BYTES")) slice_bytes = std::atoi(e);
-    int32_t target = cus * (131072 / slice_bytes);
-    if (const char *e = std::getenv("ASX_SLICE_WGS")) target = std::atoi(e);
     // pass 2: one wave per block of rows; at least 8 waves per compute unit where m allows, at most
     // 16 KiB of accumulators per wave
     int32_t rpw = 256;
-    while (rpw < (int32_t)(16384 / sizeof(T)) && (int64_t)rpw * cus * 8 < m) rpw *= 2;
-    if (const char *e = std::getenv("ASX_SLICE_RPW")) rpw = std::atoi(e);
-    st = build_sliced<T>(m, n, nnz, (int32_t)(slice_bytes / sizeof(T)), rpw, target, d_row_ptr, d_col, d_val,
-                         &p->sliced, s);
-    if (st) {
-        delete p;
-        return st;
-    }
-    p->nunits = p->sliced.ntiles;
-    p->workspace_bytes = align_up(((size_t)p->sliced.npartials + kWave) * sizeof(T), kAlign);
-    *out = p;
+    while (rpw < (int32_t)(16384 / sizeof(T)) && (int64_t)rpw * cus * 8 < p->m) rpw *= 2;
+    SlicedMatrix sm{};
+    const int st = build_sliced<T>(p->m, p->n, p->nnz, (int32_t)(kSliceBytes / sizeof(T)), rpw, cus, d_row_ptr, d_col,
+                                   d_val, &sm, s);
+    if (st) return st;
+    if (p->d_meta) (void)hipFree(p->d_meta);
+    p->d_meta = nullptr;
+    p->meta_bytes = 0;
+    p->alg = ASX_SPMV_SLICED;
+    p->sliced = sm;
+    p->nunits = sm.ntiles;
+    p->carry_pass = 0;
+    p->workspace_bytes = 0;
     return ASX_STATUS_SUCCESS;
 }
 
@@ -719,38 +611,48 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     *out = nullptr;
     if (m < 0 || n < 0 || nnz < 0) return ASX_STATUS_INVALID_SIZE;
     if (value_type != ASX_R_32F && value_type != ASX_R_64F) return ASX_STATUS_NOT_SUPPORTED;
-    if (alg == ASX_SPMV_SLICED) {
-        if (m == 0 || nnz == 0 || n == 0) return ASX_STATUS_INVALID_SIZE;
-        if (!d_row_ptr || !d_col || !d_val) return ASX_STATUS_INVALID_POINTER;
-        if (value_type == ASX_R_64F)
-            return spmv_plan_sliced<double>(out, value_type, m, n, nnz, d_row_ptr, d_col, (const double *)d_val,
-                                            (hipStream_t)stream);
-        return spmv_plan_sliced<float>(out, value_type, m, n, nnz, d_row_ptr, d_col, (const float *)d_val,
-                                       (hipStream_t)stream);
-    }
-    const bool want = alg == ASX_SPMV_PANEL;
-    const bool candidate = alg == ASX_SPMV_DEFAULT && d_col && d_val &&
-                           panel_candidate(m, n, nnz, vsize(value_type)) &&
-                           sampled_line_spread(d_col, nnz, vsize(value_type), (hipStream_t)stream) >= kPanelMinSpread;
+    const bool want = alg == ASX_SPMV_SLICED;
     if (want && (m == 0 || nnz == 0 || n == 0)) return ASX_STATUS_INVALID_SIZE;
     if (want && (!d_row_ptr || !d_col || !d_val)) return ASX_STATUS_INVALID_POINTER;
-    if (!want && !(alg == ASX_SPMV_DEFAULT && candidate))
-        return asx_plan_create(out, 0, alg, value_type, m, n, nnz, d_row_ptr, 1, stream);
-    if (value_type == ASX_R_64F)
-        return spmv_plan_with_panels<double>(out, alg, value_type, m, n, nnz, d_row_ptr, d_col, (const double *)d_val,
-                                             (hipStream_t)stream);
-    return spmv_plan_with_panels<float>(out, alg, value_type, m, n, nnz, d_row_ptr, d_col, (const float *)d_val,
-                                        (hipStream_t)stream);
+    hipStream_t s = (hipStream_t)stream;
+    // histogram, sizes and (for DEFAULT) the row-ordered kernel the histogram picks
+    asx_plan *p = nullptr;
+    int st = asx_plan_create(&p, 0, want ? ASX_SPMV_VECTOR : alg, value_type, m, n, nnz, d_row_ptr, 1, stream);
+    if (st) return st;
+    bool slices = want;
+    if (alg == ASX_SPMV_DEFAULT && d_col && d_val && sliced_pays(p->hist, m, n, nnz, vsize(value_type)))
+        slices = sampled_line_spread(d_col, nnz, vsize(value_type), s) >= kScatteredMinSpread;
+    if (slices) {
+        st = value_type == ASX_R_64F ? plan_add_slices<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
+                                     : plan_add_slices<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
+        if (st && want) {
+            asx_plan_destroy(p);
+            return st;
+        }
+        // DEFAULT: no slices (out of memory, ...) is not an error; the row-ordered plan stands
+    }
+    *out = p;
+    return ASX_STATUS_SUCCESS;
 }
 
-size_t asx_spmv_panel_workspace_bytes(int value_type, int32_t m, int32_t n, int32_t nnz)
+int asx_plan_update_values(asx_plan *plan, const void *d_val, void *stream)
 {
-    if (m <= 0 || n <= 0 || nnz <= 0) return 0;
-    const size_t sv = vsize(value_type);
-    if (!panel_candidate(m, n, nnz, sv)) return 0;
-    // a row leaves at most one partial sum per panel and no more than it has stored elements
-    const size_t partial_sums = std::min<size_t>((size_t)nnz, (size_t)kPanels * (size_t)m);
-    return spmv_panel_layout(partial_sums, (size_t)ceil_div64(nnz, kFlatTile) + kPanels, sv).bytes;
+    if (!plan) return ASX_STATUS_INVALID_POINTER;
+    if (plan->nnz > 0 && !d_val) return ASX_STATUS_INVALID_POINTER;
+    hipStream_t s = (hipStream_t)stream;
+    if (!plan->is_spmm && plan->alg == ASX_SPMV_SLICED)
+        return plan->value_type == ASX_R_64F ? sliced_update_values<double>(&plan->sliced, (const double *)d_val, s)
+                                             : sliced_update_values<float>(&plan->sliced, (const float *)d_val, s);
+    if (plan->is_spmm && plan->alg == ASX_SPMM_BLOCKED)
+        return plan->value_type == ASX_R_64F ? blocked_update_values<double>(&plan->blocked, (const double *)d_val, s)
+                                             : blocked_update_values<float>(&plan->blocked, (const float *)d_val, s);
+    return ASX_STATUS_SUCCESS;  // the other kernels read the caller's values in every call
+}
+
+int asx_plan_holds_values(const asx_plan *plan)
+{
+    if (!plan) return 0;
+    return (!plan->is_spmm && plan->alg == ASX_SPMV_SLICED) || (plan->is_spmm && plan->alg == ASX_SPMM_BLOCKED);
 }
 
 int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill)
@@ -807,8 +709,13 @@ int asx_spmv_resolve_alg(int alg, int32_t m, int32_t nnz)
 size_t asx_spmv_workspace_bytes(int alg, int value_type, int32_t m, int32_t nnz)
 {
     const int kernel = asx_spmv_resolve_alg(alg, m, nnz);
-    if (kernel == ASX_SPMV_MERGE) return spmv_merge_layout(m, nnz, vsize(value_type), true).bytes;
-    if (kernel == ASX_SPMV_FLAT) return spmv_flat_layout(nnz, vsize(value_type), true).bytes;
+    const size_t merge = spmv_merge_layout(m, nnz, vsize(value_type), true).bytes;
+    const size_t flat = spmv_flat_layout(nnz, vsize(value_type), true).bytes;
+    // DEFAULT: a plan may pick the merge-path kernel (hypersparse or very long rows), whose carry
+    // array can exceed the flat kernel's: report what every choice fits in
+    if (alg == ASX_SPMV_DEFAULT) return std::max(merge, flat);
+    if (kernel == ASX_SPMV_MERGE) return merge;
+    if (kernel == ASX_SPMV_FLAT) return flat;
     if (kernel == ASX_SPMV_STREAM)
         return align_up(((size_t)std::max(stream_blocks(nnz), 1) + 1) * 8, kAlign);
     return 0;

@@ -93,53 +93,21 @@ struct BlockedMatrix {
     int32_t *brow_ptr;  // nbrows + 1
     int32_t *bcol;      // column quad of each block
     void *bval;         // nblocks * 64 values, lane order of the MFMA A operand
+    int32_t nnz;        // stored elements of A
+    int32_t *upd_src;   // nnz: position in A's values of every stored element, in block order
+    int64_t *upd_dst;   // nnz: its slot in bval; sign bit = repeats the (row, column) before it
 };
 template <typename T>
 int build_blocked(int32_t m, int32_t k, int32_t nnz, const int32_t *row_ptr, const int32_t *col,
                   const T *val, BlockedMatrix *out, hipStream_t s);
 void free_blocked(BlockedMatrix *b);
 template <typename T>
+int blocked_update_values(const BlockedMatrix *bm, const T *val, hipStream_t s);
+template <typename T>
 int launch_spmm_blocked(int32_t m, int32_t k, int32_t ncols, T alpha, const BlockedMatrix *bm, const T *B,
                         int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t s);
 
-// ---- column-panel SpMV (asx_panel.hip builds, asx_spmv.hip runs) ----
-// The stored elements regrouped into kPanels column panels (panel = col / width).  Each panel is
-// a CSR matrix over the rows that have elements in it (rows without any are left out: with short
-// rows most panels miss most rows).  Workgroup b runs on XCD b % kXcds (consecutive workgroups
-// go to consecutive XCDs) and works on panel b % kXcds first and then, when that panel's tiles
-// are used up, on panel b % kXcds + kXcds, ...: at any time an XCD's L2 sees one panel's slice
-// of x (workgroups are dispatched in order, so the phases of one XCD barely overlap).
-// A panel writes one partial sum per row it holds.  `rowid` names the row of A of every partial
-// sum; `blk_lo` says, for every block of kPanelRowBlock rows of A, where in each panel's partial
-// sums the block's rows start, so the reduction reads contiguous ranges.
-constexpr int kXcds = 8;
-constexpr int kPanelPhases = 4;  // at most; a matrix uses 2 phases while its slices of x stay small
-constexpr int kPanels = kXcds * kPanelPhases;
-constexpr int kPanelRowBlock = 1024;  // rows of A per workgroup of the reduction
-struct PanelMatrix {
-    int32_t npanels;                // panels in use (a multiple of kXcds, <= kPanels); the rest are empty
-    int32_t width;                  // columns per panel
-    int32_t count[kPanels];         // stored elements per panel
-    int64_t elem_off[kPanels + 1];  // start of each panel in col / val (multiples of 4 elements)
-    int32_t tile_off[kPanels + 1];  // start of each panel's tiles in the carry array
-    int32_t krows[kPanels];         // rows present in each panel
-    int32_t kbase[kPanels + 1];     // start of each panel in the partial-sum array
-    int32_t max_tiles;              // largest number of tiles one XCD works through
-    int32_t *col;       // device
-    void *val;          // device, a copy of A's values in panel order
-    int32_t *row_ptr;   // device, panel j at kbase[j] + j, krows[j] + 1 entries
-    int32_t *seg_row;   // device, panel j at tile_off[j] + j, tiles_j + 1 entries
-    int32_t *rowid;     // device, kbase[kPanels]: row of A of each partial sum
-    int32_t *blk_lo;    // device, (ceil(m / kPanelRowBlock) + 1) x kPanels
-    int carry_pass;
-};
-template <typename T>
-int build_panels(int32_t m, int32_t n, int32_t nnz, int32_t npanels, const int32_t *row_ptr, const int32_t *col,
-                 const T *val, PanelMatrix *out, hipStream_t s);
-void free_panels(PanelMatrix *p);
-template <typename T>
-int launch_spmv_panel(int32_t m, T alpha, const PanelMatrix *pm, const T *x, T beta, T *y, T *partial, T *carry,
-                      hipStream_t s);
+constexpr int kXcds = 8;  // workgroups are dealt to the 8 XCDs round-robin (workgroup b runs on XCD b % 8)
 // out[r] = first i with sorted[i] >= r, r in [0, n]
 int launch_offsets_from_sorted(const int32_t *sorted, int32_t count, int32_t n, int32_t *out, hipStream_t s);
 
@@ -162,6 +130,7 @@ struct SlicedMatrix {
     int32_t rows_per_wave;  // pass 2
     int32_t nrb;            // ceil(m / rows_per_wave)
     void *val;              // ntiles * kSlicedTile values (a copy of A's, in slice order; pads are 0)
+    void *partial;          // npartials (+ 64 readable) values: the partial sums of one call
     uint16_t *cf;           // ntiles * kSlicedTile: column inside the slice, bit 15 = first element of a run
     int32_t *perm;          // where each stored copy comes from in A's val (-1 for pads)
     int32_t *tile_base;     // ntiles + 1: index of the first partial sum of each tile
@@ -176,8 +145,7 @@ void free_sliced(SlicedMatrix *p);
 template <typename T>
 int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s);
 template <typename T>
-int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, T *partial,
-                       hipStream_t s);
+int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, hipStream_t s);
 
 inline int32_t merge_tiles(int32_t m, int32_t nnz) { return (int32_t)ceil_div64((int64_t)m + nnz, kMergeTile); }
 inline int32_t flat_tiles(int32_t nnz) { int32_t t = (int32_t)ceil_div64(nnz, kFlatTile); return t < 1 ? 1 : t; }
@@ -201,6 +169,5 @@ struct asx_plan {
     int64_t stats[4];
     size_t workspace_bytes;
     asx::BlockedMatrix blocked;  // only for ASX_SPMM_BLOCKED plans
-    asx::PanelMatrix panel;      // only for ASX_SPMV_PANEL plans
     asx::SlicedMatrix sliced;    // only for ASX_SPMV_SLICED plans
 };

@@ -27,7 +27,6 @@
 #include <hipcub/hipcub.hpp>
 
 #include <algorithm>
-#include <cstdlib>
 #include <vector>
 
 #include "asx_internal.hpp"
@@ -269,6 +268,13 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const 
     const int4 wg = wg_tab[blockIdx.x];
     const int64_t c0 = (int64_t)wg.x * WIDTH;
     const int32_t cnt = n - c0 < WIDTH ? (int32_t)(n - c0) : WIDTH;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    // the first tiles' loads go out before the slice of x is fetched (they do not need it)
+    const int32_t last = wg.z - 1;
+    SlicedTile<T> tl[D];
+    int32_t t = wg.y + wave;
+#pragma unroll
+    for (int d = 0; d < D; ++d) sliced_tile_load<T>(tl[d], t + d * NW < last ? t + d * NW : last, lane, cf, val, tile_base);
     {
         // the slice of x: every load issued before the first LDS write (one memory round trip)
         constexpr int V = 16 / sizeof(T);                 // values per 16-byte load
@@ -293,16 +299,10 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const 
         for (int k = 0; k < PER; ++k) reinterpret_cast<vec_t *>(xs)[k * NW * kWave + threadIdx.x] = buf[k];
     }
     __syncthreads();
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     // D tiles in turn; a tile's loads are issued D steps ahead, right after the stores of the tile
     // that used the buffer before it.  The loads are unconditional (past the end they re-read the
     // last tile), so that the number of memory operations issued after them is known and a step
     // waits for its own loads only.
-    const int32_t last = wg.z - 1;
-    SlicedTile<T> tl[D];
-    int32_t t = wg.y + wave;
-#pragma unroll
-    for (int d = 0; d < D; ++d) sliced_tile_load<T>(tl[d], t + d * NW < last ? t + d * NW : last, lane, cf, val, tile_base);
     while (t < wg.z) {  // uniform over the wave
 #pragma unroll
         for (int d = 0; d < D; ++d) {
@@ -462,10 +462,10 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_reduce(int32_t m, int32_t 
 
 void free_sliced(SlicedMatrix *p)
 {
-    for (void *q : {p->val, (void *)p->cf, (void *)p->perm, (void *)p->tile_base, (void *)p->wg_tab, (void *)p->prow,
-                    (void *)p->chunk_lo})
+    for (void *q : {p->val, p->partial, (void *)p->cf, (void *)p->perm, (void *)p->tile_base, (void *)p->wg_tab,
+                    (void *)p->prow, (void *)p->chunk_lo})
         if (q) (void)hipFree(q);
-    p->val = nullptr;
+    p->val = p->partial = nullptr;
     p->cf = p->prow = nullptr;
     p->perm = p->tile_base = p->wg_tab = p->chunk_lo = nullptr;
 }
@@ -556,6 +556,8 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
         ASX_TRY(hipMalloc((void **)&sm.prow, sizeof(uint16_t) * ((size_t)sm.npartials + kWave)));
         ASX_TRY(hipMemsetAsync(sm.prow, 0, sizeof(uint16_t) * ((size_t)sm.npartials + kWave), s));
         ASX_TRY(hipMalloc((void **)&prow_full, sizeof(int32_t) * (size_t)sm.npartials));
+        ASX_TRY(hipMalloc(&sm.partial, sizeof(T) * ((size_t)sm.npartials + kWave)));
+        ASX_TRY(hipMemsetAsync(sm.partial, 0, sizeof(T) * ((size_t)sm.npartials + kWave), s));
         ASX_TRY(hipMalloc((void **)&sm.chunk_lo, sizeof(int32_t) * ((size_t)sm.nrb + 1) * (size_t)sm.nslices));
         hipLaunchKernelGGL(k_sliced_tile_base, dim3((unsigned)ceil_div64((int64_t)sm.ntiles + 1, kBlock)), dim3(kBlock),
                            0, s, hscan, sm.ntiles, sm.tile_base);
@@ -614,22 +616,22 @@ int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s)
 }
 
 template <typename T>
-int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, T *partial,
-                       hipStream_t s)
+int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, hipStream_t s)
 {
     if (m <= 0) return ASX_STATUS_SUCCESS;
+    T *partial = static_cast<T *>(sm->partial);
     constexpr int kSmall = 65536 / sizeof(T), kLarge = 131072 / sizeof(T);
     const int4 *tab = reinterpret_cast<const int4 *>(sm->wg_tab);
-    static const int depth = std::getenv("ASX_P1_DEPTH") ? std::atoi(std::getenv("ASX_P1_DEPTH")) : 4;
-#define ASX_PROD(W, NW, D)                                                                                          \
-    hipLaunchKernelGGL((k_sliced_products<T, W, NW, D>), dim3((unsigned)sm->nwg), dim3(NW * kWave), 0, s, n, tab, \
+    constexpr int kDepth = 2;  // tiles in flight per wave (4 and 8 measured the same or slower)
+#define ASX_PROD(W)                                                                                                 \
+    hipLaunchKernelGGL((k_sliced_products<T, W, 16, kDepth>), dim3((unsigned)sm->nwg), dim3(16 * kWave), 0, s, n, tab, \
                        sm->cf, (const T *)sm->val, sm->tile_base, x, partial)
     if (sm->nwg > 0) {
-        if (sm->width == kLarge) {
-            if (depth == 2) ASX_PROD(kLarge, 16, 2); else if (depth == 8) ASX_PROD(kLarge, 16, 8); else ASX_PROD(kLarge, 16, 4);
-        } else if (sm->width == kSmall) {
-            if (depth == 2) ASX_PROD(kSmall, 16, 2); else if (depth == 8) ASX_PROD(kSmall, 16, 8); else ASX_PROD(kSmall, 16, 4);
-        } else
+        if (sm->width == kLarge)
+            ASX_PROD(kLarge);
+        else if (sm->width == kSmall)
+            ASX_PROD(kSmall);
+        else
             return ASX_STATUS_INVALID_VALUE;
     }
 #undef ASX_PROD
@@ -637,16 +639,11 @@ int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, co
     if (sm->rows_per_wave < 1 || (size_t)sm->rows_per_wave * sizeof(T) > 16384) return ASX_STATUS_INVALID_VALUE;
     const unsigned rgrid = (unsigned)(ceil_div64(ceil_div64(sm->nrb, kWaves), kXcds) * kXcds);
     const size_t lds = (size_t)kWaves * sm->rows_per_wave * sizeof(T);
-    static const int mode_env = std::getenv("ASX_P2_MODE") ? std::atoi(std::getenv("ASX_P2_MODE")) : -1;
-    const int mode = mode_env >= 0 ? mode_env : (sizeof(T) == 4 ? 1 : 0);
-#define ASX_RED(MODE)                                                                                              \
-    hipLaunchKernelGGL((k_sliced_reduce<T, kWaves, MODE>), dim3(rgrid), dim3(kWaves * kWave), lds, s, m, sm->nrb,  \
-                       sm->rows_per_wave, sm->nslices, alpha, beta, sm->chunk_lo, sm->prow, partial, y)
-    if (mode == 1)
-        ASX_RED(1);
-    else
-        ASX_RED(0);
-#undef ASX_RED
+    // fp32: plain LDS read-add-write (LDS float atomics measured 2.5x slower on scattered rows);
+    // fp64: LDS atomic adds (no dependent read in the wave's instruction stream; measured faster)
+    constexpr int kMode = sizeof(T) == 4 ? 1 : 0;
+    hipLaunchKernelGGL((k_sliced_reduce<T, kWaves, kMode>), dim3(rgrid), dim3(kWaves * kWave), lds, s, m, sm->nrb,
+                       sm->rows_per_wave, sm->nslices, alpha, beta, sm->chunk_lo, sm->prow, partial, y);
     return check_launch();
 }
 
@@ -654,7 +651,7 @@ int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, co
     template int build_sliced<T>(int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, const int32_t *,          \
                                  const int32_t *, const T *, SlicedMatrix *, hipStream_t);                       \
     template int sliced_update_values<T>(const SlicedMatrix *, const T *, hipStream_t);                          \
-    template int launch_spmv_sliced<T>(int32_t, int32_t, T, const SlicedMatrix *, const T *, T, T *, T *, hipStream_t);
+    template int launch_spmv_sliced<T>(int32_t, int32_t, T, const SlicedMatrix *, const T *, T, T *, hipStream_t);
 ASX_INST(float)
 ASX_INST(double)
 #undef ASX_INST

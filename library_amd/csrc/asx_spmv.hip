@@ -14,9 +14,7 @@
 //            items; partial rows are joined by a segmented scan inside the workgroup and by
 //            an ordered carry pass between workgroups.  No atomics: results do not depend on
 //            scheduling.
-//   panel  : the flat kernel's tile code over column panels of a regrouped copy of A, the
-//            panels dealt to the XCDs so that each XCD's L2 holds the slice of x it gathers
-//            from; per-panel partial sums are added in panel order by a last pass.
+//   (the column-sliced kernel for scattered columns lives in asx_sliced.hip)
 //
 // The reference's kernels for the same job (hip/kernel/level2/alphasparse_spmv_csr_vector.h,
 // _flat.h, _merge_ginkgo.h, _adaptive.h) join partial rows with floating-point atomicAdd and
@@ -856,141 +854,6 @@ int launch_spmv_flat(int32_t m, int32_t nnz, T alpha, const int32_t *row_ptr, co
     return check_launch();
 }
 
-// ===========================================================================================
-// panel: the flat kernel over kPanels column panels, one panel per XCD
-// ===========================================================================================
-// Random gathers that miss the 4 MiB L2 of an XCD cost a 128-byte fill each (60 G gathers/s
-// against 180 G/s for hits).  With the stored elements regrouped by column panel and the
-// workgroups of one XCD (consecutive workgroups go to consecutive XCDs) working through that
-// XCD's panels one after the other, an XCD gathers from one slice of x at a time, which then
-// lives in its L2.  A panel is a CSR
-// matrix over the rows present in it and writes one partial sum per such row; an ordered pass
-// then adds, for every row of A, its partial sums in panel order.
-struct PanelView {
-    const int32_t *row_ptr, *col, *seg_row;
-    const void *val;
-    int64_t elem_off[kPanels];
-    int32_t count[kPanels];
-    int32_t tile_off[kPanels];
-    int32_t krows[kPanels];
-    int32_t kbase[kPanels];
-};
-
-template <typename T, bool NT>
-__global__ __launch_bounds__(kBlock) void k_spmv_panel(PanelView v, const T *__restrict__ x, T *__restrict__ partial,
-                                                       T *__restrict__ carry)
-{
-    __shared__ FlatShared<T> sh;
-    int j = blockIdx.x % kXcds;
-    int t = blockIdx.x / kXcds;
-    int32_t cnt = 0;
-    for (; j < kPanels; j += kXcds) {  // the panel of this XCD that tile t falls into
-        cnt = v.count[j];
-        const int tiles = (cnt + kFlatTile - 1) / kFlatTile;
-        if (t < tiles) break;
-        t -= tiles;
-    }
-    if (j >= kPanels) return;  // uniform over the workgroup
-    const int32_t *col = v.col + v.elem_off[j];
-    const T *val = static_cast<const T *>(v.val) + v.elem_off[j];
-    int32_t c[4];
-    T p[4];
-    flat_load<T, true, NT>(t, cnt, col, val, c, p);
-    flat_tile<T, false>(sh, t, v.krows[j], cnt, T(1), v.row_ptr + v.kbase[j] + j, c, p, x, T(0), partial + v.kbase[j],
-                        v.seg_row + v.tile_off[j] + j, carry + v.tile_off[j]);
-}
-
-template <typename T>
-__global__ __launch_bounds__(kBlock) void k_spmv_panel_fixup(PanelView v, const T *__restrict__ carry,
-                                                             T *__restrict__ partial)
-{
-    const int j = blockIdx.y;
-    const int32_t cnt = v.count[j];
-    if (cnt == 0) return;
-    const int32_t ntiles = (cnt + kFlatTile - 1) / kFlatTile;
-    if ((int64_t)blockIdx.x * kBlock >= ntiles) return;
-    fixup_tiles<T>((int64_t)blockIdx.x * kBlock + threadIdx.x, v.krows[j], ntiles, T(1), v.seg_row + v.tile_off[j] + j,
-                   carry + v.tile_off[j], partial + v.kbase[j]);
-}
-
-// y[r] = alpha * (sum of row r's partial sums, in panel order) + beta * y[r].  One workgroup per
-// block of kPanelRowBlock rows of A: the partial sums of those rows are one contiguous range of
-// every panel (blk_lo), so all loads are contiguous; they are added into an LDS accumulator per
-// row, one panel after the other (a row appears at most once in a panel, so the adds of one
-// panel never collide).
-template <typename T>
-__global__ __launch_bounds__(kBlock) void k_spmv_panel_reduce(int32_t m, int32_t npanels, T alpha, T beta,
-                                                              const int32_t *__restrict__ blk_lo,
-                                                              const int32_t *__restrict__ rowid,
-                                                              const T *__restrict__ partial, T *__restrict__ y)
-{
-    __shared__ T acc[kPanelRowBlock];
-    __shared__ int32_t s_lo[kPanels], s_hi[kPanels];
-    const int tid = threadIdx.x;
-    const int64_t b = blockIdx.x;
-    const int32_t r0 = (int32_t)(b * kPanelRowBlock);
-    if (tid < kPanels) {
-        s_lo[tid] = blk_lo[b * kPanels + tid];
-        s_hi[tid] = blk_lo[(b + 1) * kPanels + tid];
-    }
-#pragma unroll
-    for (int i = tid; i < kPanelRowBlock; i += kBlock) acc[i] = T(0);
-    __syncthreads();
-    constexpr int kChunk = 16;  // panels whose loads are in flight together
-    for (int j0 = 0; j0 < npanels; j0 += kChunk) {
-        // first kBlock entries of every panel's range: all loads issued before the first add
-        T v[kChunk];
-        int32_t rid[kChunk];
-#pragma unroll
-        for (int j = 0; j < kChunk; ++j) {
-            const int32_t k = s_lo[j0 + j] + tid;
-            const bool ok = k < s_hi[j0 + j];
-            rid[j] = ok ? rowid[k] - r0 : -1;
-            v[j] = ok ? partial[k] : T(0);
-        }
-#pragma unroll
-        for (int j = 0; j < kChunk; ++j) {
-            if (rid[j] >= 0) acc[rid[j]] += v[j];
-            for (int32_t k = s_lo[j0 + j] + kBlock + tid; k < s_hi[j0 + j]; k += kBlock) acc[rowid[k] - r0] += partial[k];
-            __syncthreads();
-        }
-    }
-#pragma unroll
-    for (int i = tid; i < kPanelRowBlock; i += kBlock) {
-        const int64_t r = (int64_t)r0 + i;
-        if (r < m) y[r] = axpby_out<T>(alpha, acc[i], beta, y, r);
-    }
-}
-
-template <typename T>
-int launch_spmv_panel(int32_t m, T alpha, const PanelMatrix *pm, const T *x, T beta, T *y, T *partial, T *carry,
-                      hipStream_t s)
-{
-    if (m <= 0) return ASX_STATUS_SUCCESS;
-    PanelView v{};
-    v.row_ptr = pm->row_ptr;
-    v.col = pm->col;
-    v.seg_row = pm->seg_row;
-    v.val = pm->val;
-    for (int j = 0; j < kPanels; ++j) {
-        v.elem_off[j] = pm->elem_off[j];
-        v.count[j] = pm->count[j];
-        v.tile_off[j] = pm->tile_off[j];
-        v.krows[j] = pm->krows[j];
-        v.kbase[j] = pm->kbase[j];
-    }
-    if (pm->max_tiles > 0) {
-        hipLaunchKernelGGL((k_spmv_panel<T, true>), dim3((unsigned)pm->max_tiles * kXcds), dim3(kBlock), 0, s, v, x,
-                           partial, carry);
-        if (pm->carry_pass)
-            hipLaunchKernelGGL((k_spmv_panel_fixup<T>), dim3((unsigned)ceil_div64(pm->max_tiles, kBlock), (unsigned)pm->npanels),
-                               dim3(kBlock), 0, s, v, carry, partial);
-    }
-    hipLaunchKernelGGL((k_spmv_panel_reduce<T>), dim3((unsigned)ceil_div64(m, kPanelRowBlock)), dim3(kBlock), 0, s, m,
-                       pm->npanels, alpha, beta, pm->blk_lo, pm->rowid, partial, y);
-    return check_launch();
-}
-
 #define ASX_INST(T)                                                                                  \
     template int launch_spmv_vector<T>(int32_t, int32_t, T, const int32_t *, const int32_t *,        \
                                        const T *, const T *, T, T *, hipStream_t);                   \
@@ -1000,8 +863,7 @@ int launch_spmv_panel(int32_t m, T alpha, const PanelMatrix *pm, const T *x, T b
                                       const T *, const T *, T, T *, const int32_t *, const int32_t *, \
                                       T *, hipStream_t);                                             \
     template int launch_spmv_flat<T>(int32_t, int32_t, T, const int32_t *, const int32_t *, const T *, \
-                                     const T *, T, T *, const int32_t *, T *, bool, hipStream_t);      \
-    template int launch_spmv_panel<T>(int32_t, T, const PanelMatrix *, const T *, T, T *, T *, T *, hipStream_t);
+                                     const T *, T, T *, const int32_t *, T *, bool, hipStream_t);
 ASX_INST(float)
 ASX_INST(double)
 #undef ASX_INST

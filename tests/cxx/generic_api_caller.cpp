@@ -101,6 +101,18 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
             s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
         }
+        if (analysis == 2) {
+            // the caller changes A's values in place (same pattern) and says so by calling the
+            // analysis again; the next product must use the new values
+            auto val2 = read_bin<T>(dir + "/val2.bin", nnz);
+            HIP_OK(hipStreamSynchronize(handle->stream));
+            HIP_OK(hipMemcpy(d_val, val2.data(), val2.size() * sizeof(T), hipMemcpyHostToDevice));
+            s = alphasparseSpMV_analysis(handle, opA, A, (alphasparseSpMVAlg_t)alg);
+            if (s) return 70 + (int)s;
+            HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
+            s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
+            if (s) return 50 + (int)s;
+        }
         if (analysis && alphasparseSpMV_clear(handle, (alphasparseSpMVAlg_t)alg)) return 7;
         alphasparseDestroyDnVec(X);
         alphasparseDestroyDnVec(Y);
@@ -124,6 +136,18 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
             if (b2 > bytes) return 8;
         }
         for (int rep = 0; rep < 2; ++rep) {
+            HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
+            s = alphasparseSpMM(handle, opA, opB, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, buffer);
+            if (s) return 50 + (int)s;
+        }
+        if (analysis == 2) {  // new values in place, preprocess again, multiply again
+            auto val2 = read_bin<T>(dir + "/val2.bin", nnz);
+            HIP_OK(hipStreamSynchronize(handle->stream));
+            HIP_OK(hipMemcpy(d_val, val2.data(), val2.size() * sizeof(T), hipMemcpyHostToDevice));
+            size_t b2 = 0;
+            s = alphasparseSpMM_preprocess(handle, opA, opB, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, &b2);
+            if (s) return 70 + (int)s;
+            if (b2 > bytes) return 8;
             HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
             s = alphasparseSpMM(handle, opA, opB, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
@@ -233,8 +257,10 @@ static int selftest()
     }
     EXPECT(alphasparseSpMV(h, (alphasparseOperation_t)7, &alpha, A, X, &beta, Y, ALPHA_R_64F,
                            ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) == ALPHA_SPARSE_STATUS_INVALID_VALUE);
-    // analysis is kept on the handle, found again, and cleared
+    // analysis is kept on the matrix (matA->info), found again, and cleared through the handle
     EXPECT(alphasparseSpMV_analysis(h, N, A, ALPHA_SPARSE_SPMV_ALG_DEFAULT) == 0 && A->analysed);
+    EXPECT(A->info && A->info->csrmv_info && A->info->csrmv_info->m == 2 && A->info->csrmv_info->nnz == 3 &&
+           A->info->csrmv_info->csr_row_ptr == d_rp);
     EXPECT(alphasparseSpMV_analysis(h, N, A, ALPHA_SPARSE_SPMV_ALG_DEFAULT) == 0);
     HIP_OK(hipMemcpy(d_y, x.data(), sizeof(double) * 2, hipMemcpyHostToDevice));
     EXPECT(alphasparseSpMV(h, N, &alpha, A, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) == 0);

@@ -41,6 +41,7 @@ def lib():
 
 def test_header_symbols_are_exported(lib):
     header = open(os.path.join(ROOT, "include", "alphasparse_amd.h")).read()
+    header += open(os.path.join(ROOT, "include", "alphasparse_amd_bench.h")).read()
     declared = sorted(set(re.findall(r"\b(asx_[a-z0-9_]+)\s*\(", header)))
     assert declared, "no declarations found"
     assert sorted(capi.EXPORTS) == declared  # the ctypes view covers the whole header
@@ -53,6 +54,35 @@ def test_generic_api_mangled_names(lib):
     exported = {line.split()[-1] for line in out.splitlines() if line.strip()}
     for name in MANGLED:
         assert name in exported, name
+
+
+def test_struct_layouts_match_the_reference_fixture(tmp_path):
+    """tests/golden/layout.json holds sizeof / offsetof of the boundary structs as the reference's
+    own headers give them (written by tests/golden/make_layout.py in the build container).  The
+    same probe compiled against this repository's include/ must print the same numbers."""
+    import json
+    want = json.load(open(os.path.join(ROOT, "tests", "golden", "layout.json")))
+    exe = str(tmp_path / "layout_probe")
+    subprocess.run(["g++", "-std=c++17", "-w", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
+                    "-I" + os.path.join(ROOT, "include"), os.path.join(ROOT, "tests", "golden", "layout_probe.cpp"),
+                    "-o", exe], check=True)
+    got = json.loads(subprocess.run([exe], check=True, capture_output=True, text=True).stdout)
+    got.pop("end", None)
+    assert got == want, {k: (got.get(k), want.get(k)) for k in set(got) | set(want) if got.get(k) != want.get(k)}
+    assert want["sizeof(alphasparse_handle_s)"] == 1608 and want["sizeof(_alphasparse_mat_descr)"] == 144
+
+
+def test_default_workspace_covers_merge_and_flat(lib):
+    """alphasparseSpMV_bufferSize(DEFAULT) reports asx_spmv_workspace_bytes(DEFAULT); a DEFAULT
+    analysis may settle on the flat or the merge-path kernel, so it must cover both, also for
+    hypersparse matrices where the merge-path carry array (one value per 2048 rows + stored
+    elements) is the larger."""
+    for vt in (capi.R_32F, capi.R_64F):
+        for m, nnz in ((2_000_000, 100_000), (1 << 22, 34_000_000), (10, 10), (1 << 24, 1 << 20), (300_000, 200_000),
+                       (1, 0), (5_000_000, 1)):
+            d = lib.asx_spmv_workspace_bytes(capi.SPMV_DEFAULT, vt, m, nnz)
+            assert d >= lib.asx_spmv_workspace_bytes(capi.SPMV_MERGE, vt, m, nnz), (vt, m, nnz)
+            assert d >= lib.asx_spmv_workspace_bytes(capi.SPMV_FLAT, vt, m, nnz), (vt, m, nnz)
 
 
 def test_alg_mapping_and_workspace(lib):

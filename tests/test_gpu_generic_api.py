@@ -15,12 +15,14 @@ EXE = os.path.join(ROOT, "tests", "cxx", "generic_api_caller")
 
 
 def _run_case(tmp_path, op, dtype, rp, col, val, x, y, ncols, alg, alpha, beta, analysis, variant=(0, 0, 0, 0, 0),
-              n=None):
+              n=None, val2=None):
     """variant = (trans_a, idx_base, col_major_b, col_major_c, trans_b); n = columns of A."""
     d = tmp_path / f"{op}_{np.dtype(dtype).name}_{alg}_{analysis}_{''.join(map(str, variant))}"
     d.mkdir()
     for name, a in (("row_ptr", rp), ("col", col), ("val", val), ("x", x), ("y", y)):
         np.ascontiguousarray(a).tofile(d / f"{name}.bin")
+    if val2 is not None:  # analysis == 2: values written over A's after the first products
+        np.ascontiguousarray(val2).tofile(d / "val2.bin")
     tag = "f64" if np.dtype(dtype) == np.float64 else "f32"
     if n is None:
         n = x.size // ncols
@@ -183,10 +185,11 @@ def test_cli_on_matrixmarket_files(tmp_path):
     assert r.returncode == 4
 
 
-def test_spmv_analysis_on_a_panel_candidate(tmp_path, oracle):
-    """A matrix whose x (8 MiB) is a candidate for the column-panel kernel: analysis with DEFAULT
-    builds the panels and times them; whichever kernel it keeps, the buffer alphasparseSpMV_bufferSize
-    reported must do and the result must match, also for opA = TRANSPOSE."""
+def test_spmv_analysis_on_a_scattered_matrix(tmp_path, oracle):
+    """A matrix DEFAULT's analysis takes the column-sliced kernel for (4 M scattered stored elements,
+    x of 8 MiB): the buffer alphasparseSpMV_bufferSize reported must do, the result must match, also
+    for opA = TRANSPOSE, and after the caller overwrites A's values and calls the analysis again the
+    product must be the one of the new values."""
     from library_amd import workloads as W
     rp, col, val = W.csr_zipf(1 << 20, 1 << 20, 20, 1.0, 5000, 0.01, np.float64, 3)
     n = 1 << 20
@@ -199,10 +202,29 @@ def test_spmv_analysis_on_a_panel_candidate(tmp_path, oracle):
     scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
     got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, alpha, beta, 1)
     assert_close(got, ref, scale, np.float64, "DEFAULT with analysis")
+    val2 = rng.uniform(-1, 1, val.size)
+    got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, alpha, beta, 2, val2=val2)
+    assert_close(got, oracle.spmv(rp, col, val2, x, alpha, beta, y0, 8), spmv_scale(rp, col, val2, x, alpha, beta, y0),
+                 np.float64, "DEFAULT, values changed, analysis called again")
     rp_t, col_t, val_t = _transpose_csr(rp, col, val, n)
     ref_t = oracle.spmv(rp_t, col_t, val_t, y0, alpha, beta, x, 8)
     got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, y0, x, 1, 0, alpha, beta, 1, (1, 0, 0, 0, 0), n=n)
     assert_close(got, ref_t, spmv_scale(rp_t, col_t, val_t, y0, alpha, beta, x), np.float64, "transpose, DEFAULT with analysis")
+
+
+def test_spmm_blocked_values_changed_after_preprocess(tmp_path, oracle):
+    """ALPHASPARSE_SPMM_CSR_ALG6 keeps a blocked copy of A's values: after the caller overwrites the
+    values and calls alphasparseSpMM_preprocess again, the product is the one of the new values."""
+    from test_gpu_parity import _block_structured
+    rng = np.random.default_rng(67)
+    m, k, n = 700, 640, 64
+    rp, col, val = _block_structured(rng, m, k, np.float32)
+    B = rng.uniform(-1, 1, k * n).astype(np.float32)
+    C0 = rng.uniform(-1, 1, m * n).astype(np.float32)
+    val2 = rng.uniform(-1, 1, val.size).astype(np.float32)
+    got = _run_case(tmp_path, "spmm", np.float32, rp, col, val, B, C0, n, 10, 2.0, 3.0, 2, val2=val2)
+    assert_close(got, oracle.spmm(rp, col, val2, B, n, 2.0, 3.0, C0, 4), spmm_scale(rp, col, val2, B, n, 2.0, 3.0, C0),
+                 np.float32, "ALG6, values changed, preprocess called again")
 
 
 def test_cli_on_the_reference_matrix():

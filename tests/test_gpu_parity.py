@@ -348,21 +348,25 @@ def test_benchmark_configs_full_size(torch, capi, oracle):
             torch.cuda.synchronize()
             assert_close(y.cpu().numpy(), ref, scale, w.dtype, f"{name} alg={alg}")
             plan.destroy()
-        if name == "powerlaw_f64":
-            # plans that may look at columns and values: the column-panel kernel, forced and as the
-            # winner of DEFAULT's timing on this matrix (x is 8 L2s large, columns are scattered)
-            for alg in (capi.SPMV_PANEL, capi.SPMV_DEFAULT):
+        if name in ("powerlaw_f64", "uniform16_f32"):
+            # plans that may look at columns and values: the column-sliced kernel, forced and as
+            # DEFAULT's choice on these matrices (scattered columns; the choice is rule-based, so two
+            # plan builds agree)
+            for alg in (capi.SPMV_SLICED, capi.SPMV_DEFAULT, capi.SPMV_DEFAULT):
                 plan = capi.Plan(False, alg, w.val.dtype, w.m, w.n, w.nnz, d[0], col=d[1], val=d[2])
-                assert plan.alg == capi.SPMV_PANEL
+                assert plan.alg == capi.SPMV_SLICED and plan.holds_values and plan.workspace_bytes == 0
+                outs = []
                 for rep in range(2):
                     y = dev(torch, w.y)
                     capi.spmv(d[0], d[1], d[2], d[3], y, w.alpha, w.beta, alg=alg, plan=plan)
                     torch.cuda.synchronize()
-                    assert_close(y.cpu().numpy(), ref, scale, w.dtype, f"{name} panel alg={alg} rep={rep}")
+                    outs.append(y.cpu().numpy())
+                    assert_close(outs[-1], ref, scale, w.dtype, f"{name} sliced alg={alg} rep={rep}")
+                assert np.array_equal(outs[0], outs[1]), "two calls through one plan must agree bit for bit"
                 plan.destroy()
-        else:  # not candidates for panels: DEFAULT with values behaves as without
+        else:  # regular columns: DEFAULT with columns and values behaves as without
             plan = capi.Plan(False, capi.SPMV_DEFAULT, w.val.dtype, w.m, w.n, w.nnz, d[0], col=d[1], val=d[2])
-            assert plan.alg == capi.SPMV_FLAT
+            assert plan.alg == capi.SPMV_FLAT and not plan.holds_values
             plan.destroy()
         del d
     w = W.spmm_zipf_f32()
@@ -413,6 +417,44 @@ def test_spmm_blocked_mfma(torch, capi, oracle, dtype):
                 torch.cuda.synchronize()
                 assert_close(Cm.cpu().numpy(), ref, scale, dtype, f"blocked m={m} k={k} n={n} a={alpha} b={beta}")
             plan.destroy()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_spmm_blocked_repeated_entries_and_value_update(torch, capi, oracle, dtype):
+    """CSR may repeat a (row, column): the blocked copy sums the repeats, as the row-wise kernels
+    and the reference do.  After the values change, one asx_plan_update_values brings the plan's
+    copy up to date."""
+    rng = np.random.default_rng(63)
+    m, k, n = 300, 260, 64
+    rp, col, val = _block_structured(rng, m, k, dtype)
+    # repeat about a fifth of the stored elements once or twice, next to the original
+    reps = rng.choice([1, 1, 1, 1, 2, 3], size=col.size)
+    rows = np.repeat(np.arange(m), np.diff(rp))
+    rows2, col2 = np.repeat(rows, reps), np.repeat(col, reps)
+    val2 = rng.uniform(-1, 1, col2.size).astype(dtype)
+    rp2 = np.zeros(m + 1, np.int32)
+    np.cumsum(np.bincount(rows2, minlength=m), out=rp2[1:])
+    col2 = col2.astype(np.int32)
+    B = rng.uniform(-1, 1, k * n).astype(dtype)
+    C0 = rng.uniform(-1, 1, m * n).astype(dtype)
+    d = [dev(torch, a) for a in (rp2, col2, val2)]
+    for alg in (capi.SPMM_BLOCKED, capi.SPMM_DEFAULT):
+        plan = capi.Plan(True, alg, np.dtype(dtype), m, k, col2.size, d[0], ncols=n, col=d[1], val=d[2])
+        assert plan.alg == capi.SPMM_BLOCKED and plan.holds_values
+        ref = oracle.spmm(rp2, col2, val2, B, n, 1.5, 0.5, C0, 4)
+        Cm = dev(torch, C0)
+        capi.spmm(d[0], d[1], d[2], dev(torch, B), Cm, n, 1.5, 0.5, alg=alg, plan=plan, k=k)
+        torch.cuda.synchronize()
+        assert_close(Cm.cpu().numpy(), ref, spmm_scale(rp2, col2, val2, B, n, 1.5, 0.5, C0), dtype, f"repeats alg={alg}")
+        val3 = rng.uniform(-1, 1, col2.size).astype(dtype)
+        d3 = dev(torch, val3)
+        plan.update_values(d3)
+        ref = oracle.spmm(rp2, col2, val3, B, n, 1.5, 0.5, C0, 4)
+        Cm = dev(torch, C0)
+        capi.spmm(d[0], d[1], d3, dev(torch, B), Cm, n, 1.5, 0.5, alg=alg, plan=plan, k=k)
+        torch.cuda.synchronize()
+        assert_close(Cm.cpu().numpy(), ref, spmm_scale(rp2, col2, val3, B, n, 1.5, 0.5, C0), dtype, f"updated alg={alg}")
+        plan.destroy()
 
 
 def test_spmm_default_picks_blocked_only_for_dense_blocks(torch, capi, oracle):
@@ -505,58 +547,111 @@ def test_csr_transpose_rebase_dense_transpose(torch, capi):
             assert np.array_equal(d_out.cpu().numpy().reshape(cols_, ld_out), want), (rows_, cols_)
 
 
-# ------------------------------------------------------------------ column-panel SpMV
+# ------------------------------------------------------------------ column-sliced SpMV
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
-def test_spmv_panel_kernel_shapes(torch, capi, oracle, dtype):
-    """The panel kernel forced on small matrices of every awkward shape: panels without elements,
-    rows that span many tiles of one panel, runs of empty rows, a single column panel in use,
-    beta = 0 over NaN, and two calls through one plan."""
+def test_spmv_sliced_kernel_shapes(torch, capi, oracle, dtype):
+    """The sliced kernel forced on small matrices of every awkward shape: slices without elements,
+    runs longer than a tile (cut into several partial sums of one row), runs of empty rows, a
+    single slice in use, a last slice narrower than the others, more than 64 slices (several
+    groups of ranges per row block), beta = 0 over NaN, two calls through one plan, and a value
+    update through the kept permutation."""
     rng = np.random.default_rng(91)
+    width = 131072 // np.dtype(dtype).itemsize
     cases = []
     for name, lens in analysis_shapes().items():
         if np.sum(lens) == 0:
             continue
         n = int(max(np.max(lens), 64)) + 29
         cases.append((name, csr_from_lengths(lens, n, 6, dtype), n))
-    # every column in the first panel; columns in the last panel only; one dense-ish long row
+    # a few columns in the first slice only; in the last (narrow) slice only; spread over 3 slices
+    n3 = 2 * width + 777
     lens = np.r_[rng.integers(0, 9, 3000), 20000]
-    rp, col, val = csr_from_lengths(lens, 30000, 8, dtype)
-    cases.append(("first_panel", (rp, (col % 100).astype(np.int32), val), 30000))
-    cases.append(("last_panel", (rp, (29999 - col % 50).astype(np.int32), val), 30000))
-    cases.append(("spread", (rp, col, val), 30000))
+    rp, col, val = csr_from_lengths(lens, n3, 8, dtype)
+    cases.append(("first_slice", (rp, (col % 100).astype(np.int32), val), n3))
+    cases.append(("last_slice", (rp, (n3 - 1 - col % 50).astype(np.int32), val), n3))
+    cases.append(("spread3", (rp, col, val), n3))
+    # 70 slices: row blocks walk two groups of ranges; rows of 300 reach most slices
+    n70 = 69 * width + 5
+    lens = np.r_[rng.integers(0, 4, 500), np.full(40, 300), 0, 0, 9000]
+    cases.append(("slices70", csr_from_lengths(lens, n70, 9, dtype), n70))
     for name, (rp, col, val), n in cases:
         m = rp.size - 1
         x = rng.uniform(-1, 1, n).astype(dtype)
         y0 = rng.uniform(-1, 1, m).astype(dtype)
         d = [dev(torch, a) for a in (rp, col, val, x)]
-        plan = capi.Plan(False, capi.SPMV_PANEL, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
-        assert plan.alg == capi.SPMV_PANEL
+        plan = capi.Plan(False, capi.SPMV_SLICED, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
+        assert plan.alg == capi.SPMV_SLICED and plan.holds_values
         for alpha, beta in ((1.5, 0.5), (1.0, 0.0), (-2.0, 1.0)):
             ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 2)
             scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
             for rep in range(2):
                 y = dev(torch, y0 if beta else np.full(m, np.nan, dtype=dtype))
-                capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_PANEL, plan=plan)
+                capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_SLICED, plan=plan)
                 torch.cuda.synchronize()
                 assert_close(y.cpu().numpy(), ref, scale, dtype, f"{name} a={alpha} b={beta} rep={rep}")
+        # new values, same pattern: stale until the plan is told, the oracle's answer afterwards
+        val2 = rng.uniform(-1, 1, val.size).astype(dtype)
+        d2 = dev(torch, val2)
+        plan.update_values(d2)
+        ref = oracle.spmv(rp, col, val2, x, dtype(1.5), dtype(0.5), y0, 2)
+        y = dev(torch, y0)
+        capi.spmv(d[0], d[1], d2, d[3], y, 1.5, 0.5, alg=capi.SPMV_SLICED, plan=plan)
+        torch.cuda.synchronize()
+        assert_close(y.cpu().numpy(), ref, spmv_scale(rp, col, val2, x, 1.5, 0.5, y0), dtype, f"{name} updated values")
         plan.destroy()
-    # the panel kernel needs its plan; a plan without columns and values cannot be a panel plan
+    # the sliced kernel needs its plan; a plan without columns and values cannot be a sliced plan
     L = capi.lib()
     h = capi.C.c_void_p()
-    assert L.asx_plan_create(capi.C.byref(h), 0, capi.SPMV_PANEL, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), 1, None) == 6
-    assert L.asx_spmv_csr_f64(None, capi.SPMV_PANEL, 1, 1, 0, 1.0, capi._ptr(d[0]), None, None, None, 0.0,
+    assert L.asx_plan_create(capi.C.byref(h), 0, capi.SPMV_SLICED, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), 1, None) == 6
+    assert L.asx_spmv_csr_f64(None, capi.SPMV_SLICED, 1, 1, 0, 1.0, capi._ptr(d[0]), None, None, None, 0.0,
                               capi._ptr(d[3]), None, 0, None) == 6
     # argument errors of the plan constructor that takes columns and values
-    for args, want in (((None, capi.SPMV_PANEL, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 7),
-                       ((capi.C.byref(h), capi.SPMV_PANEL, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), None, capi._ptr(d[2]), None), 7),
-                       ((capi.C.byref(h), capi.SPMV_PANEL, capi.R_64F, -1, 10, 10, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 10),
-                       ((capi.C.byref(h), capi.SPMV_PANEL, capi.R_64F, 10, 10, 0, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 10),
-                       ((capi.C.byref(h), capi.SPMV_PANEL, 7, 10, 10, 10, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 6),
+    for args, want in (((None, capi.SPMV_SLICED, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 7),
+                       ((capi.C.byref(h), capi.SPMV_SLICED, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), None, capi._ptr(d[2]), None), 7),
+                       ((capi.C.byref(h), capi.SPMV_SLICED, capi.R_64F, -1, 10, 10, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 10),
+                       ((capi.C.byref(h), capi.SPMV_SLICED, capi.R_64F, 10, 10, 0, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 10),
+                       ((capi.C.byref(h), capi.SPMV_SLICED, 7, 10, 10, 10, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 6),
                        ((capi.C.byref(h), 1, capi.R_64F, 10, 10, 10, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None), 6)):
         assert L.asx_spmv_plan_create(*args) == want, args
-    assert L.asx_spmv_panel_workspace_bytes(capi.R_64F, 1 << 22, 1 << 22, 1 << 25) >= 8 * (1 << 22) * 8
-    assert L.asx_spmv_panel_workspace_bytes(capi.R_64F, 1 << 26, 1 << 26, 1 << 27) == 0  # x (512 MiB) too large
-    assert L.asx_spmv_panel_workspace_bytes(capi.R_32F, 1 << 20, 1 << 20, 1 << 24) == 0  # x fits one L2
+    assert L.asx_plan_update_values(None, None, None) == 7
+    assert L.asx_plan_holds_values(None) == 0
+
+
+def test_default_workspace_covers_every_choice(torch, capi, oracle):
+    """alphasparseSpMV_bufferSize(DEFAULT) is asx_spmv_workspace_bytes(DEFAULT): whatever kernel a
+    DEFAULT plan settles on must fit in it.  Hypersparse (the plan takes the merge-path kernel,
+    whose carry array follows m + nnz) and very long rows, with an exactly sized workspace."""
+    rng = np.random.default_rng(77)
+    L = capi.lib()
+    shapes = {
+        "hypersparse": np.where(rng.random(2_000_000) < 0.05, 1, 0),
+        "long_rows": np.r_[np.full(20, 9000), rng.integers(0, 3, 300000)],
+    }
+    for name, lens in shapes.items():
+        m = lens.size
+        n = 50000
+        rp = np.zeros(m + 1, np.int32)
+        rp[1:] = np.cumsum(lens)
+        nnz = int(rp[-1])
+        col = np.sort(rng.integers(0, n, nnz).astype(np.int32))  # order inside rows does not matter here
+        rows = np.repeat(np.arange(m), lens)
+        order = np.lexsort((col, rows))
+        col = col[order]
+        val = rng.uniform(-1, 1, nnz)
+        x = rng.uniform(-1, 1, n)
+        y0 = rng.uniform(-1, 1, m)
+        d = [dev(torch, a) for a in (rp, col, val, x)]
+        plan = capi.Plan(False, capi.SPMV_DEFAULT, val.dtype, m, n, nnz, d[0], col=d[1], val=d[2])
+        budget = L.asx_spmv_workspace_bytes(capi.SPMV_DEFAULT, capi.R_64F, m, nnz)
+        assert plan.alg == capi.SPMV_MERGE, name
+        assert plan.workspace_bytes <= budget, (name, plan.workspace_bytes, budget)
+        ws = torch.empty(budget, dtype=torch.uint8, device="cuda")
+        y = dev(torch, y0)
+        capi.spmv(d[0], d[1], d[2], d[3], y, 1.5, 0.5, plan=plan, workspace=ws)
+        torch.cuda.synchronize()
+        ref = oracle.spmv(rp, col, val, x, 1.5, 0.5, y0, 4)
+        assert_close(y.cpu().numpy(), ref, spmv_scale(rp, col, val, x, 1.5, 0.5, y0), np.float64, name)
+        plan.destroy()
 
 
 # ------------------------------------------------------------------ randomised shapes, every SpMV kernel
@@ -588,37 +683,22 @@ def test_spmv_random_shapes_all_kernels(torch, capi, oracle):
         for alg in ALGS:
             got = run_spmv(torch, capi, rp, col, val, x, y0, alpha, beta, alg_id(capi, alg), use_plan=(case % 4 < 2))
             assert_close(got, ref, scale, dtype, f"case {case} kind {kind} {alg}")
-        if col.size:  # the panel kernel needs its plan
+        if col.size:  # the sliced kernel needs its plan
             d = [dev(torch, a) for a in (rp, col, val, x)]
             y = dev(torch, y0)
-            plan = capi.Plan(False, capi.SPMV_PANEL, np.dtype(dtype), rp.size - 1, ncols, col.size, d[0], col=d[1], val=d[2])
-            capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_PANEL, plan=plan)
+            plan = capi.Plan(False, capi.SPMV_SLICED, np.dtype(dtype), rp.size - 1, ncols, col.size, d[0], col=d[1], val=d[2])
+            capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_SLICED, plan=plan)
             torch.cuda.synchronize()
-            assert_close(y.cpu().numpy(), ref, scale, dtype, f"case {case} kind {kind} panel")
+            assert_close(y.cpu().numpy(), ref, scale, dtype, f"case {case} kind {kind} sliced")
             plan.destroy()
 
 
-# ------------------------------------------------------------------ measurement helpers
-def test_probes_and_copy_run(torch, capi):
-    """The measurement entry points launch, finish and write nothing but the copy's destination."""
+# ------------------------------------------------------------------ measurement helper
+def test_calibration_copy_runs(torch, capi):
+    """The benchmark's copy kernel copies, and rejects sizes that are no multiple of 16."""
     L = capi.lib()
     rng = np.random.default_rng(5)
-    n, nnz = 5000, 70001
-    col = dev(torch, rng.integers(0, n, nnz).astype(np.int32))
     stream = capi._stream()
-    for dtype, vt in ((np.float64, capi.R_64F), (np.float32, capi.R_32F)):
-        val = dev(torch, rng.uniform(-1, 1, nnz).astype(dtype))
-        x = dev(torch, rng.uniform(-1, 1, n).astype(dtype))
-        sink = torch.zeros(4, dtype=val.dtype, device="cuda")
-        for mode in (0, 1):
-            assert L.asx_probe_stream_gather(vt, mode, nnz, capi._ptr(col), capi._ptr(val), capi._ptr(x), capi._ptr(sink), stream) == 0
-        for slicing in (0, 1, 2):
-            assert L.asx_probe_sliced_gather(vt, slicing, nnz, n, capi._ptr(col), capi._ptr(val), capi._ptr(x), capi._ptr(sink), stream) == 0
-        torch.cuda.synchronize()
-        assert sink.cpu().numpy().tolist() == [0, 0, 0, 0]
-    assert L.asx_probe_stream_gather(capi.R_64F, 5, nnz, capi._ptr(col), capi._ptr(val), capi._ptr(x), capi._ptr(sink), stream) == 3
-    assert L.asx_probe_sliced_gather(capi.R_64F, 3, nnz, n, capi._ptr(col), capi._ptr(val), capi._ptr(x), capi._ptr(sink), stream) == 3
-    assert L.asx_probe_sliced_gather(capi.R_64F, 0, nnz, 8, capi._ptr(col), capi._ptr(val), capi._ptr(x), capi._ptr(sink), stream) == 10
     src = dev(torch, rng.integers(0, 255, 1 << 20).astype(np.uint8))
     dst = torch.zeros_like(src)
     assert L.asx_copy_bytes(capi._ptr(src), capi._ptr(dst), src.numel(), stream) == 0
