@@ -234,6 +234,22 @@ int asx_spmv_csr_f32(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_
                      const float *d_x, float beta, float *d_y, void *d_workspace,
                      size_t workspace_bytes, void *stream);
 
+/* asx_spmv_csr_f64 without a plan and without a workspace argument, for callers that cannot
+ * allocate device memory and have no buffer to pass (code under HIP graph capture, serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  The split points and
+ * carries that asx_spmv_csr_f64 puts into the caller's workspace live in an array inside the
+ * library, one copy per GPU, asx_spmv_noalloc_max_workspace() bytes (4 MiB) large: a call whose
+ * asx_spmv_workspace_bytes(alg, ASX_R_64F, m, nnz) exceeds that returns ASX_STATUS_INVALID_SIZE
+ * and launches nothing (the flat kernel, alg 0, needs 12 bytes per 1024 stored elements: about
+ * 350 million stored elements fit).  The call allocates nothing and frees nothing.  Every call on
+ * a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads)
+ * race; calls on one stream are safe.  Same kernels, same results as asx_spmv_csr_f64 with the
+ * same `alg`. */
+int asx_spmv_csr_f64_noalloc(int alg, int32_t m, int32_t n, int32_t nnz, double alpha,
+                             const int32_t *d_row_ptr, const int32_t *d_col, const double *d_val,
+                             const double *d_x, double beta, double *d_y, void *stream);
+size_t asx_spmv_noalloc_max_workspace(void);
+
 /* ------------------------------------------------------------------------------------
  * SpMM  C = alpha*A*B + beta*C, B (k x ncols) and C (m x ncols) row-major
  *       (alphasparseSpMM, include/alphasparse/spapi.h:6963-6974; CPU twin alphasparse_?_mm,

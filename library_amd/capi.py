@@ -30,6 +30,7 @@ EXPORTS = [
     "asx_plan_update_values", "asx_plan_holds_values", "asx_plan_create",
     "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
+    "asx_spmv_csr_f64_noalloc", "asx_spmv_noalloc_max_workspace",
     "asx_spmm_resolve_alg", "asx_spmm_workspace_bytes", "asx_spmm_csr_f32", "asx_spmm_csr_f64",
     "asx_copy_bytes",
 ]
@@ -86,6 +87,9 @@ def lib():
     L.asx_spmv_workspace_bytes.restype = sz
     L.asx_spmv_csr_f64.argtypes = [vp, C.c_int, i32, i32, i32, C.c_double, vp, vp, vp, vp, C.c_double, vp, vp, sz, vp]
     L.asx_spmv_csr_f32.argtypes = [vp, C.c_int, i32, i32, i32, C.c_float, vp, vp, vp, vp, C.c_float, vp, vp, sz, vp]
+    L.asx_spmv_csr_f64_noalloc.argtypes = [C.c_int, i32, i32, i32, C.c_double, vp, vp, vp, vp, C.c_double, vp, vp]
+    L.asx_spmv_noalloc_max_workspace.argtypes = []
+    L.asx_spmv_noalloc_max_workspace.restype = sz
     L.asx_spmm_resolve_alg.argtypes = [C.c_int, i32, i32, i32]
     L.asx_spmm_workspace_bytes.argtypes = [C.c_int, C.c_int, i32, i32, i32]
     L.asx_spmm_workspace_bytes.restype = sz

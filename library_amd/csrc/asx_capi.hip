@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -736,6 +737,58 @@ int asx_spmv_csr_f32(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_
 {
     return spmv_impl<float>(plan, alg, m, n, nnz, alpha, d_row_ptr, d_col, d_val, d_x, beta, d_y,
                             d_workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------- SpMV without any allocation
+}  // extern "C"
+
+// Split points and carries of a plan-less call, for callers that can neither allocate nor bring
+// a buffer.  One copy of the array per GPU, held until the process ends; its device address is
+// looked up once per device (the array's name is not a device address in host code).
+static constexpr size_t kNoAllocScratchBytes = (size_t)4 << 20;
+static __device__ __align__(256) unsigned char asx_noalloc_scratch[kNoAllocScratchBytes];
+static constexpr int kNoAllocMaxDevices = 64;
+static void *g_noalloc_ptr[kNoAllocMaxDevices];
+static std::mutex g_noalloc_mutex;
+
+// Device address of this device's copy of the scratch array; the device must be current.
+static int noalloc_scratch(void **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return status_of(e);
+    if (dev < 0 || dev >= kNoAllocMaxDevices) return ASX_STATUS_NOT_SUPPORTED;
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+    if (!g_noalloc_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(asx_noalloc_scratch));
+        if (e != hipSuccess) return status_of(e);
+        if (!p) return ASX_STATUS_INTERNAL_ERROR;
+        g_noalloc_ptr[dev] = p;
+    }
+    *out = g_noalloc_ptr[dev];
+    return ASX_STATUS_SUCCESS;
+}
+
+extern "C" {
+
+size_t asx_spmv_noalloc_max_workspace(void) { return kNoAllocScratchBytes; }
+
+int asx_spmv_csr_f64_noalloc(int alg, int32_t m, int32_t n, int32_t nnz, double alpha, const int32_t *d_row_ptr,
+                             const int32_t *d_col, const double *d_val, const double *d_x, double beta, double *d_y,
+                             void *stream)
+{
+    if (m < 0 || n < 0 || nnz < 0) return ASX_STATUS_INVALID_SIZE;
+    if (asx_spmv_resolve_alg(alg, m, nnz) < 0) return ASX_STATUS_NOT_SUPPORTED;
+    // what asx_spmv_csr_f64 would ask of a caller's buffer for this call must fit the array
+    const size_t need = asx_spmv_workspace_bytes(alg, ASX_R_64F, m, nnz);
+    if (need > kNoAllocScratchBytes) return ASX_STATUS_INVALID_SIZE;
+    void *ws = nullptr;
+    const int st = noalloc_scratch(&ws);
+    if (st) return st;
+    // every kernel writes the split points and carries it reads: nothing has to start at zero
+    return spmv_impl<double>(nullptr, alg, m, n, nnz, alpha, d_row_ptr, d_col, d_val, d_x, beta, d_y, ws,
+                             kNoAllocScratchBytes, (hipStream_t)stream);
 }
 
 // ---------------------------------------------------------------- SpMM
