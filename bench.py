@@ -4,12 +4,25 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only]
 
 A step is one SpMV (or SpMM) call through the C-ABI on a synthetic workload that is already
-resident in HBM; analysis (split points) is done once, outside the timed region, and reported
-separately.  Prints ONE JSON line.  `value` is effective GB/s = algorithmic bytes / time, with
+resident in HBM; analysis (split points, column slices) is done once, outside the timed region,
+and reported separately.  Prints ONE JSON line.  `value` is effective GB/s = algorithmic bytes /
+time, with
     SpMV bytes = nnz*(sv+4) + (m+1)*4 + n*sv   + m*sv  *(beta != 0 ? 2 : 1)
     SpMM bytes = nnz*(sv+4) + (m+1)*4 + k*N*sv + m*N*sv*(beta != 0 ? 2 : 1)
 All five benchmark configurations are measured (unless --only); the one named by --workload
 supplies the headline fields, the others are listed under "workloads".
+
+Per workload, on the GPU:
+  ms_per_step     K calls back to back between two synchronisations (the whole-job figure)
+  event_ms_*      one HIP event pair per call on the launch stream; when beta != 0 the output is
+                  restored from a pristine copy before every call, outside the event pair (the
+                  reference's test loop does the same, hip/test/level2/spmv_csr_r_f64_test.hip:183-198)
+  cold_ms         as event_ms, after a 1 GiB sweep that evicts the caches before every call
+  noplan_ms       the call without kept analysis (split points recomputed inside every call, as
+                  the reference does)
+and on the host (unless --no-cpu), the reference's own CPU kernels (oracle/_ref, kind
+"reference") or their C restatement (kind "port") on the same inputs: all physical cores of the
+box's share, and one thread.
 """
 import argparse
 import json
@@ -23,17 +36,19 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 ORDER = ["banded_f64", "uniform16_f32", "powerlaw_f64", "stencil5_f64", "spmm_zipf_f32"]
 EXTRA = ["spmm_banded_f32"]  # not a BASELINE configuration: dense-block matrix for the MFMA SpMM variant
-KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "k_spmv_flat", 100: "k_spmv_panel", 5: "k_spmm_row", 7: "k_spmm_merge",
-                10: "k_spmm_blocked"}
+KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "k_spmv_flat",
+                101: "k_sliced_products+k_sliced_reduce", 5: "k_spmm_row", 7: "k_spmm_merge", 10: "k_spmm_blocked"}
 
-# HBM traffic per call measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; see profiles/),
-# scaled by the same counters' reading for a plain copy of known size.  None = not measured.
+# HBM-side traffic per call measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE in KiB per
+# dispatch, summed over the kernels of one call; see profiles/), scaled by the same counters'
+# reading for a plain copy of known size (FETCH_SIZE reads half the bytes, WRITE_SIZE all of
+# them).  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "powerlaw_f64": (305282.3 * 2 + 111347.2) * 1024,     # profiles/spmv_panel_powerlaw_f64.md
-    "stencil5_f64": (679827.7 * 2 + 138992.2) * 1024,    # profiles/spmv_flat_stencil5_f64.md
-    "uniform16_f32": (215067.3 * 2 + 4699.0) * 1024,     # profiles/spmv_flat_uniform16_f32.md
-    "spmm_banded_f32": (741844.7 * 2 + 340585.3) * 1024,  # profiles/spmm_blocked_spmm_banded_f32.md
-    "spmm_zipf_f32": (2284685.2 * 2 + 278616.5) * 1024,  # profiles/spmm_merge_spmm_zipf_f32.md
+    "powerlaw_f64": None,
+    "stencil5_f64": None,
+    "uniform16_f32": None,
+    "spmm_banded_f32": None,
+    "spmm_zipf_f32": None,
 }
 
 
@@ -44,12 +59,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="powerlaw_f64", choices=ORDER + EXTRA)
     ap.add_argument("--only", action="store_true", help="measure only --workload")
-    ap.add_argument("--alg", type=int, default=0, help="kernel id (0 = pick from the histogram)")
+    ap.add_argument("--alg", type=int, default=0, help="kernel id (0 = what the analysis picks)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
-    ap.add_argument("--probe", action="store_true",
-                    help="only run the stream / stream+gather probes on --workload (what the chip sustains "
-                         "for this matrix without reduction and write)")
+    ap.add_argument("--cpu-seconds", type=float, default=60.0,
+                    help="budget of the whole CPU baseline leg (split evenly over workloads and thread counts)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run the plain copy kernel on 1 GiB (known traffic, for scaling profiler counters)")
     return ap.parse_args()
@@ -63,8 +76,10 @@ def measure(w, steps, warmup, alg):
 
     dev = lambda a: torch.from_numpy(a).cuda()
     d_rp, d_col, d_val, d_x = dev(w.row_ptr), dev(w.col), dev(w.val), dev(w.x)
-    d_y = dev(w.y.copy())
+    d_y0 = dev(w.y.copy())
+    d_y = d_y0.clone()
     spmm = w.kind == "spmm"
+    restore = w.beta != 0
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     plan = capi.Plan(spmm, alg, w.val.dtype, w.m, w.n, w.nnz, d_rp, ncols=w.ncols, col=d_col, val=d_val)
@@ -80,23 +95,37 @@ def measure(w, steps, warmup, alg):
 
     for _ in range(warmup):
         step()
-    # (a) K steps back to back, bracketed by synchronisation: the whole-job figure
+    # (a) K steps back to back, bracketed by synchronisation: the whole-job figure.  (With
+    #     beta != 0 the output feeds the next call; the values stay finite and the time per call
+    #     does not depend on them.)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    # (b) one HIP event pair per call on the launch stream: per-call device time
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    for i in range(steps):
-        starts[i].record()
-        step()
-        ends[i].record()
-    torch.cuda.synchronize()
-    per_call = np.array([s.elapsed_time(e) for s, e in zip(starts, ends)])
-    # (c) the same call without kept analysis (split points recomputed inside every call, as the
+
+    # (b) one HIP event pair per call on the launch stream, fresh output before every call
+    def timed_calls(count, before=None):
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(count)]
+        ends = [torch.cuda.Event(enable_timing=True) for _ in range(count)]
+        for i in range(count):
+            if restore:
+                d_y.copy_(d_y0)
+            if before is not None:
+                before()
+            starts[i].record()
+            step()
+            ends[i].record()
+        torch.cuda.synchronize()
+        return np.array([s.elapsed_time(e) for s, e in zip(starts, ends)])
+
+    per_call = timed_calls(steps)
+    # (c) cold caches: a 1 GiB sweep between calls evicts the L2s and the Infinity Cache
+    sweep = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    cold = timed_calls(max(5, min(20, steps // 5)), before=lambda: sweep.fill_(1))
+    del sweep
+    # (d) the same call without kept analysis (split points recomputed inside every call, as the
     #     reference does): what a caller that never calls *_analysis / *_preprocess sees
     vt = capi.value_type(w.val.dtype)
     if spmm:
@@ -133,6 +162,7 @@ def measure(w, steps, warmup, alg):
         "ms_per_step": wall_ms,
         "event_ms_mean": float(per_call.mean()), "event_ms_median": float(np.median(per_call)),
         "event_ms_min": float(per_call.min()),
+        "cold_ms_median": float(np.median(cold)),
         "noplan_ms": float(noplan_ms),
     }
     res["gbs"] = nbytes / (wall_ms * 1e-3) / 1e9
@@ -140,7 +170,7 @@ def measure(w, steps, warmup, alg):
     res["gbs_event"] = nbytes / (res["event_ms_mean"] * 1e-3) / 1e9
     res["frac_hbm_peak"] = res["gbs_event"] / HBM_PEAK_GBS
     plan.destroy()
-    del d_rp, d_col, d_val, d_x, d_y, ws, ws2
+    del d_rp, d_col, d_val, d_x, d_y, d_y0, ws, ws2
     torch.cuda.empty_cache()
     return res
 
@@ -167,86 +197,111 @@ def copy_calibration(steps, nbytes=1 << 30):
             "read_plus_write_gbs": 2 * nbytes / (ms * 1e-3) / 1e9}
 
 
-def probe(w, steps):
-    """Stream-only and stream+gather rates for workload w (no reduction, no output)."""
-    import torch
-    from library_amd import capi
-    dev = lambda a: torch.from_numpy(a).cuda()
-    d_col, d_val, d_x = dev(w.col), dev(w.val), dev(w.x)
-    sink = torch.zeros(16, dtype=d_val.dtype, device="cuda")
-    vt = capi.value_type(w.val.dtype)
-    stream = torch.cuda.current_stream().cuda_stream
-    out = {"workload": w.name, "nnz": w.nnz, "stream_bytes": w.nnz * (w.dtype.itemsize + 4)}
-    for mode, key in ((0, "stream"), (1, "stream_gather"), (10, "gather_slice_per_xcd"), (11, "gather_16_slices_2_phases"),
-                      (12, "gather_slices_mixed_over_xcds")):
-        if mode < 10:
-            call = lambda: capi.lib().asx_probe_stream_gather(vt, mode, w.nnz, d_col.data_ptr(), d_val.data_ptr(),
-                                                              d_x.data_ptr(), sink.data_ptr(), stream)
-        else:
-            call = lambda: capi.lib().asx_probe_sliced_gather(vt, mode - 10, w.nnz, w.n, d_col.data_ptr(),
-                                                              d_val.data_ptr(), d_x.data_ptr(), sink.data_ptr(), stream)
-        for _ in range(3):
-            call()
-        torch.cuda.synchronize()
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        for _ in range(steps):
-            call()
-        e.record()
-        torch.cuda.synchronize()
-        ms = s.elapsed_time(e) / steps
-        out[key + "_us"] = ms * 1e3
-        out[key + "_gbs_of_col_val"] = out["stream_bytes"] / (ms * 1e-3) / 1e9
-        out[key + "_gnnz_per_s"] = w.nnz / (ms * 1e-3) / 1e9
-    return out
+def host_cpus():
+    """nproc, sockets and physical cores of this host, and the thread count the baseline uses:
+    the physical cores, capped by the box's CPU share (OMP_NUM_THREADS, 16 on a one-GPU box)."""
+    nproc = os.cpu_count() or 1
+    sockets, cores = set(), set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("physical id"):
+                phys = line.split(":")[1].strip()
+            elif line.startswith("core id"):
+                core = line.split(":")[1].strip()
+            elif not line.strip():
+                if phys is not None and core is not None:
+                    sockets.add(phys)
+                    cores.add((phys, core))
+                phys = core = None
+    except OSError:
+        pass
+    physical = len(cores) or nproc
+    share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or nproc
+    return {"nproc": nproc, "sockets": len(sockets) or 1, "physical_cores": physical, "cpu_share": share,
+            "threads_used": max(1, min(physical, share, nproc))}
 
 
-def cpu_baseline(w, budget_s):
-    """The reference's own CPU path (oracle/_ref, kind "reference") or, where that is not
-    built, the C restatement (kind "port"), timed on this host for the same workload."""
+def _time_calls(call, budget_s, max_calls):
+    """Warm-up call (first touch, thread pool), then as many timed calls as fit the budget."""
     import numpy as np
-    from oracle.bindings import Oracle, Ref
-
-    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 16)
-    nbytes = w.bytes_algorithmic()
-    times = []
-    if Ref.available():
-        kind = "reference"
-        ref = Ref()
-        h = ref.create(w.row_ptr, w.col, w.val, w.n)
-        y = w.y.copy()
-
-        def call():
-            if w.kind == "spmm":
-                ref.mm(h, w.x, w.ncols, w.alpha, w.beta, y, threads)
-            else:
-                ref.mv(h, w.x, w.alpha, w.beta, y, threads)
-    else:
-        kind = "port"
-        orc = Oracle()
-
-        def call():
-            if w.kind == "spmm":
-                orc.spmm(w.row_ptr, w.col, w.val, w.x, w.ncols, w.alpha, w.beta, w.y, threads)
-            else:
-                orc.spmv(w.row_ptr, w.col, w.val, w.x, w.alpha, w.beta, w.y, threads)
     t_start = time.perf_counter()
-    call()  # warm-up (first touch, thread pool)
+    call()
     warm = time.perf_counter() - t_start
-    reps = 0
-    while reps < 1000 and (time.perf_counter() - t_start) < budget_s and (reps < 3 or warm * (reps + 2) < budget_s):
+    times = []
+    while len(times) < max_calls and (time.perf_counter() - t_start) + warm < budget_s:
         t0 = time.perf_counter()
         call()
         times.append(time.perf_counter() - t0)
-        reps += 1
+    warmed = bool(times)
     if not times:
-        times = [warm]
-    t = float(np.median(times))
-    if kind == "reference":
+        times = [warm]  # one call was all the budget allowed: it is the (cold) sample
+    return float(np.median(times)), len(times), warmed
+
+
+def cpu_baseline(w, threads, budget_s):
+    """The reference's own CPU path (oracle/_ref, kind "reference") or, where that is not built,
+    the C restatement (kind "port"), timed on this host for workload w with `threads` OpenMP
+    threads.  SpMV runs at full size.  The reference's SpMM builds a rows x (k/256 + 1) table of
+    ints in every call (hygon/util/partition.cpp:178-201; 17 GB and tens of seconds at this
+    shape), so it is timed on the first 1/16 of the rows of A (B and C at full width), and the
+    restatement (one K block, no table) at full size beside it."""
+    import numpy as np
+    from oracle.bindings import Oracle, Ref
+
+    def rates(nbytes, flops, t):
+        return {"gbs": nbytes / t / 1e9, "gflops": flops / t / 1e9, "ms_per_call": t * 1e3}
+
+    out = {"threads": threads}
+    have_ref = Ref.available()
+    sv = w.dtype.itemsize
+    if w.kind == "spmv":
+        y = w.y.copy()
+        if have_ref:
+            ref = Ref()
+            h = ref.create(w.row_ptr, w.col, w.val, w.n)
+            call = lambda: ref.mv(h, w.x, w.alpha, w.beta, y, threads)
+        else:
+            orc = Oracle()
+            call = lambda: orc.spmv(w.row_ptr, w.col, w.val, w.x, w.alpha, w.beta, w.y, threads)
+        t, n, warmed = _time_calls(call, budget_s, 1000)
+        if have_ref:
+            ref.destroy(h)
+        out.update(rates(w.bytes_algorithmic(), w.flops, t))
+        out.update({"kind": "reference" if have_ref else "port", "calls_timed": n, "warmed_up": warmed,
+                    "sample": f"{w.name} at full size"})
+        return out
+    # SpMM
+    orc = Oracle()
+    if have_ref:
+        rows = max(1, w.m // 16)
+        nz = int(w.row_ptr[rows])
+        rp = np.ascontiguousarray(w.row_ptr[:rows + 1])
+        ref = Ref()
+        h = ref.create(rp, w.col[:nz], w.val[:nz], w.n)
+        Cs = w.y[:rows * w.ncols].copy()
+        call = lambda: ref.mm(h, w.x, w.ncols, w.alpha, w.beta, Cs, threads)
+        t, n, warmed = _time_calls(call, budget_s * 0.6, 20)
         ref.destroy(h)
-    return {"value": nbytes / t / 1e9, "unit": "GB/s", "cores": threads, "kind": kind,
-            "sample": f"{w.name} at full size, median of {len(times)} calls after 1 warm-up, {threads} OpenMP threads",
-            "ms_per_call": t * 1e3, "gflops": w.flops / t / 1e9}
+        ymul = 2 if w.beta != 0 else 1
+        sbytes = nz * (sv + 4) + (rows + 1) * 4 + w.n * w.ncols * sv + rows * w.ncols * sv * ymul
+        out.update(rates(sbytes, 2 * nz * w.ncols, t))
+        out.update({"kind": "reference", "calls_timed": n, "warmed_up": warmed,
+                    "sample": f"{w.name}: the first {rows} of {w.m} rows of A ({nz} stored elements), B and C {w.ncols} wide; "
+                              f"the reference's per-call table of rows x (k/256 + 1) ints is {rows * (w.n // 256 + 1) * 4 / 1e9:.1f} GB "
+                              f"for the sample, {w.m * (w.n // 256 + 1) * 4 / 1e9:.1f} GB at full size"})
+        budget_s *= 0.4
+    Cf = w.y.copy()
+    call = lambda: orc.spmm(w.row_ptr, w.col, w.val, w.x, w.ncols, w.alpha, w.beta, Cf, threads)
+    t, n, warmed = _time_calls(call, budget_s, 20)
+    port = rates(w.bytes_algorithmic(), w.flops, t)
+    port.update({"kind": "port", "calls_timed": n, "warmed_up": warmed,
+                 "sample": f"{w.name} at full size, C restatement of the reference's row kernel with one K block (no table)"})
+    if have_ref:
+        out["restatement_full_size"] = port
+    else:
+        out.update(port)
+    return out
 
 
 def main():
@@ -264,26 +319,35 @@ def main():
     if a.calibrate_copy:
         print(json.dumps(copy_calibration(a.steps)))
         return
-    if a.probe:
-        print(json.dumps(probe(W.CONFIGS[a.workload](), a.steps)))
-        return
     names = [a.workload] if (a.only or a.workload in EXTRA) else ORDER
-    results = {}
-    head_w = None
+    cpus = host_cpus()
+    legs = [cpus["threads_used"]] + ([1] if cpus["threads_used"] > 1 else [])
+    leg_budget = a.cpu_seconds / (len(names) * len(legs))
+    results, cpu_by_workload = {}, {}
     for name in names:
         w = W.CONFIGS[name]()
         results[name] = measure(w, a.steps, a.warmup, a.alg if name == a.workload else 0)
-        if name == a.workload:
-            head_w = w
-        else:
-            del w
+        if not a.no_cpu:
+            rows = []
+            for threads in legs:
+                try:
+                    rows.append(cpu_baseline(w, threads, leg_budget))
+                except Exception as e:  # the baseline is a reported extra; never lose the GPU line to it
+                    rows.append({"threads": threads, "kind": "unavailable", "sample": repr(e)})
+            cpu_by_workload[name] = rows
+        del w
     head = results[a.workload]
     cpu = None
     if not a.no_cpu:
-        try:
-            cpu = cpu_baseline(head_w, a.cpu_seconds)
-        except Exception as e:  # the baseline is a reported extra; never lose the GPU line to it
-            cpu = {"value": None, "unit": "GB/s", "cores": 0, "kind": "unavailable", "sample": repr(e)}
+        c = cpu_by_workload[a.workload][0]
+        cpu = {"value": c.get("gbs"), "unit": "GB/s", "cores": c["threads"], "kind": c.get("kind"),
+               "sample": f"{c.get('sample')}; median of {c.get('calls_timed')} calls after "
+                         f"{'one' if c.get('warmed_up') else 'no'} warm-up call, {c['threads']} OpenMP threads "
+                         f"(host: nproc {cpus['nproc']}, {cpus['sockets']} socket(s), {cpus['physical_cores']} physical cores, "
+                         f"CPU share {cpus['cpu_share']})",
+               "ms_per_call": c.get("ms_per_call"), "gflops": c.get("gflops"),
+               "one_thread": next(({"value": r.get("gbs"), "ms_per_call": r.get("ms_per_call"), "calls_timed": r.get("calls_timed")}
+                                   for r in cpu_by_workload[a.workload] if r["threads"] == 1), None)}
     traffic = MEASURED_TRAFFIC_BYTES.get(a.workload)
     line = {
         "metric": "effective HBM GB/s, CSR " + ("SpMM N=64 fp32" if head["kind"] == "spmm" else f"SpMV {head['dtype']}")
@@ -299,6 +363,8 @@ def main():
                      "frac": head["frac_hbm_peak"], "traffic": traffic, "kernel": head["kernel"],
                      "bytes_per_launch": head["bytes"], "launch_ms": head["event_ms_mean"]},
         "cpu_baseline": cpu,
+        "host_cpus": cpus,
+        "cpu_baseline_by_workload": cpu_by_workload,
         "roofline_by_workload": {n: {"kernel": results[n]["kernel"], "achieved": round(results[n]["gbs_event"], 1),
                                      "frac": round(results[n]["frac_hbm_peak"], 4),
                                      "traffic": MEASURED_TRAFFIC_BYTES.get(n)} for n in names},
