@@ -50,9 +50,13 @@ enum {
     ASX_SPMV_STREAM = 3,  /* LDS-staged row blocks, segmented reduction */
     ASX_SPMV_MERGE = 9,   /* merge-path tiles + ordered carry fix-up */
     ASX_SPMV_FLAT = 15,   /* tiles of 1024 stored elements, register walk + ordered carry fix-up */
-    ASX_SPMV_SLICED = 101 /* not a reference id: stored elements regrouped by column slice, each slice of x
+    ASX_SPMV_SLICED = 101, /* not a reference id: stored elements regrouped by column slice, each slice of x
                              held in LDS; one partial sum per (row, slice), added per row by a second pass
                              (needs a plan from asx_spmv_plan_create) */
+    ASX_SPMV_WINDOW = 102 /* not a reference id: blocks of consecutive rows with their window of x in LDS and
+                             16-bit columns, for matrices whose rows reach only nearby columns
+                             (needs a plan from asx_spmv_plan_create; NOT_SUPPORTED when some 256 rows reach
+                             further than 128 KiB of x) */
 };
 
 /* SpMM kernels (alphasparseSpMMAlg_t values, include/alphasparse/spdef.h:390-402) */

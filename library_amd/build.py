@@ -16,7 +16,7 @@ LIB = os.path.join(HERE, "libalphasparse_amd.so")
 WORKLOADS = os.path.join(HERE, "libasx_workloads.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-HIP_SOURCES = ["asx_analysis.hip", "asx_spmv.hip", "asx_spmm.hip", "asx_capi.hip", "asx_blocked.hip", "asx_coo.hip", "asx_convert.hip", "asx_sliced.hip"]
+HIP_SOURCES = ["asx_analysis.hip", "asx_spmv.hip", "asx_spmm.hip", "asx_capi.hip", "asx_blocked.hip", "asx_coo.hip", "asx_convert.hip", "asx_sliced.hip", "asx_window.hip"]
 CXX_SOURCES = ["asx_rowblocks.cpp", "alphasparse_generic.cpp", "asx_mtx.cpp"]
 
 # packed-fp32 code generation is switched off for all device code

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libalphasparse_amd.so")
 
 R_32F, R_64F = 0, 1
-SPMV_DEFAULT, SPMV_STREAM, SPMV_VECTOR, SPMV_MERGE, SPMV_FLAT, SPMV_SLICED = 0, 3, 6, 9, 15, 101
+SPMV_DEFAULT, SPMV_STREAM, SPMV_VECTOR, SPMV_MERGE, SPMV_FLAT, SPMV_SLICED, SPMV_WINDOW = 0, 3, 6, 9, 15, 101, 102
 SPMM_DEFAULT, SPMM_ROW, SPMM_MERGE, SPMM_BLOCKED = 0, 5, 7, 10
 
 STATUS = {0: "SUCCESS", 1: "NOT_INITIALIZED", 2: "ALLOC_FAILED", 3: "INVALID_VALUE",

@@ -202,6 +202,12 @@ int spmv_impl(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, 
         if (!plan || !plan->sliced.cf) return ASX_STATUS_NOT_INITIALIZED;
         if (plan->n != n) return ASX_STATUS_INVALID_VALUE;
         return launch_spmv_sliced<T>(m, n, alpha, &plan->sliced, x, beta, y, s);
+    case ASX_SPMV_WINDOW:
+        // the row blocks hold a copy of A's columns and values (and the carries of a call) and are
+        // built by asx_spmv_plan_create; no workspace
+        if (!plan || !plan->window.cf) return ASX_STATUS_NOT_INITIALIZED;
+        if (plan->n != n) return ASX_STATUS_INVALID_VALUE;
+        return launch_spmv_window<T>(m, n, alpha, &plan->window, x, beta, y, s);
     default: return ASX_STATUS_NOT_SUPPORTED;
     }
 }
@@ -475,6 +481,7 @@ int asx_plan_destroy(asx_plan *plan)
     if (plan->d_meta) st = status_of(hipFree(plan->d_meta));
     free_blocked(&plan->blocked);
     free_sliced(&plan->sliced);
+    free_window(&plan->window);
     delete plan;
     return st;
 }
@@ -603,6 +610,27 @@ int plan_add_slices(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
     return ASX_STATUS_SUCCESS;
 }
 
+// Builds the row-block copy onto a plan that already holds the histogram.
+constexpr int32_t kWindowMaxRow = 2048;  // longer rows would make the ordered carry pass serial
+template <typename T>
+int plan_add_window(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, hipStream_t s)
+{
+    if (p->stats[0] > kWindowMaxRow) return ASX_STATUS_NOT_SUPPORTED;
+    WindowMatrix wm{};
+    const int st = build_window<T>(p->m, p->n, p->nnz, (int32_t)(kSliceBytes / sizeof(T)), 8192, d_row_ptr, d_col, d_val,
+                                   &wm, s);
+    if (st) return st;
+    if (p->d_meta) (void)hipFree(p->d_meta);
+    p->d_meta = nullptr;
+    p->meta_bytes = 0;
+    p->alg = ASX_SPMV_WINDOW;
+    p->window = wm;
+    p->nunits = wm.ntiles;
+    p->carry_pass = wm.has_carry;
+    p->workspace_bytes = 0;
+    return ASX_STATUS_SUCCESS;
+}
+
 extern "C" {
 
 int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
@@ -612,7 +640,7 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     *out = nullptr;
     if (m < 0 || n < 0 || nnz < 0) return ASX_STATUS_INVALID_SIZE;
     if (value_type != ASX_R_32F && value_type != ASX_R_64F) return ASX_STATUS_NOT_SUPPORTED;
-    const bool want = alg == ASX_SPMV_SLICED;
+    const bool want = alg == ASX_SPMV_SLICED || alg == ASX_SPMV_WINDOW;
     if (want && (m == 0 || nnz == 0 || n == 0)) return ASX_STATUS_INVALID_SIZE;
     if (want && (!d_row_ptr || !d_col || !d_val)) return ASX_STATUS_INVALID_POINTER;
     hipStream_t s = (hipStream_t)stream;
@@ -620,13 +648,23 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     asx_plan *p = nullptr;
     int st = asx_plan_create(&p, 0, want ? ASX_SPMV_VECTOR : alg, value_type, m, n, nnz, d_row_ptr, 1, stream);
     if (st) return st;
-    bool slices = want;
+    if (alg == ASX_SPMV_WINDOW) {
+        st = value_type == ASX_R_64F ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
+                                     : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
+        if (st) {
+            asx_plan_destroy(p);
+            return st;
+        }
+        *out = p;
+        return ASX_STATUS_SUCCESS;
+    }
+    bool slices = alg == ASX_SPMV_SLICED;
     if (alg == ASX_SPMV_DEFAULT && d_col && d_val && sliced_pays(p->hist, m, n, nnz, vsize(value_type)))
         slices = sampled_line_spread(d_col, nnz, vsize(value_type), s) >= kScatteredMinSpread;
     if (slices) {
         st = value_type == ASX_R_64F ? plan_add_slices<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
                                      : plan_add_slices<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
-        if (st && want) {
+        if (st && alg == ASX_SPMV_SLICED) {
             asx_plan_destroy(p);
             return st;
         }
@@ -644,6 +682,9 @@ int asx_plan_update_values(asx_plan *plan, const void *d_val, void *stream)
     if (!plan->is_spmm && plan->alg == ASX_SPMV_SLICED)
         return plan->value_type == ASX_R_64F ? sliced_update_values<double>(&plan->sliced, (const double *)d_val, s)
                                              : sliced_update_values<float>(&plan->sliced, (const float *)d_val, s);
+    if (!plan->is_spmm && plan->alg == ASX_SPMV_WINDOW)
+        return plan->value_type == ASX_R_64F ? window_update_values<double>(&plan->window, (const double *)d_val, s)
+                                             : window_update_values<float>(&plan->window, (const float *)d_val, s);
     if (plan->is_spmm && plan->alg == ASX_SPMM_BLOCKED)
         return plan->value_type == ASX_R_64F ? blocked_update_values<double>(&plan->blocked, (const double *)d_val, s)
                                              : blocked_update_values<float>(&plan->blocked, (const float *)d_val, s);
@@ -653,7 +694,8 @@ int asx_plan_update_values(asx_plan *plan, const void *d_val, void *stream)
 int asx_plan_holds_values(const asx_plan *plan)
 {
     if (!plan) return 0;
-    return (!plan->is_spmm && plan->alg == ASX_SPMV_SLICED) || (plan->is_spmm && plan->alg == ASX_SPMM_BLOCKED);
+    return (!plan->is_spmm && (plan->alg == ASX_SPMV_SLICED || plan->alg == ASX_SPMV_WINDOW)) ||
+           (plan->is_spmm && plan->alg == ASX_SPMM_BLOCKED);
 }
 
 int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill)

@@ -147,6 +147,33 @@ int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s);
 template <typename T>
 int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, hipStream_t s);
 
+// ---- row blocks with their window of x in LDS (asx_window.hip) ----
+// Blocks of `rows_per_block` consecutive rows whose columns all lie inside a window of at most
+// `width` - 1 columns; one workgroup per block copies the window into LDS and streams the block's
+// stored elements as tiles (16-bit column-in-window + row-start flag, as the sliced kernel's);
+// every row owns at least one slot, so a tile's runs are consecutive rows and go straight to y.
+struct WindowMatrix {
+    int32_t width;           // LDS entries per window; the last one holds the zero empty rows point at
+    int32_t rows_per_block;
+    int32_t nblocks;
+    int32_t ntiles;
+    int has_carry;           // some tile starts inside a row: the ordered carry pass is needed
+    void *val;               // ntiles * kSlicedTile values (a copy of A's; pads are 0)
+    void *carry;             // ntiles values
+    uint16_t *cf;            // ntiles * kSlicedTile: column - window start, bit 15 = first slot of a row (or tile)
+    int32_t *perm;           // where each stored copy comes from in A's val (-1 for pads)
+    int32_t *tile_word;      // ntiles: row of the tile's first slot, bit 31 = the tile starts inside that row
+    int32_t *wg_tab;         // nblocks x 4: window start, first tile, end tile, end row
+};
+template <typename T>
+int build_window(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t max_rows_per_block, const int32_t *row_ptr,
+                 const int32_t *col, const T *val, WindowMatrix *out, hipStream_t s);
+void free_window(WindowMatrix *p);
+template <typename T>
+int window_update_values(const WindowMatrix *wm, const T *val, hipStream_t s);
+template <typename T>
+int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, hipStream_t s);
+
 inline int32_t merge_tiles(int32_t m, int32_t nnz) { return (int32_t)ceil_div64((int64_t)m + nnz, kMergeTile); }
 inline int32_t flat_tiles(int32_t nnz) { int32_t t = (int32_t)ceil_div64(nnz, kFlatTile); return t < 1 ? 1 : t; }
 inline int32_t stream_blocks(int32_t nnz) { return (int32_t)ceil_div64(nnz, kStreamTile); }
@@ -170,4 +197,5 @@ struct asx_plan {
     size_t workspace_bytes;
     asx::BlockedMatrix blocked;  // only for ASX_SPMM_BLOCKED plans
     asx::SlicedMatrix sliced;    // only for ASX_SPMV_SLICED plans
+    asx::WindowMatrix window;    // only for ASX_SPMV_WINDOW plans
 };

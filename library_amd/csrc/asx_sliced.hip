@@ -30,24 +30,13 @@
 #include <vector>
 
 #include "asx_internal.hpp"
+#include "asx_tiles.hpp"
 
 namespace asx {
 
 namespace {
 
 constexpr int32_t kPadRow = 0x7fffffff;
-
-// Position of logical element e (= 4*lane + j) of a tile in the tile's value storage: the order
-// in which 16-byte loads at consecutive lanes deliver 4 consecutive elements to each lane.
-template <typename T>
-__host__ __device__ __forceinline__ int sliced_val_pos(int e)
-{
-    if (sizeof(T) == 8) {  // two loads of 2 doubles: [half][lane][2]
-        const int lane = e >> 2, j = e & 3;
-        return (j >> 1) * 128 + lane * 2 + (j & 1);
-    }
-    return e;  // one load of 4 floats
-}
 
 __global__ __launch_bounds__(kBlock) void k_sliced_keys(const int32_t *__restrict__ col, int32_t nnz, int32_t width,
                                                         int32_t *__restrict__ keys, int32_t *__restrict__ idx)
@@ -115,7 +104,7 @@ __global__ __launch_bounds__(kBlock) void k_sliced_place(const int32_t *__restri
     lhead[d] = head ? 1 : 0;
     cf[d] = (uint16_t)((col[src] - sl * width) | (head ? 0x8000 : 0));
     const int64_t t = d / kSlicedTile;
-    const int64_t phys = t * kSlicedTile + sliced_val_pos<T>((int)(d % kSlicedTile));
+    const int64_t phys = t * kSlicedTile + tile_val_pos<T>((int)(d % kSlicedTile));
     val_out[phys] = val[src];
     perm[phys] = src;
 }
@@ -178,84 +167,12 @@ __global__ __launch_bounds__(kBlock) void k_sliced_regather(const int32_t *__res
 }
 
 // ---- pass 1 ------------------------------------------------------------------------------
+// a run's sum goes to the tile's partial sums, at the run's rank
 template <typename T>
-struct SlicedTileLoad;
-template <>
-struct SlicedTileLoad<double> {
-    static __device__ __forceinline__ void load(const double *tile, int lane, double v[4])
-    {
-        typedef double f64x2 __attribute__((ext_vector_type(2)));
-        const f64x2 *q = reinterpret_cast<const f64x2 *>(tile);
-        const f64x2 a = __builtin_nontemporal_load(q + lane);
-        const f64x2 b = __builtin_nontemporal_load(q + 64 + lane);
-        v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
-    }
+struct StorePartial {
+    T *out;
+    __device__ __forceinline__ void operator()(int rank, T v) const { out[rank] = v; }
 };
-template <>
-struct SlicedTileLoad<float> {
-    static __device__ __forceinline__ void load(const float *tile, int lane, float v[4])
-    {
-        typedef float f32x4 __attribute__((ext_vector_type(4)));
-        const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(tile) + lane);
-        v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w;
-    }
-};
-
-__device__ __forceinline__ int lanes_below(unsigned long long mask)
-{
-    return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0));
-}
-
-// One tile's stored elements as the loads deliver them.
-template <typename T>
-struct SlicedTile {
-    uint32_t c01, c23;  // 4 x (column in slice | run start << 15)
-    T v[4];
-    int32_t base;  // index of the tile's first partial sum
-};
-template <typename T>
-__device__ __forceinline__ void sliced_tile_load(SlicedTile<T> &tl, int32_t t, int lane, const uint16_t *__restrict__ cf,
-                                                 const T *__restrict__ val, const int32_t *__restrict__ tile_base)
-{
-    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-    const u32x2 cw = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(cf + (int64_t)t * kSlicedTile) + lane);
-    tl.c01 = cw.x;
-    tl.c23 = cw.y;
-    SlicedTileLoad<T>::load(val + (int64_t)t * kSlicedTile, lane, tl.v);
-    tl.base = tile_base[t];
-}
-
-// Products, running sums, wave scan and the stores of one tile.
-template <typename T>
-__device__ __forceinline__ void sliced_tile_reduce(const SlicedTile<T> &tl, int lane, const T *xs, T *__restrict__ partial)
-{
-    const bool f0 = (tl.c01 >> 15) & 1, f1 = tl.c01 >> 31, f2 = (tl.c23 >> 15) & 1, f3 = tl.c23 >> 31;
-    const T p0 = tl.v[0] * xs[tl.c01 & 0x7fff], p1 = tl.v[1] * xs[(tl.c01 >> 16) & 0x7fff];
-    const T p2 = tl.v[2] * xs[tl.c23 & 0x7fff], p3 = tl.v[3] * xs[(tl.c23 >> 16) & 0x7fff];
-    // running sums that restart at every run start
-    const T r0 = p0;
-    const T r1 = f1 ? p1 : r0 + p1;
-    const T r2 = f2 ? p2 : r1 + p2;
-    const T r3 = f3 ? p3 : r2 + p3;
-    const int nh = (int)f0 + (int)f1 + (int)f2 + (int)f3;
-    const unsigned long long m0 = __ballot(f0), m1 = __ballot(f1), m2 = __ballot(f2), m3 = __ballot(f3);
-    const int before = lanes_below(m0) + lanes_below(m1) + lanes_below(m2) + lanes_below(m3);
-    const int total = __popcll(m0) + __popcll(m1) + __popcll(m2) + __popcll(m3);
-    // sum of the run that is open at the end of each lane, over the lanes it spans
-    const T open = wave_segsum_dpp<T>(r3, nh != 0);
-    const T cin = wave_shift_up1<T>(open);  // what earlier lanes hold of the run open at this lane's start
-    // a run start closes the run before it
-    T *out = partial + tl.base;
-    int hb = before;
-    if (f0 && hb > 0) out[hb - 1] = cin;
-    hb += f0;
-    if (f1) out[hb - 1] = f0 ? r0 : cin + r0;
-    hb += f1;
-    if (f2) out[hb - 1] = (f0 | f1) ? r1 : cin + r1;
-    hb += f2;
-    if (f3) out[hb - 1] = (f0 | f1 | f2) ? r2 : cin + r2;
-    if (lane == kWave - 1) out[total - 1] = open;
-}
 
 template <typename T, int WIDTH, int NW, int D>
 __global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const int4 *__restrict__ wg_tab,
@@ -271,33 +188,11 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const 
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     // the first tiles' loads go out before the slice of x is fetched (they do not need it)
     const int32_t last = wg.z - 1;
-    SlicedTile<T> tl[D];
+    Tile<T> tl[D];
     int32_t t = wg.y + wave;
 #pragma unroll
-    for (int d = 0; d < D; ++d) sliced_tile_load<T>(tl[d], t + d * NW < last ? t + d * NW : last, lane, cf, val, tile_base);
-    {
-        // the slice of x: every load issued before the first LDS write (one memory round trip)
-        constexpr int V = 16 / sizeof(T);                 // values per 16-byte load
-        constexpr int PER = WIDTH / (NW * kWave * V);     // loads per thread
-        static_assert(PER * NW * kWave * V == WIDTH, "slice width must be a multiple of the workgroup's loads");
-        typedef T vec_t __attribute__((ext_vector_type(V)));
-        vec_t buf[PER];
-        const bool whole = cnt == WIDTH && ((uintptr_t)(x + c0) % 16) == 0;
-        if (whole) {
-#pragma unroll
-            for (int k = 0; k < PER; ++k)
-                buf[k] = reinterpret_cast<const vec_t *>(x + c0)[k * NW * kWave + threadIdx.x];
-        } else {
-#pragma unroll
-            for (int k = 0; k < PER; ++k) {
-                const int i0 = (k * NW * kWave + (int)threadIdx.x) * V;
-#pragma unroll
-                for (int e = 0; e < V; ++e) buf[k][e] = i0 + e < cnt ? x[c0 + i0 + e] : T(0);
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < PER; ++k) reinterpret_cast<vec_t *>(xs)[k * NW * kWave + threadIdx.x] = buf[k];
-    }
+    for (int d = 0; d < D; ++d) tile_load<T>(tl[d], t + d * NW < last ? t + d * NW : last, lane, cf, val, tile_base);
+    load_x_window<T, WIDTH, NW * kWave>(xs, x, c0, cnt);
     __syncthreads();
     // D tiles in turn; a tile's loads are issued D steps ahead, right after the stores of the tile
     // that used the buffer before it.  The loads are unconditional (past the end they re-read the
@@ -306,8 +201,8 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const 
     while (t < wg.z) {  // uniform over the wave
 #pragma unroll
         for (int d = 0; d < D; ++d) {
-            if (t + d * NW < wg.z) sliced_tile_reduce<T>(tl[d], lane, xs, partial);
-            sliced_tile_load<T>(tl[d], t + (D + d) * NW < last ? t + (D + d) * NW : last, lane, cf, val, tile_base);
+            if (t + d * NW < wg.z) tile_reduce<T>(tl[d], lane, xs, StorePartial<T>{partial + tl[d].base});
+            tile_load<T>(tl[d], t + (D + d) * NW < last ? t + (D + d) * NW : last, lane, cf, val, tile_base);
         }
         t += D * NW;
     }
