@@ -166,8 +166,8 @@ struct WindowMatrix {
     int32_t *wg_tab;         // nblocks x 4: window start, first tile, end tile, end row
 };
 template <typename T>
-int build_window(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t max_rows_per_block, const int32_t *row_ptr,
-                 const int32_t *col, const T *val, WindowMatrix *out, hipStream_t s);
+int build_window(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t max_rows_per_block, int32_t max_reload,
+                 const int32_t *row_ptr, const int32_t *col, const T *val, WindowMatrix *out, hipStream_t s);
 void free_window(WindowMatrix *p);
 template <typename T>
 int window_update_values(const WindowMatrix *wm, const T *val, hipStream_t s);

@@ -259,8 +259,8 @@ void free_window(WindowMatrix *p)
 }
 
 template <typename T>
-int build_window(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t max_rows_per_block, const int32_t *row_ptr,
-                 const int32_t *col, const T *val, WindowMatrix *out, hipStream_t s)
+int build_window(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t max_rows_per_block, int32_t max_reload,
+                 const int32_t *row_ptr, const int32_t *col, const T *val, WindowMatrix *out, hipStream_t s)
 {
     WindowMatrix wm{};
     if (m <= 0 || nnz <= 0 || n <= 0) return ASX_STATUS_INVALID_SIZE;
@@ -310,8 +310,12 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t max_r
         ASX_TRY(hipMemcpyAsync(h_small, d_small, sizeof(int32_t), hipMemcpyDeviceToHost, s));
         ASX_TRY(hipStreamSynchronize(s));
         if (h_small[0] <= width - 1) {
-            wm.rows_per_block = rows;
-            wm.nblocks = nb;
+            // every workgroup fetches its whole window: with a bound on that (max_reload > 0), blocks
+            // whose window is more than max_reload times their rows wide are turned down
+            if (max_reload <= 0 || h_small[0] <= (int64_t)max_reload * rows) {
+                wm.rows_per_block = rows;
+                wm.nblocks = nb;
+            }
             break;
         }
     }
@@ -393,11 +397,19 @@ template <typename T>
 int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, hipStream_t s)
 {
     if (m <= 0) return ASX_STATUS_SUCCESS;
-    constexpr int kWidth = 131072 / sizeof(T);
-    if (wm->width != kWidth) return ASX_STATUS_INVALID_VALUE;
-    hipLaunchKernelGGL((k_spmv_window<T, kWidth, 16, 2>), dim3((unsigned)wm->nblocks), dim3(16 * kWave), 0, s, n, alpha,
-                       beta, reinterpret_cast<const int4 *>(wm->wg_tab), wm->cf, (const T *)wm->val, wm->tile_word, x, y,
-                       (T *)wm->carry);
+#define ASX_WIN(W)                                                                                                  \
+    hipLaunchKernelGGL((k_spmv_window<T, W, 16, 2>), dim3((unsigned)wm->nblocks), dim3(16 * kWave), 0, s, n, alpha, beta, \
+                       reinterpret_cast<const int4 *>(wm->wg_tab), wm->cf, (const T *)wm->val, wm->tile_word, x, y,     \
+                       (T *)wm->carry)
+    if (wm->width == (int)(131072 / sizeof(T)))
+        ASX_WIN(131072 / sizeof(T));
+    else if (wm->width == (int)(81920 / sizeof(T)))
+        ASX_WIN(81920 / sizeof(T));
+    else if (sizeof(T) == 8 && wm->width == 20480)
+        ASX_WIN(20480);
+    else
+        return ASX_STATUS_INVALID_VALUE;
+#undef ASX_WIN
     if (wm->has_carry)
         hipLaunchKernelGGL((k_window_fixup<T>), dim3((unsigned)ceil_div64(wm->ntiles, kBlock)), dim3(kBlock), 0, s,
                            wm->ntiles, alpha, wm->tile_word, (const T *)wm->carry, y);
@@ -405,8 +417,8 @@ int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, co
 }
 
 #define ASX_INST(T)                                                                                               \
-    template int build_window<T>(int32_t, int32_t, int32_t, int32_t, int32_t, const int32_t *, const int32_t *,  \
-                                 const T *, WindowMatrix *, hipStream_t);                                        \
+    template int build_window<T>(int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, const int32_t *,         \
+                                 const int32_t *, const T *, WindowMatrix *, hipStream_t);                                        \
     template int window_update_values<T>(const WindowMatrix *, const T *, hipStream_t);                           \
     template int launch_spmv_window<T>(int32_t, int32_t, T, const WindowMatrix *, const T *, T, T *, hipStream_t);
 ASX_INST(float)

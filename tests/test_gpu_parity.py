@@ -364,8 +364,22 @@ def test_benchmark_configs_full_size(torch, capi, oracle):
                     assert_close(outs[-1], ref, scale, w.dtype, f"{name} sliced alg={alg} rep={rep}")
                 assert np.array_equal(outs[0], outs[1]), "two calls through one plan must agree bit for bit"
                 plan.destroy()
-        else:  # regular columns: DEFAULT with columns and values behaves as without
-            plan = capi.Plan(False, capi.SPMV_DEFAULT, w.val.dtype, w.m, w.n, w.nnz, d[0], col=d[1], val=d[2])
+        else:
+            # rows that reach only nearby columns: the row-block kernel with its window of x in LDS,
+            # forced and as DEFAULT's choice; without columns and values DEFAULT stays row-ordered
+            for alg in (capi.SPMV_WINDOW, capi.SPMV_DEFAULT):
+                plan = capi.Plan(False, alg, w.val.dtype, w.m, w.n, w.nnz, d[0], col=d[1], val=d[2])
+                assert plan.alg == capi.SPMV_WINDOW and plan.holds_values and plan.workspace_bytes == 0
+                outs = []
+                for rep in range(2):
+                    y = dev(torch, w.y)
+                    capi.spmv(d[0], d[1], d[2], d[3], y, w.alpha, w.beta, alg=alg, plan=plan)
+                    torch.cuda.synchronize()
+                    outs.append(y.cpu().numpy())
+                    assert_close(outs[-1], ref, scale, w.dtype, f"{name} window alg={alg} rep={rep}")
+                assert np.array_equal(outs[0], outs[1])
+                plan.destroy()
+            plan = capi.Plan(False, capi.SPMV_DEFAULT, w.val.dtype, w.m, w.n, w.nnz, d[0])
             assert plan.alg == capi.SPMV_FLAT and not plan.holds_values
             plan.destroy()
         del d
@@ -617,6 +631,74 @@ def test_spmv_sliced_kernel_shapes(torch, capi, oracle, dtype):
     assert L.asx_plan_holds_values(None) == 0
 
 
+def _banded_random(rng, m, n, half, dens, dtype, empty=0.1, longrow=None):
+    """Rows around the (scaled) diagonal: columns within +-half of it, a fraction `dens` of them
+    stored, some rows empty, optionally one row that takes every column in reach."""
+    rp = np.zeros(m + 1, np.int32)
+    cl = []
+    for r in range(m):
+        c = int(r * (n - 1) / max(m - 1, 1))
+        lo, hi = max(0, c - half), min(n, c + half + 1)
+        k = 0 if rng.random() < empty else max(1, int(rng.binomial(hi - lo, dens)))
+        if longrow is not None and r == longrow:
+            k = hi - lo
+        cs = np.sort(rng.choice(np.arange(lo, hi), size=min(k, hi - lo), replace=False))
+        cl.append(cs)
+        rp[r + 1] = rp[r] + cs.size
+    col = np.concatenate(cl).astype(np.int32)
+    return rp, col, rng.uniform(-1, 1, col.size).astype(dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
+    """The row-block kernel forced on banded matrices: empty rows (a slot of their own), rows cut by
+    tile starts (carry pass), a row of 1401 spanning six tiles, a block whose last tile is mostly
+    padding, a rectangular matrix, the 5-point stencil, beta = 0 over NaN, two calls through one
+    plan, a value update; and NOT_SUPPORTED for rows that reach further than a window."""
+    rng = np.random.default_rng(93)
+    from library_amd import workloads as W
+    cases = []
+    for (m, n, half, dens, lr) in ((3000, 3000, 40, 0.3, None), (5000, 9000, 700, 0.02, 2500), (700, 700, 300, 0.9, 10),
+                                   (20000, 20000, 3, 1.0, None), (257, 300, 100, 0.2, None), (1, 5, 2, 1.0, None)):
+        cases.append((f"band {m}x{n} +-{half}", _banded_random(rng, m, n, half, dens, dtype, longrow=lr), n))
+    st = W.stencil5_f64(300, 200)
+    cases.append(("stencil 300x200", (st.row_ptr, st.col, st.val.astype(dtype)), st.n))
+    for name, (rp, col, val), n in cases:
+        m = rp.size - 1
+        x = rng.uniform(-1, 1, n).astype(dtype)
+        y0 = rng.uniform(-1, 1, m).astype(dtype)
+        d = [dev(torch, a) for a in (rp, col, val, x)]
+        plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
+        assert plan.alg == capi.SPMV_WINDOW and plan.holds_values and plan.workspace_bytes == 0
+        for alpha, beta in ((1.5, 0.5), (1.0, 0.0), (-2.0, 1.0)):
+            ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 2)
+            scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
+            for rep in range(2):
+                y = dev(torch, y0 if beta else np.full(m, np.nan, dtype=dtype))
+                capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_WINDOW, plan=plan)
+                torch.cuda.synchronize()
+                assert_close(y.cpu().numpy(), ref, scale, dtype, f"{name} a={alpha} b={beta} rep={rep}")
+        val2 = rng.uniform(-1, 1, val.size).astype(dtype)
+        d2 = dev(torch, val2)
+        plan.update_values(d2)
+        y = dev(torch, y0)
+        capi.spmv(d[0], d[1], d2, d[3], y, 1.5, 0.5, alg=capi.SPMV_WINDOW, plan=plan)
+        torch.cuda.synchronize()
+        assert_close(y.cpu().numpy(), oracle.spmv(rp, col, val2, x, dtype(1.5), dtype(0.5), y0, 2),
+                     spmv_scale(rp, col, val2, x, 1.5, 0.5, y0), dtype, f"{name} updated values")
+        plan.destroy()
+    # rows that reach far (uniform random columns over 200 000) are not this kernel's matrix; a row
+    # longer than 2048 is not either
+    L = capi.lib()
+    for lens, ncols in ((rng.integers(1, 9, 2000), 200000), (np.r_[np.full(50, 3), 2500, np.full(50, 3)], 2600)):
+        rp, col, val = csr_from_lengths(lens, ncols, 5, dtype)
+        d = [dev(torch, a) for a in (rp, col, val)]
+        h = capi.C.c_void_p()
+        assert L.asx_spmv_plan_create(capi.C.byref(h), capi.SPMV_WINDOW, capi.value_type(np.dtype(dtype)), rp.size - 1,
+                                      ncols, col.size, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None) == 6
+        assert not h.value
+
+
 def test_default_workspace_covers_every_choice(torch, capi, oracle):
     """alphasparseSpMV_bufferSize(DEFAULT) is asx_spmv_workspace_bytes(DEFAULT): whatever kernel a
     DEFAULT plan settles on must fit in it.  Hypersparse (the plan takes the merge-path kernel,
@@ -691,6 +773,20 @@ def test_spmv_random_shapes_all_kernels(torch, capi, oracle):
             torch.cuda.synchronize()
             assert_close(y.cpu().numpy(), ref, scale, dtype, f"case {case} kind {kind} sliced")
             plan.destroy()
+            # the row-block kernel where it applies (columns within reach, no row longer than 2048)
+            h = capi.C.c_void_p()
+            rc = capi.lib().asx_spmv_plan_create(capi.C.byref(h), capi.SPMV_WINDOW, capi.value_type(np.dtype(dtype)),
+                                                 rp.size - 1, ncols, col.size, capi._ptr(d[0]), capi._ptr(d[1]),
+                                                 capi._ptr(d[2]), None)
+            assert rc in (0, 6), rc
+            if rc == 0:
+                y = dev(torch, y0)
+                fn = capi.lib().asx_spmv_csr_f64 if dtype == np.float64 else capi.lib().asx_spmv_csr_f32
+                assert fn(h, capi.SPMV_WINDOW, rp.size - 1, ncols, col.size, alpha, capi._ptr(d[0]), capi._ptr(d[1]),
+                          capi._ptr(d[2]), capi._ptr(d[3]), beta, capi._ptr(y), None, 0, capi._stream()) == 0
+                torch.cuda.synchronize()
+                assert_close(y.cpu().numpy(), ref, scale, dtype, f"case {case} kind {kind} window")
+                capi.lib().asx_plan_destroy(h)
 
 
 # ------------------------------------------------------------------ measurement helper
