@@ -53,10 +53,10 @@ enum {
     ASX_SPMV_SLICED = 101, /* not a reference id: stored elements regrouped by column slice, each slice of x
                              held in LDS; one partial sum per (row, slice), added per row by a second pass
                              (needs a plan from asx_spmv_plan_create) */
-    ASX_SPMV_WINDOW = 102 /* not a reference id: blocks of consecutive rows with their window of x in LDS and
-                             16-bit columns, for matrices whose rows reach only nearby columns
+    ASX_SPMV_WINDOW = 102 /* not a reference id: chains of blocks of consecutive rows with a sliding window of x
+                             in LDS and 16-bit columns, for matrices whose rows reach only nearby columns
                              (needs a plan from asx_spmv_plan_create; NOT_SUPPORTED when some 256 rows reach
-                             further than 128 KiB of x) */
+                             over 16376 columns or more, or a row is longer than 2048) */
 };
 
 /* SpMM kernels (alphasparseSpMMAlg_t values, include/alphasparse/spdef.h:390-402) */
@@ -196,10 +196,14 @@ int asx_spmm_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, in
  * distinct 128-byte lines of x per tile) and a cost model over the row-length histogram and the
  * sizes puts it at least 10 % ahead of the row-ordered kernels; the choice depends on the matrix
  * alone, not on timings.  Otherwise as asx_plan_create.  No counterpart in the reference (its
- * alphasparseSpMV_analysis is a stub).  Synchronises `stream`. */
+ * alphasparseSpMV_analysis is a stub).  alg = ASX_SPMV_WINDOW builds the row-block copy for the
+ * kernel that keeps a sliding window of x in LDS (again a COPY of columns and values, and the
+ * carry slots of a call); DEFAULT picks it, when the sliced kernel is not chosen, for nnz >= 2^21
+ * and rows no longer than 2048 whenever the matrix qualifies (every 256 consecutive rows reach
+ * over fewer than 16376 columns).  Synchronises `stream`. */
 int asx_spmv_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
                          const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, void *stream);
-/* Brings a plan that holds a copy of A's values (ASX_SPMV_SLICED, ASX_SPMM_BLOCKED) up to date
+/* Brings a plan that holds a copy of A's values (ASX_SPMV_SLICED, ASX_SPMV_WINDOW, ASX_SPMM_BLOCKED) up to date
  * with d_val (same sparsity pattern as when the plan was built); asynchronous on `stream`.  For
  * the other kernels, which read the caller's values in every call, it does nothing.
  * asx_plan_holds_values tells the two kinds apart.  No counterpart in the reference. */

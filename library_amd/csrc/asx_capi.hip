@@ -613,13 +613,14 @@ int plan_add_slices(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
 // Builds the row-block copy onto a plan that already holds the histogram.
 constexpr int32_t kWindowMaxRow = 2048;  // longer rows would make the ordered carry pass serial
 template <typename T>
-int plan_add_window(asx_plan *p, int32_t max_reload, const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val,
-                    hipStream_t s)
+int plan_add_window(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, hipStream_t s)
 {
     if (p->stats[0] > kWindowMaxRow) return ASX_STATUS_NOT_SUPPORTED;
+    int cus = 256;
+    (void)asx_device_info(&cus, nullptr);
     WindowMatrix wm{};
-    const int st = build_window<T>(p->m, p->n, p->nnz, (int32_t)(kSliceBytes / sizeof(T)), 8192, max_reload, d_row_ptr,
-                                   d_col, d_val, &wm, s);
+    // one chain of row blocks per compute unit for fp64 (128 KiB of LDS each), two for fp32
+    const int st = build_window<T>(p->m, p->n, p->nnz, cus * (sizeof(T) == 4 ? 2 : 1), d_row_ptr, d_col, d_val, &wm, s);
     if (st) return st;
     if (p->d_meta) (void)hipFree(p->d_meta);
     p->d_meta = nullptr;
@@ -650,8 +651,8 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     int st = asx_plan_create(&p, 0, want ? ASX_SPMV_VECTOR : alg, value_type, m, n, nnz, d_row_ptr, 1, stream);
     if (st) return st;
     if (alg == ASX_SPMV_WINDOW) {
-        st = value_type == ASX_R_64F ? plan_add_window<double>(p, 0, d_row_ptr, d_col, (const double *)d_val, s)
-                                     : plan_add_window<float>(p, 0, d_row_ptr, d_col, (const float *)d_val, s);
+        st = value_type == ASX_R_64F ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
+                                     : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
         if (st) {
             asx_plan_destroy(p);
             return st;
@@ -672,13 +673,12 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
         // DEFAULT: no slices (out of memory, ...) is not an error; the row-ordered plan stands
     } else if (alg == ASX_SPMV_DEFAULT && d_col && d_val && nnz >= kSlicedMinNnz && p->stats[0] <= kWindowMaxRow &&
                (p->alg == ASX_SPMV_FLAT || p->alg == ASX_SPMV_MERGE)) {
-        // rows that reach only nearby columns: row blocks with their window of x in LDS (measured
-        // 14 % faster than the flat kernel on the 5-point stencil, 23 % on a band of 19); the build
+        // rows that reach only nearby columns: row blocks with a sliding window of x in LDS (measured
+        // 23 % faster than the flat kernel on the 5-point stencil, 20 % on a band of 19); the build
         // reports NOT_SUPPORTED when some 256 rows reach further than a window, and then, as after
-        // any other failure, the row-ordered plan stands.  A workgroup fetches its whole window:
-        // blocks whose window is more than 4 times their rows wide are turned down
-        (void)(value_type == ASX_R_64F ? plan_add_window<double>(p, 4, d_row_ptr, d_col, (const double *)d_val, s)
-                                       : plan_add_window<float>(p, 4, d_row_ptr, d_col, (const float *)d_val, s));
+        // any other failure, the row-ordered plan stands
+        (void)(value_type == ASX_R_64F ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
+                                       : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, s));
     }
     *out = p;
     return ASX_STATUS_SUCCESS;

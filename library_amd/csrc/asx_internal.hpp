@@ -147,27 +147,29 @@ int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s);
 template <typename T>
 int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, hipStream_t s);
 
-// ---- row blocks with their window of x in LDS (asx_window.hip) ----
-// Blocks of `rows_per_block` consecutive rows whose columns all lie inside a window of at most
-// `width` - 1 columns; one workgroup per block copies the window into LDS and streams the block's
-// stored elements as tiles (16-bit column-in-window + row-start flag, as the sliced kernel's);
-// every row owns at least one slot, so a tile's runs are consecutive rows and go straight to y.
+// ---- row blocks with a sliding window of x in LDS (asx_window.hip) ----
+// Blocks of `rows_per_block` consecutive rows whose columns all lie inside fewer than 16384
+// columns, chained: a workgroup walks a chain of blocks with LDS as a ring over the columns of x
+// and fetches, per block, only the columns that are new.  The stored elements stream as tiles
+// (16-bit column mod 16384 + row-start flag, as the sliced kernel's); every row owns at least one
+// slot, so a tile's runs are consecutive rows and go straight to y.
 struct WindowMatrix {
-    int32_t width;           // LDS entries per window; the last one holds the zero empty rows point at
     int32_t rows_per_block;
     int32_t nblocks;
+    int32_t nchains;         // workgroups
     int32_t ntiles;
     int has_carry;           // some tile starts inside a row: the ordered carry pass is needed
     void *val;               // ntiles * kSlicedTile values (a copy of A's; pads are 0)
     void *carry;             // ntiles values
-    uint16_t *cf;            // ntiles * kSlicedTile: column - window start, bit 15 = first slot of a row (or tile)
+    uint16_t *cf;            // ntiles * kSlicedTile: column mod 16384, bit 15 = first slot of a row (or tile)
     int32_t *perm;           // where each stored copy comes from in A's val (-1 for pads)
-    int32_t *tile_word;      // ntiles: row of the tile's first slot, bit 31 = the tile starts inside that row
-    int32_t *wg_tab;         // nblocks x 4: window start, first tile, end tile, end row
+    int32_t *tile_info;      // ntiles x 2: row of the tile's first slot (bit 31: the tile starts inside it), rows in the tile
+    int32_t *blocks;         // nblocks x 4: first tile, end tile, columns to fetch before the block (from, to)
+    int32_t *chains;         // nchains x 2: first block, end block
 };
 template <typename T>
-int build_window(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t max_rows_per_block, int32_t max_reload,
-                 const int32_t *row_ptr, const int32_t *col, const T *val, WindowMatrix *out, hipStream_t s);
+int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const int32_t *row_ptr, const int32_t *col,
+                 const T *val, WindowMatrix *out, hipStream_t s);
 void free_window(WindowMatrix *p);
 template <typename T>
 int window_update_values(const WindowMatrix *wm, const T *val, hipStream_t s);

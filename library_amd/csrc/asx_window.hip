@@ -1,16 +1,20 @@
-// Row-block CSR SpMV with the block's window of x in LDS, for matrices whose rows reach only
+// Row-block CSR SpMV with a sliding window of x in LDS, for matrices whose rows reach only
 // nearby columns (stencils, banded and finite-element matrices).
 //
 // The row-ordered kernels read 4 bytes of column index per stored element, the row offsets, and
 // gather x through the L2 (one request per stored element).  Here the rows are cut, once (plan
-// build), into blocks of R consecutive rows whose columns all lie inside a window of at most
-// 128 KiB of x; a workgroup copies its window into LDS and streams its block's stored elements as
-// tiles of 256 with a 16-bit column-in-window and a "first element of a row" flag per element
+// build), into blocks of R consecutive rows whose columns all lie inside a window of fewer than
+// kWindowCols columns, and consecutive blocks are chained: a workgroup walks its chain of blocks
+// with LDS as a ring over the columns of x (column c lives at c mod kWindowCols), so that from
+// one block to the next only the columns that are new are fetched - while the block before is
+// still being multiplied - and x crosses the L2 once.  The block's stored elements stream as
+// tiles of 256 with a 16-bit column-mod-window and a "first element of a row" flag per element
 // (10 instead of 12.8 bytes per stored element in fp64; no row offsets are read).  Every row owns
-// at least one slot (an empty row gets a zero that points at a zero in LDS), so the runs of a
-// tile are consecutive rows and a run's sum goes straight to y.  A tile that starts inside a row
-// puts that first sum into a carry slot instead, and an ordered pass adds the carries to y
-// afterwards (no atomics; results are bit-reproducible).
+// at least one slot (an empty row gets a zero that points at a zero in LDS), so the runs of a tile
+// are consecutive rows and a run's sum goes straight to y.  Rows of up to 16 stored elements are
+// never cut by a tile start (the tile is padded instead); a longer row that is cut leaves its
+// later pieces in carry slots, which an ordered pass adds to y afterwards (no atomics; results are
+// bit-reproducible).
 //
 // The reference has no counterpart (its CSR kernels read 32-bit columns and gather x from global
 // memory: hip/kernel/level2/alphasparse_spmv_csr_vector.h:99-126).
@@ -27,12 +31,15 @@ namespace asx {
 namespace {
 
 constexpr int32_t kNoCol = 0x7fffffff;
+constexpr int kWindowCols = 16384;    // ring size in columns: 128 KiB of fp64, 64 KiB of fp32
+constexpr int kWindowSlack = 8;       // a block's window is kept this much narrower (aligned fetches)
+constexpr int kWindowWaves = 16;
+constexpr int32_t kAlignRowLen = 16;  // rows up to this length are not cut by tile starts
 
-// first and last column of every row (cmin = kNoCol, cmax = -1 for an empty row), its emptiness
+// first and last column of every row (cmin = kNoCol, cmax = -1 for an empty row)
 __global__ __launch_bounds__(kBlock) void k_window_row_span(const int32_t *__restrict__ row_ptr,
                                                             const int32_t *__restrict__ col, int32_t m,
-                                                            int32_t *__restrict__ cmin, int32_t *__restrict__ cmax,
-                                                            int32_t *__restrict__ empty)
+                                                            int32_t *__restrict__ cmin, int32_t *__restrict__ cmax)
 {
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= m) return;
@@ -44,7 +51,6 @@ __global__ __launch_bounds__(kBlock) void k_window_row_span(const int32_t *__res
     }
     cmin[r] = lo;
     cmax[r] = hi;
-    empty[r] = hi < 0 ? 1 : 0;
 }
 
 // bmin / bmax of every block of `rows` rows (bmin preset to kNoCol, bmax to -1)
@@ -73,24 +79,30 @@ __global__ __launch_bounds__(kBlock) void k_window_max_span(const int32_t *__res
     atomicMax(out, bmax[b] - (bmin[b] & ~3) + 1);
 }
 
-// start (in slots, from the start of its block) of row r: stored elements and empty rows before it
-__device__ __forceinline__ int32_t window_row_start(const int32_t *__restrict__ row_ptr,
-                                                    const int32_t *__restrict__ empties_before, int32_t r0, int32_t r)
-{
-    return (row_ptr[r] - row_ptr[r0]) + (empties_before[r] - empties_before[r0]);
-}
-
-// tiles of every block
-__global__ __launch_bounds__(kBlock) void k_window_block_tiles(const int32_t *__restrict__ row_ptr,
-                                                               const int32_t *__restrict__ empties_before, int32_t m,
-                                                               int32_t rows, int32_t nblocks,
-                                                               int32_t *__restrict__ tiles)
+// Slot (from the start of its block) at which every row starts, and the tiles of every block.  A
+// row takes max(1, length) slots; a row of at most kAlignRowLen slots that would cross a tile
+// start begins at that tile start instead.  One thread walks one block's rows in order.
+__global__ __launch_bounds__(kBlock) void k_window_row_starts(const int32_t *__restrict__ row_ptr, int32_t m,
+                                                              int32_t rows, int32_t nblocks,
+                                                              int32_t *__restrict__ row_start,
+                                                              int32_t *__restrict__ block_tiles)
 {
     const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (b >= nblocks) return;
     const int32_t r0 = (int32_t)(b * rows);
     const int32_t r1 = (int64_t)r0 + rows < m ? r0 + rows : m;
-    tiles[b] = (window_row_start(row_ptr, empties_before, r0, r1) + kSlicedTile - 1) / kSlicedTile;
+    int32_t pos = 0;
+    int32_t next = row_ptr[r0];
+    for (int32_t r = r0; r < r1; ++r) {
+        const int32_t cur = next;
+        next = row_ptr[r + 1];
+        const int32_t len = next - cur > 0 ? next - cur : 1;
+        const int32_t in_tile = pos % kSlicedTile;
+        if (len <= kAlignRowLen && in_tile + len > kSlicedTile) pos += kSlicedTile - in_tile;
+        row_start[r] = pos;
+        pos += len;
+    }
+    block_tiles[b] = (pos + kSlicedTile - 1) / kSlicedTile;
 }
 
 template <typename T>
@@ -108,9 +120,8 @@ template <typename T>
 __global__ __launch_bounds__(kBlock) void k_window_place(const int32_t *__restrict__ row_ptr,
                                                          const int32_t *__restrict__ col, const T *__restrict__ val,
                                                          int32_t m, int32_t nnz, int32_t rows,
-                                                         const int32_t *__restrict__ empties_before,
-                                                         const int32_t *__restrict__ tile_off,
-                                                         const int32_t *__restrict__ bmin, uint16_t *__restrict__ cf,
+                                                         const int32_t *__restrict__ row_start,
+                                                         const int32_t *__restrict__ tile_off, uint16_t *__restrict__ cf,
                                                          T *__restrict__ val_out, int32_t *__restrict__ perm)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -123,22 +134,22 @@ __global__ __launch_bounds__(kBlock) void k_window_place(const int32_t *__restri
         else
             hi = mid - 1;
     }
-    const int32_t r = lo, b = r / rows, r0 = b * rows;
-    const int32_t o = window_row_start(row_ptr, empties_before, r0, r) + (int32_t)(i - row_ptr[r]);
+    const int32_t r = lo, b = r / rows;
+    const int32_t o = row_start[r] + (int32_t)(i - row_ptr[r]);
     const int64_t d = (int64_t)tile_off[b] * kSlicedTile + o;
     const bool head = i == row_ptr[r] || o % kSlicedTile == 0;
-    cf[d] = (uint16_t)((col[i] - (bmin[b] & ~3)) | (head ? 0x8000 : 0));
+    cf[d] = (uint16_t)((col[i] % kWindowCols) | (head ? 0x8000 : 0));
     const int64_t phys = d / kSlicedTile * kSlicedTile + tile_val_pos<T>((int)(d % kSlicedTile));
     val_out[phys] = val[i];
     perm[phys] = (int32_t)i;
 }
 
-// per tile: the row its first slot belongs to, bit 31 set when the tile starts inside that row
-__global__ __launch_bounds__(kBlock) void k_window_tile_words(const int32_t *__restrict__ row_ptr,
-                                                              const int32_t *__restrict__ empties_before, int32_t m,
-                                                              int32_t rows, int32_t nblocks,
-                                                              const int32_t *__restrict__ tile_off, int32_t ntiles,
-                                                              int32_t *__restrict__ tile_word, int32_t *__restrict__ any_cont)
+// per tile: x = the row its first slot belongs to, bit 31 set when the tile starts inside that
+// row; y = the number of runs of the tile that are rows (the slots behind them are padding)
+__global__ __launch_bounds__(kBlock) void k_window_tile_info(const int32_t *__restrict__ row_start, int32_t m,
+                                                             int32_t rows, int32_t nblocks,
+                                                             const int32_t *__restrict__ tile_off, int32_t ntiles,
+                                                             int2 *__restrict__ tile_info, int32_t *__restrict__ any_cont)
 {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= ntiles) return;
@@ -156,13 +167,21 @@ __global__ __launch_bounds__(kBlock) void k_window_tile_words(const int32_t *__r
     int32_t a = r0, z = r1 - 1;  // largest row whose start is <= o
     while (a < z) {
         const int32_t mid = a + (z - a + 1) / 2;
-        if (window_row_start(row_ptr, empties_before, r0, mid) <= o)
+        if (row_start[mid] <= o)
             a = mid;
         else
             z = mid - 1;
     }
-    const bool cont = window_row_start(row_ptr, empties_before, r0, a) != o;
-    tile_word[t] = a | (cont ? (int32_t)0x80000000 : 0);
+    int32_t u = a + 1, v = r1;  // first row that starts at or behind the end of the tile
+    while (u < v) {
+        const int32_t mid = u + (v - u) / 2;
+        if (row_start[mid] < o + kSlicedTile)
+            u = mid + 1;
+        else
+            v = mid;
+    }
+    const bool cont = row_start[a] != o;
+    tile_info[t] = make_int2(a | (cont ? (int32_t)0x80000000 : 0), u - a);
     if (cont) *any_cont = 1;
 }
 
@@ -177,12 +196,12 @@ __global__ __launch_bounds__(kBlock) void k_window_regather(const int32_t *__res
 }
 
 // ---- the kernel ----------------------------------------------------------------------------
-// rank k of a tile is row (first row of the tile) + k; the first sum of a tile that starts inside
-// a row goes to the tile's carry slot
+// run k of a tile is row (first row of the tile) + k, for the `limit` runs that are rows; the
+// first sum of a tile that starts inside a row goes to the tile's carry slot
 template <typename T>
 struct StoreRows {
     T *y, *carry_slot;
-    int32_t row0, r1;
+    int32_t row0, limit;
     bool cont;
     T alpha, beta;
     __device__ __forceinline__ void operator()(int rank, T v) const
@@ -191,58 +210,140 @@ struct StoreRows {
             *carry_slot = v;
             return;
         }
-        const int64_t r = (int64_t)row0 + rank;
-        if (r < r1) y[r] = beta == T(0) ? alpha * v : fma_t<T>(alpha, v, beta * y[r]);
+        if (rank < limit) {
+            const int64_t r = (int64_t)row0 + rank;
+            y[r] = beta == T(0) ? alpha * v : fma_t<T>(alpha, v, beta * y[r]);
+        }
     }
 };
 
-template <typename T, int WIDTH, int NW, int D>
-__global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T beta, const int4 *__restrict__ wg_tab,
+template <typename T>
+struct WindowTile : Tile<T> {
+    int32_t limit;
+};
+template <typename T>
+__device__ __forceinline__ void window_tile_load(WindowTile<T> &tl, int32_t t, int lane, const uint16_t *__restrict__ cf,
+                                                 const T *__restrict__ val, const int2 *__restrict__ tile_info)
+{
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 cw = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(cf + (int64_t)t * kSlicedTile) + lane);
+    tl.c01 = cw.x;
+    tl.c23 = cw.y;
+    TileValues<T>::load(val + (int64_t)t * kSlicedTile, lane, tl.v);
+    const int2 info = tile_info[t];
+    tl.base = info.x;
+    tl.limit = info.y;
+}
+
+// The columns [lo, hi) of x (lo a multiple of 4, hi - lo <= kWindowCols) into registers, one
+// 16-byte piece per thread and step; columns at or past n read as 0.
+template <typename T, int THREADS>
+struct XFetch {
+    static constexpr int V = 16 / sizeof(T);
+    static constexpr int PER = kWindowCols / (THREADS * V);
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    vec_t buf[PER];
+    __device__ __forceinline__ void load(const T *__restrict__ x, int32_t n, int32_t lo, int32_t hi)
+    {
+        const bool aligned = ((uintptr_t)x % 16) == 0;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const int64_t c = (int64_t)lo + ((int64_t)k * THREADS + threadIdx.x) * V;
+            if (c + V <= hi && c + V <= n && aligned) {
+                buf[k] = *reinterpret_cast<const vec_t *>(x + c);
+            } else {
+#pragma unroll
+                for (int e = 0; e < V; ++e) buf[k][e] = (c + e < hi && c + e < n) ? x[c + e] : T(0);
+            }
+        }
+    }
+    __device__ __forceinline__ void store(T *xs, int32_t lo, int32_t hi) const
+    {
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const int64_t c = (int64_t)lo + ((int64_t)k * THREADS + threadIdx.x) * V;
+            if (c < hi) *reinterpret_cast<vec_t *>(xs + (c % kWindowCols)) = buf[k];
+        }
+    }
+};
+
+template <typename T, int NW>
+__global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T beta, const int2 *__restrict__ chains,
+                                                           const int4 *__restrict__ blocks,
                                                            const uint16_t *__restrict__ cf, const T *__restrict__ val,
-                                                           const int32_t *__restrict__ tile_word,
+                                                           const int2 *__restrict__ tile_info,
                                                            const T *__restrict__ x, T *__restrict__ y,
                                                            T *__restrict__ carry)
 {
-    __shared__ T xs[WIDTH];
-    const int4 wg = wg_tab[blockIdx.x];  // window start, first tile, end tile, end row
-    const int64_t c0 = wg.x;
-    const int32_t cnt = n - c0 < WIDTH ? (int32_t)(n - c0) : WIDTH;
+    // ring over the columns of x, then the zero the pads point at
+    __shared__ __align__(16) T xs[kWindowCols + 16 / sizeof(T)];
+    const int2 chain = chains[blockIdx.x];  // first block, end block
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    // the first tiles' loads go out before the window of x is fetched (they do not need it)
-    const int32_t last = wg.z - 1;
-    Tile<T> tl[D];
-    int32_t t = wg.y + wave;
-#pragma unroll
-    for (int d = 0; d < D; ++d) tile_load<T>(tl[d], t + d * NW < last ? t + d * NW : last, lane, cf, val, tile_word);
-    load_x_window<T, WIDTH, NW * kWave>(xs, x, c0, cnt);
-    if (threadIdx.x == NW * kWave - 1) xs[WIDTH - 1] = T(0);  // what the slots of empty rows and the padding point at
-    __syncthreads();
-    while (t < wg.z) {  // uniform over the wave
-#pragma unroll
-        for (int d = 0; d < D; ++d) {
-            const int32_t td = t + d * NW;
-            if (td < wg.z)
-                tile_reduce<T>(tl[d], lane, xs,
-                               StoreRows<T>{y, carry + td, tl[d].base & 0x7fffffff, wg.w, tl[d].base < 0, alpha, beta});
-            tile_load<T>(tl[d], t + (D + d) * NW < last ? t + (D + d) * NW : last, lane, cf, val, tile_word);
-        }
-        t += D * NW;
+    const int32_t chain_last = blocks[chain.y - 1].y - 1;  // last tile of the chain
+    // this wave's tiles are those congruent to its number, across the blocks of the chain; two are
+    // in flight (loaded two steps ahead; past the end of the chain the last tile is re-read)
+    WindowTile<T> ta, tb;
+    int32_t t = blocks[chain.x].x + wave;
+    window_tile_load<T>(ta, t < chain_last ? t : chain_last, lane, cf, val, tile_info);
+    window_tile_load<T>(tb, t + NW < chain_last ? t + NW : chain_last, lane, cf, val, tile_info);
+    if (threadIdx.x == 0) xs[kWindowCols] = T(0);
+    XFetch<T, NW * kWave> xf;
+    int4 blk = blocks[chain.x];  // first tile, end tile, columns to fetch before the block: from, to
+    xf.load(x, n, blk.z, blk.w);
+    int32_t b = chain.x, tile_hi;
+    // Start of block b: the columns fetched for it go into the ring once every wave is done with
+    // the block before; the next block's new columns are fetched while this one is multiplied.
+#define ASX_BLOCK_BEGIN()                      \
+    {                                          \
+        __syncthreads();                       \
+        xf.store(xs, blk.z, blk.w);            \
+        __syncthreads();                       \
+        tile_hi = blk.y;                       \
+        if (b + 1 < chain.y) {                 \
+            blk = blocks[b + 1];               \
+            xf.load(x, n, blk.z, blk.w);       \
+        }                                      \
     }
+#define ASX_STEP(TL, TT)                                                                                             \
+    tile_reduce<T>(TL, lane, xs, StoreRows<T>{y, carry + (TT), TL.base & 0x7fffffff, TL.limit, TL.base < 0, alpha, beta})
+#define ASX_NEXT(TL, TT) window_tile_load<T>(TL, (TT) < chain_last ? (TT) : chain_last, lane, cf, val, tile_info)
+    // Every wave passes the start of every block of the chain (the barriers count all waves),
+    // whether it has tiles in the block or not.  ta and tb take turns without changing places.
+    ASX_BLOCK_BEGIN()
+    for (;;) {  // all conditions are uniform over the wave
+        while (t >= tile_hi) {
+            if (++b >= chain.y) return;
+            ASX_BLOCK_BEGIN()
+        }
+        ASX_STEP(ta, t);
+        ASX_NEXT(ta, t + 2 * NW);
+        t += NW;
+        while (t >= tile_hi) {
+            if (++b >= chain.y) return;
+            ASX_BLOCK_BEGIN()
+        }
+        ASX_STEP(tb, t);
+        ASX_NEXT(tb, t + 2 * NW);
+        t += NW;
+    }
+#undef ASX_BLOCK_BEGIN
+#undef ASX_STEP
+#undef ASX_NEXT
 }
 
 // Adds the carries to their rows, in tile order: the thread of the first tile of a run of tiles
 // that start inside the same row sums the run's carries and adds the total once.
 template <typename T>
-__global__ __launch_bounds__(kBlock) void k_window_fixup(int32_t ntiles, T alpha, const int32_t *__restrict__ tile_word,
+__global__ __launch_bounds__(kBlock) void k_window_fixup(int32_t ntiles, T alpha, const int2 *__restrict__ tile_info,
                                                          const T *__restrict__ carry, T *__restrict__ y)
 {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= ntiles) return;
-    const int32_t w = tile_word[t];
-    if (w >= 0) return;                         // starts at a row start
-    if (t > 0 && tile_word[t - 1] == w) return;  // a later tile of its run
+    const int32_t w = tile_info[t].x;
+    if (w >= 0) return;                            // starts at a row start
+    if (t > 0 && tile_info[t - 1].x == w) return;  // a later tile of its run
     T s = carry[t];
-    for (int64_t j = t + 1; j < ntiles && tile_word[j] == w; ++j) s += carry[j];
+    for (int64_t j = t + 1; j < ntiles && tile_info[j].x == w; ++j) s += carry[j];
     const int32_t r = w & 0x7fffffff;
     y[r] = fma_t<T>(alpha, s, y[r]);
 }
@@ -251,86 +352,79 @@ __global__ __launch_bounds__(kBlock) void k_window_fixup(int32_t ntiles, T alpha
 
 void free_window(WindowMatrix *p)
 {
-    for (void *q : {p->val, p->carry, (void *)p->cf, (void *)p->perm, (void *)p->tile_word, (void *)p->wg_tab})
+    for (void *q : {p->val, p->carry, (void *)p->cf, (void *)p->perm, (void *)p->tile_info, (void *)p->blocks,
+                    (void *)p->chains})
         if (q) (void)hipFree(q);
     p->val = p->carry = nullptr;
     p->cf = nullptr;
-    p->perm = p->tile_word = p->wg_tab = nullptr;
+    p->perm = p->tile_info = p->blocks = p->chains = nullptr;
 }
 
 template <typename T>
-int build_window(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t max_rows_per_block, int32_t max_reload,
-                 const int32_t *row_ptr, const int32_t *col, const T *val, WindowMatrix *out, hipStream_t s)
+int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const int32_t *row_ptr, const int32_t *col,
+                 const T *val, WindowMatrix *out, hipStream_t s)
 {
     WindowMatrix wm{};
     if (m <= 0 || nnz <= 0 || n <= 0) return ASX_STATUS_INVALID_SIZE;
-    if (width < 64 || width > 32768) return ASX_STATUS_INVALID_VALUE;
-    wm.width = width;
+    if (target_wgs < 1) return ASX_STATUS_INVALID_VALUE;
     int st = ASX_STATUS_SUCCESS;
-    int32_t *cmin = nullptr, *cmax = nullptr, *empty = nullptr, *ebefore = nullptr;  // m (+1) each
+    int32_t *cmin = nullptr, *cmax = nullptr, *row_start = nullptr;  // m each
     int32_t *bmin = nullptr, *bmax = nullptr, *btiles = nullptr, *tile_off = nullptr, *d_small = nullptr;
     void *tmp = nullptr;
-    size_t tmp_bytes = 0, tb = 0;
-    std::vector<int32_t> h_bmin, h_off, tab;
+    size_t tmp_bytes = 0;
+    std::vector<int32_t> h_bmin, h_bmax, h_off, blk, chains;
     int64_t slots = 0;
     int32_t h_small[2] = {0, 0};
     const unsigned mgrid = (unsigned)ceil_div64(m, kBlock);
-    const int32_t min_blocks = 1024;  // larger blocks only while at least this many row blocks remain
+    const int32_t min_blocks = 4 * target_wgs;  // larger blocks only while at least this many blocks remain
     const int32_t max_nb = (int32_t)ceil_div64(m, 256);
 #define ASX_TRY(expr)         \
     do {                      \
         st = status_of(expr); \
         if (st) goto done;    \
     } while (0)
-    for (int32_t **q : {&cmin, &cmax, &empty, &ebefore}) ASX_TRY(hipMalloc((void **)q, sizeof(int32_t) * ((size_t)m + 1)));
-    for (int32_t **q : {&bmin, &bmax, &btiles, &tile_off}) ASX_TRY(hipMalloc((void **)q, sizeof(int32_t) * ((size_t)max_nb + 1)));
+    for (int32_t **q : {&cmin, &cmax, &row_start}) ASX_TRY(hipMalloc((void **)q, sizeof(int32_t) * (size_t)m));
+    for (int32_t **q : {&bmin, &bmax, &btiles, &tile_off})
+        ASX_TRY(hipMalloc((void **)q, sizeof(int32_t) * ((size_t)max_nb + 1)));
     ASX_TRY(hipMalloc((void **)&d_small, sizeof(int32_t) * 2));
-    ASX_TRY(hipcub::DeviceScan::ExclusiveSum(nullptr, tmp_bytes, empty, ebefore, m + 1, s));
-    ASX_TRY(hipcub::DeviceScan::ExclusiveSum(nullptr, tb, btiles, tile_off, max_nb + 1, s));
-    tmp_bytes = std::max(tmp_bytes, tb);
+    ASX_TRY(hipcub::DeviceScan::ExclusiveSum(nullptr, tmp_bytes, btiles, tile_off, max_nb + 1, s));
     ASX_TRY(hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1));
 
-    // 1. column span and emptiness of every row; empty rows before each row
-    hipLaunchKernelGGL(k_window_row_span, dim3(mgrid), dim3(kBlock), 0, s, row_ptr, col, m, cmin, cmax, empty);
-    ASX_TRY(hipMemsetAsync(empty + m, 0, sizeof(int32_t), s));
-    ASX_TRY(hipcub::DeviceScan::ExclusiveSum(tmp, tmp_bytes, empty, ebefore, m + 1, s));
-
-    // 2. the largest block of rows (at most max_rows_per_block, a multiple of 256) whose widest
-    //    window fits; the last LDS entry is kept for the zero that empty rows point at
+    // 1. column span of every row
+    hipLaunchKernelGGL(k_window_row_span, dim3(mgrid), dim3(kBlock), 0, s, row_ptr, col, m, cmin, cmax);
+    // 2. the largest block of rows (a multiple of 256) whose widest window fits the ring
     wm.rows_per_block = 0;
     for (int32_t rows : {8192, 6144, 4096, 3072, 2048, 1536, 1024, 768, 512, 384, 256}) {
-        if (rows > max_rows_per_block) continue;
-        if (rows > 256 && ceil_div64(m, rows) < min_blocks) continue;  // too few workgroups
+        if (rows > 256 && ceil_div64(m, rows) < min_blocks) continue;  // too few blocks to share out
         const int32_t nb = (int32_t)ceil_div64(m, rows);
-        hipLaunchKernelGGL(k_window_fill_i32, dim3((unsigned)ceil_div64(nb, kBlock)), dim3(kBlock), 0, s, bmin, (int64_t)nb, kNoCol);
-        hipLaunchKernelGGL(k_window_fill_i32, dim3((unsigned)ceil_div64(nb, kBlock)), dim3(kBlock), 0, s, bmax, (int64_t)nb, -1);
+        const unsigned bgrid = (unsigned)ceil_div64(nb, kBlock);
+        hipLaunchKernelGGL(k_window_fill_i32, dim3(bgrid), dim3(kBlock), 0, s, bmin, (int64_t)nb, kNoCol);
+        hipLaunchKernelGGL(k_window_fill_i32, dim3(bgrid), dim3(kBlock), 0, s, bmax, (int64_t)nb, -1);
         ASX_TRY(hipMemsetAsync(d_small, 0, sizeof(int32_t) * 2, s));
         hipLaunchKernelGGL(k_window_block_span, dim3(mgrid), dim3(kBlock), 0, s, cmin, cmax, m, rows, bmin, bmax);
-        hipLaunchKernelGGL(k_window_max_span, dim3((unsigned)ceil_div64(nb, kBlock)), dim3(kBlock), 0, s, bmin, bmax, nb, d_small);
+        hipLaunchKernelGGL(k_window_max_span, dim3(bgrid), dim3(kBlock), 0, s, bmin, bmax, nb, d_small);
         ASX_TRY(hipMemcpyAsync(h_small, d_small, sizeof(int32_t), hipMemcpyDeviceToHost, s));
         ASX_TRY(hipStreamSynchronize(s));
-        if (h_small[0] <= width - 1) {
-            // every workgroup fetches its whole window: with a bound on that (max_reload > 0), blocks
-            // whose window is more than max_reload times their rows wide are turned down
-            if (max_reload <= 0 || h_small[0] <= (int64_t)max_reload * rows) {
-                wm.rows_per_block = rows;
-                wm.nblocks = nb;
-            }
+        if (h_small[0] <= kWindowCols - kWindowSlack) {
+            wm.rows_per_block = rows;
+            wm.nblocks = nb;
             break;
         }
     }
     if (wm.rows_per_block == 0) {
-        st = ASX_STATUS_NOT_SUPPORTED;  // some 256 rows reach further than a window: not this kernel's matrix
+        st = ASX_STATUS_NOT_SUPPORTED;  // some 256 rows reach further than the ring: not this kernel's matrix
         goto done;
     }
-    // 3. tiles of every block
-    hipLaunchKernelGGL(k_window_block_tiles, dim3((unsigned)ceil_div64(wm.nblocks, kBlock)), dim3(kBlock), 0, s, row_ptr,
-                       ebefore, m, wm.rows_per_block, wm.nblocks, btiles);
+    // 3. where every row starts inside its block; tiles of every block
+    hipLaunchKernelGGL(k_window_row_starts, dim3((unsigned)ceil_div64(wm.nblocks, kBlock)), dim3(kBlock), 0, s, row_ptr, m,
+                       wm.rows_per_block, wm.nblocks, row_start, btiles);
     ASX_TRY(hipMemsetAsync(btiles + wm.nblocks, 0, sizeof(int32_t), s));
     ASX_TRY(hipcub::DeviceScan::ExclusiveSum(tmp, tmp_bytes, btiles, tile_off, wm.nblocks + 1, s));
     h_bmin.resize((size_t)wm.nblocks);
+    h_bmax.resize((size_t)wm.nblocks);
     h_off.resize((size_t)wm.nblocks + 1);
     ASX_TRY(hipMemcpyAsync(h_bmin.data(), bmin, sizeof(int32_t) * h_bmin.size(), hipMemcpyDeviceToHost, s));
+    ASX_TRY(hipMemcpyAsync(h_bmax.data(), bmax, sizeof(int32_t) * h_bmax.size(), hipMemcpyDeviceToHost, s));
     ASX_TRY(hipMemcpyAsync(h_off.data(), tile_off, sizeof(int32_t) * h_off.size(), hipMemcpyDeviceToHost, s));
     ASX_TRY(hipStreamSynchronize(s));
     wm.ntiles = h_off[(size_t)wm.nblocks];
@@ -342,37 +436,76 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t max_r
     ASX_TRY(hipMalloc(&wm.val, sizeof(T) * (size_t)slots));
     ASX_TRY(hipMalloc((void **)&wm.cf, sizeof(uint16_t) * (size_t)slots));
     ASX_TRY(hipMalloc((void **)&wm.perm, sizeof(int32_t) * (size_t)slots));
-    ASX_TRY(hipMalloc((void **)&wm.tile_word, sizeof(int32_t) * (size_t)wm.ntiles));
+    ASX_TRY(hipMalloc((void **)&wm.tile_info, sizeof(int2) * (size_t)wm.ntiles));
     ASX_TRY(hipMalloc(&wm.carry, sizeof(T) * (size_t)wm.ntiles));
     ASX_TRY(hipMemsetAsync(wm.carry, 0, sizeof(T) * (size_t)wm.ntiles, s));
-    // 4. every slot starts as a zero that points at the zero in LDS and opens a row of its own (the
-    //    slots of empty rows and the padding behind a block's last row stay that way)
+    // 4. every slot starts as a zero that points at the zero behind the ring and opens a run of its
+    //    own (the slots of empty rows and the padding stay that way)
     hipLaunchKernelGGL((k_window_fill_pads<T>), dim3((unsigned)ceil_div64(slots, kBlock)), dim3(kBlock), 0, s, slots,
-                       (uint16_t)(0x8000 | (width - 1)), wm.cf, (T *)wm.val, wm.perm);
+                       (uint16_t)(0x8000 | kWindowCols), wm.cf, (T *)wm.val, wm.perm);
     hipLaunchKernelGGL((k_window_place<T>), dim3((unsigned)ceil_div64(nnz, kBlock)), dim3(kBlock), 0, s, row_ptr, col, val,
-                       m, nnz, wm.rows_per_block, ebefore, tile_off, bmin, wm.cf, (T *)wm.val, wm.perm);
-    // 5. first row of every tile
+                       m, nnz, wm.rows_per_block, row_start, tile_off, wm.cf, (T *)wm.val, wm.perm);
+    // 5. first row and number of rows of every tile
     ASX_TRY(hipMemsetAsync(d_small, 0, sizeof(int32_t) * 2, s));
-    hipLaunchKernelGGL(k_window_tile_words, dim3((unsigned)ceil_div64(wm.ntiles, kBlock)), dim3(kBlock), 0, s, row_ptr,
-                       ebefore, m, wm.rows_per_block, wm.nblocks, tile_off, wm.ntiles, wm.tile_word, d_small);
+    hipLaunchKernelGGL(k_window_tile_info, dim3((unsigned)ceil_div64(wm.ntiles, kBlock)), dim3(kBlock), 0, s, row_start, m,
+                       wm.rows_per_block, wm.nblocks, tile_off, wm.ntiles, (int2 *)wm.tile_info, d_small);
     ASX_TRY(hipMemcpyAsync(h_small, d_small, sizeof(int32_t), hipMemcpyDeviceToHost, s));
-    // 6. one workgroup per block: window start, tiles, end row
-    tab.resize((size_t)wm.nblocks * 4);
-    for (int32_t b = 0; b < wm.nblocks; ++b) {
-        const int64_t r1 = std::min<int64_t>(m, ((int64_t)b + 1) * wm.rows_per_block);
-        tab[(size_t)b * 4 + 0] = h_bmin[(size_t)b] == kNoCol ? 0 : (h_bmin[(size_t)b] & ~3);
-        tab[(size_t)b * 4 + 1] = h_off[(size_t)b];
-        tab[(size_t)b * 4 + 2] = h_off[(size_t)b + 1];
-        tab[(size_t)b * 4 + 3] = (int32_t)r1;
+    // 6. chains of blocks, one per workgroup, of about equal numbers of tiles.  Inside a chain a
+    //    block fetches only the columns behind those already in the ring; a block whose columns
+    //    start before what the ring still holds begins a new chain (and fetches its whole window).
+    {
+        const int64_t per_chain = std::max<int64_t>(1, ceil_div64(wm.ntiles, target_wgs));
+        blk.resize((size_t)wm.nblocks * 4);
+        int64_t have = -1;  // columns [.., have) are in the ring (-1: nothing yet)
+        int32_t chain_lo = 0;
+        int64_t chain_tiles = 0;
+        for (int32_t b = 0; b < wm.nblocks; ++b) {
+            const bool empty = h_bmax[(size_t)b] < 0;
+            const int64_t lo = empty ? 0 : (h_bmin[(size_t)b] & ~3);
+            const int64_t hi = empty ? 0 : ((int64_t)h_bmax[(size_t)b] + 4) & ~(int64_t)3;  // past the last, rounded up
+            bool fresh = false;
+            if (b != chain_lo) {
+                if (!empty && have >= 0 && lo < std::max(have, hi) - kWindowCols) fresh = true;  // already overwritten
+                if (chain_tiles >= per_chain) fresh = true;
+            }
+            if (fresh) {
+                chains.push_back(chain_lo);
+                chains.push_back(b);
+                chain_lo = b;
+                chain_tiles = 0;
+                have = -1;
+            }
+            int64_t from = 0, to = 0;
+            if (!empty) {
+                if (have < 0 || lo >= have) {  // nothing useful in the ring: the whole window
+                    from = lo;
+                    to = hi;
+                } else {
+                    from = have;
+                    to = std::max(have, hi);
+                }
+                have = to;
+            }
+            blk[(size_t)b * 4 + 0] = h_off[(size_t)b];
+            blk[(size_t)b * 4 + 1] = h_off[(size_t)b + 1];
+            blk[(size_t)b * 4 + 2] = (int32_t)from;
+            blk[(size_t)b * 4 + 3] = (int32_t)to;
+            chain_tiles += h_off[(size_t)b + 1] - h_off[(size_t)b];
+        }
+        chains.push_back(chain_lo);
+        chains.push_back(wm.nblocks);
+        wm.nchains = (int32_t)(chains.size() / 2);
     }
-    ASX_TRY(hipMalloc((void **)&wm.wg_tab, sizeof(int32_t) * tab.size()));
-    ASX_TRY(hipMemcpyAsync(wm.wg_tab, tab.data(), sizeof(int32_t) * tab.size(), hipMemcpyHostToDevice, s));
+    ASX_TRY(hipMalloc((void **)&wm.blocks, sizeof(int32_t) * blk.size()));
+    ASX_TRY(hipMalloc((void **)&wm.chains, sizeof(int32_t) * chains.size()));
+    ASX_TRY(hipMemcpyAsync(wm.blocks, blk.data(), sizeof(int32_t) * blk.size(), hipMemcpyHostToDevice, s));
+    ASX_TRY(hipMemcpyAsync(wm.chains, chains.data(), sizeof(int32_t) * chains.size(), hipMemcpyHostToDevice, s));
     ASX_TRY(hipStreamSynchronize(s));
     ASX_TRY(hipGetLastError());
     wm.has_carry = h_small[0] != 0;
 #undef ASX_TRY
 done:
-    for (void *p : {(void *)cmin, (void *)cmax, (void *)empty, (void *)ebefore, (void *)bmin, (void *)bmax, (void *)btiles,
+    for (void *p : {(void *)cmin, (void *)cmax, (void *)row_start, (void *)bmin, (void *)bmax, (void *)btiles,
                     (void *)tile_off, (void *)d_small, tmp})
         if (p) (void)hipFree(p);
     if (st) {
@@ -397,28 +530,18 @@ template <typename T>
 int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, hipStream_t s)
 {
     if (m <= 0) return ASX_STATUS_SUCCESS;
-#define ASX_WIN(W)                                                                                                  \
-    hipLaunchKernelGGL((k_spmv_window<T, W, 16, 2>), dim3((unsigned)wm->nblocks), dim3(16 * kWave), 0, s, n, alpha, beta, \
-                       reinterpret_cast<const int4 *>(wm->wg_tab), wm->cf, (const T *)wm->val, wm->tile_word, x, y,     \
-                       (T *)wm->carry)
-    if (wm->width == (int)(131072 / sizeof(T)))
-        ASX_WIN(131072 / sizeof(T));
-    else if (wm->width == (int)(81920 / sizeof(T)))
-        ASX_WIN(81920 / sizeof(T));
-    else if (sizeof(T) == 8 && wm->width == 20480)
-        ASX_WIN(20480);
-    else
-        return ASX_STATUS_INVALID_VALUE;
-#undef ASX_WIN
+    hipLaunchKernelGGL((k_spmv_window<T, kWindowWaves>), dim3((unsigned)wm->nchains), dim3(kWindowWaves * kWave), 0, s, n,
+                       alpha, beta, reinterpret_cast<const int2 *>(wm->chains), reinterpret_cast<const int4 *>(wm->blocks),
+                       wm->cf, (const T *)wm->val, reinterpret_cast<const int2 *>(wm->tile_info), x, y, (T *)wm->carry);
     if (wm->has_carry)
         hipLaunchKernelGGL((k_window_fixup<T>), dim3((unsigned)ceil_div64(wm->ntiles, kBlock)), dim3(kBlock), 0, s,
-                           wm->ntiles, alpha, wm->tile_word, (const T *)wm->carry, y);
+                           wm->ntiles, alpha, reinterpret_cast<const int2 *>(wm->tile_info), (const T *)wm->carry, y);
     return check_launch();
 }
 
 #define ASX_INST(T)                                                                                               \
-    template int build_window<T>(int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, const int32_t *,         \
-                                 const int32_t *, const T *, WindowMatrix *, hipStream_t);                                        \
+    template int build_window<T>(int32_t, int32_t, int32_t, int32_t, const int32_t *, const int32_t *, const T *, \
+                                 WindowMatrix *, hipStream_t);                                                    \
     template int window_update_values<T>(const WindowMatrix *, const T *, hipStream_t);                           \
     template int launch_spmv_window<T>(int32_t, int32_t, T, const WindowMatrix *, const T *, T, T *, hipStream_t);
 ASX_INST(float)
