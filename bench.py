@@ -37,18 +37,20 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 ORDER = ["banded_f64", "uniform16_f32", "powerlaw_f64", "stencil5_f64", "spmm_zipf_f32"]
 EXTRA = ["spmm_banded_f32"]  # not a BASELINE configuration: dense-block matrix for the MFMA SpMM variant
 KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "k_spmv_flat",
-                101: "k_sliced_products+k_sliced_reduce", 5: "k_spmm_row", 7: "k_spmm_merge", 10: "k_spmm_blocked"}
+                101: "k_sliced_products+k_sliced_reduce", 102: "k_spmv_window", 5: "k_spmm_row", 7: "k_spmm_merge", 10: "k_spmm_blocked"}
 
-# HBM-side traffic per call measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE in KiB per
-# dispatch, summed over the kernels of one call; see profiles/), scaled by the same counters'
-# reading for a plain copy of known size (FETCH_SIZE reads half the bytes, WRITE_SIZE all of
-# them).  None = not measured.
+# Traffic beyond the L2s per call measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE in KiB per
+# dispatch, summed over the kernels of one call with kept analysis; see profiles/), scaled by the
+# same counters' reading for a plain copy of known size (FETCH_SIZE reads half the bytes,
+# WRITE_SIZE all of them).  The Infinity Cache serves part of it: the counters read the same with
+# warm and with cold caches.
 MEASURED_TRAFFIC_BYTES = {
-    "powerlaw_f64": None,
-    "stencil5_f64": None,
-    "uniform16_f32": None,
-    "spmm_banded_f32": None,
-    "spmm_zipf_f32": None,
+    "banded_f64": 458_667,             # profiles/spmv_vector_banded_f64.md
+    "uniform16_f32": 279_700_064,      # profiles/spmv_sliced_uniform16_f32.md
+    "powerlaw_f64": 723_138_155,       # profiles/spmv_sliced_powerlaw_f64.md
+    "stencil5_f64": 1_134_700_565,     # profiles/spmv_window_stencil5_f64.md
+    "spmm_zipf_f32": 4_964_363_985,    # profiles/spmm_merge_spmm_zipf_f32.md
+    "spmm_banded_f32": 1_868_512_068,  # profiles/spmm_blocked_spmm_banded_f32.md
 }
 
 

@@ -59,10 +59,18 @@ __global__ __launch_bounds__(kBlock) void k_window_block_span(const int32_t *__r
                                                               int32_t rows, int32_t *__restrict__ bmin,
                                                               int32_t *__restrict__ bmax)
 {
+    // `rows` is a multiple of 256, so the 64 rows of a wave lie in one block: one pair of atomics a wave
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (r >= m || cmax[r] < 0) return;
-    atomicMin(bmin + r / rows, cmin[r]);
-    atomicMax(bmax + r / rows, cmax[r]);
+    int32_t lo = kNoCol, hi = -1;
+    if (r < m && cmax[r] >= 0) lo = cmin[r], hi = cmax[r];
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        lo = min(lo, __shfl_xor(lo, d, kWave));
+        hi = max(hi, __shfl_xor(hi, d, kWave));
+    }
+    if (__lane_id() != 0 || hi < 0) return;
+    atomicMin(bmin + r / rows, lo);
+    atomicMax(bmax + r / rows, hi);
 }
 __global__ __launch_bounds__(kBlock) void k_window_fill_i32(int32_t *p, int64_t n, int32_t v)
 {
