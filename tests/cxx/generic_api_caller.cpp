@@ -113,6 +113,34 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
             s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
         }
+        if (analysis == 3) {
+            // a second descriptor that shares A's row offsets and columns but has its own values
+            // (the usual "same pattern, new values" set-up): each descriptor must multiply with its
+            // own values.  Its product goes to out2.bin; A's product is computed again afterwards.
+            auto val2 = read_bin<T>(dir + "/val2.bin", nnz);
+            T *d_val2 = to_device(val2);
+            alphasparseSpMatDescr_t A2;
+            if (alphasparseCreateCsr(&A2, (int)m, (int)n, (int)nnz, d_rp, d_col, d_val2, ALPHA_SPARSE_INDEXTYPE_I32,
+                                     ALPHA_SPARSE_INDEXTYPE_I32,
+                                     v.base ? ALPHA_SPARSE_INDEX_BASE_ONE : ALPHA_SPARSE_INDEX_BASE_ZERO, dt))
+                return 5;
+            s = alphasparseSpMV_analysis(handle, opA, A2, (alphasparseSpMVAlg_t)alg);
+            if (s) return 70 + (int)s;
+            HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
+            s = alphasparseSpMV(handle, opA, &alpha, A2, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
+            if (s) return 50 + (int)s;
+            HIP_OK(hipStreamSynchronize(handle->stream));
+            std::vector<T> out2(yin.size());
+            HIP_OK(hipMemcpy(out2.data(), d_y, out2.size() * sizeof(T), hipMemcpyDeviceToHost));
+            FILE *f2 = std::fopen((dir + "/out2.bin").c_str(), "wb");
+            if (!f2 || std::fwrite(out2.data(), sizeof(T), out2.size(), f2) != out2.size()) return 9;
+            std::fclose(f2);
+            alphasparseDestroySpMat(A2);
+            (void)hipFree(d_val2);
+            HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
+            s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
+            if (s) return 50 + (int)s;
+        }
         if (analysis && alphasparseSpMV_clear(handle, (alphasparseSpMVAlg_t)alg)) return 7;
         alphasparseDestroyDnVec(X);
         alphasparseDestroyDnVec(Y);

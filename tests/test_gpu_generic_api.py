@@ -21,7 +21,7 @@ def _run_case(tmp_path, op, dtype, rp, col, val, x, y, ncols, alg, alpha, beta, 
     d.mkdir()
     for name, a in (("row_ptr", rp), ("col", col), ("val", val), ("x", x), ("y", y)):
         np.ascontiguousarray(a).tofile(d / f"{name}.bin")
-    if val2 is not None:  # analysis == 2: values written over A's after the first products
+    if val2 is not None:  # analysis == 2: values written over A's after the first products; 3: a second descriptor's
         np.ascontiguousarray(val2).tofile(d / "val2.bin")
     tag = "f64" if np.dtype(dtype) == np.float64 else "f32"
     if n is None:
@@ -206,6 +206,13 @@ def test_spmv_analysis_on_a_scattered_matrix(tmp_path, oracle):
     got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, alpha, beta, 2, val2=val2)
     assert_close(got, oracle.spmv(rp, col, val2, x, alpha, beta, y0, 8), spmv_scale(rp, col, val2, x, alpha, beta, y0),
                  np.float64, "DEFAULT, values changed, analysis called again")
+    # two descriptors that share row offsets and columns, each with its own values (analysis = 3):
+    # out2.bin is the second descriptor's product, out.bin the first one's, computed after it
+    got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, alpha, beta, 3, val2=val2)
+    assert_close(got, ref, scale, np.float64, "DEFAULT, first of two descriptors sharing row_ptr")
+    got2 = np.fromfile(next(tmp_path.glob("spmv_float64_0_3_*")) / "out2.bin", dtype=np.float64)
+    assert_close(got2, oracle.spmv(rp, col, val2, x, alpha, beta, y0, 8), spmv_scale(rp, col, val2, x, alpha, beta, y0),
+                 np.float64, "DEFAULT, second of two descriptors sharing row_ptr")
     rp_t, col_t, val_t = _transpose_csr(rp, col, val, n)
     ref_t = oracle.spmv(rp_t, col_t, val_t, y0, alpha, beta, x, 8)
     got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, y0, x, 1, 0, alpha, beta, 1, (1, 0, 0, 0, 0), n=n)
