@@ -591,10 +591,16 @@ int plan_add_slices(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
 {
     int cus = 256;
     (void)asx_device_info(&cus, nullptr);
-    // pass 2: one wave per block of rows; at least 8 waves per compute unit where m allows, at most
-    // 16 KiB of accumulators per wave
+    // pass 2: one wave per block of rows with at most 16 KiB of accumulators.  Blocks of 256 rows,
+    // doubled while that leaves more than 8 waves per compute unit and the block's partial sums
+    // inside one slice (expected from the row-length histogram) are too few to fill the 64-wide
+    // steps in which a wave reads them (measured: 16 rows of 16 over 32 slices, 100 per range, run
+    // 5 % faster with 256 rows than with 512; the power-law matrix, 4 per range at 256 rows, runs
+    // 2x faster with 2048).
+    const int32_t nslices = (int32_t)ceil_div64((int64_t)p->n * (int64_t)sizeof(T), kSliceBytes);
+    const double per_row_slice = sliced_expected_partials(p->hist, nslices) / ((double)p->m * (double)nslices);
     int32_t rpw = 256;
-    while (rpw < (int32_t)(16384 / sizeof(T)) && (int64_t)rpw * cus * 8 < p->m) rpw *= 2;
+    while (rpw < (int32_t)(16384 / sizeof(T)) && (int64_t)rpw * cus * 8 < p->m && per_row_slice * rpw < 96.0) rpw *= 2;
     SlicedMatrix sm{};
     const int st = build_sliced<T>(p->m, p->n, p->nnz, (int32_t)(kSliceBytes / sizeof(T)), rpw, cus, d_row_ptr, d_col,
                                    d_val, &sm, s);

@@ -204,11 +204,17 @@ __global__ __launch_bounds__(kBlock) void k_window_regather(const int32_t *__res
 }
 
 // ---- the kernel ----------------------------------------------------------------------------
-// run k of a tile is row (first row of the tile) + k, for the `limit` runs that are rows; the
-// first sum of a tile that starts inside a row goes to the tile's carry slot
+// Run k of a tile is row (first row of the tile) + k, for the `limit` runs that are rows; the
+// first sum of a tile that starts inside a row goes to the tile's carry slot.  The sums of the
+// first kStageRows rows of a tile pass through a staging area of the wave in LDS and leave as
+// stores of consecutive lanes to consecutive rows: stored straight from the lanes that close the
+// runs (4 or 5 masked stores a tile, 8 bytes every 32 to 40), the same 134 MB of y cost 66 us of
+// the 5-point stencil's 220; staged, a third of that.  Rows past kStageRows (a tile of rows shorter
+// than 2 on average) are stored directly.
+constexpr int kStageRows = 128;
 template <typename T>
 struct StoreRows {
-    T *y, *carry_slot;
+    T *y, *carry_slot, *stage;
     int32_t row0, limit;
     bool cont;
     T alpha, beta;
@@ -218,10 +224,31 @@ struct StoreRows {
             *carry_slot = v;
             return;
         }
-        if (rank < limit) {
+        if (rank < kStageRows) {
+            stage[rank] = v;  // ranks at or past `limit` are written too and never read
+        } else if (rank < limit) {
             const int64_t r = (int64_t)row0 + rank;
             y[r] = beta == T(0) ? alpha * v : fma_t<T>(alpha, v, beta * y[r]);
         }
+    }
+    // after the tile's runs are staged: the wave's LDS writes and reads execute in order
+    __device__ __forceinline__ void flush(int lane) const
+    {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const int32_t first = cont ? 1 : 0, end = limit < kStageRows ? limit : kStageRows;
+#pragma unroll
+        for (int k = 0; k < kStageRows / kWave; ++k) {
+            const int32_t i = k * kWave + lane;
+            if (k * kWave < end) {  // uniform
+                if (i >= first && i < end) {
+                    const int64_t r = (int64_t)row0 + i;
+                    const T v = stage[i];
+                    y[r] = beta == T(0) ? alpha * v : fma_t<T>(alpha, v, beta * y[r]);
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
     }
 };
 
@@ -244,38 +271,55 @@ __device__ __forceinline__ void window_tile_load(WindowTile<T> &tl, int32_t t, i
 }
 
 // The columns [lo, hi) of x (lo a multiple of 4, hi - lo <= kWindowCols) into registers, one
-// 16-byte piece per thread and step; columns at or past n read as 0.
-template <typename T, int THREADS>
+// 16-byte piece per thread and step; columns at or past n read as 0.  Every register is written by
+// one load instruction only (predicated, after a zero fill), never by two alternative ones: with
+// alternatives the compiler orders them with a full s_waitcnt between the steps and the fetch
+// takes one memory round trip per step.  ALIGNED (x on a 16-byte boundary): whole pieces inside x
+// with one 16-byte load; the piece that straddles the end of x (n no multiple of the piece),
+// element by element into `tail` by the one thread that owns it.  Otherwise element by element.
+template <typename T, int THREADS, bool ALIGNED>
 struct XFetch {
     static constexpr int V = 16 / sizeof(T);
     static constexpr int PER = kWindowCols / (THREADS * V);
     typedef T vec_t __attribute__((ext_vector_type(V)));
     vec_t buf[PER];
+    vec_t tail;
     __device__ __forceinline__ void load(const T *__restrict__ x, int32_t n, int32_t lo, int32_t hi)
     {
-        const bool aligned = ((uintptr_t)x % 16) == 0;
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
             const int64_t c = (int64_t)lo + ((int64_t)k * THREADS + threadIdx.x) * V;
-            if (c + V <= hi && c + V <= n && aligned) {
-                buf[k] = *reinterpret_cast<const vec_t *>(x + c);
+            buf[k] = vec_t(T(0));
+            if (ALIGNED) {
+                if (c < hi && c + V <= n) buf[k] = *reinterpret_cast<const vec_t *>(x + c);
             } else {
 #pragma unroll
-                for (int e = 0; e < V; ++e) buf[k][e] = (c + e < hi && c + e < n) ? x[c + e] : T(0);
+                for (int e = 0; e < V; ++e)
+                    if (c + e < hi && c + e < n) buf[k][e] = x[c + e];
+            }
+        }
+        if (ALIGNED) {
+            tail = vec_t(T(0));
+            const int64_t cs = (int64_t)n & ~(int64_t)(V - 1);  // start of the piece that straddles the end of x
+            if (cs < n && cs >= lo && cs < hi && ((cs - lo) / V) % THREADS == (int64_t)threadIdx.x) {
+#pragma unroll
+                for (int e = 0; e < V - 1; ++e)
+                    if (cs + e < n) tail[e] = x[cs + e];
             }
         }
     }
-    __device__ __forceinline__ void store(T *xs, int32_t lo, int32_t hi) const
+    __device__ __forceinline__ void store(T *xs, int32_t n, int32_t lo, int32_t hi) const
     {
+        const int64_t cs = (int64_t)n & ~(int64_t)(V - 1);
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
             const int64_t c = (int64_t)lo + ((int64_t)k * THREADS + threadIdx.x) * V;
-            if (c < hi) *reinterpret_cast<vec_t *>(xs + (c % kWindowCols)) = buf[k];
+            if (c < hi) *reinterpret_cast<vec_t *>(xs + (c % kWindowCols)) = (ALIGNED && c == cs) ? tail : buf[k];
         }
     }
 };
 
-template <typename T, int NW>
+template <typename T, int NW, bool ALIGNED>
 __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T beta, const int2 *__restrict__ chains,
                                                            const int4 *__restrict__ blocks,
                                                            const uint16_t *__restrict__ cf, const T *__restrict__ val,
@@ -285,8 +329,10 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
 {
     // ring over the columns of x, then the zero the pads point at
     __shared__ __align__(16) T xs[kWindowCols + 16 / sizeof(T)];
+    __shared__ T stage_all[NW * kStageRows];
     const int2 chain = chains[blockIdx.x];  // first block, end block
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    T *stage = stage_all + wave * kStageRows;
     const int32_t chain_last = blocks[chain.y - 1].y - 1;  // last tile of the chain
     // this wave's tiles are those congruent to its number, across the blocks of the chain; two are
     // in flight (loaded two steps ahead; past the end of the chain the last tile is re-read)
@@ -295,7 +341,7 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
     window_tile_load<T>(ta, t < chain_last ? t : chain_last, lane, cf, val, tile_info);
     window_tile_load<T>(tb, t + NW < chain_last ? t + NW : chain_last, lane, cf, val, tile_info);
     if (threadIdx.x == 0) xs[kWindowCols] = T(0);
-    XFetch<T, NW * kWave> xf;
+    XFetch<T, NW * kWave, ALIGNED> xf;
     int4 blk = blocks[chain.x];  // first tile, end tile, columns to fetch before the block: from, to
     xf.load(x, n, blk.z, blk.w);
     int32_t b = chain.x, tile_hi;
@@ -304,7 +350,7 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
 #define ASX_BLOCK_BEGIN()                      \
     {                                          \
         __syncthreads();                       \
-        xf.store(xs, blk.z, blk.w);            \
+        xf.store(xs, n, blk.z, blk.w);         \
         __syncthreads();                       \
         tile_hi = blk.y;                       \
         if (b + 1 < chain.y) {                 \
@@ -312,8 +358,12 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
             xf.load(x, n, blk.z, blk.w);       \
         }                                      \
     }
-#define ASX_STEP(TL, TT)                                                                                             \
-    tile_reduce<T>(TL, lane, xs, StoreRows<T>{y, carry + (TT), TL.base & 0x7fffffff, TL.limit, TL.base < 0, alpha, beta})
+#define ASX_STEP(TL, TT)                                                                                          \
+    {                                                                                                             \
+        const StoreRows<T> out{y, carry + (TT), stage, TL.base & 0x7fffffff, TL.limit, TL.base < 0, alpha, beta}; \
+        tile_reduce<T>(TL, lane, xs, out);                                                                        \
+        out.flush(lane);                                                                                          \
+    }
 #define ASX_NEXT(TL, TT) window_tile_load<T>(TL, (TT) < chain_last ? (TT) : chain_last, lane, cf, val, tile_info)
     // Every wave passes the start of every block of the chain (the barriers count all waves),
     // whether it has tiles in the block or not.  ta and tb take turns without changing places.
@@ -538,9 +588,11 @@ template <typename T>
 int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, hipStream_t s)
 {
     if (m <= 0) return ASX_STATUS_SUCCESS;
-    hipLaunchKernelGGL((k_spmv_window<T, kWindowWaves>), dim3((unsigned)wm->nchains), dim3(kWindowWaves * kWave), 0, s, n,
-                       alpha, beta, reinterpret_cast<const int2 *>(wm->chains), reinterpret_cast<const int4 *>(wm->blocks),
-                       wm->cf, (const T *)wm->val, reinterpret_cast<const int2 *>(wm->tile_info), x, y, (T *)wm->carry);
+    // x on a 16-byte boundary (every allocation is): 16-byte fetches; else element by element
+    const auto kernel = ((uintptr_t)x % 16) == 0 ? k_spmv_window<T, kWindowWaves, true> : k_spmv_window<T, kWindowWaves, false>;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)wm->nchains), dim3(kWindowWaves * kWave), 0, s, n, alpha, beta,
+                       reinterpret_cast<const int2 *>(wm->chains), reinterpret_cast<const int4 *>(wm->blocks), wm->cf,
+                       (const T *)wm->val, reinterpret_cast<const int2 *>(wm->tile_info), x, y, (T *)wm->carry);
     if (wm->has_carry)
         hipLaunchKernelGGL((k_window_fixup<T>), dim3((unsigned)ceil_div64(wm->ntiles, kBlock)), dim3(kBlock), 0, s,
                            wm->ntiles, alpha, reinterpret_cast<const int2 *>(wm->tile_info), (const T *)wm->carry, y);
