@@ -167,12 +167,28 @@ __global__ __launch_bounds__(kBlock) void k_sliced_regather(const int32_t *__res
 }
 
 // ---- pass 1 ------------------------------------------------------------------------------
-// a run's sum goes to the tile's partial sums, at the run's rank
+// A run's sum goes, at the run's rank, into the wave's staging area in LDS; the tile's sums then
+// leave as stores of consecutive lanes to consecutive partial sums.
+constexpr int kStageRuns = kSlicedTile;  // every run of a tile
 template <typename T>
-struct StorePartial {
-    T *out;
-    __device__ __forceinline__ void operator()(int rank, T v) const { out[rank] = v; }
+struct StageRun {
+    T *stage;
+    __device__ __forceinline__ void operator()(int rank, T v) const { stage[rank] = v; }
 };
+template <typename T>
+__device__ __forceinline__ void store_staged(const T *stage, int lane, int total, T *__restrict__ out)
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int k = 0; k < kStageRuns / kWave; ++k) {
+        const int i = k * kWave + lane;
+        if (k * kWave < total) {  // uniform
+            if (i < total) out[i] = stage[i];
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+}
 
 template <typename T, int WIDTH, int NW, int D>
 __global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const int4 *__restrict__ wg_tab,
@@ -182,10 +198,12 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const 
                                                                const T *__restrict__ x, T *__restrict__ partial)
 {
     __shared__ T xs[WIDTH];
+    __shared__ T stage_all[NW * kStageRuns];
     const int4 wg = wg_tab[blockIdx.x];
     const int64_t c0 = (int64_t)wg.x * WIDTH;
     const int32_t cnt = n - c0 < WIDTH ? (int32_t)(n - c0) : WIDTH;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    T *stage = stage_all + wave * kStageRuns;
     // the first tiles' loads go out before the slice of x is fetched (they do not need it)
     const int32_t last = wg.z - 1;
     Tile<T> tl[D];
@@ -201,7 +219,10 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const 
     while (t < wg.z) {  // uniform over the wave
 #pragma unroll
         for (int d = 0; d < D; ++d) {
-            if (t + d * NW < wg.z) tile_reduce<T>(tl[d], lane, xs, StorePartial<T>{partial + tl[d].base});
+            if (t + d * NW < wg.z) {
+                const int total = tile_reduce<T>(tl[d], lane, xs, StageRun<T>{stage});
+                store_staged<T>(stage, lane, total, partial + tl[d].base);
+            }
             tile_load<T>(tl[d], t + (D + d) * NW < last ? t + (D + d) * NW : last, lane, cf, val, tile_base);
         }
         t += D * NW;

@@ -66,10 +66,11 @@ __device__ __forceinline__ void tile_load(Tile<T> &tl, int32_t t, int lane, cons
 }
 
 // Products, running sums and wave scan of one tile; `emit(rank, sum)` is called once for every run
-// of the tile, rank = position of the run in the tile (a tile starts with a run start).  Lane l
+// of the tile, rank = position of the run in the tile (a tile starts with a run start); returns the
+// number of runs.  Lane l
 // holds elements 4l .. 4l+3; a run start closes the run before it; lane 63 closes the last one.
 template <typename T, typename Emit>
-__device__ __forceinline__ void tile_reduce(const Tile<T> &tl, int lane, const T *xs, Emit emit)
+__device__ __forceinline__ int tile_reduce(const Tile<T> &tl, int lane, const T *xs, Emit emit)
 {
     const bool f0 = (tl.c01 >> 15) & 1, f1 = tl.c01 >> 31, f2 = (tl.c23 >> 15) & 1, f3 = tl.c23 >> 31;
     const T p0 = tl.v[0] * xs[tl.c01 & 0x7fff], p1 = tl.v[1] * xs[(tl.c01 >> 16) & 0x7fff];
@@ -95,6 +96,7 @@ __device__ __forceinline__ void tile_reduce(const Tile<T> &tl, int lane, const T
     hb += f2;
     if (f3) emit(hb - 1, (f0 | f1 | f2) ? r2 : cin + r2);
     if (lane == kWave - 1) emit(total - 1, open);
+    return total;
 }
 
 // The workgroup's window of x (WIDTH values from x + c0, `cnt` of them valid, the rest 0) into
