@@ -37,6 +37,7 @@ namespace asx {
 namespace {
 
 constexpr int32_t kPadRow = 0x7fffffff;
+constexpr int kReducePad = 4 * kWave;  // entries of prow / partial that pass 2 may read past the last partial sum
 
 __global__ __launch_bounds__(kBlock) void k_sliced_keys(const int32_t *__restrict__ col, int32_t nnz, int32_t width,
                                                         int32_t *__restrict__ keys, int32_t *__restrict__ idx)
@@ -250,7 +251,8 @@ __device__ __forceinline__ void lds_add(T *acc, uint16_t id, T v, bool on)
     }
 }
 
-// Walks the ranges of one row block, 64 entries per step.
+// Walks the ranges of one row block, STEP entries per step.
+template <int STEP>
 struct RangeWalk {
     int32_t lo_v, len_v;  // per lane: start and length of range `lane` of the current 64 slices
     int32_t ns;           // ranges in the current group
@@ -261,13 +263,13 @@ struct RangeWalk {
         a = __builtin_amdgcn_readlane(lo_v, j & (kWave - 1));
         len = j < ns ? __builtin_amdgcn_readlane(len_v, j & (kWave - 1)) : 0;
     }
-    // start (an index that is safe to load from for 64 lanes) and count of the next step
+    // start (an index that is safe to load STEP entries from) and count of the next step
     __device__ __forceinline__ void next(int32_t &start, int32_t &count)
     {
         const int32_t left = len - k0;
-        count = left < kWave ? (left > 0 ? left : 0) : kWave;
+        count = left < STEP ? (left > 0 ? left : 0) : STEP;
         start = j < ns ? a + k0 : 0;
-        k0 += kWave;
+        k0 += STEP;
         if (k0 >= len && j < ns) {
             ++j;
             k0 = 0;
@@ -276,7 +278,24 @@ struct RangeWalk {
     }
 };
 
-template <typename T, int NW, int MODE>
+// W consecutive entries of a lane (row ids and partial sums), loaded with one instruction each;
+// the addresses are only aligned to one entry.
+template <typename T, int W>
+struct Entries {
+    typedef uint16_t id_vec __attribute__((ext_vector_type(W)));
+    typedef T pv_vec __attribute__((ext_vector_type(W)));
+    typedef id_vec id_vec_u __attribute__((aligned(2)));
+    typedef pv_vec pv_vec_u __attribute__((aligned(sizeof(T))));
+    id_vec id;
+    pv_vec pv;
+    __device__ __forceinline__ void load(const uint16_t *__restrict__ prow, const T *__restrict__ partial, int64_t at)
+    {
+        id = *reinterpret_cast<const id_vec_u *>(prow + at);
+        pv = *reinterpret_cast<const pv_vec_u *>(partial + at);
+    }
+};
+
+template <typename T, int NW, int MODE, int W>
 __global__ __launch_bounds__(NW *kWave) void k_sliced_reduce(int32_t m, int32_t nrb, int32_t rw, int32_t nslices, T alpha,
                                                              T beta, const int32_t *__restrict__ chunk_lo,
                                                              const uint16_t *__restrict__ prow,
@@ -295,6 +314,49 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_reduce(int32_t m, int32_t 
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     const int32_t *lo_row = chunk_lo + b * nslices;
     const int32_t *hi_row = lo_row + nslices;
+    if (W > 1) {
+        // Long ranges (chosen by the launcher from the mean range length): steps of 64 W entries, W
+        // consecutive ones per lane from one load of the row ids and one of the sums; U steps per
+        // batch, two batches in turn.  Loads are unconditional (prow and partial are readable for
+        // kReducePad entries past the last partial sum); entries past a range's end are dropped at
+        // the add.  A lane adds its W entries in order, so rows repeated inside a lane are safe.
+        constexpr int UW = 8;
+        for (int32_t s0 = 0; s0 < nslices; s0 += kWave) {
+            RangeWalk<kWave * W> w;
+            w.ns = nslices - s0 < kWave ? nslices - s0 : kWave;
+            w.lo_v = lane < w.ns ? lo_row[s0 + lane] : 0;
+            w.len_v = lane < w.ns ? hi_row[s0 + lane] - w.lo_v : 0;
+            w.j = 0;
+            w.k0 = 0;
+            w.fetch();
+            Entries<T, W> ea[UW], eb[UW];
+            int32_t na[UW], nb[UW];
+#define ASX_LOADW(E, N)                            \
+    _Pragma("unroll") for (int u = 0; u < UW; ++u) \
+    {                                              \
+        int32_t start;                             \
+        w.next(start, N[u]);                       \
+        E[u].load(prow, partial, (int64_t)start + lane * W); \
+    }
+#define ASX_ADDW(E, N)                             \
+    _Pragma("unroll") for (int u = 0; u < UW; ++u) \
+    {                                              \
+        _Pragma("unroll") for (int e = 0; e < W; ++e) lds_add<MODE, T>(acc, E[u].id[e], E[u].pv[e], lane * W + e < N[u]); \
+    }
+            ASX_LOADW(ea, na)
+            ASX_LOADW(eb, nb)
+            while (true) {  // uniform over the wave
+                ASX_ADDW(ea, na)
+                const bool more_a = w.j < w.ns;
+                ASX_LOADW(ea, na)
+                ASX_ADDW(eb, nb)
+                if (!more_a) break;  // nothing was left when batch a was reloaded: a and b are spent
+                ASX_LOADW(eb, nb)
+            }
+#undef ASX_LOADW
+#undef ASX_ADDW
+        }
+    } else {
     // Steps of 64 (row, partial sum) pairs, U steps per batch, two batches in turn: a batch's loads
     // are issued before the other batch is added.  Loads are unconditional (prow and partial are
     // readable for 64 entries past the last partial sum; a step past the end reads entry 0 on);
@@ -336,7 +398,7 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_reduce(int32_t m, int32_t 
 #undef ASX_LOAD
 #undef ASX_ADDJ
         } else {
-            RangeWalk w;
+            RangeWalk<kWave> w;
             w.ns = ns;
             w.lo_v = lo_v;
             w.len_v = len_v;
@@ -365,6 +427,7 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_reduce(int32_t m, int32_t 
 #undef ASX_LOAD
         }
 #undef ASX_ADD
+    }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const int64_t r0 = b * rw;
@@ -469,11 +532,11 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
         ASX_TRY(hipMemcpyAsync(&sm.npartials, hscan + (slots - 1), sizeof(int32_t), hipMemcpyDeviceToHost, s));
         ASX_TRY(hipStreamSynchronize(s));
         ASX_TRY(hipMalloc((void **)&sm.tile_base, sizeof(int32_t) * ((size_t)sm.ntiles + 1)));
-        ASX_TRY(hipMalloc((void **)&sm.prow, sizeof(uint16_t) * ((size_t)sm.npartials + kWave)));
-        ASX_TRY(hipMemsetAsync(sm.prow, 0, sizeof(uint16_t) * ((size_t)sm.npartials + kWave), s));
+        ASX_TRY(hipMalloc((void **)&sm.prow, sizeof(uint16_t) * ((size_t)sm.npartials + kReducePad)));
+        ASX_TRY(hipMemsetAsync(sm.prow, 0, sizeof(uint16_t) * ((size_t)sm.npartials + kReducePad), s));
         ASX_TRY(hipMalloc((void **)&prow_full, sizeof(int32_t) * (size_t)sm.npartials));
-        ASX_TRY(hipMalloc(&sm.partial, sizeof(T) * ((size_t)sm.npartials + kWave)));
-        ASX_TRY(hipMemsetAsync(sm.partial, 0, sizeof(T) * ((size_t)sm.npartials + kWave), s));
+        ASX_TRY(hipMalloc(&sm.partial, sizeof(T) * ((size_t)sm.npartials + kReducePad)));
+        ASX_TRY(hipMemsetAsync(sm.partial, 0, sizeof(T) * ((size_t)sm.npartials + kReducePad), s));
         ASX_TRY(hipMalloc((void **)&sm.chunk_lo, sizeof(int32_t) * ((size_t)sm.nrb + 1) * (size_t)sm.nslices));
         hipLaunchKernelGGL(k_sliced_tile_base, dim3((unsigned)ceil_div64((int64_t)sm.ntiles + 1, kBlock)), dim3(kBlock),
                            0, s, hscan, sm.ntiles, sm.tile_base);
@@ -558,8 +621,20 @@ int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, co
     // fp32: plain LDS read-add-write (LDS float atomics measured 2.5x slower on scattered rows);
     // fp64: LDS atomic adds (no dependent read in the wave's instruction stream; measured faster)
     constexpr int kMode = sizeof(T) == 4 ? 1 : 0;
-    hipLaunchKernelGGL((k_sliced_reduce<T, kWaves, kMode>), dim3(rgrid), dim3(kWaves * kWave), lds, s, m, sm->nrb,
-                       sm->rows_per_wave, sm->nslices, alpha, beta, sm->chunk_lo, sm->prow, partial, y);
+    // entries per lane and step, from the mean number of partial sums a row block has in one slice
+    // (a step should be mostly full): 64-wide steps below 80, 128-wide below 160, else 256-wide (fp32)
+    const double mean_range = (double)sm->npartials / ((double)sm->nrb * (double)sm->nslices);
+    const int wide = mean_range < 80.0 ? 1 : (mean_range < 160.0 || sizeof(T) == 8) ? 2 : 4;
+#define ASX_RED(WW)                                                                                                   \
+    hipLaunchKernelGGL((k_sliced_reduce<T, kWaves, kMode, WW>), dim3(rgrid), dim3(kWaves * kWave), lds, s, m, sm->nrb, \
+                       sm->rows_per_wave, sm->nslices, alpha, beta, sm->chunk_lo, sm->prow, partial, y)
+    if (wide == 1)
+        ASX_RED(1);
+    else if (wide == 2)
+        ASX_RED(2);
+    else
+        ASX_RED(4);
+#undef ASX_RED
     return check_launch();
 }
 
