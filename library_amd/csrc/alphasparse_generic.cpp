@@ -662,6 +662,22 @@ alphasparseStatus_t alphasparseSpMV_bufferSize(alphasparseHandle_t handle, alpha
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
+// Analysis on first use, for callers written against the reference, where alphasparseSpMV_analysis
+// and alphasparseSpMM_preprocess are stubs or cheap and therefore often never called
+// (hip/kernel/level2/alphasparse_spmv.hip:229-256): with ALPHASPARSE_AMD_AUTO_ANALYSIS=1 in the
+// environment the first alphasparseSpMV / alphasparseSpMM on a descriptor runs the analysis itself
+// (allocates and synchronises once; later calls are kernels only).  Off by default, because kept
+// analysis may hold a copy of A's values that a caller who updates them in place would not know
+// to refresh.  Read once per process.
+static bool auto_analysis()
+{
+    static const bool on = [] {
+        const char *e = std::getenv("ALPHASPARSE_AMD_AUTO_ANALYSIS");
+        return e && e[0] && e[0] != '0';
+    }();
+    return on;
+}
+
 alphasparseStatus_t alphasparseSpMV_analysis(alphasparseHandle_t handle, alphasparseOperation_t opA,
                                              alphasparseSpMatDescr_t matA, alphasparseSpMVAlg_t alg)
 {
@@ -728,6 +744,14 @@ alphasparseStatus_t alphasparseSpMV(alphasparseHandle_t handle, alphasparseOpera
     const _alphasparseSpMatDescr *A = &eff.d;
     const int32_t m = (int32_t)A->rows, n = (int32_t)A->cols, nnz = (int32_t)A->nnz;
     const asx_plan *plan = find_plan(matA, false, (int)alg, A, 1);
+    if (!plan && auto_analysis()) {
+        release_effective(handle, &eff);
+        s = alphasparseSpMV_analysis(handle, opA, matA, alg);
+        if (s) return s;
+        s = make_effective(handle, matA, opA, &eff);
+        if (s) return s;
+        plan = find_plan(matA, false, (int)alg, A, 1);
+    }
     const size_t need = plan ? asx_plan_workspace_bytes(plan)
                              : asx_spmv_workspace_bytes((int)alg, (int)A->data_type, m, nnz);
     bool ok;
@@ -869,6 +893,15 @@ alphasparseStatus_t alphasparseSpMM(alphasparseHandle_t handle, alphasparseOpera
     const int32_t m = (int32_t)A->rows, k = (int32_t)A->cols, nnz = (int32_t)A->nnz;
     const int vt = (int)A->data_type;
     const asx_plan *plan = find_plan(matA, true, (int)alg, A, ncols);
+    if (!plan && auto_analysis()) {
+        release_effective(handle, &eff);
+        size_t unused = 0;
+        s = alphasparseSpMM_preprocess(handle, opA, opB, alpha, matA, matB, beta, matC, computeType, alg, &unused);
+        if (s) return s;
+        s = make_effective(handle, matA, opA, &eff);
+        if (s) return s;
+        plan = find_plan(matA, true, (int)alg, A, ncols);
+    }
     const size_t kernel_need =
         plan ? asx_plan_workspace_bytes(plan) : asx_spmm_workspace_bytes((int)alg, vt, m, nnz, ncols);
     size_t b_bytes, c_bytes;

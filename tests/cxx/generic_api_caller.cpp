@@ -101,6 +101,12 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
             s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
         }
+        // analysis on first use (ALPHASPARSE_AMD_AUTO_ANALYSIS=1): the calls above must have left
+        // kept analysis on the descriptor although alphasparseSpMV_analysis was never called
+        if (!analysis) {
+            const char *e = std::getenv("ALPHASPARSE_AMD_AUTO_ANALYSIS");
+            if ((e && e[0] == '1') != A->analysed) return 12;
+        }
         if (analysis == 2) {
             // the caller changes A's values in place (same pattern) and says so by calling the
             // analysis again; the next product must use the new values
@@ -167,6 +173,10 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
             HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
             s = alphasparseSpMM(handle, opA, opB, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
+        }
+        if (!analysis) {
+            const char *e = std::getenv("ALPHASPARSE_AMD_AUTO_ANALYSIS");
+            if ((e && e[0] == '1') != A->analysed) return 12;
         }
         if (analysis == 2) {  // new values in place, preprocess again, multiply again
             auto val2 = read_bin<T>(dir + "/val2.bin", nnz);

@@ -15,9 +15,9 @@ EXE = os.path.join(ROOT, "tests", "cxx", "generic_api_caller")
 
 
 def _run_case(tmp_path, op, dtype, rp, col, val, x, y, ncols, alg, alpha, beta, analysis, variant=(0, 0, 0, 0, 0),
-              n=None, val2=None):
+              n=None, val2=None, env=None):
     """variant = (trans_a, idx_base, col_major_b, col_major_c, trans_b); n = columns of A."""
-    d = tmp_path / f"{op}_{np.dtype(dtype).name}_{alg}_{analysis}_{''.join(map(str, variant))}"
+    d = tmp_path / f"{op}_{np.dtype(dtype).name}_{alg}_{analysis}_{''.join(map(str, variant))}{'_env' if env else ''}"
     d.mkdir()
     for name, a in (("row_ptr", rp), ("col", col), ("val", val), ("x", x), ("y", y)):
         np.ascontiguousarray(a).tofile(d / f"{name}.bin")
@@ -28,7 +28,8 @@ def _run_case(tmp_path, op, dtype, rp, col, val, x, y, ncols, alg, alpha, beta, 
         n = x.size // ncols
     (d / "meta.txt").write_text(f"{op} {tag} {rp.size - 1} {n} {col.size} {ncols} {alg} {alpha!r} {beta!r} {analysis}\n"
                                 + " ".join(map(str, variant)) + "\n")
-    r = subprocess.run([EXE, str(d)], capture_output=True, text=True, timeout=120)
+    r = subprocess.run([EXE, str(d)], capture_output=True, text=True, timeout=120,
+                       env=dict(os.environ, **env) if env else None)
     assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
     return np.fromfile(d / "out.bin", dtype=dtype)
 
@@ -217,6 +218,32 @@ def test_spmv_analysis_on_a_scattered_matrix(tmp_path, oracle):
     ref_t = oracle.spmv(rp_t, col_t, val_t, y0, alpha, beta, x, 8)
     got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, y0, x, 1, 0, alpha, beta, 1, (1, 0, 0, 0, 0), n=n)
     assert_close(got, ref_t, spmv_scale(rp_t, col_t, val_t, y0, alpha, beta, x), np.float64, "transpose, DEFAULT with analysis")
+
+
+def test_analysis_on_first_use(tmp_path, oracle):
+    """ALPHASPARSE_AMD_AUTO_ANALYSIS=1: a caller that never calls alphasparseSpMV_analysis /
+    alphasparseSpMM_preprocess (the reference's own test loops do not) gets kept analysis from its
+    first call on; the caller program checks that the descriptor ends up analysed, and without the
+    variable does not."""
+    from library_amd import workloads as W
+    rp, col, val = W.csr_zipf(1 << 20, 1 << 20, 20, 1.0, 5000, 0.01, np.float64, 5)
+    n = 1 << 20
+    rng = np.random.default_rng(71)
+    x = rng.uniform(-1, 1, n)
+    y0 = rng.uniform(-1, 1, rp.size - 1)
+    got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, 2.1, 3.2, 0,
+                    env={"ALPHASPARSE_AMD_AUTO_ANALYSIS": "1"})
+    assert_close(got, oracle.spmv(rp, col, val, x, 2.1, 3.2, y0, 8), spmv_scale(rp, col, val, x, 2.1, 3.2, y0),
+                 np.float64, "SpMV, analysis on first use")
+    from test_gpu_parity import _block_structured
+    m, k, nc = 700, 640, 64
+    rp, col, val = _block_structured(rng, m, k, np.float32)
+    B = rng.uniform(-1, 1, k * nc).astype(np.float32)
+    C0 = rng.uniform(-1, 1, m * nc).astype(np.float32)
+    got = _run_case(tmp_path, "spmm", np.float32, rp, col, val, B, C0, nc, 0, 2.0, 3.0, 0,
+                    env={"ALPHASPARSE_AMD_AUTO_ANALYSIS": "1"})
+    assert_close(got, oracle.spmm(rp, col, val, B, nc, 2.0, 3.0, C0, 4), spmm_scale(rp, col, val, B, nc, 2.0, 3.0, C0),
+                 np.float32, "SpMM, analysis on first use")
 
 
 def test_spmm_blocked_values_changed_after_preprocess(tmp_path, oracle):
