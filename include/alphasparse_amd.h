@@ -197,10 +197,13 @@ int asx_spmm_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, in
  * sizes puts it at least 10 % ahead of the row-ordered kernels; the choice depends on the matrix
  * alone, not on timings.  Otherwise as asx_plan_create.  No counterpart in the reference (its
  * alphasparseSpMV_analysis is a stub).  alg = ASX_SPMV_WINDOW builds the row-block copy for the
- * kernel that keeps a sliding window of x in LDS (again a COPY of columns and values, and the
+ * kernel that keeps sliding windows of x in LDS (again a COPY of columns and values, and the
  * carry slots of a call); DEFAULT picks it, when the sliced kernel is not chosen, for nnz >= 2^21
- * and rows no longer than 2048 whenever the matrix qualifies (every 256 consecutive rows reach
- * over fewer than 16376 columns).  Synchronises `stream`. */
+ * and rows no longer than 2048 whenever the matrix qualifies: every 256 consecutive rows reach
+ * over fewer than 16376 columns, or the stored elements lie on at most 4 bands of diagonals whose
+ * windows fit the LDS together (stencils on three-dimensional grids); otherwise
+ * ASX_STATUS_NOT_SUPPORTED for the explicit id, the row-ordered plan for DEFAULT.  Synchronises
+ * `stream`. */
 int asx_spmv_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
                          const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, void *stream);
 /* Brings a plan that holds a copy of A's values (ASX_SPMV_SLICED, ASX_SPMV_WINDOW, ASX_SPMM_BLOCKED) up to date

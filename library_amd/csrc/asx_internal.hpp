@@ -147,24 +147,27 @@ int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s);
 template <typename T>
 int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, hipStream_t s);
 
-// ---- row blocks with a sliding window of x in LDS (asx_window.hip) ----
-// Blocks of `rows_per_block` consecutive rows whose columns all lie inside fewer than 16384
-// columns, chained: a workgroup walks a chain of blocks with LDS as a ring over the columns of x
-// and fetches, per block, only the columns that are new.  The stored elements stream as tiles
-// (16-bit column mod 16384 + row-start flag, as the sliced kernel's); every row owns at least one
-// slot, so a tile's runs are consecutive rows and go straight to y.
+// ---- row blocks with sliding windows of x in LDS (asx_window.hip) ----
+// Blocks of `rows_per_block` consecutive rows whose columns all lie inside at most kWindowBands
+// bands that together span fewer than 16384 columns, chained: a workgroup walks a chain of blocks
+// with a ring in LDS per band and fetches, per block, only the columns that are new.  The stored
+// elements stream as tiles (16-bit LDS slot + row-start flag, as the sliced kernel's); every row
+// owns at least one slot, so a tile's runs are consecutive rows and go straight to y.
+constexpr int kWindowBands = 4;
 struct WindowMatrix {
     int32_t rows_per_block;
     int32_t nblocks;
     int32_t nchains;         // workgroups
     int32_t ntiles;
+    int32_t nbands;          // 1: one window per block; 2..kWindowBands: bands of diagonals
     int has_carry;           // some tile starts inside a row: the ordered carry pass is needed
     void *val;               // ntiles * kSlicedTile values (a copy of A's; pads are 0)
     void *carry;             // ntiles values
-    uint16_t *cf;            // ntiles * kSlicedTile: column mod 16384, bit 15 = first slot of a row (or tile)
+    uint16_t *cf;            // ntiles * kSlicedTile: LDS slot of the column, bit 15 = first slot of a row (or tile)
     int32_t *perm;           // where each stored copy comes from in A's val (-1 for pads)
     int32_t *tile_info;      // ntiles x 2: row of the tile's first slot (bit 31: the tile starts inside it), rows in the tile
-    int32_t *blocks;         // nblocks x 4: first tile, end tile, columns to fetch before the block (from, to)
+    int32_t *blocks;         // nblocks x 4: first tile, end tile, first piece, end piece
+    int32_t *pieces;         // x 4: columns of x to fetch before a block (from, to), first LDS slot and size of their ring
     int32_t *chains;         // nchains x 2: first block, end block
 };
 template <typename T>

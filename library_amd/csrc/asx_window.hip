@@ -1,5 +1,6 @@
-// Row-block CSR SpMV with a sliding window of x in LDS, for matrices whose rows reach only
-// nearby columns (stencils, banded and finite-element matrices).
+// Row-block CSR SpMV with sliding windows of x in LDS, for matrices whose rows reach only
+// nearby columns (stencils, banded and finite-element matrices) or a few bands of diagonals
+// (stencils on three-dimensional grids).
 //
 // The row-ordered kernels read 4 bytes of column index per stored element, the row offsets, and
 // gather x through the L2 (one request per stored element).  Here the rows are cut, once (plan
@@ -7,14 +8,17 @@
 // kWindowCols columns, and consecutive blocks are chained: a workgroup walks its chain of blocks
 // with LDS as a ring over the columns of x (column c lives at c mod kWindowCols), so that from
 // one block to the next only the columns that are new are fetched - while the block before is
-// still being multiplied - and x crosses the L2 once.  The block's stored elements stream as
-// tiles of 256 with a 16-bit column-mod-window and a "first element of a row" flag per element
-// (10 instead of 12.8 bytes per stored element in fp64; no row offsets are read).  Every row owns
-// at least one slot (an empty row gets a zero that points at a zero in LDS), so the runs of a tile
-// are consecutive rows and a run's sum goes straight to y.  Rows of up to 16 stored elements are
-// never cut by a tile start (the tile is padded instead); a longer row that is cut leaves its
-// later pieces in carry slots, which an ordered pass adds to y afterwards (no atomics; results are
-// bit-reproducible).
+// still being multiplied - and x crosses the L2 once.  Where no such window exists but the
+// stored elements lie on at most kWindowBands bands of diagonals (column minus row inside a few
+// narrow intervals: the planes of a 7- or 27-point stencil), every band gets a ring of its own in
+// LDS and a block fetches the new columns of every band (x then crosses the L2 once per band).
+// The block's stored elements stream as tiles of 256 with a 16-bit LDS slot and a "first element
+// of a row" flag per element (10 instead of 12.8 bytes per stored element in fp64; no row offsets
+// are read).  Every row owns at least one slot (an empty row gets a zero that points at a zero in
+// LDS), so the runs of a tile are consecutive rows and a run's sum goes straight to y.  Rows of up
+// to 16 stored elements are never cut by a tile start (the tile is padded instead); a longer row
+// that is cut leaves its later pieces in carry slots, which an ordered pass adds to y afterwards
+// (no atomics; results are bit-reproducible).
 //
 // The reference has no counterpart (its CSR kernels read 32-bit columns and gather x from global
 // memory: hip/kernel/level2/alphasparse_spmv_csr_vector.h:99-126).
@@ -124,10 +128,37 @@ __global__ __launch_bounds__(kBlock) void k_window_fill_pads(int64_t slots, uint
     perm[d] = -1;
 }
 
+// Where the columns of x live in LDS.  One band (nbands = 1): column c at c mod kWindowCols.
+// Several: the stored elements whose offset from the diagonal, c - floor(r n / m), lies in
+// [dlo[k], dhi[k]] use ring k: column c at base[k] + c mod width[k].
+struct BandTable {
+    int32_t nbands;
+    int32_t dlo[kWindowBands], dhi[kWindowBands], base[kWindowBands], width[kWindowBands];
+};
+__host__ __device__ __forceinline__ int64_t band_centre(int64_t r, int64_t m, int64_t n) { return r * n / m; }
+
+// bit b of `bits` set = some stored element has (c - centre(r) + n) / 64 == b
+__global__ __launch_bounds__(kBlock) void k_window_offset_bins(const int32_t *__restrict__ row_ptr,
+                                                               const int32_t *__restrict__ col, int32_t m, int32_t n,
+                                                               uint32_t *__restrict__ bits)
+{
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= m) return;
+    const int64_t shift = (int64_t)n - band_centre(r, m, n);
+    int64_t last = -1;
+    for (int32_t k = row_ptr[r]; k < row_ptr[r + 1]; ++k) {
+        const int64_t bin = ((int64_t)col[k] + shift) >> 6;
+        if (bin == last) continue;
+        last = bin;
+        const uint32_t mask = 1u << (bin & 31);
+        if (!(bits[bin >> 5] & mask)) atomicOr(bits + (bin >> 5), mask);  // mostly set already: few atomics
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_window_place(const int32_t *__restrict__ row_ptr,
                                                          const int32_t *__restrict__ col, const T *__restrict__ val,
-                                                         int32_t m, int32_t nnz, int32_t rows,
+                                                         int32_t m, int32_t n, int32_t nnz, int32_t rows, BandTable bands,
                                                          const int32_t *__restrict__ row_start,
                                                          const int32_t *__restrict__ tile_off, uint16_t *__restrict__ cf,
                                                          T *__restrict__ val_out, int32_t *__restrict__ perm)
@@ -146,7 +177,15 @@ __global__ __launch_bounds__(kBlock) void k_window_place(const int32_t *__restri
     const int32_t o = row_start[r] + (int32_t)(i - row_ptr[r]);
     const int64_t d = (int64_t)tile_off[b] * kSlicedTile + o;
     const bool head = i == row_ptr[r] || o % kSlicedTile == 0;
-    cf[d] = (uint16_t)((col[i] % kWindowCols) | (head ? 0x8000 : 0));
+    const int32_t c = col[i];
+    int k = 0;
+    if (bands.nbands > 1) {
+        const int64_t off = (int64_t)c - band_centre(r, m, n);
+        for (int j = 1; j < kWindowBands; ++j)
+            if (j < bands.nbands && off >= bands.dlo[j]) k = j;  // bands ascend and cover every offset
+    }
+    const int32_t slot = bands.base[k] + c % bands.width[k];
+    cf[d] = (uint16_t)(slot | (head ? 0x8000 : 0));
     const int64_t phys = d / kSlicedTile * kSlicedTile + tile_val_pos<T>((int)(d % kSlicedTile));
     val_out[phys] = val[i];
     perm[phys] = (int32_t)i;
@@ -270,64 +309,115 @@ __device__ __forceinline__ void window_tile_load(WindowTile<T> &tl, int32_t t, i
     tl.limit = info.y;
 }
 
-// The columns [lo, hi) of x (lo a multiple of 4, hi - lo <= kWindowCols) into registers, one
-// 16-byte piece per thread and step; columns at or past n read as 0.  Every register is written by
-// one load instruction only (predicated, after a zero fill), never by two alternative ones: with
+// The pieces of x a block needs before it is multiplied (at most kWindowBands ranges of columns
+// [from, to), from a multiple of 4, together at most kWindowCols columns; ring of piece q: slots
+// base .. base + width) into registers, one 16-byte unit per thread and step, and later from the
+// registers into the rings.  Columns at or past n read as 0.  Every register is written by one
+// load instruction only (predicated, after a zero fill), never by two alternative ones: with
 // alternatives the compiler orders them with a full s_waitcnt between the steps and the fetch
-// takes one memory round trip per step.  ALIGNED (x on a 16-byte boundary): whole pieces inside x
-// with one 16-byte load; the piece that straddles the end of x (n no multiple of the piece),
-// element by element into `tail` by the one thread that owns it.  Otherwise element by element.
-template <typename T, int THREADS, bool ALIGNED>
+// takes one memory round trip per step.  VEC (x on a 16-byte boundary, n at least one unit): one
+// 16-byte load per unit; the unit that straddles the end of x is read from the last whole unit
+// inside x (an unaligned address) and shifted into place when it is stored.  Otherwise element by
+// element.  NB = 1: one piece, ring of kWindowCols slots from slot 0 (no piece search, constant modulus).
+template <typename T, int THREADS, bool VEC, int NB>
 struct XFetch {
     static constexpr int V = 16 / sizeof(T);
     static constexpr int PER = kWindowCols / (THREADS * V);
     typedef T vec_t __attribute__((ext_vector_type(V)));
+    typedef vec_t vec_u __attribute__((aligned(sizeof(T))));
     vec_t buf[PER];
-    vec_t tail;
-    __device__ __forceinline__ void load(const T *__restrict__ x, int32_t n, int32_t lo, int32_t hi)
+    // the pending fetch (uniform values): its pieces, the first unit of each and the ring slot of
+    // its first column
+    int32_t from[NB], to[NB], base[NB], width[NB], ustart[NB], fslot[NB];
+
+    __device__ __forceinline__ void set(const int4 *__restrict__ pieces, int32_t lo, int32_t hi)
+    {
+        int32_t u = 0;
+#pragma unroll
+        for (int q = 0; q < NB; ++q) {
+            int4 pc = make_int4(0, 0, 0, 4);
+            if (lo + q < hi) pc = pieces[lo + q];  // uniform
+            from[q] = __builtin_amdgcn_readfirstlane(pc.x);
+            to[q] = __builtin_amdgcn_readfirstlane(pc.y);
+            base[q] = NB == 1 ? 0 : __builtin_amdgcn_readfirstlane(pc.z);
+            width[q] = NB == 1 ? kWindowCols : __builtin_amdgcn_readfirstlane(pc.w);
+            fslot[q] = (int32_t)((uint32_t)from[q] % (uint32_t)width[q]);
+            ustart[q] = u;
+            u += (to[q] - from[q] + V - 1) / V;
+        }
+    }
+    // unit u: first column, end of its piece, LDS slot (a unit past the last piece lands at or past
+    // `to` of the last one).  A piece is no longer than its ring, so one wrap suffices.
+    __device__ __forceinline__ void locate(int32_t u, int32_t &c, int32_t &c_to, int32_t &slot) const
+    {
+        int32_t f = from[0], s = 0, fs = fslot[0], b = base[0], w = width[0];
+        c_to = to[0];
+#pragma unroll
+        for (int q = 1; q < NB; ++q) {
+            const bool in = u >= ustart[q];
+            f = in ? from[q] : f;
+            s = in ? ustart[q] : s;
+            fs = in ? fslot[q] : fs;
+            b = in ? base[q] : b;
+            w = in ? width[q] : w;
+            c_to = in ? to[q] : c_to;
+        }
+        const int32_t off = (u - s) * V;
+        c = f + off;
+        const int32_t sl = fs + off;
+        slot = b + (sl >= w ? sl - w : sl);
+    }
+    __device__ __forceinline__ void load(const T *__restrict__ x, int32_t n)
     {
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
-            const int64_t c = (int64_t)lo + ((int64_t)k * THREADS + threadIdx.x) * V;
+            int32_t c, c_to, slot;
+            locate(k * THREADS + (int)threadIdx.x, c, c_to, slot);
             buf[k] = vec_t(T(0));
-            if (ALIGNED) {
-                if (c < hi && c + V <= n) buf[k] = *reinterpret_cast<const vec_t *>(x + c);
+            if (VEC) {
+                if (c < c_to && c < n) buf[k] = *reinterpret_cast<const vec_u *>(x + (n - c >= V ? (int64_t)c : (int64_t)n - V));
             } else {
 #pragma unroll
                 for (int e = 0; e < V; ++e)
-                    if (c + e < hi && c + e < n) buf[k][e] = x[c + e];
-            }
-        }
-        if (ALIGNED) {
-            tail = vec_t(T(0));
-            const int64_t cs = (int64_t)n & ~(int64_t)(V - 1);  // start of the piece that straddles the end of x
-            if (cs < n && cs >= lo && cs < hi && ((cs - lo) / V) % THREADS == (int64_t)threadIdx.x) {
-#pragma unroll
-                for (int e = 0; e < V - 1; ++e)
-                    if (cs + e < n) tail[e] = x[cs + e];
+                    if (c_to - c > e && n - c > e) buf[k][e] = x[(int64_t)c + e];
             }
         }
     }
-    __device__ __forceinline__ void store(T *xs, int32_t n, int32_t lo, int32_t hi) const
+    __device__ __forceinline__ void store(T *xs, int32_t n) const
     {
-        const int64_t cs = (int64_t)n & ~(int64_t)(V - 1);
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
-            const int64_t c = (int64_t)lo + ((int64_t)k * THREADS + threadIdx.x) * V;
-            if (c < hi) *reinterpret_cast<vec_t *>(xs + (c % kWindowCols)) = (ALIGNED && c == cs) ? tail : buf[k];
+            int32_t c, c_to, slot;
+            locate(k * THREADS + (int)threadIdx.x, c, c_to, slot);
+            if (c < c_to) {
+                vec_t v = buf[k];
+                if (VEC && c < n && n - c < V) {
+                    // holds x[n - V .. n): the columns c .. n - 1 move to the front, zeros behind them
+                    const int cnt = n - c;
+                    vec_t w = vec_t(T(0));
+#pragma unroll
+                    for (int e = 0; e < V - 1; ++e)
+#pragma unroll
+                        for (int j = 1; j < V; ++j)
+                            if (e < cnt && j == V - cnt + e) w[e] = v[j];
+                    v = w;
+                }
+                *reinterpret_cast<vec_t *>(xs + slot) = v;
+            }
         }
     }
 };
 
-template <typename T, int NW, bool ALIGNED>
+template <typename T, int NW, bool VEC, int NB>
 __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T beta, const int2 *__restrict__ chains,
                                                            const int4 *__restrict__ blocks,
+                                                           const int4 *__restrict__ pieces,
                                                            const uint16_t *__restrict__ cf, const T *__restrict__ val,
                                                            const int2 *__restrict__ tile_info,
                                                            const T *__restrict__ x, T *__restrict__ y,
                                                            T *__restrict__ carry)
 {
-    // ring over the columns of x, then the zero the pads point at
+    // the rings over the columns of x, then the zero the pads point at
     __shared__ __align__(16) T xs[kWindowCols + 16 / sizeof(T)];
     __shared__ T stage_all[NW * kStageRows];
     const int2 chain = chains[blockIdx.x];  // first block, end block
@@ -341,21 +431,23 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
     window_tile_load<T>(ta, t < chain_last ? t : chain_last, lane, cf, val, tile_info);
     window_tile_load<T>(tb, t + NW < chain_last ? t + NW : chain_last, lane, cf, val, tile_info);
     if (threadIdx.x == 0) xs[kWindowCols] = T(0);
-    XFetch<T, NW * kWave, ALIGNED> xf;
-    int4 blk = blocks[chain.x];  // first tile, end tile, columns to fetch before the block: from, to
-    xf.load(x, n, blk.z, blk.w);
+    XFetch<T, NW * kWave, VEC, NB> xf;
+    int4 blk = blocks[chain.x];  // first tile, end tile, pieces of x to fetch before the block: first, end
+    xf.set(pieces, blk.z, blk.w);
+    xf.load(x, n);
     int32_t b = chain.x, tile_hi;
     // Start of block b: the columns fetched for it go into the ring once every wave is done with
     // the block before; the next block's new columns are fetched while this one is multiplied.
 #define ASX_BLOCK_BEGIN()                      \
     {                                          \
         __syncthreads();                       \
-        xf.store(xs, n, blk.z, blk.w);         \
+        xf.store(xs, n);                       \
         __syncthreads();                       \
         tile_hi = blk.y;                       \
         if (b + 1 < chain.y) {                 \
             blk = blocks[b + 1];               \
-            xf.load(x, n, blk.z, blk.w);       \
+            xf.set(pieces, blk.z, blk.w);      \
+            xf.load(x, n);                     \
         }                                      \
     }
 #define ASX_STEP(TL, TT)                                                                                          \
@@ -411,11 +503,11 @@ __global__ __launch_bounds__(kBlock) void k_window_fixup(int32_t ntiles, T alpha
 void free_window(WindowMatrix *p)
 {
     for (void *q : {p->val, p->carry, (void *)p->cf, (void *)p->perm, (void *)p->tile_info, (void *)p->blocks,
-                    (void *)p->chains})
+                    (void *)p->pieces, (void *)p->chains})
         if (q) (void)hipFree(q);
     p->val = p->carry = nullptr;
     p->cf = nullptr;
-    p->perm = p->tile_info = p->blocks = p->chains = nullptr;
+    p->perm = p->tile_info = p->blocks = p->pieces = p->chains = nullptr;
 }
 
 template <typename T>
@@ -430,7 +522,10 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     int32_t *bmin = nullptr, *bmax = nullptr, *btiles = nullptr, *tile_off = nullptr, *d_small = nullptr;
     void *tmp = nullptr;
     size_t tmp_bytes = 0;
-    std::vector<int32_t> h_bmin, h_bmax, h_off, blk, chains;
+    std::vector<int32_t> h_bmin, h_bmax, h_off, blk, pcs, chains;
+    std::vector<uint32_t> h_bits;
+    uint32_t *d_bits = nullptr;
+    BandTable bands{};
     int64_t slots = 0;
     int32_t h_small[2] = {0, 0};
     const unsigned mgrid = (unsigned)ceil_div64(m, kBlock);
@@ -469,10 +564,69 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
             break;
         }
     }
+    bands.nbands = 1;
+    bands.base[0] = 0;
+    bands.width[0] = kWindowCols;
     if (wm.rows_per_block == 0) {
-        st = ASX_STATUS_NOT_SUPPORTED;  // some 256 rows reach further than the ring: not this kernel's matrix
-        goto done;
+        // 2b. some 256 rows reach further than the ring.  Bands of diagonals instead: which offsets
+        //     c - centre(r) occur (a bit per 64 of them), the runs of occupied offsets, and the
+        //     largest block whose bands (block's advance along the diagonal + width of the run) fit
+        //     the LDS together.  More runs than rings: the closest runs are joined.
+        const int64_t nbins = (2 * (int64_t)n >> 6) + 2;
+        const size_t words = (size_t)(nbins + 31) / 32;
+        ASX_TRY(hipMalloc((void **)&d_bits, sizeof(uint32_t) * words));
+        ASX_TRY(hipMemsetAsync(d_bits, 0, sizeof(uint32_t) * words, s));
+        hipLaunchKernelGGL(k_window_offset_bins, dim3(mgrid), dim3(kBlock), 0, s, row_ptr, col, m, n, d_bits);
+        h_bits.resize(words);
+        ASX_TRY(hipMemcpyAsync(h_bits.data(), d_bits, sizeof(uint32_t) * words, hipMemcpyDeviceToHost, s));
+        ASX_TRY(hipStreamSynchronize(s));
+        std::vector<std::pair<int64_t, int64_t>> runs;  // first and last occupied bin
+        for (int64_t b = 0; b < nbins; ++b) {
+            if (!(h_bits[(size_t)(b >> 5)] >> (b & 31) & 1u)) continue;
+            if (!runs.empty() && runs.back().second + 1 >= b)
+                runs.back().second = b;
+            else
+                runs.emplace_back(b, b);
+        }
+        while ((int)runs.size() > kWindowBands) {  // join the two runs with the smallest gap
+            size_t best = 0;
+            for (size_t i = 1; i + 1 < runs.size(); ++i)
+                if (runs[i + 1].first - runs[i].second < runs[best + 1].first - runs[best].second) best = i;
+            runs[best].second = runs[best + 1].second;
+            runs.erase(runs.begin() + (long)best + 1);
+        }
+        if (runs.empty()) {
+            st = ASX_STATUS_NOT_SUPPORTED;
+            goto done;
+        }
+        bands.nbands = (int32_t)runs.size();
+        for (int k = 0; k < bands.nbands; ++k) {
+            bands.dlo[k] = (int32_t)std::max<int64_t>((runs[(size_t)k].first << 6) - n, -(int64_t)n);
+            bands.dhi[k] = (int32_t)std::min<int64_t>(((runs[(size_t)k].second + 1) << 6) - 1 - n, n);
+        }
+        for (int32_t rows : {8192, 7168, 6144, 5120, 4608, 4096, 3584, 3072, 2560, 2048, 1792, 1536, 1280, 1024, 768, 512, 384, 256}) {
+            if (rows > 256 && ceil_div64(m, rows) < min_blocks) continue;
+            const int64_t advance = ceil_div64((int64_t)rows * n, m) + 1;  // of the centre over a block
+            int64_t total = 0;
+            for (int k = 0; k < bands.nbands; ++k)
+                total += (advance + ((int64_t)bands.dhi[k] - bands.dlo[k]) + 1 + kWindowSlack + 3 + 3) & ~(int64_t)3;
+            if (total > kWindowCols) continue;
+            wm.rows_per_block = rows;
+            wm.nblocks = (int32_t)ceil_div64(m, rows);
+            int32_t at = 0;
+            for (int k = 0; k < bands.nbands; ++k) {
+                bands.base[k] = at;
+                bands.width[k] = (int32_t)((advance + ((int64_t)bands.dhi[k] - bands.dlo[k]) + 1 + kWindowSlack + 3 + 3) & ~(int64_t)3);
+                at += bands.width[k];
+            }
+            break;
+        }
+        if (wm.rows_per_block == 0) {
+            st = ASX_STATUS_NOT_SUPPORTED;  // the bands of 256 rows do not fit the LDS: not this kernel's matrix
+            goto done;
+        }
     }
+    wm.nbands = bands.nbands;
     // 3. where every row starts inside its block; tiles of every block
     hipLaunchKernelGGL(k_window_row_starts, dim3((unsigned)ceil_div64(wm.nblocks, kBlock)), dim3(kBlock), 0, s, row_ptr, m,
                        wm.rows_per_block, wm.nblocks, row_start, btiles);
@@ -481,8 +635,10 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     h_bmin.resize((size_t)wm.nblocks);
     h_bmax.resize((size_t)wm.nblocks);
     h_off.resize((size_t)wm.nblocks + 1);
-    ASX_TRY(hipMemcpyAsync(h_bmin.data(), bmin, sizeof(int32_t) * h_bmin.size(), hipMemcpyDeviceToHost, s));
-    ASX_TRY(hipMemcpyAsync(h_bmax.data(), bmax, sizeof(int32_t) * h_bmax.size(), hipMemcpyDeviceToHost, s));
+    if (bands.nbands == 1) {
+        ASX_TRY(hipMemcpyAsync(h_bmin.data(), bmin, sizeof(int32_t) * h_bmin.size(), hipMemcpyDeviceToHost, s));
+        ASX_TRY(hipMemcpyAsync(h_bmax.data(), bmax, sizeof(int32_t) * h_bmax.size(), hipMemcpyDeviceToHost, s));
+    }
     ASX_TRY(hipMemcpyAsync(h_off.data(), tile_off, sizeof(int32_t) * h_off.size(), hipMemcpyDeviceToHost, s));
     ASX_TRY(hipStreamSynchronize(s));
     wm.ntiles = h_off[(size_t)wm.nblocks];
@@ -502,28 +658,44 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     hipLaunchKernelGGL((k_window_fill_pads<T>), dim3((unsigned)ceil_div64(slots, kBlock)), dim3(kBlock), 0, s, slots,
                        (uint16_t)(0x8000 | kWindowCols), wm.cf, (T *)wm.val, wm.perm);
     hipLaunchKernelGGL((k_window_place<T>), dim3((unsigned)ceil_div64(nnz, kBlock)), dim3(kBlock), 0, s, row_ptr, col, val,
-                       m, nnz, wm.rows_per_block, row_start, tile_off, wm.cf, (T *)wm.val, wm.perm);
+                       m, n, nnz, wm.rows_per_block, bands, row_start, tile_off, wm.cf, (T *)wm.val, wm.perm);
     // 5. first row and number of rows of every tile
     ASX_TRY(hipMemsetAsync(d_small, 0, sizeof(int32_t) * 2, s));
     hipLaunchKernelGGL(k_window_tile_info, dim3((unsigned)ceil_div64(wm.ntiles, kBlock)), dim3(kBlock), 0, s, row_start, m,
                        wm.rows_per_block, wm.nblocks, tile_off, wm.ntiles, (int2 *)wm.tile_info, d_small);
     ASX_TRY(hipMemcpyAsync(h_small, d_small, sizeof(int32_t), hipMemcpyDeviceToHost, s));
     // 6. chains of blocks, one per workgroup, of about equal numbers of tiles.  Inside a chain a
-    //    block fetches only the columns behind those already in the ring; a block whose columns
-    //    start before what the ring still holds begins a new chain (and fetches its whole window).
+    //    block fetches, per band, only the columns behind those already in the band's ring; a block
+    //    whose columns start before what a ring still holds begins a new chain (and fetches its
+    //    whole windows).
     {
         const int64_t per_chain = std::max<int64_t>(1, ceil_div64(wm.ntiles, target_wgs));
         blk.resize((size_t)wm.nblocks * 4);
-        int64_t have = -1;  // columns [.., have) are in the ring (-1: nothing yet)
+        int64_t have[kWindowBands];  // columns [.., have) are in the ring (-1: nothing yet)
+        for (int k = 0; k < kWindowBands; ++k) have[k] = -1;
         int32_t chain_lo = 0;
         int64_t chain_tiles = 0;
         for (int32_t b = 0; b < wm.nblocks; ++b) {
-            const bool empty = h_bmax[(size_t)b] < 0;
-            const int64_t lo = empty ? 0 : (h_bmin[(size_t)b] & ~3);
-            const int64_t hi = empty ? 0 : ((int64_t)h_bmax[(size_t)b] + 4) & ~(int64_t)3;  // past the last, rounded up
+            // columns the block needs in every band, rounded to multiples of 4: [lo, hi)
+            int64_t lo[kWindowBands], hi[kWindowBands];
+            const int64_t r0 = (int64_t)b * wm.rows_per_block, r1 = std::min<int64_t>(r0 + wm.rows_per_block, m);
+            for (int k = 0; k < bands.nbands; ++k) {
+                if (bands.nbands == 1) {
+                    const bool empty = h_bmax[(size_t)b] < 0;
+                    lo[k] = empty ? 0 : (h_bmin[(size_t)b] & ~3);
+                    hi[k] = empty ? 0 : ((int64_t)h_bmax[(size_t)b] + 4) & ~(int64_t)3;  // past the last, rounded up
+                } else {
+                    const int64_t a = std::min<int64_t>(std::max<int64_t>(band_centre(r0, m, n) + bands.dlo[k], 0), n);
+                    const int64_t z = std::min<int64_t>(std::max<int64_t>(band_centre(r1 - 1, m, n) + bands.dhi[k] + 1, 0), n);
+                    lo[k] = a & ~(int64_t)3;
+                    hi[k] = z > a ? (z + 3) & ~(int64_t)3 : lo[k];
+                }
+            }
             bool fresh = false;
             if (b != chain_lo) {
-                if (!empty && have >= 0 && lo < std::max(have, hi) - kWindowCols) fresh = true;  // already overwritten
+                for (int k = 0; k < bands.nbands; ++k)  // already overwritten, or the band moved backwards
+                    if (hi[k] > lo[k] && have[k] >= 0 && lo[k] < std::max(have[k], hi[k]) - bands.width[k] + kWindowSlack)
+                        fresh = true;
                 if (chain_tiles >= per_chain) fresh = true;
             }
             if (fresh) {
@@ -531,29 +703,37 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
                 chains.push_back(b);
                 chain_lo = b;
                 chain_tiles = 0;
-                have = -1;
-            }
-            int64_t from = 0, to = 0;
-            if (!empty) {
-                if (have < 0 || lo >= have) {  // nothing useful in the ring: the whole window
-                    from = lo;
-                    to = hi;
-                } else {
-                    from = have;
-                    to = std::max(have, hi);
-                }
-                have = to;
+                for (int k = 0; k < kWindowBands; ++k) have[k] = -1;
             }
             blk[(size_t)b * 4 + 0] = h_off[(size_t)b];
             blk[(size_t)b * 4 + 1] = h_off[(size_t)b + 1];
-            blk[(size_t)b * 4 + 2] = (int32_t)from;
-            blk[(size_t)b * 4 + 3] = (int32_t)to;
+            blk[(size_t)b * 4 + 2] = (int32_t)(pcs.size() / 4);
+            for (int k = 0; k < bands.nbands; ++k) {
+                int64_t from = lo[k], to = lo[k];
+                if (hi[k] > lo[k]) {
+                    if (have[k] < 0 || lo[k] >= have[k]) {  // nothing useful in the ring: the whole window
+                        from = lo[k];
+                        to = hi[k];
+                    } else {
+                        from = have[k];
+                        to = std::max(have[k], hi[k]);
+                    }
+                    have[k] = to;
+                }
+                pcs.push_back((int32_t)from);
+                pcs.push_back((int32_t)to);
+                pcs.push_back(bands.base[k]);
+                pcs.push_back(bands.width[k]);
+            }
+            blk[(size_t)b * 4 + 3] = (int32_t)(pcs.size() / 4);
             chain_tiles += h_off[(size_t)b + 1] - h_off[(size_t)b];
         }
         chains.push_back(chain_lo);
         chains.push_back(wm.nblocks);
         wm.nchains = (int32_t)(chains.size() / 2);
     }
+    ASX_TRY(hipMalloc((void **)&wm.pieces, sizeof(int32_t) * pcs.size()));
+    ASX_TRY(hipMemcpyAsync(wm.pieces, pcs.data(), sizeof(int32_t) * pcs.size(), hipMemcpyHostToDevice, s));
     ASX_TRY(hipMalloc((void **)&wm.blocks, sizeof(int32_t) * blk.size()));
     ASX_TRY(hipMalloc((void **)&wm.chains, sizeof(int32_t) * chains.size()));
     ASX_TRY(hipMemcpyAsync(wm.blocks, blk.data(), sizeof(int32_t) * blk.size(), hipMemcpyHostToDevice, s));
@@ -564,7 +744,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
 #undef ASX_TRY
 done:
     for (void *p : {(void *)cmin, (void *)cmax, (void *)row_start, (void *)bmin, (void *)bmax, (void *)btiles,
-                    (void *)tile_off, (void *)d_small, tmp})
+                    (void *)tile_off, (void *)d_small, (void *)d_bits, tmp})
         if (p) (void)hipFree(p);
     if (st) {
         free_window(&wm);
@@ -588,11 +768,16 @@ template <typename T>
 int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, hipStream_t s)
 {
     if (m <= 0) return ASX_STATUS_SUCCESS;
-    // x on a 16-byte boundary (every allocation is): 16-byte fetches; else element by element
-    const auto kernel = ((uintptr_t)x % 16) == 0 ? k_spmv_window<T, kWindowWaves, true> : k_spmv_window<T, kWindowWaves, false>;
+    // x on a 16-byte boundary (every allocation is) and at least one 16-byte unit long: 16-byte
+    // fetches; else element by element
+    const bool vec = ((uintptr_t)x % 16) == 0 && (size_t)n * sizeof(T) >= 16;
+    const auto kernel = wm->nbands == 1 ? (vec ? k_spmv_window<T, kWindowWaves, true, 1> : k_spmv_window<T, kWindowWaves, false, 1>)
+                                        : (vec ? k_spmv_window<T, kWindowWaves, true, kWindowBands>
+                                               : k_spmv_window<T, kWindowWaves, false, kWindowBands>);
     hipLaunchKernelGGL(kernel, dim3((unsigned)wm->nchains), dim3(kWindowWaves * kWave), 0, s, n, alpha, beta,
-                       reinterpret_cast<const int2 *>(wm->chains), reinterpret_cast<const int4 *>(wm->blocks), wm->cf,
-                       (const T *)wm->val, reinterpret_cast<const int2 *>(wm->tile_info), x, y, (T *)wm->carry);
+                       reinterpret_cast<const int2 *>(wm->chains), reinterpret_cast<const int4 *>(wm->blocks),
+                       reinterpret_cast<const int4 *>(wm->pieces), wm->cf, (const T *)wm->val,
+                       reinterpret_cast<const int2 *>(wm->tile_info), x, y, (T *)wm->carry);
     if (wm->has_carry)
         hipLaunchKernelGGL((k_window_fixup<T>), dim3((unsigned)ceil_div64(wm->ntiles, kBlock)), dim3(kBlock), 0, s,
                            wm->ntiles, alpha, reinterpret_cast<const int2 *>(wm->tile_info), (const T *)wm->carry, y);

@@ -699,6 +699,89 @@ def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
         assert not h.value
 
 
+def _diagonal_bands(rng, m, n, bands, dens, dtype, empty=0.05):
+    """Rows whose columns lie on bands of diagonals: for every (lo, hi) in `bands` the columns
+    centre + lo .. centre + hi (centre = r n // m) that fall inside the matrix, a fraction `dens`
+    of them stored; some rows empty."""
+    r = np.arange(m, dtype=np.int64)
+    centre = r * n // m
+    keys = []
+    for lo, hi in bands:
+        for off in range(lo, hi + 1):
+            c = centre + off
+            keep = (c >= 0) & (c < n) & (rng.random(m) < dens)
+            keys.append(r[keep] * n + c[keep])
+    key = np.unique(np.concatenate(keys))
+    rows = key // n
+    rows_empty = rng.random(m) < empty
+    key = key[~rows_empty[rows]]
+    rows = key // n
+    rp = np.zeros(m + 1, np.int64)
+    np.add.at(rp, rows + 1, 1)
+    rp = np.cumsum(rp).astype(np.int32)
+    col = (key % n).astype(np.int32)
+    return rp, col, rng.uniform(-1, 1, col.size).astype(dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_spmv_window_kernel_bands_of_diagonals(torch, capi, oracle, dtype):
+    """Matrices no single window holds but a few bands of diagonals do (the planes of a stencil on
+    a three-dimensional grid): a 7-point and a 27-point stencil on 96 x 96 x 12, random bands on a
+    rectangular matrix with an odd number of columns, five bands (the two closest are joined), long
+    rows that tiles cut (carry pass); and NOT_SUPPORTED where the bands are too wide for the LDS."""
+    rng = np.random.default_rng(131)
+    nx, ny, nz = 96, 96, 12
+    plane = nx * ny
+    cases = []
+
+    def stencil3d(points):
+        idx = np.arange(nx * ny * nz, dtype=np.int64)
+        i, j, k = idx % nx, (idx // nx) % ny, idx // plane
+        rng3 = (-1, 0, 1)
+        offs = [(di, dj, dk) for dk in rng3 for dj in rng3 for di in rng3
+                if points == 27 or abs(di) + abs(dj) + abs(dk) <= 1]
+        keys = []
+        for di, dj, dk in offs:
+            ii, jj, kk = i + di, j + dj, k + dk
+            ok = (ii >= 0) & (ii < nx) & (jj >= 0) & (jj < ny) & (kk >= 0) & (kk < nz)
+            keys.append(idx[ok] * idx.size + (ii + nx * (jj + ny * kk))[ok])
+        key = np.sort(np.concatenate(keys))
+        rp = np.zeros(idx.size + 1, np.int64)
+        np.add.at(rp, key // idx.size + 1, 1)
+        return np.cumsum(rp).astype(np.int32), (key % idx.size).astype(np.int32), rng.uniform(-1, 1, key.size).astype(dtype)
+
+    for pts in (7, 27):
+        cases.append((f"stencil {pts} points", stencil3d(pts), nx * ny * nz))
+    cases.append(("two far bands, rectangular", _diagonal_bands(rng, 50000, 70001, [(-30000, -29990), (-5, 40)], 0.5, dtype), 70001))
+    cases.append(("five bands", _diagonal_bands(rng, 40000, 40000, [(-20000, -20000), (-9000, -8990), (0, 0), (300, 310), (15000, 15001)],
+                                                0.9, dtype), 40000))
+    cases.append(("long rows", _diagonal_bands(rng, 9000, 60000, [(-25000, -24400), (0, 500)], 0.8, dtype), 60000))
+    L = capi.lib()
+    for name, (rp, col, val), n in cases:
+        m = rp.size - 1
+        x = rng.uniform(-1, 1, n).astype(dtype)
+        y0 = rng.uniform(-1, 1, m).astype(dtype)
+        d = [dev(torch, a) for a in (rp, col, val, x)]
+        plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
+        assert plan.alg == capi.SPMV_WINDOW and plan.holds_values and plan.workspace_bytes == 0
+        for alpha, beta in ((1.5, 0.5), (1.0, 0.0)):
+            ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 2)
+            scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
+            for rep in range(2):
+                y = dev(torch, y0 if beta else np.full(m, np.nan, dtype=dtype))
+                capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_WINDOW, plan=plan)
+                torch.cuda.synchronize()
+                assert_close(y.cpu().numpy(), ref, scale, dtype, f"{name} a={alpha} b={beta} rep={rep}")
+        plan.destroy()
+    # three bands of 9000 diagonals each: 27000 columns a block, more than the LDS holds
+    rp, col, val = _diagonal_bands(rng, 30000, 90000, [(-40000, -31000), (0, 9000), (30000, 39000)], 0.002, dtype)
+    d = [dev(torch, a) for a in (rp, col, val)]
+    h = capi.C.c_void_p()
+    assert L.asx_spmv_plan_create(capi.C.byref(h), capi.SPMV_WINDOW, capi.value_type(np.dtype(dtype)), rp.size - 1, 90000,
+                                  col.size, capi._ptr(d[0]), capi._ptr(d[1]), capi._ptr(d[2]), None) == 6
+    assert not h.value
+
+
 def test_default_workspace_covers_every_choice(torch, capi, oracle):
     """alphasparseSpMV_bufferSize(DEFAULT) is asx_spmv_workspace_bytes(DEFAULT): whatever kernel a
     DEFAULT plan settles on must fit in it.  Hypersparse (the plan takes the merge-path kernel,
