@@ -782,6 +782,46 @@ def test_spmv_window_kernel_bands_of_diagonals(torch, capi, oracle, dtype):
     assert not h.value
 
 
+def test_sliced_and_window_calls_replay_in_a_hip_graph(torch, capi, oracle):
+    """A call with a sliced or window plan is kernels only (no allocation, copy, memset or
+    synchronisation): captured once in a HIP graph it must give the eager result on every replay,
+    with eager work and synchronisations of the program between the replays."""
+    rng = np.random.default_rng(151)
+    lens = np.minimum(rng.zipf(1.6, 20000), 3000)
+    cases = [(capi.SPMV_SLICED, csr_from_lengths(lens, 90000, 7, np.float64), 90000),
+             (capi.SPMV_WINDOW, _banded_random(rng, 20000, 20000, 300, 0.05, np.float64, longrow=700), 20000)]
+    for alg, (rp, col, val), n in cases:
+        m = rp.size - 1
+        x = rng.uniform(-1, 1, n)
+        y0 = rng.uniform(-1, 1, m)
+        d = [dev(torch, a) for a in (rp, col, val, x)]
+        plan = capi.Plan(False, alg, val.dtype, m, n, col.size, d[0], col=d[1], val=d[2])
+        assert plan.workspace_bytes == 0
+        y_eager = dev(torch, y0)
+        capi.spmv(d[0], d[1], d[2], d[3], y_eager, 1.5, 0.5, alg=alg, plan=plan)
+        torch.cuda.synchronize()
+        eager = y_eager.cpu().numpy()
+        assert_close(eager, oracle.spmv(rp, col, val, x, 1.5, 0.5, y0, 2), spmv_scale(rp, col, val, x, 1.5, 0.5, y0),
+                     np.float64, f"eager alg {alg}")
+        y = dev(torch, y0)
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                capi.spmv(d[0], d[1], d[2], d[3], y, 1.5, 0.5, alg=alg, plan=plan)
+        torch.cuda.synchronize()
+        for rep in range(3):
+            y.copy_(dev(torch, y0))                      # eager work between the replays
+            scratch = (d[3] * 2.0).sum().item()          # and a synchronisation
+            assert np.isfinite(scratch)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert np.array_equal(y.cpu().numpy(), eager), f"alg {alg} replay {rep}"
+        del graph
+        plan.destroy()
+
+
 def test_default_workspace_covers_every_choice(torch, capi, oracle):
     """alphasparseSpMV_bufferSize(DEFAULT) is asx_spmv_workspace_bytes(DEFAULT): whatever kernel a
     DEFAULT plan settles on must fit in it.  Hypersparse (the plan takes the merge-path kernel,
