@@ -450,13 +450,16 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
             xf.load(x, n);                     \
         }                                      \
     }
+#define ASX_NEXT(TL, TT) window_tile_load<T>(TL, (TT) < chain_last ? (TT) : chain_last, lane, cf, val, tile_info)
+    // one tile: its rows' sums into the staging area, the loads of the tile two steps ahead (into
+    // the registers this one has just left), then the staged sums to y
 #define ASX_STEP(TL, TT)                                                                                          \
     {                                                                                                             \
         const StoreRows<T> out{y, carry + (TT), stage, TL.base & 0x7fffffff, TL.limit, TL.base < 0, alpha, beta}; \
         tile_reduce<T>(TL, lane, xs, out);                                                                        \
+        ASX_NEXT(TL, (TT) + 2 * NW);                                                                              \
         out.flush(lane);                                                                                          \
     }
-#define ASX_NEXT(TL, TT) window_tile_load<T>(TL, (TT) < chain_last ? (TT) : chain_last, lane, cf, val, tile_info)
     // Every wave passes the start of every block of the chain (the barriers count all waves),
     // whether it has tiles in the block or not.  ta and tb take turns without changing places.
     ASX_BLOCK_BEGIN()
@@ -466,14 +469,12 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
             ASX_BLOCK_BEGIN()
         }
         ASX_STEP(ta, t);
-        ASX_NEXT(ta, t + 2 * NW);
         t += NW;
         while (t >= tile_hi) {
             if (++b >= chain.y) return;
             ASX_BLOCK_BEGIN()
         }
         ASX_STEP(tb, t);
-        ASX_NEXT(tb, t + 2 * NW);
         t += NW;
     }
 #undef ASX_BLOCK_BEGIN
