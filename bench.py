@@ -65,6 +65,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=60.0,
                     help="budget of the whole CPU baseline leg (split evenly over workloads and thread counts)")
+    ap.add_argument("--calibrate-gather", action="store_true",
+                    help="only run the random-line gather kernel (lines per second the memory system delivers "
+                         "past the L2s: the bound of a gather without reuse)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run the plain copy kernel on 1 GiB (known traffic, for scaling profiler counters)")
     return ap.parse_args()
@@ -199,6 +202,44 @@ def copy_calibration(steps, nbytes=1 << 30):
             "read_plus_write_gbs": 2 * nbytes / (ms * 1e-3) / 1e9}
 
 
+def gather_calibration(loads_per_lane=128):
+    """Independent random reads that miss the L2s: one 128-byte line per lane, or one 256-byte row
+    (two lines) per wave, from buffers that fit the 256 MB Infinity Cache (64 MiB), are as large as
+    config 5's B (256 MiB) or exceed every cache (2 GiB).  Lines per second = the ceiling for a
+    gather without reuse, whatever the kernel around it."""
+    import torch
+    from library_amd import capi
+    import ctypes as C
+    L = capi.lib()
+    nthreads = C.c_int(0)
+    L.asx_gather_lines(None, 0, 1, 8, None, C.byref(nthreads), None)
+    out = torch.empty(nthreads.value, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+    for mib in (64, 256, 2048):
+        buf = torch.zeros(mib << 20, dtype=torch.uint8, device="cuda")
+        for group in (1, 64):
+            per_lane = loads_per_lane * (16 if group == 64 else 1)  # a wave's load is 2 lines, not 64
+            for _ in range(2):
+                rc = L.asx_gather_lines(buf.data_ptr(), buf.numel(), group, per_lane, out.data_ptr(), None, stream)
+                assert rc == 0, rc
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = 5
+            s.record()
+            for _ in range(reps):
+                L.asx_gather_lines(buf.data_ptr(), buf.numel(), group, per_lane, out.data_ptr(), None, stream)
+            e.record()
+            torch.cuda.synchronize()
+            ms = s.elapsed_time(e) / reps
+            loads = nthreads.value * per_lane                  # lane loads
+            lines = loads if group == 1 else loads // 64 * 2    # 128-byte lines fetched
+            rows.append({"buffer_mib": mib, "group_lanes": group, "ms": ms, "lines": lines,
+                         "g_lines_per_s": lines / (ms * 1e-3) / 1e9, "tb_per_s_of_lines": lines * 128 / (ms * 1e-3) / 1e12})
+        del buf
+    return {"gather": rows}
+
+
 def host_cpus():
     """nproc, sockets and physical cores of this host, and the thread count the baseline uses:
     the physical cores, capped by the box's CPU share (OMP_NUM_THREADS, 16 on a one-GPU box)."""
@@ -318,6 +359,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     capi.lib()
 
+    if a.calibrate_gather:
+        print(json.dumps(gather_calibration()))
+        return
     if a.calibrate_copy:
         print(json.dumps(copy_calibration(a.steps)))
         return

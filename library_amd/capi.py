@@ -32,7 +32,7 @@ EXPORTS = [
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
     "asx_spmv_csr_f64_noalloc", "asx_spmv_noalloc_max_workspace",
     "asx_spmm_resolve_alg", "asx_spmm_workspace_bytes", "asx_spmm_csr_f32", "asx_spmm_csr_f64",
-    "asx_copy_bytes",
+    "asx_copy_bytes", "asx_gather_lines",
 ]
 
 
@@ -96,6 +96,7 @@ def lib():
     L.asx_spmm_csr_f32.argtypes = [vp, C.c_int, i32, i32, i32, i32, C.c_float, vp, vp, vp, vp, i64, C.c_float, vp, i64, vp, sz, vp]
     L.asx_spmm_csr_f64.argtypes = [vp, C.c_int, i32, i32, i32, i32, C.c_double, vp, vp, vp, vp, i64, C.c_double, vp, i64, vp, sz, vp]
     L.asx_copy_bytes.argtypes = [vp, vp, sz, vp]
+    L.asx_gather_lines.argtypes = [vp, sz, C.c_int, C.c_int, vp, C.POINTER(C.c_int), vp]
     _lib = L
     return L
 

@@ -254,4 +254,54 @@ int launch_copy_bytes(const void *d_src, void *d_dst, size_t bytes, hipStream_t 
     return check_launch();
 }
 
+// -------------------------------------------------------------------------------------------
+// Calibration gather: groups of G consecutive lanes read G consecutive 32-bit words at pseudo-
+// random places of a buffer (G = 1: every lane its own 128-byte line; G = 64: the wave reads a
+// 256-byte row, the access of an N = 64 fp32 SpMM), 8 loads in flight per lane.  Measures how many
+// independent lines per second the memory system delivers past the L2s.
+// -------------------------------------------------------------------------------------------
+template <int G>
+__global__ __launch_bounds__(256) void k_gather_lines(const uint32_t *__restrict__ buf, uint64_t units, int per_lane,
+                                                      uint32_t *__restrict__ out)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t state = (tid / G) * 0x9E3779B97F4A7C15ull + 0x2545F4914F6CDD1Dull;
+    const uint32_t in_group = (uint32_t)(tid % G);
+    uint32_t sum = 0;
+    for (int i = 0; i < per_lane; i += 8) {
+        uint32_t v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            state = state * 6364136223846793005ull + 1442695040888963407ull;
+            const uint64_t u = __umul64hi(state, units);  // uniform in [0, units)
+            // a unit is G words for G >= 32, else a 128-byte line of which the lane reads one word
+            v[j] = buf[G >= 32 ? u * G + in_group : u * 32 + in_group];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sum += v[j];
+    }
+    out[tid] = sum;
+}
+
+int launch_gather_lines(const void *d_buf, size_t bytes, int group_lanes, int per_lane, void *d_out, int *nthreads,
+                        hipStream_t s)
+{
+    const int grid = 256 * 8, threads = grid * 256;
+    if (nthreads) *nthreads = threads;
+    if (!d_out) return ASX_STATUS_SUCCESS;  // size query
+    if (per_lane < 8 || per_lane % 8) return ASX_STATUS_INVALID_VALUE;
+    if (group_lanes == 1) {
+        if (bytes < 128) return ASX_STATUS_INVALID_SIZE;
+        hipLaunchKernelGGL(k_gather_lines<1>, dim3(grid), dim3(256), 0, s, (const uint32_t *)d_buf, (uint64_t)(bytes / 128),
+                           per_lane, (uint32_t *)d_out);
+    } else if (group_lanes == 64) {
+        if (bytes < 256) return ASX_STATUS_INVALID_SIZE;
+        hipLaunchKernelGGL(k_gather_lines<64>, dim3(grid), dim3(256), 0, s, (const uint32_t *)d_buf, (uint64_t)(bytes / 256),
+                           per_lane, (uint32_t *)d_out);
+    } else {
+        return ASX_STATUS_INVALID_VALUE;
+    }
+    return check_launch();
+}
+
 }  // namespace asx

@@ -898,4 +898,11 @@ int asx_copy_bytes(const void *d_src, void *d_dst, size_t bytes, void *stream)
     return launch_copy_bytes(d_src, d_dst, bytes, (hipStream_t)stream);
 }
 
+int asx_gather_lines(const void *d_buf, size_t bytes, int group_lanes, int loads_per_lane, void *d_out, int *nthreads,
+                     void *stream)
+{
+    if (d_out && !d_buf) return ASX_STATUS_INVALID_POINTER;
+    return launch_gather_lines(d_buf, bytes, group_lanes, loads_per_lane, d_out, nthreads, (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -52,6 +52,8 @@ int launch_loadbalance_partition(const int32_t *d_row_ptr, int32_t m, int32_t nn
 int launch_stream_row_blocks(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t *d_blocks,
                              hipStream_t s);
 int launch_copy_bytes(const void *d_src, void *d_dst, size_t bytes, hipStream_t s);
+int launch_gather_lines(const void *d_buf, size_t bytes, int group_lanes, int per_lane, void *d_out, int *nthreads,
+                        hipStream_t s);
 
 // ---- SpMV launchers (asx_spmv.hip) ----
 template <typename T>

@@ -924,3 +924,15 @@ def test_calibration_copy_runs(torch, capi):
     torch.cuda.synchronize()
     assert torch.equal(src, dst)
     assert L.asx_copy_bytes(capi._ptr(src), capi._ptr(dst), 17, stream) == 10
+    # the random-line gather of the benchmark: runs for both group sizes, refuses others
+    import ctypes as C
+    nthreads = C.c_int(0)
+    assert L.asx_gather_lines(None, 0, 1, 8, None, C.byref(nthreads), None) == 0 and nthreads.value > 0
+    out = torch.zeros(nthreads.value, dtype=torch.int32, device="cuda")
+    buf = torch.ones(1 << 22, dtype=torch.int32, device="cuda")
+    for group in (1, 64):
+        assert L.asx_gather_lines(capi._ptr(buf), buf.numel() * 4, group, 16, capi._ptr(out), None, stream) == 0
+        torch.cuda.synchronize()
+        assert int(out.min()) == 16 and int(out.max()) == 16  # 16 loads of the value 1 per lane
+    assert L.asx_gather_lines(capi._ptr(buf), buf.numel() * 4, 3, 16, capi._ptr(out), None, stream) == 3
+    assert L.asx_gather_lines(capi._ptr(buf), buf.numel() * 4, 1, 12, capi._ptr(out), None, stream) == 3
