@@ -672,8 +672,9 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     {
         const int64_t per_chain = std::max<int64_t>(1, ceil_div64(wm.ntiles, target_wgs));
         blk.resize((size_t)wm.nblocks * 4);
-        int64_t have[kWindowBands];  // columns [.., have) are in the ring (-1: nothing yet)
-        for (int k = 0; k < kWindowBands; ++k) have[k] = -1;
+        int64_t have[kWindowBands];  // columns [low, have) were fetched in this chain (have = -1: nothing yet)
+        int64_t low[kWindowBands];
+        for (int k = 0; k < kWindowBands; ++k) have[k] = -1, low[k] = 0;
         int32_t chain_lo = 0;
         int64_t chain_tiles = 0;
         for (int32_t b = 0; b < wm.nblocks; ++b) {
@@ -694,8 +695,9 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
             }
             bool fresh = false;
             if (b != chain_lo) {
-                for (int k = 0; k < bands.nbands; ++k)  // already overwritten, or the band moved backwards
-                    if (hi[k] > lo[k] && have[k] >= 0 && lo[k] < std::max(have[k], hi[k]) - bands.width[k] + kWindowSlack)
+                for (int k = 0; k < bands.nbands; ++k)  // columns never fetched in this chain, or already overwritten
+                    if (hi[k] > lo[k] && have[k] >= 0 &&
+                        (lo[k] < low[k] || lo[k] < std::max(have[k], hi[k]) - bands.width[k] + kWindowSlack))
                         fresh = true;
                 if (chain_tiles >= per_chain) fresh = true;
             }
@@ -704,7 +706,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
                 chains.push_back(b);
                 chain_lo = b;
                 chain_tiles = 0;
-                for (int k = 0; k < kWindowBands; ++k) have[k] = -1;
+                for (int k = 0; k < kWindowBands; ++k) have[k] = -1, low[k] = 0;
             }
             blk[(size_t)b * 4 + 0] = h_off[(size_t)b];
             blk[(size_t)b * 4 + 1] = h_off[(size_t)b + 1];
@@ -715,6 +717,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
                     if (have[k] < 0 || lo[k] >= have[k]) {  // nothing useful in the ring: the whole window
                         from = lo[k];
                         to = hi[k];
+                        low[k] = lo[k];
                     } else {
                         from = have[k];
                         to = std::max(have[k], hi[k]);

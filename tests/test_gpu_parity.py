@@ -663,6 +663,21 @@ def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
         cases.append((f"band {m}x{n} +-{half}", _banded_random(rng, m, n, half, dens, dtype, longrow=lr), n))
     st = W.stencil5_f64(300, 200)
     cases.append(("stencil 300x200", (st.row_ptr, st.col, st.val.astype(dtype)), st.n))
+    # windows that move backwards from one block of rows to the next, inside what a ring could still
+    # hold: the columns below the chain's first window were never fetched.  Large enough (2^20 rows)
+    # for chains of several blocks.
+    zig = [(1000, 1400), (200, 600), (5000, 5300), (4000, 4200), (4100, 4900), (0, 50), (9000, 9900), (8990, 9100)]
+    groups = 4096
+    lens = rng.integers(0, 9, 256 * groups)
+    rp = np.zeros(lens.size + 1, np.int32)
+    rp[1:] = np.cumsum(lens)
+    g = (np.repeat(np.arange(lens.size), lens) // 256) % len(zig)
+    zlo = np.array([z[0] for z in zig])[g]
+    zw = np.array([z[1] - z[0] for z in zig])[g]
+    # distinct ascending columns inside a row: a random start and a stride that keeps 8 of them in range
+    within = np.arange(rp[-1]) - np.repeat(rp[:-1], lens)
+    col = (zlo + (rng.integers(0, 5, rp[-1])[np.repeat(rp[:-1], lens)] + within * (zw // 9))).astype(np.int32)
+    cases.append(("windows moving backwards", (rp, col, rng.uniform(-1, 1, col.size).astype(dtype)), 10000))
     for name, (rp, col, val), n in cases:
         m = rp.size - 1
         x = rng.uniform(-1, 1, n).astype(dtype)
