@@ -218,6 +218,19 @@ int asx_plan_destroy(asx_plan *plan);
 /* Kernel the plan resolved to, and bytes of per-call workspace its launches need. */
 int asx_plan_alg(const asx_plan *plan);
 size_t asx_plan_workspace_bytes(const asx_plan *plan);
+/* What a plan that holds a regrouped copy of A looks like (for logs and tests; -1 where the
+ * figure does not apply to the plan's kernel).  No counterpart in the reference. */
+enum {
+    ASX_PLAN_INFO_TILES = 0,          /* tiles of 256 slots (sliced, window) */
+    ASX_PLAN_INFO_SLICES = 1,         /* column slices (sliced) */
+    ASX_PLAN_INFO_PARTIAL_SUMS = 2,   /* partial sums per call (sliced) */
+    ASX_PLAN_INFO_ROWS_PER_WAVE = 3,  /* rows of a row block of pass 2 (sliced) */
+    ASX_PLAN_INFO_ROWS_PER_BLOCK = 4, /* rows of a block (window) */
+    ASX_PLAN_INFO_BANDS = 5,          /* rings of x in LDS: 1 = one window, 2..4 = bands of diagonals (window) */
+    ASX_PLAN_INFO_CHAINS = 6,         /* chains of blocks = workgroups (window) */
+    ASX_PLAN_INFO_CARRY_PASS = 7      /* 1 if a call runs the ordered carry pass (window) */
+};
+int64_t asx_plan_info(const asx_plan *plan, int what);
 /* Copies the plan's histogram (33 bins) and stats (4) to host arrays. */
 int asx_plan_histogram(const asx_plan *plan, int64_t h_hist[33], int64_t h_stats[4]);
 

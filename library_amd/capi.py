@@ -27,7 +27,7 @@ EXPORTS = [
     "asx_nnz_split_rows", "asx_merge_path_search", "asx_loadbalance_nwarps",
     "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_coo2csr", "asx_coo_sort", "asx_csr_transpose", "asx_csr_rebase",
     "asx_dense_transpose", "asx_mtx_read", "asx_host_free", "asx_spmv_plan_create",
-    "asx_plan_update_values", "asx_plan_holds_values", "asx_plan_create",
+    "asx_plan_update_values", "asx_plan_holds_values", "asx_plan_info", "asx_plan_create",
     "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
     "asx_spmv_csr_f64_noalloc", "asx_spmv_noalloc_max_workspace",
@@ -96,6 +96,8 @@ def lib():
     L.asx_spmm_csr_f32.argtypes = [vp, C.c_int, i32, i32, i32, i32, C.c_float, vp, vp, vp, vp, i64, C.c_float, vp, i64, vp, sz, vp]
     L.asx_spmm_csr_f64.argtypes = [vp, C.c_int, i32, i32, i32, i32, C.c_double, vp, vp, vp, vp, i64, C.c_double, vp, i64, vp, sz, vp]
     L.asx_copy_bytes.argtypes = [vp, vp, sz, vp]
+    L.asx_plan_info.argtypes = [vp, C.c_int]
+    L.asx_plan_info.restype = i64
     L.asx_gather_lines.argtypes = [vp, sz, C.c_int, C.c_int, vp, C.POINTER(C.c_int), vp]
     _lib = L
     return L
@@ -281,6 +283,13 @@ class Plan:
     def update_values(self, val):
         _check(lib().asx_plan_update_values(self.h, _ptr(val), _stream()), "asx_plan_update_values")
         self._keep = (self._keep[0], self._keep[1], val)
+
+    INFO = {"tiles": 0, "slices": 1, "partial_sums": 2, "rows_per_wave": 3, "rows_per_block": 4, "bands": 5,
+            "chains": 6, "carry_pass": 7}
+
+    def info(self, what):
+        """A figure of a sliced or window plan (asx_plan_info); -1 where it does not apply."""
+        return int(lib().asx_plan_info(self.h, self.INFO[what]))
 
     @property
     def holds_values(self):

@@ -725,6 +725,22 @@ int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill)
 
 int asx_plan_alg(const asx_plan *plan) { return plan ? plan->alg : -1; }
 size_t asx_plan_workspace_bytes(const asx_plan *plan) { return plan ? plan->workspace_bytes : 0; }
+int64_t asx_plan_info(const asx_plan *plan, int what)
+{
+    if (!plan || plan->is_spmm) return -1;
+    const bool sliced = plan->alg == ASX_SPMV_SLICED, window = plan->alg == ASX_SPMV_WINDOW;
+    switch (what) {
+    case ASX_PLAN_INFO_TILES: return sliced ? plan->sliced.ntiles : window ? plan->window.ntiles : -1;
+    case ASX_PLAN_INFO_SLICES: return sliced ? plan->sliced.nslices : -1;
+    case ASX_PLAN_INFO_PARTIAL_SUMS: return sliced ? plan->sliced.npartials : -1;
+    case ASX_PLAN_INFO_ROWS_PER_WAVE: return sliced ? plan->sliced.rows_per_wave : -1;
+    case ASX_PLAN_INFO_ROWS_PER_BLOCK: return window ? plan->window.rows_per_block : -1;
+    case ASX_PLAN_INFO_BANDS: return window ? plan->window.nbands : -1;
+    case ASX_PLAN_INFO_CHAINS: return window ? plan->window.nchains : -1;
+    case ASX_PLAN_INFO_CARRY_PASS: return window ? plan->window.has_carry : -1;
+    default: return -1;
+    }
+}
 int asx_plan_histogram(const asx_plan *plan, int64_t h_hist[33], int64_t h_stats[4])
 {
     if (!plan || !h_hist || !h_stats) return ASX_STATUS_INVALID_POINTER;

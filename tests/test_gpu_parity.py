@@ -685,6 +685,9 @@ def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
         d = [dev(torch, a) for a in (rp, col, val, x)]
         plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
         assert plan.alg == capi.SPMV_WINDOW and plan.holds_values and plan.workspace_bytes == 0
+        assert plan.info("bands") == 1 and plan.info("rows_per_block") % 256 == 0 and plan.info("tiles") > 0
+        if name == "windows moving backwards":
+            assert plan.info("chains") < -(-m // plan.info("rows_per_block")), "chains of several blocks expected"
         for alpha, beta in ((1.5, 0.5), (1.0, 0.0), (-2.0, 1.0)):
             ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 2)
             scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
@@ -779,6 +782,9 @@ def test_spmv_window_kernel_bands_of_diagonals(torch, capi, oracle, dtype):
         d = [dev(torch, a) for a in (rp, col, val, x)]
         plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
         assert plan.alg == capi.SPMV_WINDOW and plan.holds_values and plan.workspace_bytes == 0
+        assert 2 <= plan.info("bands") <= 4 and plan.info("slices") == -1, (name, plan.info("bands"))
+        if name in ("stencil 7 points", "long rows"):  # rows of at most 16 are never cut by tiles
+            assert plan.info("carry_pass") == (1 if name == "long rows" else 0), name
         for alpha, beta in ((1.5, 0.5), (1.0, 0.0)):
             ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 2)
             scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
