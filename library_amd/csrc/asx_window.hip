@@ -424,12 +424,14 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     T *stage = stage_all + wave * kStageRows;
     const int32_t chain_last = blocks[chain.y - 1].y - 1;  // last tile of the chain
-    // this wave's tiles are those congruent to its number, across the blocks of the chain; two are
-    // in flight (loaded two steps ahead; past the end of the chain the last tile is re-read)
-    WindowTile<T> ta, tb;
+    // this wave's tiles are those congruent to its number, across the blocks of the chain; three
+    // are in flight (loaded three steps ahead; past the end of the chain the last tile is re-read;
+    // measured 1-2 % ahead of two)
+    WindowTile<T> ta, tb, tc;
     int32_t t = blocks[chain.x].x + wave;
     window_tile_load<T>(ta, t < chain_last ? t : chain_last, lane, cf, val, tile_info);
     window_tile_load<T>(tb, t + NW < chain_last ? t + NW : chain_last, lane, cf, val, tile_info);
+    window_tile_load<T>(tc, t + 2 * NW < chain_last ? t + 2 * NW : chain_last, lane, cf, val, tile_info);
     if (threadIdx.x == 0) xs[kWindowCols] = T(0);
     XFetch<T, NW * kWave, VEC, NB> xf;
     int4 blk = blocks[chain.x];  // first tile, end tile, pieces of x to fetch before the block: first, end
@@ -451,17 +453,17 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
         }                                      \
     }
 #define ASX_NEXT(TL, TT) window_tile_load<T>(TL, (TT) < chain_last ? (TT) : chain_last, lane, cf, val, tile_info)
-    // one tile: its rows' sums into the staging area, the loads of the tile two steps ahead (into
+    // one tile: its rows' sums into the staging area, the loads of the tile three steps ahead (into
     // the registers this one has just left), then the staged sums to y
 #define ASX_STEP(TL, TT)                                                                                          \
     {                                                                                                             \
         const StoreRows<T> out{y, carry + (TT), stage, TL.base & 0x7fffffff, TL.limit, TL.base < 0, alpha, beta}; \
         tile_reduce<T>(TL, lane, xs, out);                                                                        \
-        ASX_NEXT(TL, (TT) + 2 * NW);                                                                              \
+        ASX_NEXT(TL, (TT) + 3 * NW);                                                                              \
         out.flush(lane);                                                                                          \
     }
     // Every wave passes the start of every block of the chain (the barriers count all waves),
-    // whether it has tiles in the block or not.  ta and tb take turns without changing places.
+    // whether it has tiles in the block or not.  ta, tb and tc take turns without changing places.
     ASX_BLOCK_BEGIN()
     for (;;) {  // all conditions are uniform over the wave
         while (t >= tile_hi) {
@@ -475,6 +477,12 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
             ASX_BLOCK_BEGIN()
         }
         ASX_STEP(tb, t);
+        t += NW;
+        while (t >= tile_hi) {
+            if (++b >= chain.y) return;
+            ASX_BLOCK_BEGIN()
+        }
+        ASX_STEP(tc, t);
         t += NW;
     }
 #undef ASX_BLOCK_BEGIN
