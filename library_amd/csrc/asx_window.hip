@@ -604,7 +604,9 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
             runs[best].second = runs[best + 1].second;
             runs.erase(runs.begin() + (long)best + 1);
         }
-        if (runs.empty()) {
+        // one run of offsets: the rows fill a band too wide for the single window tried above
+        // (the one-ring kernel places column c at c mod kWindowCols; it is not built from here)
+        if (runs.size() < 2) {
             st = ASX_STATUS_NOT_SUPPORTED;
             goto done;
         }
