@@ -717,6 +717,35 @@ def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
         assert not h.value
 
 
+def test_spmv_sliced_wide_steps(torch, capi, oracle):
+    """Pass 2 of the sliced kernel reads a row block's partial sums inside a slice 64 at a time, or,
+    when those ranges are long, 128 (fp64) or 256 (fp32) at a time, several consecutive ones per
+    lane from unaligned addresses.  Matrices whose mean range is beyond the thresholds."""
+    W = pytest.importorskip("library_amd.workloads")
+    rng = np.random.default_rng(171)
+    for dtype, m, n, k, want in ((np.float32, 120000, 40000, 48, 160.0), (np.float64, 200000, 180000, 16, 80.0)):
+        rp, col, val = W.csr_fixed(m, n, k, dtype, seed=3)
+        x = rng.uniform(-1, 1, n).astype(dtype)
+        y0 = rng.uniform(-1, 1, m).astype(dtype)
+        d = [dev(torch, a) for a in (rp, col, val, x)]
+        plan = capi.Plan(False, capi.SPMV_SLICED, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
+        nrb = -(-m // plan.info("rows_per_wave"))
+        mean_range = plan.info("partial_sums") / (nrb * plan.info("slices"))
+        assert mean_range >= want, (mean_range, plan.info("rows_per_wave"), plan.info("slices"))
+        for alpha, beta in ((1.5, 0.5), (1.0, 0.0)):
+            ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 4)
+            scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
+            outs = []
+            for rep in range(2):
+                y = dev(torch, y0 if beta else np.full(m, np.nan, dtype=dtype))
+                capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_SLICED, plan=plan)
+                torch.cuda.synchronize()
+                outs.append(y.cpu().numpy())
+                assert_close(outs[-1], ref, scale, dtype, f"{np.dtype(dtype).name} a={alpha} b={beta} rep={rep}")
+            assert np.array_equal(outs[0], outs[1]), "two calls through one plan must agree bit for bit"
+        plan.destroy()
+
+
 def _diagonal_bands(rng, m, n, bands, dens, dtype, empty=0.05):
     """Rows whose columns lie on bands of diagonals: for every (lo, hi) in `bands` the columns
     centre + lo .. centre + hi (centre = r n // m) that fall inside the matrix, a fraction `dens`
