@@ -35,7 +35,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 ORDER = ["banded_f64", "uniform16_f32", "powerlaw_f64", "stencil5_f64", "spmm_zipf_f32"]
-EXTRA = ["spmm_banded_f32"]  # not a BASELINE configuration: dense-block matrix for the MFMA SpMM variant
+# not BASELINE configurations: a dense-block matrix for the MFMA SpMM variant; config 2's matrix in fp64
+EXTRA = ["spmm_banded_f32", "uniform16_f64"]
 KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "k_spmv_flat",
                 101: "k_sliced_products+k_sliced_reduce", 102: "k_spmv_window", 5: "k_spmm_row", 7: "k_spmm_merge", 10: "k_spmm_blocked"}
 

@@ -161,6 +161,12 @@ def uniform16_f32(m=1 << 20, k=16, seed=0):
     return _spmv("uniform16_f32", np.float32, rp, col, val, m, 1.5, 0.5, seed)
 
 
+def uniform16_f64(m=1 << 20, k=16, seed=0):
+    """Not a BASELINE configuration: config 2's matrix in fp64 (y = 1.5*A*x + 0.5*y)."""
+    rp, col, val = csr_fixed(m, m, k, np.float64, seed)
+    return _spmv("uniform16_f64", np.float64, rp, col, val, m, 1.5, 0.5, seed)
+
+
 def powerlaw_f64(m=1 << 22, max_len=200000, empty_frac=0.01, seed=0, alpha=1.0, beta=0.0):
     """Config 3: Zipf(2.0) row lengths clipped to [1, max_len], 1% empty rows, fp64."""
     rp, col, val = csr_zipf(m, m, 20, 1.0, min(max_len, m), empty_frac, np.float64, seed)
@@ -198,4 +204,5 @@ CONFIGS = {
     "stencil5_f64": stencil5_f64,
     "spmm_zipf_f32": spmm_zipf_f32,
     "spmm_banded_f32": spmm_banded_f32,
+    "uniform16_f64": uniform16_f64,
 }
