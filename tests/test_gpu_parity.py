@@ -352,6 +352,7 @@ def test_benchmark_configs_full_size(torch, capi, oracle):
             # plans that may look at columns and values: the column-sliced kernel, forced and as
             # DEFAULT's choice on these matrices (scattered columns; the choice is rule-based, so two
             # plan builds agree)
+            across_plans = []
             for alg in (capi.SPMV_SLICED, capi.SPMV_DEFAULT, capi.SPMV_DEFAULT):
                 plan = capi.Plan(False, alg, w.val.dtype, w.m, w.n, w.nnz, d[0], col=d[1], val=d[2])
                 assert plan.alg == capi.SPMV_SLICED and plan.holds_values and plan.workspace_bytes == 0
@@ -363,10 +364,14 @@ def test_benchmark_configs_full_size(torch, capi, oracle):
                     outs.append(y.cpu().numpy())
                     assert_close(outs[-1], ref, scale, w.dtype, f"{name} sliced alg={alg} rep={rep}")
                 assert np.array_equal(outs[0], outs[1]), "two calls through one plan must agree bit for bit"
+                across_plans.append(outs[0])
                 plan.destroy()
+            assert all(np.array_equal(across_plans[0], o) for o in across_plans[1:]), \
+                "plans built again from the same matrix must give the same bits"
         else:
             # rows that reach only nearby columns: the row-block kernel with its window of x in LDS,
             # forced and as DEFAULT's choice; without columns and values DEFAULT stays row-ordered
+            across_plans = []
             for alg in (capi.SPMV_WINDOW, capi.SPMV_DEFAULT):
                 plan = capi.Plan(False, alg, w.val.dtype, w.m, w.n, w.nnz, d[0], col=d[1], val=d[2])
                 assert plan.alg == capi.SPMV_WINDOW and plan.holds_values and plan.workspace_bytes == 0
@@ -378,7 +383,9 @@ def test_benchmark_configs_full_size(torch, capi, oracle):
                     outs.append(y.cpu().numpy())
                     assert_close(outs[-1], ref, scale, w.dtype, f"{name} window alg={alg} rep={rep}")
                 assert np.array_equal(outs[0], outs[1])
+                across_plans.append(outs[0])
                 plan.destroy()
+            assert np.array_equal(across_plans[0], across_plans[1]), "plans built again must give the same bits"
             plan = capi.Plan(False, capi.SPMV_DEFAULT, w.val.dtype, w.m, w.n, w.nnz, d[0])
             assert plan.alg == capi.SPMV_FLAT and not plan.holds_values
             plan.destroy()
