@@ -565,6 +565,18 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
             }
         }
         sm.nwg = (int32_t)(tab.size() / 4);
+        // The workgroups of a slice all fetch that slice of x: keep them on one XCD, whose L2 then
+        // fetches it once (workgroup i runs on XCD i mod kXcds; entry j of the list above goes to
+        // position (j mod per_xcd) * kXcds + j / per_xcd, so consecutive entries share an XCD).
+        if (sm.nwg > sm.nslices && sm.nwg % kXcds == 0) {
+            const int32_t per_xcd = sm.nwg / kXcds;
+            std::vector<int32_t> placed(tab.size());
+            for (int32_t j = 0; j < sm.nwg; ++j) {
+                const int32_t i = (j % per_xcd) * kXcds + j / per_xcd;
+                for (int q = 0; q < 4; ++q) placed[(size_t)i * 4 + q] = tab[(size_t)j * 4 + q];
+            }
+            tab.swap(placed);
+        }
         ASX_TRY(hipMalloc((void **)&sm.wg_tab, sizeof(int32_t) * std::max<size_t>(tab.size(), 4)));
         ASX_TRY(hipMemcpyAsync(sm.wg_tab, tab.data(), sizeof(int32_t) * tab.size(), hipMemcpyHostToDevice, s));
     }
