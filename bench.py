@@ -47,7 +47,7 @@ KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "
 # warm and with cold caches.
 MEASURED_TRAFFIC_BYTES = {
     "banded_f64": 458_667,             # profiles/spmv_vector_banded_f64.md
-    "uniform16_f32": 278_201_324,      # profiles/spmv_sliced_uniform16_f32.md
+    "uniform16_f32": 248_805_417,      # profiles/spmv_sliced_uniform16_f32.md
     "powerlaw_f64": 719_379_833,       # profiles/spmv_sliced_powerlaw_f64.md
     "stencil5_f64": 1_135_154_025,     # profiles/spmv_window_stencil5_f64.md
     "spmm_zipf_f32": 4_964_370_644,    # profiles/spmm_merge_spmm_zipf_f32.md
