@@ -465,7 +465,17 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
     while ((1 << key_bits) < sm.nslices) ++key_bits;
 
     int st = ASX_STATUS_SUCCESS;
-    int32_t *a = nullptr, *b = nullptr, *c = nullptr, *d = nullptr;  // nnz-sized scratch
+    // Scratch of the build, in one allocation (every hipMalloc / hipFree of this size costs a
+    // fraction of a millisecond): five arrays of `cap` ints, cap = the most slots there can be
+    // (every slice padded to whole tiles), used in turn as
+    //   a: sort keys in, then row of each sorted element, then (after the placing) the scan of run starts
+    //   b: sorted keys = slice of each sorted element, then (after the placing) the row of each partial sum
+    //   c: sort values in, then row of each slot
+    //   d: sorted values = position in A of each sorted element
+    //   e: run-start flag of each slot
+    // followed by the slice offsets (elements, tiles) and the sort / scan workspace.
+    int32_t *arena = nullptr;
+    int32_t *a = nullptr, *b = nullptr, *c = nullptr, *d = nullptr, *e = nullptr;
     int32_t *lrow = nullptr, *lhead = nullptr, *hscan = nullptr, *prow_full = nullptr;
     int32_t *d_pstart = nullptr, *d_tile_off = nullptr;
     void *tmp = nullptr;
@@ -474,7 +484,10 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
     std::vector<int32_t> tab;
     int64_t slots = 0;
     const unsigned grid = (unsigned)ceil_div64(nnz, kBlock);
-    const size_t nb = sizeof(int32_t) * (size_t)nnz;
+    const int64_t cap64 = (int64_t)nnz + (int64_t)(kSlicedTile - 1) * sm.nslices;
+    if (cap64 > 0x7fffffff) return ASX_STATUS_INVALID_SIZE;
+    const size_t cap = ((size_t)cap64 + 63) & ~(size_t)63;
+    const size_t noff = ((size_t)sm.nslices + 1 + 63) & ~(size_t)63;
 #define ASX_TRY(expr)         \
     do {                      \
         st = status_of(expr); \
@@ -485,22 +498,23 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
         st = (expr);       \
         if (st) goto done; \
     } while (0)
-    for (int32_t **q : {&a, &b, &c, &d}) ASX_TRY(hipMalloc((void **)q, nb));
-    ASX_TRY(hipMalloc((void **)&d_pstart, sizeof(int32_t) * ((size_t)sm.nslices + 1)));
-    ASX_TRY(hipMalloc((void **)&d_tile_off, sizeof(int32_t) * ((size_t)sm.nslices + 1)));
+    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_sort, a, b, c, d, nnz, 0, key_bits, s));
+    ASX_TRY(hipcub::DeviceScan::InclusiveSum(nullptr, tmp_scan, lhead, hscan, (int)cap64, s));
+    tmp_bytes = std::max<size_t>(std::max(tmp_sort, tmp_scan), 256);
+    ASX_TRY(hipMalloc((void **)&arena, sizeof(int32_t) * (5 * cap + 2 * noff) + tmp_bytes));
+    a = arena, b = a + cap, c = b + cap, d = c + cap, e = d + cap;
+    d_pstart = e + cap;
+    d_tile_off = d_pstart + noff;
+    tmp = d_tile_off + noff;
 
     // 1. stored elements by slice (stable: row order, then column order, survives inside a slice)
-    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_sort, a, b, c, d, nnz, 0, key_bits, s));
-    ASX_TRY(hipMalloc(&tmp, tmp_sort ? tmp_sort : 1));
     hipLaunchKernelGGL(k_sliced_keys, dim3(grid), dim3(kBlock), 0, s, col, nnz, width, a, c);
-    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_sort, a, b, c, d, nnz, 0, key_bits, s));
+    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, a, b, c, d, nnz, 0, key_bits, s));
     // b = slice of each sorted element, d = its position in A; a = its row
     hipLaunchKernelGGL(k_sliced_rows, dim3(grid), dim3(kBlock), 0, s, d, nnz, row_ptr, m, a);
     ASX_TRY_ST(launch_offsets_from_sorted(b, nnz, sm.nslices, d_pstart, s));
     ASX_TRY(hipMemcpyAsync(pstart.data(), d_pstart, sizeof(int32_t) * pstart.size(), hipMemcpyDeviceToHost, s));
     ASX_TRY(hipStreamSynchronize(s));
-    (void)hipFree(tmp);
-    tmp = nullptr;
 
     // 2. tiles: every slice starts a new tile
     for (int32_t sl = 0; sl < sm.nslices; ++sl)
@@ -515,9 +529,8 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
     ASX_TRY(hipMalloc(&sm.val, sizeof(T) * (size_t)slots));
     ASX_TRY(hipMalloc((void **)&sm.cf, sizeof(uint16_t) * (size_t)slots));
     ASX_TRY(hipMalloc((void **)&sm.perm, sizeof(int32_t) * (size_t)slots));
-    ASX_TRY(hipMalloc((void **)&lrow, sizeof(int32_t) * (size_t)slots));
-    ASX_TRY(hipMalloc((void **)&lhead, sizeof(int32_t) * (size_t)slots));
-    ASX_TRY(hipMalloc((void **)&hscan, sizeof(int32_t) * (size_t)slots));
+    lrow = c;   // the sort's input values are spent
+    lhead = e;
     {
         const unsigned sgrid = (unsigned)ceil_div64(slots, kBlock);
         hipLaunchKernelGGL((k_sliced_fill_pads<T>), dim3(sgrid), dim3(kBlock), 0, s, slots, lrow, lhead, sm.cf,
@@ -525,16 +538,14 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
         hipLaunchKernelGGL((k_sliced_place<T>), dim3(grid), dim3(kBlock), 0, s, b, d, a, nnz, width, d_pstart, d_tile_off,
                            col, val, lrow, lhead, sm.cf, (T *)sm.val, sm.perm);
         // 3. partial sums: one per run start
-        ASX_TRY(hipcub::DeviceScan::InclusiveSum(nullptr, tmp_scan, lhead, hscan, (int)slots, s));
-        tmp_bytes = tmp_scan;
-        ASX_TRY(hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1));
+        hscan = a;      // the placing has read the rows, slices and positions of the sorted elements:
+        prow_full = b;  // their arrays are free (kernels run in stream order)
         ASX_TRY(hipcub::DeviceScan::InclusiveSum(tmp, tmp_bytes, lhead, hscan, (int)slots, s));
         ASX_TRY(hipMemcpyAsync(&sm.npartials, hscan + (slots - 1), sizeof(int32_t), hipMemcpyDeviceToHost, s));
         ASX_TRY(hipStreamSynchronize(s));
         ASX_TRY(hipMalloc((void **)&sm.tile_base, sizeof(int32_t) * ((size_t)sm.ntiles + 1)));
         ASX_TRY(hipMalloc((void **)&sm.prow, sizeof(uint16_t) * ((size_t)sm.npartials + kReducePad)));
         ASX_TRY(hipMemsetAsync(sm.prow, 0, sizeof(uint16_t) * ((size_t)sm.npartials + kReducePad), s));
-        ASX_TRY(hipMalloc((void **)&prow_full, sizeof(int32_t) * (size_t)sm.npartials));
         ASX_TRY(hipMalloc(&sm.partial, sizeof(T) * ((size_t)sm.npartials + kReducePad)));
         ASX_TRY(hipMemsetAsync(sm.partial, 0, sizeof(T) * ((size_t)sm.npartials + kReducePad), s));
         ASX_TRY(hipMalloc((void **)&sm.chunk_lo, sizeof(int32_t) * ((size_t)sm.nrb + 1) * (size_t)sm.nslices));
@@ -585,9 +596,7 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
 #undef ASX_TRY
 #undef ASX_TRY_ST
 done:
-    for (void *p : {(void *)a, (void *)b, (void *)c, (void *)d, (void *)lrow, (void *)lhead, (void *)hscan,
-                    (void *)prow_full, (void *)d_pstart, (void *)d_tile_off, tmp})
-        if (p) (void)hipFree(p);
+    if (arena) (void)hipFree(arena);
     if (st) {
         free_sliced(&sm);
         return st;
