@@ -527,6 +527,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     if (m <= 0 || nnz <= 0 || n <= 0) return ASX_STATUS_INVALID_SIZE;
     if (target_wgs < 1) return ASX_STATUS_INVALID_VALUE;
     int st = ASX_STATUS_SUCCESS;
+    int32_t *arena = nullptr;
     int32_t *cmin = nullptr, *cmax = nullptr, *row_start = nullptr;  // m each
     int32_t *bmin = nullptr, *bmax = nullptr, *btiles = nullptr, *tile_off = nullptr, *d_small = nullptr;
     void *tmp = nullptr;
@@ -545,12 +546,17 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
         st = status_of(expr); \
         if (st) goto done;    \
     } while (0)
-    for (int32_t **q : {&cmin, &cmax, &row_start}) ASX_TRY(hipMalloc((void **)q, sizeof(int32_t) * (size_t)m));
-    for (int32_t **q : {&bmin, &bmax, &btiles, &tile_off})
-        ASX_TRY(hipMalloc((void **)q, sizeof(int32_t) * ((size_t)max_nb + 1)));
-    ASX_TRY(hipMalloc((void **)&d_small, sizeof(int32_t) * 2));
+    // the scratch of the build in one allocation: three arrays of m ints, four of max_nb + 1, two
+    // counters, the scan's workspace
     ASX_TRY(hipcub::DeviceScan::ExclusiveSum(nullptr, tmp_bytes, btiles, tile_off, max_nb + 1, s));
-    ASX_TRY(hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1));
+    {
+        const size_t per_row = ((size_t)m + 63) & ~(size_t)63, per_block = ((size_t)max_nb + 1 + 63) & ~(size_t)63;
+        ASX_TRY(hipMalloc((void **)&arena, sizeof(int32_t) * (3 * per_row + 4 * per_block + 64) + std::max<size_t>(tmp_bytes, 256)));
+        cmin = arena, cmax = cmin + per_row, row_start = cmax + per_row;
+        bmin = row_start + per_row, bmax = bmin + per_block, btiles = bmax + per_block, tile_off = btiles + per_block;
+        d_small = tile_off + per_block;
+        tmp = d_small + 64;
+    }
 
     // 1. column span of every row
     hipLaunchKernelGGL(k_window_row_span, dim3(mgrid), dim3(kBlock), 0, s, row_ptr, col, m, cmin, cmax);
@@ -757,8 +763,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     wm.has_carry = h_small[0] != 0;
 #undef ASX_TRY
 done:
-    for (void *p : {(void *)cmin, (void *)cmax, (void *)row_start, (void *)bmin, (void *)bmax, (void *)btiles,
-                    (void *)tile_off, (void *)d_small, (void *)d_bits, tmp})
+    for (void *p : {(void *)arena, (void *)d_bits})
         if (p) (void)hipFree(p);
     if (st) {
         free_window(&wm);
