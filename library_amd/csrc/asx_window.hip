@@ -93,28 +93,52 @@ __global__ __launch_bounds__(kBlock) void k_window_max_span(const int32_t *__res
 
 // Slot (from the start of its block) at which every row starts, and the tiles of every block.  A
 // row takes max(1, length) slots; a row of at most kAlignRowLen slots that would cross a tile
-// start begins at that tile start instead.  One thread walks one block's rows in order.
+// start begins at that tile start instead.  One wave walks one block's rows in order, 64 at a time:
+// starts from a scan of the lengths; at the first row of the 64 that has to move to the next tile
+// the walk restarts behind that row (the rows after it shift).
 __global__ __launch_bounds__(kBlock) void k_window_row_starts(const int32_t *__restrict__ row_ptr, int32_t m,
                                                               int32_t rows, int32_t nblocks,
                                                               int32_t *__restrict__ row_start,
                                                               int32_t *__restrict__ block_tiles)
 {
-    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (b >= nblocks) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t b = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+    if (b >= nblocks) return;  // whole waves leave
     const int32_t r0 = (int32_t)(b * rows);
     const int32_t r1 = (int64_t)r0 + rows < m ? r0 + rows : m;
     int32_t pos = 0;
-    int32_t next = row_ptr[r0];
-    for (int32_t r = r0; r < r1; ++r) {
-        const int32_t cur = next;
-        next = row_ptr[r + 1];
-        const int32_t len = next - cur > 0 ? next - cur : 1;
-        const int32_t in_tile = pos % kSlicedTile;
-        if (len <= kAlignRowLen && in_tile + len > kSlicedTile) pos += kSlicedTile - in_tile;
-        row_start[r] = pos;
-        pos += len;
+    int32_t r = r0;
+    while (r < r1) {  // uniform over the wave
+        const int32_t rr = r + lane;
+        int32_t len = 0;
+        if (rr < r1) {
+            len = row_ptr[rr + 1] - row_ptr[rr];
+            len = len > 0 ? len : 1;
+        }
+        int32_t incl = len;
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+            const int32_t t = __shfl_up(incl, d, kWave);
+            if (lane >= d) incl += t;
+        }
+        const int32_t start = pos + incl - len;
+        const bool moves = rr < r1 && len <= kAlignRowLen && start % kSlicedTile + len > kSlicedTile;
+        const unsigned long long mask = __ballot(moves);
+        if (mask == 0) {
+            if (rr < r1) row_start[rr] = start;
+            const int32_t cnt = r1 - r < kWave ? r1 - r : kWave;
+            pos += __builtin_amdgcn_readlane(incl, cnt - 1);
+            r += cnt;
+        } else {
+            const int f = __builtin_ctzll(mask);
+            const int32_t moved = (__builtin_amdgcn_readlane(start, f) / kSlicedTile + 1) * kSlicedTile;
+            if (lane < f) row_start[rr] = start;
+            if (lane == f) row_start[rr] = moved;
+            pos = moved + __builtin_amdgcn_readlane(len, f);
+            r += f + 1;
+        }
     }
-    block_tiles[b] = (pos + kSlicedTile - 1) / kSlicedTile;
+    if (lane == 0) block_tiles[b] = (pos + kSlicedTile - 1) / kSlicedTile;
 }
 
 template <typename T>
@@ -645,7 +669,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     }
     wm.nbands = bands.nbands;
     // 3. where every row starts inside its block; tiles of every block
-    hipLaunchKernelGGL(k_window_row_starts, dim3((unsigned)ceil_div64(wm.nblocks, kBlock)), dim3(kBlock), 0, s, row_ptr, m,
+    hipLaunchKernelGGL(k_window_row_starts, dim3((unsigned)ceil_div64((int64_t)wm.nblocks * kWave, kBlock)), dim3(kBlock), 0, s, row_ptr, m,
                        wm.rows_per_block, wm.nblocks, row_start, btiles);
     ASX_TRY(hipMemsetAsync(btiles + wm.nblocks, 0, sizeof(int32_t), s));
     ASX_TRY(hipcub::DeviceScan::ExclusiveSum(tmp, tmp_bytes, btiles, tile_off, wm.nblocks + 1, s));
