@@ -46,12 +46,12 @@ KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "
 # WRITE_SIZE all of them).  The Infinity Cache serves part of it: the counters read the same with
 # warm and with cold caches.
 MEASURED_TRAFFIC_BYTES = {
-    "banded_f64": 458_667,             # profiles/spmv_vector_banded_f64.md
-    "uniform16_f32": 248_805_417,      # profiles/spmv_sliced_uniform16_f32.md
-    "powerlaw_f64": 719_379_833,       # profiles/spmv_sliced_powerlaw_f64.md
-    "stencil5_f64": 1_135_154_025,     # profiles/spmv_window_stencil5_f64.md
-    "spmm_zipf_f32": 4_964_370_644,    # profiles/spmm_merge_spmm_zipf_f32.md
-    "spmm_banded_f32": 1_867_973_049,  # profiles/spmm_blocked_spmm_banded_f32.md
+    "banded_f64": 458_340,             # profiles/spmv_vector_banded_f64.md
+    "uniform16_f32": 248_822_414,      # profiles/spmv_sliced_uniform16_f32.md
+    "powerlaw_f64": 719_477_964,       # profiles/spmv_sliced_powerlaw_f64.md
+    "stencil5_f64": 1_135_140_117,     # profiles/spmv_window_stencil5_f64.md
+    "spmm_zipf_f32": 4_964_377_910,    # profiles/spmm_merge_spmm_zipf_f32.md
+    "spmm_banded_f32": 1_868_805_358,  # profiles/spmm_blocked_spmm_banded_f32.md
 }
 
 
