@@ -432,7 +432,7 @@ struct XFetch {
     }
 };
 
-template <typename T, int NW, bool VEC, int NB>
+template <typename T, int NW, bool VEC, int NB, int D>
 __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T beta, const int2 *__restrict__ chains,
                                                            const int4 *__restrict__ blocks,
                                                            const int4 *__restrict__ pieces,
@@ -448,14 +448,13 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     T *stage = stage_all + wave * kStageRows;
     const int32_t chain_last = blocks[chain.y - 1].y - 1;  // last tile of the chain
-    // this wave's tiles are those congruent to its number, across the blocks of the chain; three
-    // are in flight (loaded three steps ahead; past the end of the chain the last tile is re-read;
-    // measured 1-2 % ahead of two)
-    WindowTile<T> ta, tb, tc;
+    // this wave's tiles are those congruent to its number, across the blocks of the chain; D are
+    // in flight (loaded D steps ahead; past the end of the chain the last tile is re-read)
+    WindowTile<T> tl[D];
     int32_t t = blocks[chain.x].x + wave;
-    window_tile_load<T>(ta, t < chain_last ? t : chain_last, lane, cf, val, tile_info);
-    window_tile_load<T>(tb, t + NW < chain_last ? t + NW : chain_last, lane, cf, val, tile_info);
-    window_tile_load<T>(tc, t + 2 * NW < chain_last ? t + 2 * NW : chain_last, lane, cf, val, tile_info);
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+        window_tile_load<T>(tl[d], t + d * NW < chain_last ? t + d * NW : chain_last, lane, cf, val, tile_info);
     if (threadIdx.x == 0) xs[kWindowCols] = T(0);
     XFetch<T, NW * kWave, VEC, NB> xf;
     int4 blk = blocks[chain.x];  // first tile, end tile, pieces of x to fetch before the block: first, end
@@ -477,37 +476,29 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
         }                                      \
     }
 #define ASX_NEXT(TL, TT) window_tile_load<T>(TL, (TT) < chain_last ? (TT) : chain_last, lane, cf, val, tile_info)
-    // one tile: its rows' sums into the staging area, the loads of the tile three steps ahead (into
+    // one tile: its rows' sums into the staging area, the loads of the tile D steps ahead (into
     // the registers this one has just left), then the staged sums to y
 #define ASX_STEP(TL, TT)                                                                                          \
     {                                                                                                             \
         const StoreRows<T> out{y, carry + (TT), stage, TL.base & 0x7fffffff, TL.limit, TL.base < 0, alpha, beta}; \
         tile_reduce<T>(TL, lane, xs, out);                                                                        \
-        ASX_NEXT(TL, (TT) + 3 * NW);                                                                              \
+        ASX_NEXT(TL, (TT) + D * NW);                                                                              \
         out.flush(lane);                                                                                          \
     }
     // Every wave passes the start of every block of the chain (the barriers count all waves),
-    // whether it has tiles in the block or not.  ta, tb and tc take turns without changing places.
+    // whether it has tiles in the block or not.  The D tile buffers take turns without changing
+    // places (the loop over them is unrolled).
     ASX_BLOCK_BEGIN()
     for (;;) {  // all conditions are uniform over the wave
-        while (t >= tile_hi) {
-            if (++b >= chain.y) return;
-            ASX_BLOCK_BEGIN()
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            while (t >= tile_hi) {
+                if (++b >= chain.y) return;
+                ASX_BLOCK_BEGIN()
+            }
+            ASX_STEP(tl[d], t);
+            t += NW;
         }
-        ASX_STEP(ta, t);
-        t += NW;
-        while (t >= tile_hi) {
-            if (++b >= chain.y) return;
-            ASX_BLOCK_BEGIN()
-        }
-        ASX_STEP(tb, t);
-        t += NW;
-        while (t >= tile_hi) {
-            if (++b >= chain.y) return;
-            ASX_BLOCK_BEGIN()
-        }
-        ASX_STEP(tc, t);
-        t += NW;
     }
 #undef ASX_BLOCK_BEGIN
 #undef ASX_STEP
@@ -814,9 +805,12 @@ int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, co
     // x on a 16-byte boundary (every allocation is) and at least one 16-byte unit long: 16-byte
     // fetches; else element by element
     const bool vec = ((uintptr_t)x % 16) == 0 && (size_t)n * sizeof(T) >= 16;
-    const auto kernel = wm->nbands == 1 ? (vec ? k_spmv_window<T, kWindowWaves, true, 1> : k_spmv_window<T, kWindowWaves, false, 1>)
-                                        : (vec ? k_spmv_window<T, kWindowWaves, true, kWindowBands>
-                                               : k_spmv_window<T, kWindowWaves, false, kWindowBands>);
+    // tiles in flight per wave: three with one window (measured 1-2 % ahead of two); two with bands,
+    // where three no longer fit the 128 registers a lane of a 1024-thread workgroup may use
+    const auto kernel = wm->nbands == 1
+                            ? (vec ? k_spmv_window<T, kWindowWaves, true, 1, 3> : k_spmv_window<T, kWindowWaves, false, 1, 3>)
+                            : (vec ? k_spmv_window<T, kWindowWaves, true, kWindowBands, 2>
+                                   : k_spmv_window<T, kWindowWaves, false, kWindowBands, 2>);
     hipLaunchKernelGGL(kernel, dim3((unsigned)wm->nchains), dim3(kWindowWaves * kWave), 0, s, n, alpha, beta,
                        reinterpret_cast<const int2 *>(wm->chains), reinterpret_cast<const int4 *>(wm->blocks),
                        reinterpret_cast<const int4 *>(wm->pieces), wm->cf, (const T *)wm->val,
