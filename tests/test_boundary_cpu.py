@@ -172,3 +172,31 @@ def test_workload_generator_is_deterministic():
         assert np.all(np.diff(c) > 0)
     s = W.spmm_zipf_f32(m=1 << 12, ncols=8)
     assert s.x.size == (1 << 12) * 8 and s.y.size == (1 << 12) * 8
+
+
+def test_build_reads_the_compilers_kernel_resources():
+    """library_amd.build turns the compiler's kernel-resource-usage remarks into a table and refuses
+    kernels that spill registers to scratch memory; the table of the library that is built here
+    lists the hot kernels without scratch."""
+    from library_amd import build
+    text = """
+/x/asx_spmm.hip:133:1: remark: Function Name: _ZN3asx18k_spmm_snap_splitsEiiPKiS1_S1_PiS2_ [-Rpass-analysis=kernel-resource-usage]
+  133 | {
+      | ^
+/x/asx_spmm.hip:133:1: remark:     TotalSGPRs: 20 [-Rpass-analysis=kernel-resource-usage]
+/x/asx_spmm.hip:133:1: remark:     VGPRs: 11 [-Rpass-analysis=kernel-resource-usage]
+/x/asx_spmm.hip:133:1: remark:     ScratchSize [bytes/lane]: 60 [-Rpass-analysis=kernel-resource-usage]
+/x/asx_spmm.hip:133:1: remark:     Occupancy [waves/SIMD]: 8 [-Rpass-analysis=kernel-resource-usage]
+/x/asx_spmm.hip:133:1: remark:     LDS Size [bytes/block]: 4112 [-Rpass-analysis=kernel-resource-usage]
+/x/other.hip:1:1: remark: Function Name: _ZN7rocprim6kernelEv [-Rpass-analysis=kernel-resource-usage]
+/x/other.hip:1:1: remark:     VGPRs: 99 [-Rpass-analysis=kernel-resource-usage]
+"""
+    table = build.kernel_resources(text)
+    assert list(table) == ["_ZN3asx18k_spmm_snap_splitsEiiPKiS1_S1_PiS2_"]  # only this library's kernels
+    r = table["_ZN3asx18k_spmm_snap_splitsEiiPKiS1_S1_PiS2_"]
+    assert (r["TotalSGPRs"], r["VGPRs"], r["ScratchSize"], r["Occupancy"], r["LDS Size"]) == (20, 11, 60, 8, 4112)
+    path = os.path.join(ROOT, "library_amd", "build", "kernel_resources.txt")
+    if os.path.exists(path):
+        lines = open(path).read().splitlines()
+        assert lines and all(" scratch=0 " in l for l in lines)
+        assert any("k_spmv_window" in l for l in lines) and any("k_sliced_products" in l for l in lines)
