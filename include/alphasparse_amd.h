@@ -215,7 +215,12 @@ int asx_plan_holds_values(const asx_plan *plan);
 /* Number of 16x4 blocks and their fill of a blocked plan. */
 int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill);
 int asx_plan_destroy(asx_plan *plan);
-/* Kernel the plan resolved to, and bytes of per-call workspace its launches need. */
+/* Kernel the plan resolved to, and bytes of per-call workspace its launches need (carries; for a
+ * sliced plan the partial sums of a call, for a window plan with cut rows its carries).  A sliced
+ * or window plan also keeps a buffer of that size of its own, used by calls whose workspace is
+ * NULL or smaller: such calls share it and must not overlap, while calls that each bring a
+ * workspace of this size may run at the same time on different streams (the plan itself is only
+ * read). */
 int asx_plan_alg(const asx_plan *plan);
 size_t asx_plan_workspace_bytes(const asx_plan *plan);
 /* What a plan that holds a regrouped copy of A looks like (for logs and tests; -1 where the
@@ -228,9 +233,41 @@ enum {
     ASX_PLAN_INFO_ROWS_PER_BLOCK = 4, /* rows of a block (window) */
     ASX_PLAN_INFO_BANDS = 5,          /* rings of x in LDS: 1 = one window, 2..4 = bands of diagonals (window) */
     ASX_PLAN_INFO_CHAINS = 6,         /* chains of blocks = workgroups (window) */
-    ASX_PLAN_INFO_CARRY_PASS = 7      /* 1 if a call runs the ordered carry pass (window) */
+    ASX_PLAN_INFO_CARRY_PASS = 7,     /* 1 if a call runs the ordered carry pass (window) */
+    ASX_PLAN_INFO_ROW_BLOCKS = 8,     /* row blocks of pass 2 (sliced), blocks of rows (window) */
+    ASX_PLAN_INFO_STEPS = 9,          /* steps of pass 2, each up to 64 partial sums (sliced) */
+    ASX_PLAN_INFO_WIDTH = 10,         /* columns per slice (sliced), columns the rings hold together (window) */
+    ASX_PLAN_INFO_WORKGROUPS = 11,    /* workgroups of pass 1 (sliced), chains (window) */
+    ASX_PLAN_INFO_PIECES = 12         /* pieces of x fetched over all blocks (window) */
 };
 int64_t asx_plan_info(const asx_plan *plan, int what);
+/* Frees the buffer a sliced or window plan keeps for the partial sums / carries of a call.  Calls
+ * through the plan then need a workspace of asx_plan_workspace_bytes(plan) bytes (without one they
+ * return ASX_STATUS_INVALID_POINTER); for callers who always bring their own buffer and want the
+ * memory back.  The plan must not be in use by a call that is still running.  No counterpart in
+ * the reference. */
+int asx_plan_release_scratch(asx_plan *plan);
+/* Bytes of the buffer the plan itself keeps for that purpose (0: none, or released). */
+size_t asx_plan_own_scratch_bytes(const asx_plan *plan);
+/* Copies one array of a plan that holds a regrouped copy of A to the host (for tests that check a
+ * built plan on the host, and for debugging; synchronises `stream`).  `*bytes` receives the
+ * array's size; with h_dst == NULL nothing is copied (sizing call), else `cap` must be at least
+ * that.  ASX_STATUS_INVALID_VALUE when the plan's kernel has no such array.  No counterpart in the
+ * reference. */
+enum {
+    ASX_PLAN_ARRAY_VAL = 0,          /* slots x value: the regrouped values, in the order the loads deliver them */
+    ASX_PLAN_ARRAY_CF = 1,           /* slots x u16: local column | first-of-run << 15 */
+    ASX_PLAN_ARRAY_PERM = 2,         /* slots x i32: position in A's values of each stored copy (-1: pad) */
+    ASX_PLAN_ARRAY_TILE_WORDS = 3,   /* sliced: (tiles + 1) x i32 first partial sum of each tile; window: tiles x 2 i32 */
+    ASX_PLAN_ARRAY_WORKGROUPS = 4,   /* sliced: workgroups x 4 i32 (slice, first tile, end tile, 0); window: chains x 2 i32 */
+    ASX_PLAN_ARRAY_PARTIAL_ROWS = 5, /* sliced: partial sums x u16 row inside the row block | may-repeat << 15 */
+    ASX_PLAN_ARRAY_RANGES = 6,       /* sliced: (row blocks + 1) x slices i32: first partial sum of block b in slice s */
+    ASX_PLAN_ARRAY_STEP_PTR = 7,     /* sliced: (row blocks + 1) x i32: first step of each row block */
+    ASX_PLAN_ARRAY_STEPS = 8,        /* sliced: steps x 4 i32 */
+    ASX_PLAN_ARRAY_BLOCKS = 9,       /* window: blocks x 4 i32 (first tile, end tile, first piece, end piece) */
+    ASX_PLAN_ARRAY_PIECES = 10       /* window: pieces x 4 i32 (from column, to column, ring base, ring size) */
+};
+int asx_plan_export(const asx_plan *plan, int what, void *h_dst, size_t cap, size_t *bytes, void *stream);
 /* Copies the plan's histogram (33 bins) and stats (4) to host arrays. */
 int asx_plan_histogram(const asx_plan *plan, int64_t h_hist[33], int64_t h_stats[4]);
 

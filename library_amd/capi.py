@@ -29,6 +29,7 @@ EXPORTS = [
     "asx_dense_transpose", "asx_mtx_read", "asx_host_free", "asx_spmv_plan_create",
     "asx_plan_update_values", "asx_plan_holds_values", "asx_plan_info", "asx_plan_create",
     "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
+    "asx_plan_release_scratch", "asx_plan_own_scratch_bytes", "asx_plan_export",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
     "asx_spmv_csr_f64_noalloc", "asx_spmv_noalloc_max_workspace",
     "asx_spmm_resolve_alg", "asx_spmm_workspace_bytes", "asx_spmm_csr_f32", "asx_spmm_csr_f64",
@@ -82,6 +83,10 @@ def lib():
     L.asx_plan_workspace_bytes.argtypes = [vp]
     L.asx_plan_workspace_bytes.restype = sz
     L.asx_plan_histogram.argtypes = [vp, vp, vp]
+    L.asx_plan_release_scratch.argtypes = [vp]
+    L.asx_plan_own_scratch_bytes.argtypes = [vp]
+    L.asx_plan_own_scratch_bytes.restype = sz
+    L.asx_plan_export.argtypes = [vp, C.c_int, vp, sz, C.POINTER(sz), vp]
     L.asx_spmv_resolve_alg.argtypes = [C.c_int, i32, i32]
     L.asx_spmv_workspace_bytes.argtypes = [C.c_int, C.c_int, i32, i32]
     L.asx_spmv_workspace_bytes.restype = sz
@@ -285,7 +290,26 @@ class Plan:
         self._keep = (self._keep[0], self._keep[1], val)
 
     INFO = {"tiles": 0, "slices": 1, "partial_sums": 2, "rows_per_wave": 3, "rows_per_block": 4, "bands": 5,
-            "chains": 6, "carry_pass": 7}
+            "chains": 6, "carry_pass": 7, "row_blocks": 8, "steps": 9, "width": 10, "workgroups": 11, "pieces": 12}
+    # asx_plan_export: name -> (id, element type; "value" = the plan's value type)
+    ARRAYS = {"val": (0, "value"), "cf": (1, np.uint16), "perm": (2, np.int32), "tile_words": (3, np.int32),
+              "workgroups": (4, np.int32), "partial_rows": (5, np.uint16), "ranges": (6, np.int32),
+              "step_ptr": (7, np.int32), "steps": (8, np.int32), "blocks": (9, np.int32), "pieces": (10, np.int32)}
+
+    def export(self, name, value_dtype=None):
+        """One array of a sliced or window plan as a flat numpy array (asx_plan_export)."""
+        what, dt = self.ARRAYS[name]
+        dt = np.dtype(value_dtype if dt == "value" else dt)
+        nbytes = C.c_size_t(0)
+        _check(lib().asx_plan_export(self.h, what, None, 0, C.byref(nbytes), _stream()), "asx_plan_export")
+        out = np.empty(nbytes.value // dt.itemsize, dtype=dt)
+        if nbytes.value:
+            _check(lib().asx_plan_export(self.h, what, out.ctypes.data_as(C.c_void_p), out.nbytes, C.byref(nbytes),
+                                         _stream()), "asx_plan_export")
+        return out
+
+    def release_scratch(self):
+        _check(lib().asx_plan_release_scratch(self.h), "asx_plan_release_scratch")
 
     def info(self, what):
         """A figure of a sliced or window plan (asx_plan_info); -1 where it does not apply."""
@@ -314,7 +338,8 @@ def _workspace(nbytes, device):
 
 # ------------------------------------------------------------------------------ SpMV / SpMM
 def spmv(row_ptr, col, val, x, y, alpha, beta, alg=SPMV_DEFAULT, plan=None, workspace=None, n=None):
-    """y <- alpha*A*x + beta*y in place (torch CUDA tensors).  Returns y."""
+    """y <- alpha*A*x + beta*y in place (torch CUDA tensors).  Returns y.  workspace=None allocates
+    what the call needs; workspace=False passes none (a sliced or window plan then uses its own buffer)."""
     m = row_ptr.numel() - 1
     n = x.numel() if n is None else n
     nnz = col.numel()
@@ -322,9 +347,10 @@ def spmv(row_ptr, col, val, x, y, alpha, beta, alg=SPMV_DEFAULT, plan=None, work
     need = plan.workspace_bytes if plan is not None else lib().asx_spmv_workspace_bytes(alg, vt, m, nnz)
     if workspace is None:
         workspace = _workspace(need, val.device)
+    ws_ptr, ws_bytes = (None, 0) if workspace is False else (_ptr(workspace), workspace.numel() * workspace.element_size())
     fn = lib().asx_spmv_csr_f64 if vt == R_64F else lib().asx_spmv_csr_f32
     _check(fn(plan.h if plan is not None else None, alg, m, n, nnz, alpha, _ptr(row_ptr), _ptr(col), _ptr(val),
-              _ptr(x), beta, _ptr(y), _ptr(workspace), workspace.numel(), _stream()), "asx_spmv_csr")
+              _ptr(x), beta, _ptr(y), ws_ptr, ws_bytes, _stream()), "asx_spmv_csr")
     return y
 
 

@@ -17,6 +17,7 @@
 // one-based CSR is honoured (the reference's CSR kernels ignore idx_base); column-major B / C
 // and opB go through a tiled device transpose into the call's workspace (the reference
 // transposes B and C in place and rewrites their descriptors, alphasparse_spmm.hip:186-216).
+#include <algorithm>
 #include <cstddef>
 #include <cstdlib>
 #include <new>
@@ -127,12 +128,19 @@ struct DerivedCsr {
     void *val;  // owned only when transposed (otherwise the caller's values)
 };
 constexpr uint64_t kInfoMagic = 0x415358494e464f31ull;  // "ASXINFO1"
+// What alphasparseSpMV_bufferSize last reported for (matrix, algorithm): the size the caller's
+// externalBuffer is taken to have (its size is not part of alphasparseSpMV's signature).
+struct PromisedBuffer {
+    int alg;
+    size_t bytes;
+};
 struct MatInfoExt {
     _alphasparse_mat_info info;
     _alphasparse_csrmv_info csrmv;
     uint64_t magic;
     alphasparseHandle_t owner;  // null once that handle is gone
     std::vector<KeptPlan> plans;
+    std::vector<PromisedBuffer> promised;
     std::vector<DerivedCsr> derived;  // kept by alphasparseSpMV_analysis / alphasparseSpMM_preprocess
 };
 struct HandleRegistry {
@@ -204,6 +212,13 @@ asx_plan *find_plan(const _alphasparseSpMatDescr *owner, bool spmm, int alg, con
             return k.plan;
     return nullptr;
 }
+size_t promised_bytes(const _alphasparseSpMatDescr *A, int alg)
+{
+    if (MatInfoExt *e = ext_of(A))
+        for (const PromisedBuffer &p : e->promised)
+            if (p.alg == alg) return p.bytes;
+    return 0;
+}
 void drop_plans(alphasparseHandle_t h, bool spmm, int alg, bool all)
 {
     HandleRegistry *reg = registry_of(h, false);
@@ -215,6 +230,25 @@ bool is_transpose(alphasparseOperation_t op)
 {
     // real value types only: the conjugate transpose is the transpose
     return op == ALPHA_SPARSE_OPERATION_TRANSPOSE || op == ALPHA_SPARSE_OPERATION_CONJUGATE_TRANSPOSE;
+}
+bool same_source(const DerivedCsr &d, const _alphasparseSpMatDescr *A, bool transposed);
+// The kept plan a call with (A, opA, alg) would find, without building anything.
+const asx_plan *kept_plan(const _alphasparseSpMatDescr *A, alphasparseOperation_t opA, bool spmm, int alg, int ncols)
+{
+    MatInfoExt *x = ext_of(A);
+    if (!x) return nullptr;
+    const bool tr = is_transpose(opA);
+    if (!tr && A->idx_base == ALPHA_SPARSE_INDEX_BASE_ZERO) return find_plan(A, spmm, alg, A, ncols);
+    for (const DerivedCsr &d : x->derived) {
+        if (!same_source(d, A, tr)) continue;
+        _alphasparseSpMatDescr e = *A;
+        e.row_data = d.row_ptr;
+        e.col_data = d.col;
+        e.val_data = d.val;
+        if (tr) e.rows = A->cols, e.cols = A->rows;
+        return find_plan(A, spmm, alg, &e, ncols);
+    }
+    return nullptr;
 }
 
 void free_derived(DerivedCsr &d)
@@ -655,10 +689,23 @@ alphasparseStatus_t alphasparseSpMV_bufferSize(alphasparseHandle_t handle, alpha
     const int32_t m_eff = (int32_t)(is_transpose(opA) ? matA->cols : matA->rows);
     if (asx_spmv_resolve_alg((int)alg, m_eff, (int32_t)matA->nnz) < 0)
         return ALPHA_SPARSE_STATUS_NOT_SUPPORTED;
-    // sized for a call without kept analysis, and for DEFAULT for every kernel a later
-    // alphasparseSpMV_analysis may settle on: a call with kept analysis needs no more than this
-    const size_t need = asx_spmv_workspace_bytes((int)alg, (int)matA->data_type, m_eff, (int32_t)matA->nnz);
+    // sized for a call without kept analysis, and for DEFAULT for the row-ordered kernels a later
+    // alphasparseSpMV_analysis may settle on.  Kept analysis that regrouped A (column slices, row
+    // blocks) needs room for the partial sums or carries of a call: reported when the analysis is
+    // there already (call this after alphasparseSpMV_analysis to run calls with buffers of their
+    // own at the same time; a buffer sized before the analysis is too small for them and such
+    // calls use the buffer the analysis keeps, one at a time)
+    size_t need = asx_spmv_workspace_bytes((int)alg, (int)matA->data_type, m_eff, (int32_t)matA->nnz);
+    if (const asx_plan *plan = kept_plan(matA, opA, false, (int)alg, 1))
+        need = std::max(need, asx_plan_workspace_bytes(plan));
     *bufferSize = need;
+    // remember what the caller's buffer is now taken to hold
+    if (MatInfoExt *x = ext_create(handle, matA)) {
+        bool found = false;
+        for (PromisedBuffer &p : x->promised)
+            if (p.alg == (int)alg) p.bytes = need, found = true;
+        if (!found) x->promised.push_back(PromisedBuffer{(int)alg, need});
+    }
     return ALPHA_SPARSE_STATUS_SUCCESS;
 }
 
@@ -754,15 +801,25 @@ alphasparseStatus_t alphasparseSpMV(alphasparseHandle_t handle, alphasparseOpera
     }
     const size_t need = plan ? asx_plan_workspace_bytes(plan)
                              : asx_spmv_workspace_bytes((int)alg, (int)A->data_type, m, nnz);
-    bool ok;
-    void *ws = pick_workspace(handle, externalBuffer, need, &ok);
-    if (!ok) {
-        release_effective(handle, &eff);
-        return ALPHA_SPARSE_STATUS_INVALID_POINTER;
-    }
     // the size of a caller's buffer is not part of the signature: it is trusted to be what
-    // alphasparseSpMV_bufferSize reported
-    const size_t ws_bytes = need;
+    // alphasparseSpMV_bufferSize last reported for this matrix and algorithm (never queried: what
+    // a call without kept analysis needs)
+    void *ws;
+    size_t ws_bytes = need;
+    if (plan && asx_plan_own_scratch_bytes(plan) >= need && need > 0) {
+        // kept analysis with a buffer of its own for the partial sums / carries of a call: the
+        // caller's buffer is used only when it was sized after the analysis
+        const size_t have = externalBuffer ? promised_bytes(matA, (int)alg) : 0;
+        ws = have >= need ? externalBuffer : nullptr;
+        ws_bytes = have >= need ? have : 0;
+    } else {
+        bool ok;
+        ws = pick_workspace(handle, externalBuffer, need, &ok);
+        if (!ok) {
+            release_effective(handle, &eff);
+            return ALPHA_SPARSE_STATUS_INVALID_POINTER;
+        }
+    }
     int rc;
     if (A->data_type == ALPHA_R_64F)
         rc = asx_spmv_csr_f64(plan, (int)alg, m, n, nnz, *(const double *)alpha, A->row_data, A->col_data,

@@ -3,6 +3,7 @@
 // point launches HIP kernels or returns an error status.
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -196,18 +197,27 @@ int spmv_impl(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, 
         return launch_spmv_flat<T>(m, nnz, alpha, row_ptr, col, val, x, beta, y, seg, (T *)(w + L.carry_off),
                                    plan ? plan->carry_pass != 0 : true, s);
     }
-    case ASX_SPMV_SLICED:
-        // the slices hold a copy of A's columns and values (and the partial sums of a call) and are
-        // built by asx_spmv_plan_create; no workspace
+    case ASX_SPMV_SLICED: {
+        // the slices hold a copy of A's columns and values and are built by asx_spmv_plan_create.
+        // The partial sums of the call go into the caller's workspace when it is large enough, else
+        // into the plan's own buffer (which calls that overlap would share)
         if (!plan || !plan->sliced.cf) return ASX_STATUS_NOT_INITIALIZED;
         if (plan->n != n) return ASX_STATUS_INVALID_VALUE;
-        return launch_spmv_sliced<T>(m, n, alpha, &plan->sliced, x, beta, y, s);
-    case ASX_SPMV_WINDOW:
-        // the row blocks hold a copy of A's columns and values (and the carries of a call) and are
-        // built by asx_spmv_plan_create; no workspace
+        const size_t need = sliced_scratch_bytes(&plan->sliced, sizeof(T));
+        T *scratch = ws && ws_bytes >= need ? (T *)ws : (T *)plan->sliced.partial;
+        if (!scratch) return ws ? ASX_STATUS_INVALID_SIZE : ASX_STATUS_INVALID_POINTER;
+        return launch_spmv_sliced<T>(m, n, alpha, &plan->sliced, x, beta, y, scratch, s);
+    }
+    case ASX_SPMV_WINDOW: {
+        // the row blocks hold a copy of A's columns and values and are built by asx_spmv_plan_create;
+        // the carries of the call (plans with cut rows only) go where the sliced kernel's partial sums go
         if (!plan || !plan->window.cf) return ASX_STATUS_NOT_INITIALIZED;
         if (plan->n != n) return ASX_STATUS_INVALID_VALUE;
-        return launch_spmv_window<T>(m, n, alpha, &plan->window, x, beta, y, s);
+        const size_t need = window_scratch_bytes(&plan->window, sizeof(T));
+        T *scratch = ws && ws_bytes >= need ? (T *)ws : (T *)plan->window.carry;
+        if (need && !scratch) return ws ? ASX_STATUS_INVALID_SIZE : ASX_STATUS_INVALID_POINTER;
+        return launch_spmv_window<T>(m, n, alpha, &plan->window, x, beta, y, scratch, s);
+    }
     default: return ASX_STATUS_NOT_SUPPORTED;
     }
 }
@@ -557,7 +567,7 @@ int asx_spmm_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
 // Sliced is chosen when its estimate is at least 10 % lower.
 constexpr int32_t kSlicedMinNnz = 1 << 21;
 constexpr int32_t kSliceBytes = 131072;  // of x per slice: one workgroup of 16 waves per compute unit
-double sliced_expected_partials(const int64_t hist[33], int32_t nslices)
+static double sliced_expected_partials(const int64_t hist[33], int32_t nslices)
 {
     double p = 0.0;
     const double q = nslices > 1 ? std::log1p(-1.0 / (double)nslices) : 0.0;
@@ -568,7 +578,7 @@ double sliced_expected_partials(const int64_t hist[33], int32_t nslices)
     }
     return p;
 }
-bool sliced_pays(const int64_t hist[33], int32_t m, int32_t n, int32_t nnz, size_t sv)
+static bool sliced_pays(const int64_t hist[33], int32_t m, int32_t n, int32_t nnz, size_t sv)
 {
     if (nnz < kSlicedMinNnz || m <= 0 || n <= 0) return false;
     const double xbytes = (double)n * (double)sv;
@@ -591,16 +601,17 @@ int plan_add_slices(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
 {
     int cus = 256;
     (void)asx_device_info(&cus, nullptr);
-    // pass 2: one wave per block of rows with at most 16 KiB of accumulators.  Blocks of 256 rows,
-    // doubled while that leaves more than 8 waves per compute unit and the block's partial sums
-    // inside one slice (expected from the row-length histogram) are too few to fill the 64-wide
-    // steps in which a wave reads them (measured: 16 rows of 16 over 32 slices, 100 per range, run
-    // 5 % faster with 256 rows than with 512; the power-law matrix, 4 per range at 256 rows, runs
-    // 2x faster with 2048).
+    // pass 2: one wave per block of rows, its accumulators (8 bytes a row) in LDS.  Blocks of 256
+    // rows, doubled up to 1024 while that leaves more than 8 waves per compute unit and the block's
+    // partial sums inside one slice (expected from the row-length histogram) are fewer than 12: a
+    // step of pass 2 takes its 64 entries from at most three ranges.  Small blocks mean many waves
+    // in flight.  Measured: the power-law matrix (4 per range at 256 rows) 50 / 34.5 / 36.6 us with
+    // 512 / 1024 / 2048 rows; 16 per row over 32 slices (100 per range at 256 rows) 17.5 / 20 us
+    // with 256 / 512 rows; the same in fp64 over 64 slices 26.5 / 27.5 / 36.8 us with 256 / 512 / 1024.
     const int32_t nslices = (int32_t)ceil_div64((int64_t)p->n * (int64_t)sizeof(T), kSliceBytes);
     const double per_row_slice = sliced_expected_partials(p->hist, nslices) / ((double)p->m * (double)nslices);
     int32_t rpw = 256;
-    while (rpw < (int32_t)(16384 / sizeof(T)) && (int64_t)rpw * cus * 8 < p->m && per_row_slice * rpw < 96.0) rpw *= 2;
+    while (rpw < 1024 && (int64_t)rpw * cus * 8 < p->m && per_row_slice * rpw < 12.0) rpw *= 2;
     SlicedMatrix sm{};
     const int st = build_sliced<T>(p->m, p->n, p->nnz, (int32_t)(kSliceBytes / sizeof(T)), rpw, cus, d_row_ptr, d_col,
                                    d_val, &sm, s);
@@ -612,7 +623,7 @@ int plan_add_slices(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
     p->sliced = sm;
     p->nunits = sm.ntiles;
     p->carry_pass = 0;
-    p->workspace_bytes = 0;
+    p->workspace_bytes = sliced_scratch_bytes(&sm, sizeof(T));
     return ASX_STATUS_SUCCESS;
 }
 
@@ -635,7 +646,7 @@ int plan_add_window(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
     p->window = wm;
     p->nunits = wm.ntiles;
     p->carry_pass = wm.has_carry;
-    p->workspace_bytes = 0;
+    p->workspace_bytes = window_scratch_bytes(&wm, sizeof(T));
     return ASX_STATUS_SUCCESS;
 }
 
@@ -723,6 +734,83 @@ int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill)
     return ASX_STATUS_SUCCESS;
 }
 
+size_t asx_plan_own_scratch_bytes(const asx_plan *plan)
+{
+    if (!plan || plan->is_spmm) return 0;
+    if (plan->alg == ASX_SPMV_SLICED && plan->sliced.partial) return sliced_scratch_bytes(&plan->sliced, vsize(plan->value_type));
+    if (plan->alg == ASX_SPMV_WINDOW && plan->window.carry) return window_scratch_bytes(&plan->window, vsize(plan->value_type));
+    return 0;
+}
+
+int asx_plan_release_scratch(asx_plan *plan)
+{
+    if (!plan) return ASX_STATUS_INVALID_POINTER;
+    int st = ASX_STATUS_SUCCESS;
+    if (plan->sliced.partial) {
+        st = status_of(hipFree(plan->sliced.partial));
+        plan->sliced.partial = nullptr;
+    }
+    if (plan->window.carry) {
+        const int st2 = status_of(hipFree(plan->window.carry));
+        plan->window.carry = nullptr;
+        if (!st) st = st2;
+    }
+    return st;
+}
+
+// The arrays of a plan that holds a regrouped copy of A: device address and bytes.
+static bool plan_array(const asx_plan *p, int what, const void **ptr, size_t *bytes)
+{
+    const size_t sv = vsize(p->value_type);
+    *ptr = nullptr;
+    *bytes = 0;
+    if (!p->is_spmm && p->alg == ASX_SPMV_SLICED) {
+        const SlicedMatrix &m = p->sliced;
+        const size_t slots = (size_t)m.ntiles * kSlicedTile;
+        switch (what) {
+        case ASX_PLAN_ARRAY_VAL: *ptr = m.val, *bytes = slots * sv; return true;
+        case ASX_PLAN_ARRAY_CF: *ptr = m.cf, *bytes = slots * 2; return true;
+        case ASX_PLAN_ARRAY_PERM: *ptr = m.perm, *bytes = slots * 4; return true;
+        case ASX_PLAN_ARRAY_TILE_WORDS: *ptr = m.tile_base, *bytes = ((size_t)m.ntiles + 1) * 4; return true;
+        case ASX_PLAN_ARRAY_WORKGROUPS: *ptr = m.wg_tab, *bytes = (size_t)m.nwg * 16; return true;
+        case ASX_PLAN_ARRAY_PARTIAL_ROWS: *ptr = m.prow, *bytes = (size_t)m.npartials * 2; return true;
+        case ASX_PLAN_ARRAY_RANGES: *ptr = m.chunk_lo, *bytes = ((size_t)m.nrb + 1) * (size_t)m.nslices * 4; return true;
+        case ASX_PLAN_ARRAY_STEP_PTR: *ptr = m.pstep_ptr, *bytes = ((size_t)m.nrb + 1) * 4; return true;
+        case ASX_PLAN_ARRAY_STEPS: *ptr = m.psteps, *bytes = (size_t)m.npsteps * 16; return true;
+        default: return false;
+        }
+    }
+    if (!p->is_spmm && p->alg == ASX_SPMV_WINDOW) {
+        const WindowMatrix &m = p->window;
+        const size_t slots = (size_t)m.ntiles * kSlicedTile;
+        switch (what) {
+        case ASX_PLAN_ARRAY_VAL: *ptr = m.val, *bytes = slots * sv; return true;
+        case ASX_PLAN_ARRAY_CF: *ptr = m.cf, *bytes = slots * 2; return true;
+        case ASX_PLAN_ARRAY_PERM: *ptr = m.perm, *bytes = slots * 4; return true;
+        case ASX_PLAN_ARRAY_TILE_WORDS: *ptr = m.tile_info, *bytes = (size_t)m.ntiles * 8; return true;
+        case ASX_PLAN_ARRAY_WORKGROUPS: *ptr = m.chains, *bytes = (size_t)m.nchains * 8; return true;
+        case ASX_PLAN_ARRAY_BLOCKS: *ptr = m.blocks, *bytes = (size_t)m.nblocks * 16; return true;
+        case ASX_PLAN_ARRAY_PIECES: *ptr = m.pieces, *bytes = (size_t)m.npieces * 16; return true;
+        default: return false;
+        }
+    }
+    return false;
+}
+
+int asx_plan_export(const asx_plan *plan, int what, void *h_dst, size_t cap, size_t *bytes, void *stream)
+{
+    if (!plan || !bytes) return ASX_STATUS_INVALID_POINTER;
+    const void *src;
+    if (!plan_array(plan, what, &src, bytes)) return ASX_STATUS_INVALID_VALUE;
+    if (!h_dst) return ASX_STATUS_SUCCESS;  // sizing call
+    if (cap < *bytes) return ASX_STATUS_INVALID_SIZE;
+    if (*bytes == 0) return ASX_STATUS_SUCCESS;
+    hipStream_t s = (hipStream_t)stream;
+    int st = status_of(hipMemcpyAsync(h_dst, src, *bytes, hipMemcpyDeviceToHost, s));
+    if (!st) st = status_of(hipStreamSynchronize(s));
+    return st;
+}
+
 int asx_plan_alg(const asx_plan *plan) { return plan ? plan->alg : -1; }
 size_t asx_plan_workspace_bytes(const asx_plan *plan) { return plan ? plan->workspace_bytes : 0; }
 int64_t asx_plan_info(const asx_plan *plan, int what)
@@ -738,6 +826,11 @@ int64_t asx_plan_info(const asx_plan *plan, int what)
     case ASX_PLAN_INFO_BANDS: return window ? plan->window.nbands : -1;
     case ASX_PLAN_INFO_CHAINS: return window ? plan->window.nchains : -1;
     case ASX_PLAN_INFO_CARRY_PASS: return window ? plan->window.has_carry : -1;
+    case ASX_PLAN_INFO_ROW_BLOCKS: return sliced ? plan->sliced.nrb : window ? plan->window.nblocks : -1;
+    case ASX_PLAN_INFO_STEPS: return sliced ? plan->sliced.npsteps : -1;
+    case ASX_PLAN_INFO_WIDTH: return sliced ? plan->sliced.width : window ? 16384 : -1;
+    case ASX_PLAN_INFO_WORKGROUPS: return sliced ? plan->sliced.nwg : window ? plan->window.nchains : -1;
+    case ASX_PLAN_INFO_PIECES: return window ? plan->window.npieces : -1;
     default: return -1;
     }
 }

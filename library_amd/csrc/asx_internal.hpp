@@ -132,14 +132,20 @@ struct SlicedMatrix {
     int32_t rows_per_wave;  // pass 2
     int32_t nrb;            // ceil(m / rows_per_wave)
     void *val;              // ntiles * kSlicedTile values (a copy of A's, in slice order; pads are 0)
-    void *partial;          // npartials (+ 64 readable) values: the partial sums of one call
+    void *partial;          // npartials + kSlicedReducePad values: the partial sums of one call, for callers
+                            // that bring no buffer of their own (null once released)
     uint16_t *cf;           // ntiles * kSlicedTile: column inside the slice, bit 15 = first element of a run
     int32_t *perm;          // where each stored copy comes from in A's val (-1 for pads)
     int32_t *tile_base;     // ntiles + 1: index of the first partial sum of each tile
     int32_t *wg_tab;        // nwg x 4: slice, first tile, end tile, 0
-    uint16_t *prow;         // npartials: row of each partial sum inside its row block
+    uint16_t *prow;         // npartials + kSlicedReducePad: row of each partial sum inside its row block
     int32_t *chunk_lo;      // (nrb + 1) x nslices: first partial sum of row block b in slice s
+    int32_t npsteps;        // steps of pass 2, all row blocks
+    int32_t *pstep_ptr;     // nrb + 1: first step of each row block
+    int32_t *psteps;        // npsteps (+ kSlicedStepPad) x 4: up to 64 partial sums from up to 3 pieces of ranges
 };
+constexpr int kSlicedStepPad = 64;     // readable step descriptors past the last one
+constexpr int kSlicedReducePad = 256;  // entries of prow / partial that pass 2 may read past the last partial sum
 template <typename T>
 int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_per_wave, int32_t target_wgs,
                  const int32_t *row_ptr, const int32_t *col, const T *val, SlicedMatrix *out, hipStream_t s);
@@ -147,7 +153,9 @@ void free_sliced(SlicedMatrix *p);
 template <typename T>
 int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s);
 template <typename T>
-int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, hipStream_t s);
+int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, T *partial,
+                       hipStream_t s);
+inline size_t sliced_scratch_bytes(const SlicedMatrix *sm, size_t sv) { return ((size_t)sm->npartials + kSlicedReducePad) * sv; }
 
 // ---- row blocks with sliding windows of x in LDS (asx_window.hip) ----
 // Blocks of `rows_per_block` consecutive rows whose columns all lie inside at most kWindowBands
@@ -160,11 +168,12 @@ struct WindowMatrix {
     int32_t rows_per_block;
     int32_t nblocks;
     int32_t nchains;         // workgroups
+    int32_t npieces;         // entries of `pieces`
     int32_t ntiles;
     int32_t nbands;          // 1: one window per block; 2..kWindowBands: bands of diagonals
     int has_carry;           // some tile starts inside a row: the ordered carry pass is needed
     void *val;               // ntiles * kSlicedTile values (a copy of A's; pads are 0)
-    void *carry;             // ntiles values
+    void *carry;             // ntiles values: the carries of one call, for callers that bring no buffer (null once released)
     uint16_t *cf;            // ntiles * kSlicedTile: LDS slot of the column, bit 15 = first slot of a row (or tile)
     int32_t *perm;           // where each stored copy comes from in A's val (-1 for pads)
     int32_t *tile_info;      // ntiles x 2: row of the tile's first slot (bit 31: the tile starts inside it), rows in the tile
@@ -179,7 +188,9 @@ void free_window(WindowMatrix *p);
 template <typename T>
 int window_update_values(const WindowMatrix *wm, const T *val, hipStream_t s);
 template <typename T>
-int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, hipStream_t s);
+int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, T *carry,
+                       hipStream_t s);
+inline size_t window_scratch_bytes(const WindowMatrix *wm, size_t sv) { return wm->has_carry ? (size_t)wm->ntiles * sv : 0; }
 
 inline int32_t merge_tiles(int32_t m, int32_t nnz) { return (int32_t)ceil_div64((int64_t)m + nnz, kMergeTile); }
 inline int32_t flat_tiles(int32_t nnz) { int32_t t = (int32_t)ceil_div64(nnz, kFlatTile); return t < 1 ? 1 : t; }

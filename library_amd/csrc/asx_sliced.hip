@@ -26,6 +26,8 @@
 // kernels gather x from global memory: hip/kernel/level2/alphasparse_spmv_csr_vector.h:99-126).
 #include <hipcub/hipcub.hpp>
 
+#include <rocprim/rocprim.hpp>
+
 #include <algorithm>
 #include <vector>
 
@@ -37,7 +39,6 @@ namespace asx {
 namespace {
 
 constexpr int32_t kPadRow = 0x7fffffff;
-constexpr int kReducePad = 4 * kWave;  // entries of prow / partial that pass 2 may read past the last partial sum
 
 __global__ __launch_bounds__(kBlock) void k_sliced_keys(const int32_t *__restrict__ col, int32_t nnz, int32_t width,
                                                         int32_t *__restrict__ keys, int32_t *__restrict__ idx)
@@ -231,209 +232,166 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const 
 }
 
 // ---- pass 2 ------------------------------------------------------------------------------
-// acc[id & 0x7fff] += v for the lanes that are `on`.  MODE 0: LDS atomic adds.  MODE 1: plain
-// read-add-write for entries whose row differs from the entry before them (sorted rows: no two
-// such lanes share an address), atomic adds afterwards for the marked rest (rare).  The wave owns
-// its accumulators and its LDS operations execute in order, so either way the sums are added in
-// a fixed order.
-template <int MODE, typename T>
-__device__ __forceinline__ void lds_add(T *acc, uint16_t id, T v, bool on)
+// The partial sums of a row block, range after range in slice order, are cut (when the plan is
+// built) into steps of up to 64 entries.  A step takes its entries from up to kPieces consecutive
+// pieces of ranges (a range may be split between steps); lane l reads entry base[p] + l of the
+// piece p it falls in.  Descriptor of a step: base[0..2], then
+// first lane of piece 1 | first lane of piece 2 << 8 | entries << 16.
+constexpr int kPieces = 3;
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+
+// One thread per row block walks the block's ranges; `psteps == nullptr`: only count.
+__global__ __launch_bounds__(kBlock) void k_sliced_pack(const int32_t *__restrict__ chunk_lo, int32_t nrb,
+                                                         int32_t nslices, const int32_t *__restrict__ pstep_ptr,
+                                                         int32_t *__restrict__ count, i32x4 *__restrict__ psteps)
 {
-    T *p = acc + (id & 0x7fff);
-    if (MODE == 0) {
-        if (on) __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);  // ds_add_f32 / _f64
-    } else {
-        const bool cont = (id & 0x8000) != 0;
-        if (on && !cont) *p += v;
-        if (__ballot(on && cont) != 0) {
-            if (on && cont) __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const int32_t b = (int32_t)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (b >= nrb) return;
+    const int32_t *lo_row = chunk_lo + (int64_t)b * nslices, *hi_row = lo_row + nslices;
+    i32x4 *out = psteps ? psteps + pstep_ptr[b] : nullptr;
+    int32_t nsteps = 0, fill = 0, pieces = 0;
+    int32_t base[kPieces] = {0, 0, 0}, first[kPieces] = {0, kWave, kWave};
+    for (int32_t sl = 0; sl < nslices; ++sl) {
+        int32_t lo = lo_row[sl], len = hi_row[sl] - lo;
+        while (len > 0) {
+            if (pieces == kPieces || fill == kWave) {
+                if (out) out[nsteps] = i32x4{base[0], base[1], base[2], first[1] | first[2] << 8 | fill << 16};
+                ++nsteps;
+                fill = pieces = 0;
+                first[1] = first[2] = kWave;
+            }
+            const int32_t take = len < kWave - fill ? len : kWave - fill;
+            base[pieces] = lo - fill;
+            first[pieces] = fill;
+            ++pieces;
+            fill += take;
+            lo += take;
+            len -= take;
         }
+    }
+    if (fill > 0) {
+        if (out) out[nsteps] = i32x4{base[0], base[1], base[2], first[1] | first[2] << 8 | fill << 16};
+        ++nsteps;
+    }
+    if (!psteps) count[b] = nsteps;
+}
+
+// U steps whose loads are issued together.
+template <typename T, int U>
+struct StepBatch {
+    uint16_t id[U];
+    T pv[U];
+    uint32_t valid;  // bit u: the lane's entry of step u counts
+};
+
+template <int U>
+__device__ __forceinline__ void steps_describe(i32x4 (&d)[U], int32_t first, const i32x4 *__restrict__ psteps)
+{
+#pragma unroll
+    for (int u = 0; u < U; ++u) d[u] = psteps[first + u];  // uniform addresses: scalar loads
+}
+
+// Every load is unconditional: a step past the block's last one reads entries 0..63 and counts
+// nothing; a lane past a step's entries reads a neighbour's entry (prow and partial are readable
+// for kSlicedReducePad entries past the last partial sum) and drops it at the add.
+template <typename T, int U>
+__device__ __forceinline__ void steps_issue(StepBatch<T, U> &bt, const i32x4 (&d)[U], int32_t first, int32_t end,
+                                            int lane, const uint16_t *__restrict__ prow, const T *__restrict__ partial)
+{
+    uint32_t valid = 0;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const bool live = first + u < end;
+        const int32_t w = live ? d[u].w : (kWave | kWave << 8);
+        const int32_t f1 = w & 0xff, f2 = (w >> 8) & 0xff, total = w >> 16;
+        int32_t base = d[u].x;
+        base = lane >= f1 ? d[u].y : base;
+        base = lane >= f2 ? d[u].z : base;
+        const int64_t at = live ? (int64_t)base + lane : lane;
+        bt.id[u] = prow[at];
+        bt.pv[u] = partial[at];
+        valid |= (uint32_t)(lane < total) << u;
+    }
+    bt.valid = valid;
+}
+
+// Entries that do not count go to a spare accumulator of the lane's own behind the block's rows
+// (64 lanes adding to one address would be serialised).
+template <typename T, int U>
+__device__ __forceinline__ void steps_add(const StepBatch<T, U> &bt, double *acc, int32_t spare)
+{
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const bool on = (bt.valid >> u) & 1;
+        double *p = acc + (on ? (int32_t)(bt.id[u] & 0x7fff) : spare);
+        __hip_atomic_fetch_add(p, (double)bt.pv[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);  // ds_add_f64
     }
 }
 
-// Walks the ranges of one row block, STEP entries per step.
-template <int STEP>
-struct RangeWalk {
-    int32_t lo_v, len_v;  // per lane: start and length of range `lane` of the current 64 slices
-    int32_t ns;           // ranges in the current group
-    int32_t j, k0;        // current range and offset inside it
-    int32_t a, len;       // start and length of the current range (uniform)
-    __device__ __forceinline__ void fetch()
-    {
-        a = __builtin_amdgcn_readlane(lo_v, j & (kWave - 1));
-        len = j < ns ? __builtin_amdgcn_readlane(len_v, j & (kWave - 1)) : 0;
-    }
-    // start (an index that is safe to load STEP entries from) and count of the next step
-    __device__ __forceinline__ void next(int32_t &start, int32_t &count)
-    {
-        const int32_t left = len - k0;
-        count = left < STEP ? (left > 0 ? left : 0) : STEP;
-        start = j < ns ? a + k0 : 0;
-        k0 += STEP;
-        if (k0 >= len && j < ns) {
-            ++j;
-            k0 = 0;
-            fetch();
-        }
-    }
-};
-
-// W consecutive entries of a lane (row ids and partial sums), loaded with one instruction each;
-// the addresses are only aligned to one entry.
-template <typename T, int W>
-struct Entries {
-    typedef uint16_t id_vec __attribute__((ext_vector_type(W)));
-    typedef T pv_vec __attribute__((ext_vector_type(W)));
-    typedef id_vec id_vec_u __attribute__((aligned(2)));
-    typedef pv_vec pv_vec_u __attribute__((aligned(sizeof(T))));
-    id_vec id;
-    pv_vec pv;
-    __device__ __forceinline__ void load(const uint16_t *__restrict__ prow, const T *__restrict__ partial, int64_t at)
-    {
-        id = *reinterpret_cast<const id_vec_u *>(prow + at);
-        pv = *reinterpret_cast<const pv_vec_u *>(partial + at);
-    }
-};
-
-template <typename T, int NW, int MODE, int W>
-__global__ __launch_bounds__(NW *kWave) void k_sliced_reduce(int32_t m, int32_t nrb, int32_t rw, int32_t nslices, T alpha,
-                                                             T beta, const int32_t *__restrict__ chunk_lo,
-                                                             const uint16_t *__restrict__ prow,
-                                                             const T *__restrict__ partial, T *__restrict__ y)
+// One wave (= one workgroup) per row block.  The wave reads its steps' descriptors with scalar
+// loads, one batch ahead, and keeps NB batches of U steps in flight, so that a batch waits for its
+// own loads only.  Accumulators are fp64 for both value types: the LDS has a native fp64 atomic
+// add (no dependent read in the wave's instruction stream), and the fp32 one measured 2.5 times
+// slower.  Only this wave touches its accumulators and a wave's LDS operations execute in order,
+// so the order of additions is fixed.
+template <typename T, int U, int NB>
+__global__ __launch_bounds__(kWave) void k_sliced_reduce(int32_t m, int32_t nrb, int32_t rw, T alpha, T beta,
+                                                         const int32_t *__restrict__ pstep_ptr,
+                                                         const i32x4 *__restrict__ psteps,
+                                                         const uint16_t *__restrict__ prow,
+                                                         const T *__restrict__ partial, T *__restrict__ y)
 {
     extern __shared__ __align__(16) unsigned char sliced_lds[];
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    double *acc = reinterpret_cast<double *>(sliced_lds);
+    const int lane = threadIdx.x;
     // neighbouring row blocks share the cache lines at the ends of their ranges: keep them on one XCD
     // (the grid is a multiple of kXcds workgroups, dealt to the XCDs round-robin)
     const int32_t per_xcd = (int32_t)gridDim.x / kXcds;
-    const int32_t wg = ((int32_t)blockIdx.x % kXcds) * per_xcd + (int32_t)blockIdx.x / kXcds;
-    const int64_t b = (int64_t)wg * NW + wave;
-    if (b >= nrb) return;  // whole waves leave; no workgroup barrier below
-    T *acc = reinterpret_cast<T *>(sliced_lds) + (size_t)wave * rw;
-    for (int i = lane; i < rw; i += kWave) acc[i] = T(0);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    const int32_t *lo_row = chunk_lo + b * nslices;
-    const int32_t *hi_row = lo_row + nslices;
-    if (W > 1) {
-        // Long ranges (chosen by the launcher from the mean range length): steps of 64 W entries, W
-        // consecutive ones per lane from one load of the row ids and one of the sums; U steps per
-        // batch, two batches in turn.  Loads are unconditional (prow and partial are readable for
-        // kReducePad entries past the last partial sum); entries past a range's end are dropped at
-        // the add.  A lane adds its W entries in order, so rows repeated inside a lane are safe.
-        constexpr int UW = 8;
-        for (int32_t s0 = 0; s0 < nslices; s0 += kWave) {
-            RangeWalk<kWave * W> w;
-            w.ns = nslices - s0 < kWave ? nslices - s0 : kWave;
-            w.lo_v = lane < w.ns ? lo_row[s0 + lane] : 0;
-            w.len_v = lane < w.ns ? hi_row[s0 + lane] - w.lo_v : 0;
-            w.j = 0;
-            w.k0 = 0;
-            w.fetch();
-            Entries<T, W> ea[UW], eb[UW];
-            int32_t na[UW], nb[UW];
-#define ASX_LOADW(E, N)                            \
-    _Pragma("unroll") for (int u = 0; u < UW; ++u) \
-    {                                              \
-        int32_t start;                             \
-        w.next(start, N[u]);                       \
-        E[u].load(prow, partial, (int64_t)start + lane * W); \
+    const int32_t b = ((int32_t)blockIdx.x % kXcds) * per_xcd + (int32_t)blockIdx.x / kXcds;
+    if (b >= nrb) return;
+    const int32_t s0 = pstep_ptr[b], s1 = pstep_ptr[b + 1];
+    StepBatch<T, U> bt[NB];
+    i32x4 d[U];
+    steps_describe<U>(d, s0, psteps);
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        steps_issue<T, U>(bt[j], d, s0 + j * U, s1, lane, prow, partial);
+        steps_describe<U>(d, s0 + (j + 1) * U, psteps);
+        __builtin_amdgcn_sched_barrier(0);
     }
-#define ASX_ADDW(E, N)                             \
-    _Pragma("unroll") for (int u = 0; u < UW; ++u) \
-    {                                              \
-        _Pragma("unroll") for (int e = 0; e < W; ++e) lds_add<MODE, T>(acc, E[u].id[e], E[u].pv[e], lane * W + e < N[u]); \
-    }
-            ASX_LOADW(ea, na)
-            ASX_LOADW(eb, nb)
-            while (true) {  // uniform over the wave
-                ASX_ADDW(ea, na)
-                const bool more_a = w.j < w.ns;
-                ASX_LOADW(ea, na)
-                ASX_ADDW(eb, nb)
-                if (!more_a) break;  // nothing was left when batch a was reloaded: a and b are spent
-                ASX_LOADW(eb, nb)
-            }
-#undef ASX_LOADW
-#undef ASX_ADDW
+    for (int i = lane; i < rw + kWave; i += kWave) acc[i] = 0.0;  // rw + lane: the lane's spare accumulator
+    int32_t k = s0;
+    for (; k + NB * U < s1; k += NB * U) {  // uniform
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            steps_add<T, U>(bt[j], acc, rw + lane);
+            __builtin_amdgcn_sched_barrier(0);  // keep a later batch's address arithmetic (and its wait) behind these adds
+            steps_issue<T, U>(bt[j], d, k + (NB + j) * U, s1, lane, prow, partial);
+            steps_describe<U>(d, k + (NB + j + 1) * U, psteps);
+            __builtin_amdgcn_sched_barrier(0);
         }
-    } else {
-    // Steps of 64 (row, partial sum) pairs, U steps per batch, two batches in turn: a batch's loads
-    // are issued before the other batch is added.  Loads are unconditional (prow and partial are
-    // readable for 64 entries past the last partial sum; a step past the end reads entry 0 on);
-    // entries past a range's end are dropped at the add.
-    constexpr int U = 16;
-    for (int32_t s0 = 0; s0 < nslices; s0 += kWave) {
-        const int32_t ns = nslices - s0 < kWave ? nslices - s0 : kWave;
-        const int32_t lo_v = lane < ns ? lo_row[s0 + lane] : 0;
-        const int32_t len_v = lane < ns ? hi_row[s0 + lane] - lo_v : 0;
-        uint16_t ida[U], idb[U];
-        T pa[U], pb[U];
-#define ASX_ADD(ID, PV, N)                        \
-    _Pragma("unroll") for (int u = 0; u < U; ++u) \
-    {                                             \
-        lds_add<MODE, T>(acc, ID[u], PV[u], lane < N[u]); \
     }
-        if (__ballot(len_v > kWave) == 0) {
-            // every range fits one step: range j is step j
-#define ASX_LOAD(ID, PV, J)                                         \
-    _Pragma("unroll") for (int u = 0; u < U; ++u)                   \
-    {                                                               \
-        const int32_t a = __builtin_amdgcn_readlane(lo_v, (J) + u); \
-        ID[u] = prow[a + lane];                                     \
-        PV[u] = partial[a + lane];                                  \
-    }
-#define ASX_ADDJ(ID, PV, J)                       \
-    _Pragma("unroll") for (int u = 0; u < U; ++u) \
-    {                                             \
-        lds_add<MODE, T>(acc, ID[u], PV[u], lane < __builtin_amdgcn_readlane(len_v, (J) + u)); \
-    }
-            ASX_LOAD(ida, pa, 0)
-            if (ns > U) ASX_LOAD(idb, pb, U)
-            ASX_ADDJ(ida, pa, 0)
-            if (ns > 2 * U) ASX_LOAD(ida, pa, 2 * U)
-            if (ns > U) ASX_ADDJ(idb, pb, U)
-            if (ns > 3 * U) ASX_LOAD(idb, pb, 3 * U)
-            if (ns > 2 * U) ASX_ADDJ(ida, pa, 2 * U)
-            if (ns > 3 * U) ASX_ADDJ(idb, pb, 3 * U)
-#undef ASX_LOAD
-#undef ASX_ADDJ
-        } else {
-            RangeWalk<kWave> w;
-            w.ns = ns;
-            w.lo_v = lo_v;
-            w.len_v = len_v;
-            w.j = 0;
-            w.k0 = 0;
-            w.fetch();
-            int32_t na[U], nb[U];
-#define ASX_LOAD(ID, PV, N)                       \
-    _Pragma("unroll") for (int u = 0; u < U; ++u) \
-    {                                             \
-        int32_t start;                            \
-        w.next(start, N[u]);                      \
-        ID[u] = prow[start + lane];               \
-        PV[u] = partial[start + lane];            \
-    }
-            ASX_LOAD(ida, pa, na)
-            ASX_LOAD(idb, pb, nb)
-            while (true) {  // uniform over the wave
-                ASX_ADD(ida, pa, na)
-                const bool more_a = w.j < w.ns;
-                ASX_LOAD(ida, pa, na)
-                ASX_ADD(idb, pb, nb)
-                if (!more_a) break;  // nothing was left when batch a was reloaded: a and b are spent
-                ASX_LOAD(idb, pb, nb)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) steps_add<T, U>(bt[j], acc, rw + lane);
+    const int64_t r0 = (int64_t)b * rw;
+    constexpr int Q = 8;  // rows of y per lane whose old values are requested together
+    for (int i0 = 0; i0 < rw; i0 += Q * kWave) {
+        T yv[Q];
+        if (beta != T(0)) {
+#pragma unroll
+            for (int q = 0; q < Q; ++q) {
+                const int i = i0 + q * kWave + lane;
+                yv[q] = (i < rw && r0 + i < m) ? y[r0 + i] : T(0);
             }
-#undef ASX_LOAD
         }
-#undef ASX_ADD
-    }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const int64_t r0 = b * rw;
-    for (int i = lane; i < rw; i += kWave) {
-        const int64_t r = r0 + i;
-        if (r < m) y[r] = beta == T(0) ? alpha * acc[i] : fma_t<T>(alpha, acc[i], beta * y[r]);
+#pragma unroll
+        for (int q = 0; q < Q; ++q) {
+            const int i = i0 + q * kWave + lane;
+            if (i < rw && r0 + i < m) {
+                const T a = (T)acc[i];
+                y[r0 + i] = beta == T(0) ? alpha * a : fma_t<T>(alpha, a, beta * yv[q]);
+            }
+        }
     }
 }
 
@@ -442,11 +400,11 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_reduce(int32_t m, int32_t 
 void free_sliced(SlicedMatrix *p)
 {
     for (void *q : {p->val, p->partial, (void *)p->cf, (void *)p->perm, (void *)p->tile_base, (void *)p->wg_tab,
-                    (void *)p->prow, (void *)p->chunk_lo})
+                    (void *)p->prow, (void *)p->chunk_lo, (void *)p->pstep_ptr, (void *)p->psteps})
         if (q) (void)hipFree(q);
     p->val = p->partial = nullptr;
     p->cf = p->prow = nullptr;
-    p->perm = p->tile_base = p->wg_tab = p->chunk_lo = nullptr;
+    p->perm = p->tile_base = p->wg_tab = p->chunk_lo = p->pstep_ptr = p->psteps = nullptr;
 }
 
 template <typename T>
@@ -479,6 +437,8 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
     int32_t *lrow = nullptr, *lhead = nullptr, *hscan = nullptr, *prow_full = nullptr;
     int32_t *d_pstart = nullptr, *d_tile_off = nullptr;
     void *tmp = nullptr;
+    int32_t *pack_tmp = nullptr;
+    void *pack_scan_tmp = nullptr;
     size_t tmp_sort = 0, tmp_scan = 0, tmp_bytes = 0;
     std::vector<int32_t> pstart((size_t)sm.nslices + 1), tile_off((size_t)sm.nslices + 1, 0);
     std::vector<int32_t> tab;
@@ -544,10 +504,10 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
         ASX_TRY(hipMemcpyAsync(&sm.npartials, hscan + (slots - 1), sizeof(int32_t), hipMemcpyDeviceToHost, s));
         ASX_TRY(hipStreamSynchronize(s));
         ASX_TRY(hipMalloc((void **)&sm.tile_base, sizeof(int32_t) * ((size_t)sm.ntiles + 1)));
-        ASX_TRY(hipMalloc((void **)&sm.prow, sizeof(uint16_t) * ((size_t)sm.npartials + kReducePad)));
-        ASX_TRY(hipMemsetAsync(sm.prow, 0, sizeof(uint16_t) * ((size_t)sm.npartials + kReducePad), s));
-        ASX_TRY(hipMalloc(&sm.partial, sizeof(T) * ((size_t)sm.npartials + kReducePad)));
-        ASX_TRY(hipMemsetAsync(sm.partial, 0, sizeof(T) * ((size_t)sm.npartials + kReducePad), s));
+        ASX_TRY(hipMalloc((void **)&sm.prow, sizeof(uint16_t) * ((size_t)sm.npartials + kSlicedReducePad)));
+        ASX_TRY(hipMemsetAsync(sm.prow, 0, sizeof(uint16_t) * ((size_t)sm.npartials + kSlicedReducePad), s));
+        ASX_TRY(hipMalloc(&sm.partial, sizeof(T) * ((size_t)sm.npartials + kSlicedReducePad)));
+        ASX_TRY(hipMemsetAsync(sm.partial, 0, sizeof(T) * ((size_t)sm.npartials + kSlicedReducePad), s));
         ASX_TRY(hipMalloc((void **)&sm.chunk_lo, sizeof(int32_t) * ((size_t)sm.nrb + 1) * (size_t)sm.nslices));
         hipLaunchKernelGGL(k_sliced_tile_base, dim3((unsigned)ceil_div64((int64_t)sm.ntiles + 1, kBlock)), dim3(kBlock),
                            0, s, hscan, sm.ntiles, sm.tile_base);
@@ -557,6 +517,27 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
         const int64_t nchunks = ((int64_t)sm.nrb + 1) * sm.nslices;
         hipLaunchKernelGGL(k_sliced_chunks, dim3((unsigned)ceil_div64(nchunks, kBlock)), dim3(kBlock), 0, s, prow_full,
                            sm.tile_base, d_tile_off, sm.nslices, sm.nrb, rows_per_wave, sm.chunk_lo);
+    }
+    // 4b. the steps in which pass 2 reads each row block's ranges
+    {
+        size_t scan_bytes = 0;
+        int32_t *cnt = nullptr;
+        ASX_TRY(hipMalloc((void **)&pack_tmp, sizeof(int32_t) * ((size_t)sm.nrb + 1)));
+        cnt = pack_tmp;
+        ASX_TRY(hipMalloc((void **)&sm.pstep_ptr, sizeof(int32_t) * ((size_t)sm.nrb + 1)));
+        ASX_TRY(hipMemsetAsync(cnt, 0, sizeof(int32_t) * ((size_t)sm.nrb + 1), s));
+        ASX_TRY(rocprim::exclusive_scan(nullptr, scan_bytes, cnt, sm.pstep_ptr, 0, (size_t)sm.nrb + 1, rocprim::plus<int32_t>(), s));
+        ASX_TRY(hipMalloc(&pack_scan_tmp, std::max<size_t>(scan_bytes, 256)));
+        const unsigned pgrid = (unsigned)ceil_div64(sm.nrb, kBlock);
+        hipLaunchKernelGGL(k_sliced_pack, dim3(pgrid), dim3(kBlock), 0, s, sm.chunk_lo, sm.nrb, sm.nslices, nullptr, cnt,
+                           nullptr);
+        ASX_TRY(rocprim::exclusive_scan(pack_scan_tmp, scan_bytes, cnt, sm.pstep_ptr, 0, (size_t)sm.nrb + 1, rocprim::plus<int32_t>(), s));
+        ASX_TRY(hipMemcpyAsync(&sm.npsteps, sm.pstep_ptr + sm.nrb, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+        ASX_TRY(hipStreamSynchronize(s));
+        ASX_TRY(hipMalloc((void **)&sm.psteps, sizeof(int32_t) * 4 * ((size_t)sm.npsteps + kSlicedStepPad)));
+        ASX_TRY(hipMemsetAsync(sm.psteps, 0, sizeof(int32_t) * 4 * ((size_t)sm.npsteps + kSlicedStepPad), s));
+        hipLaunchKernelGGL(k_sliced_pack, dim3(pgrid), dim3(kBlock), 0, s, sm.chunk_lo, sm.nrb, sm.nslices, sm.pstep_ptr,
+                           nullptr, reinterpret_cast<i32x4 *>(sm.psteps));
     }
     // 5. workgroups of pass 1: every slice gets its share of about `target_wgs` workgroups (at
     //    least one, and no workgroup smaller than 32 tiles unless the slice is), its tiles in equal
@@ -597,6 +578,8 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
 #undef ASX_TRY_ST
 done:
     if (arena) (void)hipFree(arena);
+    if (pack_tmp) (void)hipFree(pack_tmp);
+    if (pack_scan_tmp) (void)hipFree(pack_scan_tmp);
     if (st) {
         free_sliced(&sm);
         return st;
@@ -616,13 +599,14 @@ int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s)
 }
 
 template <typename T>
-int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, hipStream_t s)
+int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, T *partial,
+                       hipStream_t s)
 {
     if (m <= 0) return ASX_STATUS_SUCCESS;
-    T *partial = static_cast<T *>(sm->partial);
+    if (!partial) return ASX_STATUS_INVALID_POINTER;
     constexpr int kSmall = 65536 / sizeof(T), kLarge = 131072 / sizeof(T);
     const int4 *tab = reinterpret_cast<const int4 *>(sm->wg_tab);
-    constexpr int kDepth = 2;  // tiles in flight per wave (4 and 8 measured the same or slower)
+    constexpr int kDepth = 2;  // tiles in flight per wave (3 and 4 measured the same or slower)
 #define ASX_PROD(W)                                                                                                 \
     hipLaunchKernelGGL((k_sliced_products<T, W, 16, kDepth>), dim3((unsigned)sm->nwg), dim3(16 * kWave), 0, s, n, tab, \
                        sm->cf, (const T *)sm->val, sm->tile_base, x, partial)
@@ -635,27 +619,15 @@ int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, co
             return ASX_STATUS_INVALID_VALUE;
     }
 #undef ASX_PROD
-    constexpr int kWaves = 4;
-    if (sm->rows_per_wave < 1 || (size_t)sm->rows_per_wave * sizeof(T) > 16384) return ASX_STATUS_INVALID_VALUE;
-    const unsigned rgrid = (unsigned)(ceil_div64(ceil_div64(sm->nrb, kWaves), kXcds) * kXcds);
-    const size_t lds = (size_t)kWaves * sm->rows_per_wave * sizeof(T);
-    // fp32: plain LDS read-add-write (LDS float atomics measured 2.5x slower on scattered rows);
-    // fp64: LDS atomic adds (no dependent read in the wave's instruction stream; measured faster)
-    constexpr int kMode = sizeof(T) == 4 ? 1 : 0;
-    // entries per lane and step, from the mean number of partial sums a row block has in one slice
-    // (a step should be mostly full): 64-wide steps below 80, 128-wide below 160, else 256-wide (fp32)
-    const double mean_range = (double)sm->npartials / ((double)sm->nrb * (double)sm->nslices);
-    const int wide = mean_range < 80.0 ? 1 : (mean_range < 160.0 || sizeof(T) == 8) ? 2 : 4;
-#define ASX_RED(WW)                                                                                                   \
-    hipLaunchKernelGGL((k_sliced_reduce<T, kWaves, kMode, WW>), dim3(rgrid), dim3(kWaves * kWave), lds, s, m, sm->nrb, \
-                       sm->rows_per_wave, sm->nslices, alpha, beta, sm->chunk_lo, sm->prow, partial, y)
-    if (wide == 1)
-        ASX_RED(1);
-    else if (wide == 2)
-        ASX_RED(2);
-    else
-        ASX_RED(4);
-#undef ASX_RED
+    // steps per batch and batches in flight: 4 x 2 measured best (8 x 2, 4 x 4: the same or 1-3 % slower)
+    constexpr int kSteps = 4, kBatches = 2;
+    static_assert((kBatches + 1) * kSteps <= kSlicedStepPad, "descriptors are read this far past a block's last step");
+    const int32_t rw = sm->rows_per_wave;
+    const size_t lds = align_up(((size_t)rw + kWave) * sizeof(double), 16);
+    if (rw < 1 || rw > 32767 || lds > 65536) return ASX_STATUS_INVALID_VALUE;
+    const unsigned rgrid = (unsigned)(ceil_div64(sm->nrb, kXcds) * kXcds);
+    hipLaunchKernelGGL((k_sliced_reduce<T, kSteps, kBatches>), dim3(rgrid), dim3(kWave), lds, s, m, sm->nrb, rw, alpha, beta,
+                       sm->pstep_ptr, reinterpret_cast<const i32x4 *>(sm->psteps), sm->prow, partial, y);
     return check_launch();
 }
 
@@ -663,7 +635,7 @@ int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, co
     template int build_sliced<T>(int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, const int32_t *,          \
                                  const int32_t *, const T *, SlicedMatrix *, hipStream_t);                       \
     template int sliced_update_values<T>(const SlicedMatrix *, const T *, hipStream_t);                          \
-    template int launch_spmv_sliced<T>(int32_t, int32_t, T, const SlicedMatrix *, const T *, T, T *, hipStream_t);
+    template int launch_spmv_sliced<T>(int32_t, int32_t, T, const SlicedMatrix *, const T *, T, T *, T *, hipStream_t);
 ASX_INST(float)
 ASX_INST(double)
 #undef ASX_INST

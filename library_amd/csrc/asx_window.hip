@@ -766,6 +766,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
         chains.push_back(chain_lo);
         chains.push_back(wm.nblocks);
         wm.nchains = (int32_t)(chains.size() / 2);
+        wm.npieces = (int32_t)(pcs.size() / 4);
     }
     ASX_TRY(hipMalloc((void **)&wm.pieces, sizeof(int32_t) * pcs.size()));
     ASX_TRY(hipMemcpyAsync(wm.pieces, pcs.data(), sizeof(int32_t) * pcs.size(), hipMemcpyHostToDevice, s));
@@ -799,9 +800,11 @@ int window_update_values(const WindowMatrix *wm, const T *val, hipStream_t s)
 }
 
 template <typename T>
-int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, hipStream_t s)
+int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, T *carry,
+                       hipStream_t s)
 {
     if (m <= 0) return ASX_STATUS_SUCCESS;
+    if (wm->has_carry && !carry) return ASX_STATUS_INVALID_POINTER;
     // x on a 16-byte boundary (every allocation is) and at least one 16-byte unit long: 16-byte
     // fetches; else element by element
     const bool vec = ((uintptr_t)x % 16) == 0 && (size_t)n * sizeof(T) >= 16;
@@ -814,10 +817,10 @@ int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, co
     hipLaunchKernelGGL(kernel, dim3((unsigned)wm->nchains), dim3(kWindowWaves * kWave), 0, s, n, alpha, beta,
                        reinterpret_cast<const int2 *>(wm->chains), reinterpret_cast<const int4 *>(wm->blocks),
                        reinterpret_cast<const int4 *>(wm->pieces), wm->cf, (const T *)wm->val,
-                       reinterpret_cast<const int2 *>(wm->tile_info), x, y, (T *)wm->carry);
+                       reinterpret_cast<const int2 *>(wm->tile_info), x, y, carry);
     if (wm->has_carry)
         hipLaunchKernelGGL((k_window_fixup<T>), dim3((unsigned)ceil_div64(wm->ntiles, kBlock)), dim3(kBlock), 0, s,
-                           wm->ntiles, alpha, reinterpret_cast<const int2 *>(wm->tile_info), (const T *)wm->carry, y);
+                           wm->ntiles, alpha, reinterpret_cast<const int2 *>(wm->tile_info), (const T *)carry, y);
     return check_launch();
 }
 
@@ -825,7 +828,7 @@ int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, co
     template int build_window<T>(int32_t, int32_t, int32_t, int32_t, const int32_t *, const int32_t *, const T *, \
                                  WindowMatrix *, hipStream_t);                                                    \
     template int window_update_values<T>(const WindowMatrix *, const T *, hipStream_t);                           \
-    template int launch_spmv_window<T>(int32_t, int32_t, T, const WindowMatrix *, const T *, T, T *, hipStream_t);
+    template int launch_spmv_window<T>(int32_t, int32_t, T, const WindowMatrix *, const T *, T, T *, T *, hipStream_t);
 ASX_INST(float)
 ASX_INST(double)
 #undef ASX_INST

@@ -147,6 +147,47 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
             s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
         }
+        if (analysis == 4) {
+            // two handles, each on a stream of its own, multiply the one analysed descriptor at the
+            // same time, each call with its own buffer, sized after the analysis (it then holds the
+            // call's partial sums or carries when the analysis regrouped A): x -> y as before,
+            // x2 -> y2 (out2.bin)
+            auto x2 = read_bin<T>(dir + "/x2.bin", in_len);
+            T *d_x2 = to_device(x2), *d_y2 = to_device(yin);
+            alphasparseHandle_t h2 = nullptr;
+            if (alphasparseGetHandle(&h2) != ALPHA_SPARSE_STATUS_SUCCESS) return 4;
+            handle->stream = handle->streams[0];
+            h2->stream = h2->streams[0];
+            alphasparseDnVecDescr_t X2, Y2;
+            if (alphasparseCreateDnVec(&X2, in_len, d_x2, dt) || alphasparseCreateDnVec(&Y2, out_len, d_y2, dt)) return 6;
+            size_t nb = 0;
+            s = alphasparseSpMV_bufferSize(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, &nb);
+            if (s) return 10 + (int)s;
+            if (nb < bytes) return 8;
+            void *b1 = nullptr, *b2 = nullptr;
+            HIP_OK(hipMalloc(&b1, nb ? nb : 1));
+            HIP_OK(hipMalloc(&b2, nb ? nb : 1));
+            for (int rep = 0; rep < 6; ++rep) {
+                HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
+                HIP_OK(hipMemcpy(d_y2, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
+                s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, b1);
+                if (s) return 50 + (int)s;
+                s = alphasparseSpMV(h2, opA, &alpha, A, X2, &beta, Y2, dt, (alphasparseSpMVAlg_t)alg, b2);
+                if (s) return 50 + (int)s;
+                HIP_OK(hipStreamSynchronize(handle->stream));
+                HIP_OK(hipStreamSynchronize(h2->stream));
+            }
+            std::vector<T> out2(yin.size());
+            HIP_OK(hipMemcpy(out2.data(), d_y2, out2.size() * sizeof(T), hipMemcpyDeviceToHost));
+            FILE *f2 = std::fopen((dir + "/out2.bin").c_str(), "wb");
+            if (!f2 || std::fwrite(out2.data(), sizeof(T), out2.size(), f2) != out2.size()) return 9;
+            std::fclose(f2);
+            std::printf("buffer bytes before analysis %zu after %zu\n", bytes, nb);
+            alphasparseDestroyDnVec(X2);
+            alphasparseDestroyDnVec(Y2);
+            alphasparse_destory_handle(h2);
+            for (void *q : {(void *)b1, (void *)b2, (void *)d_x2, (void *)d_y2}) (void)hipFree(q);
+        }
         if (analysis && alphasparseSpMV_clear(handle, (alphasparseSpMVAlg_t)alg)) return 7;
         alphasparseDestroyDnVec(X);
         alphasparseDestroyDnVec(Y);

@@ -15,14 +15,16 @@ EXE = os.path.join(ROOT, "tests", "cxx", "generic_api_caller")
 
 
 def _run_case(tmp_path, op, dtype, rp, col, val, x, y, ncols, alg, alpha, beta, analysis, variant=(0, 0, 0, 0, 0),
-              n=None, val2=None, env=None):
+              n=None, val2=None, env=None, x2=None, tag=""):
     """variant = (trans_a, idx_base, col_major_b, col_major_c, trans_b); n = columns of A."""
-    d = tmp_path / f"{op}_{np.dtype(dtype).name}_{alg}_{analysis}_{''.join(map(str, variant))}{'_env' if env else ''}"
+    d = tmp_path / f"{op}_{np.dtype(dtype).name}_{alg}_{analysis}_{''.join(map(str, variant))}{'_env' if env else ''}{tag}"
     d.mkdir()
     for name, a in (("row_ptr", rp), ("col", col), ("val", val), ("x", x), ("y", y)):
         np.ascontiguousarray(a).tofile(d / f"{name}.bin")
     if val2 is not None:  # analysis == 2: values written over A's after the first products; 3: a second descriptor's
         np.ascontiguousarray(val2).tofile(d / "val2.bin")
+    if x2 is not None:  # analysis == 4: the second stream's input vector
+        np.ascontiguousarray(x2).tofile(d / "x2.bin")
     tag = "f64" if np.dtype(dtype) == np.float64 else "f32"
     if n is None:
         n = x.size // ncols
@@ -218,6 +220,37 @@ def test_spmv_analysis_on_a_scattered_matrix(tmp_path, oracle):
     ref_t = oracle.spmv(rp_t, col_t, val_t, y0, alpha, beta, x, 8)
     got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, y0, x, 1, 0, alpha, beta, 1, (1, 0, 0, 0, 0), n=n)
     assert_close(got, ref_t, spmv_scale(rp_t, col_t, val_t, y0, alpha, beta, x), np.float64, "transpose, DEFAULT with analysis")
+
+
+def test_two_streams_share_one_analysed_descriptor(tmp_path, oracle):
+    """Two handles, each on a stream of its own, call alphasparseSpMV on one analysed descriptor at
+    the same time, each with a buffer of its own sized by alphasparseSpMV_bufferSize after the
+    analysis (analysis = 4 in the caller program): both products must be the oracle's.  On the
+    scattered matrix the analysis keeps column slices, whose per-call partial sums then live in the
+    callers' buffers; on the band matrix with long rows it keeps row blocks with a carry pass."""
+    from library_amd import workloads as W
+    rng = np.random.default_rng(67)
+    rp, col, val = W.csr_zipf(1 << 20, 1 << 20, 20, 1.0, 5000, 0.01, np.float64, 9)
+    cases = [("scattered", rp, col, val, 1 << 20)]
+    m, offs = 100000, np.arange(-60, 61)  # a band of 121 diagonals, a fifth of it stored: rows of about 24
+    cols = np.arange(m)[:, None] + offs[None, :]
+    mask = (rng.random(cols.shape) < 0.2) & (cols >= 0) & (cols < m)
+    rp = np.zeros(m + 1, np.int32)
+    np.cumsum(mask.sum(1), out=rp[1:])
+    col = cols[mask].astype(np.int32)
+    cases.append(("band", rp, col, rng.uniform(-1, 1, col.size), m))
+    for name, rp, col, val, n in cases:
+        assert col.size >= 1 << 21, name
+        x = rng.uniform(-1, 1, n)
+        x2 = rng.uniform(-1, 1, n)
+        y0 = rng.uniform(-1, 1, rp.size - 1)
+        alpha, beta = 2.1, 3.2
+        got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, alpha, beta, 4, x2=x2, tag=name)
+        assert_close(got, oracle.spmv(rp, col, val, x, alpha, beta, y0, 8), spmv_scale(rp, col, val, x, alpha, beta, y0),
+                     np.float64, f"{name}: first stream")
+        got2 = np.fromfile(next(tmp_path.glob(f"spmv_float64_0_4_*{name}")) / "out2.bin", dtype=np.float64)
+        assert_close(got2, oracle.spmv(rp, col, val, x2, alpha, beta, y0, 8), spmv_scale(rp, col, val, x2, alpha, beta, y0),
+                     np.float64, f"{name}: second stream")
 
 
 def test_analysis_on_first_use(tmp_path, oracle):

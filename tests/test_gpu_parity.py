@@ -334,7 +334,7 @@ def test_spmm_padded_leading_dimensions_and_integers(torch, capi, oracle):
 # ------------------------------------------------------------------ benchmark configurations at full size
 def test_benchmark_configs_full_size(torch, capi, oracle):
     from library_amd import workloads as W
-    for name in ("uniform16_f32", "powerlaw_f64", "stencil5_f64"):
+    for name in ("uniform16_f32", "uniform16_f64", "powerlaw_f64", "stencil5_f64"):
         w = W.CONFIGS[name]()
         ref = oracle.spmv(w.row_ptr, w.col, w.val, w.x, w.alpha, w.beta, w.y, 16)
         scale = spmv_scale(w.row_ptr, w.col, w.val, w.x, w.alpha, w.beta, w.y)
@@ -348,18 +348,21 @@ def test_benchmark_configs_full_size(torch, capi, oracle):
             torch.cuda.synchronize()
             assert_close(y.cpu().numpy(), ref, scale, w.dtype, f"{name} alg={alg}")
             plan.destroy()
-        if name in ("powerlaw_f64", "uniform16_f32"):
+        if name in ("powerlaw_f64", "uniform16_f32", "uniform16_f64"):
             # plans that may look at columns and values: the column-sliced kernel, forced and as
             # DEFAULT's choice on these matrices (scattered columns; the choice is rule-based, so two
             # plan builds agree)
             across_plans = []
             for alg in (capi.SPMV_SLICED, capi.SPMV_DEFAULT, capi.SPMV_DEFAULT):
                 plan = capi.Plan(False, alg, w.val.dtype, w.m, w.n, w.nnz, d[0], col=d[1], val=d[2])
-                assert plan.alg == capi.SPMV_SLICED and plan.holds_values and plan.workspace_bytes == 0
+                assert plan.alg == capi.SPMV_SLICED and plan.holds_values
+                # the partial sums of a call: a workspace of this size, or the plan's own buffer
+                assert plan.workspace_bytes == (plan.info("partial_sums") + 256) * w.val.dtype.itemsize
                 outs = []
                 for rep in range(2):
                     y = dev(torch, w.y)
-                    capi.spmv(d[0], d[1], d[2], d[3], y, w.alpha, w.beta, alg=alg, plan=plan)
+                    capi.spmv(d[0], d[1], d[2], d[3], y, w.alpha, w.beta, alg=alg, plan=plan,
+                              workspace=None if rep == 0 else False)
                     torch.cuda.synchronize()
                     outs.append(y.cpu().numpy())
                     assert_close(outs[-1], ref, scale, w.dtype, f"{name} sliced alg={alg} rep={rep}")
@@ -374,7 +377,7 @@ def test_benchmark_configs_full_size(torch, capi, oracle):
             across_plans = []
             for alg in (capi.SPMV_WINDOW, capi.SPMV_DEFAULT):
                 plan = capi.Plan(False, alg, w.val.dtype, w.m, w.n, w.nnz, d[0], col=d[1], val=d[2])
-                assert plan.alg == capi.SPMV_WINDOW and plan.holds_values and plan.workspace_bytes == 0
+                assert plan.alg == capi.SPMV_WINDOW and plan.holds_values and plan.workspace_bytes == 0  # no row is cut
                 outs = []
                 for rep in range(2):
                     y = dev(torch, w.y)
@@ -691,7 +694,8 @@ def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
         y0 = rng.uniform(-1, 1, m).astype(dtype)
         d = [dev(torch, a) for a in (rp, col, val, x)]
         plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
-        assert plan.alg == capi.SPMV_WINDOW and plan.holds_values and plan.workspace_bytes == 0
+        assert plan.alg == capi.SPMV_WINDOW and plan.holds_values
+        assert plan.workspace_bytes == plan.info("carry_pass") * plan.info("tiles") * np.dtype(dtype).itemsize
         assert plan.info("bands") == 1 and plan.info("rows_per_block") % 256 == 0 and plan.info("tiles") > 0
         if name == "windows moving backwards":
             assert plan.info("chains") < -(-m // plan.info("rows_per_block")), "chains of several blocks expected"
@@ -817,7 +821,8 @@ def test_spmv_window_kernel_bands_of_diagonals(torch, capi, oracle, dtype):
         y0 = rng.uniform(-1, 1, m).astype(dtype)
         d = [dev(torch, a) for a in (rp, col, val, x)]
         plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
-        assert plan.alg == capi.SPMV_WINDOW and plan.holds_values and plan.workspace_bytes == 0
+        assert plan.alg == capi.SPMV_WINDOW and plan.holds_values
+        assert plan.workspace_bytes == plan.info("carry_pass") * plan.info("tiles") * np.dtype(dtype).itemsize
         assert 2 <= plan.info("bands") <= 4 and plan.info("slices") == -1, (name, plan.info("bands"))
         if name in ("stencil 7 points", "long rows"):  # rows of at most 16 are never cut by tiles
             assert plan.info("carry_pass") == (1 if name == "long rows" else 0), name
@@ -853,9 +858,9 @@ def test_sliced_and_window_calls_replay_in_a_hip_graph(torch, capi, oracle):
         y0 = rng.uniform(-1, 1, m)
         d = [dev(torch, a) for a in (rp, col, val, x)]
         plan = capi.Plan(False, alg, val.dtype, m, n, col.size, d[0], col=d[1], val=d[2])
-        assert plan.workspace_bytes == 0
+        ws = torch.empty(max(plan.workspace_bytes, 256), dtype=torch.uint8, device="cuda")  # no allocation while capturing
         y_eager = dev(torch, y0)
-        capi.spmv(d[0], d[1], d[2], d[3], y_eager, 1.5, 0.5, alg=alg, plan=plan)
+        capi.spmv(d[0], d[1], d[2], d[3], y_eager, 1.5, 0.5, alg=alg, plan=plan, workspace=ws)
         torch.cuda.synchronize()
         eager = y_eager.cpu().numpy()
         assert_close(eager, oracle.spmv(rp, col, val, x, 1.5, 0.5, y0, 2), spmv_scale(rp, col, val, x, 1.5, 0.5, y0),
@@ -866,7 +871,7 @@ def test_sliced_and_window_calls_replay_in_a_hip_graph(torch, capi, oracle):
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             with torch.cuda.graph(graph, stream=side):
-                capi.spmv(d[0], d[1], d[2], d[3], y, 1.5, 0.5, alg=alg, plan=plan)
+                capi.spmv(d[0], d[1], d[2], d[3], y, 1.5, 0.5, alg=alg, plan=plan, workspace=ws)
         torch.cuda.synchronize()
         for rep in range(3):
             y.copy_(dev(torch, y0))                      # eager work between the replays
@@ -876,6 +881,49 @@ def test_sliced_and_window_calls_replay_in_a_hip_graph(torch, capi, oracle):
             torch.cuda.synchronize()
             assert np.array_equal(y.cpu().numpy(), eager), f"alg {alg} replay {rep}"
         del graph
+        plan.destroy()
+
+
+def test_one_plan_two_streams_two_workspaces(torch, capi, oracle):
+    """Calls through one sliced (window) plan that each bring a workspace of plan.workspace_bytes keep
+    their partial sums (carries) apart: two streams run them at the same time on different x, and
+    both results are the oracle's.  After asx_plan_release_scratch a call without a workspace is
+    refused and one with a workspace still works."""
+    rng = np.random.default_rng(163)
+    lens = np.minimum(rng.zipf(1.5, 60000), 4000)
+    cases = [(capi.SPMV_SLICED, csr_from_lengths(lens, 120000, 11, np.float64), 120000),
+             (capi.SPMV_WINDOW, _banded_random(rng, 20000, 20000, 300, 0.05, np.float64, longrow=700), 20000)]
+    for alg, (rp, col, val), n in cases:
+        m = rp.size - 1
+        xs = [rng.uniform(-1, 1, n) for _ in range(2)]
+        y0 = rng.uniform(-1, 1, m)
+        refs = [oracle.spmv(rp, col, val, x, 1.5, 0.5, y0, 2) for x in xs]
+        scales = [spmv_scale(rp, col, val, x, 1.5, 0.5, y0) for x in xs]
+        d = [dev(torch, a) for a in (rp, col, val)]
+        dx = [dev(torch, x) for x in xs]
+        plan = capi.Plan(False, alg, val.dtype, m, n, col.size, d[0], col=d[1], val=d[2])
+        need = plan.workspace_bytes
+        assert need > 0 and capi.lib().asx_plan_own_scratch_bytes(plan.h) == need, alg
+        ws = [torch.empty(need, dtype=torch.uint8, device="cuda") for _ in range(2)]
+        streams = [torch.cuda.Stream() for _ in range(2)]
+        torch.cuda.synchronize()
+        for rep in range(5):
+            ys = [dev(torch, y0) for _ in range(2)]
+            torch.cuda.synchronize()
+            for k in range(2):
+                with torch.cuda.stream(streams[k]):
+                    capi.spmv(d[0], d[1], d[2], dx[k], ys[k], 1.5, 0.5, alg=alg, plan=plan, workspace=ws[k])
+            torch.cuda.synchronize()
+            for k in range(2):
+                assert_close(ys[k].cpu().numpy(), refs[k], scales[k], np.float64, f"alg {alg} rep {rep} stream {k}")
+        plan.release_scratch()
+        assert capi.lib().asx_plan_own_scratch_bytes(plan.h) == 0
+        y = dev(torch, y0)
+        with pytest.raises(capi.AsxError):
+            capi.spmv(d[0], d[1], d[2], dx[0], y, 1.5, 0.5, alg=alg, plan=plan, workspace=False)
+        capi.spmv(d[0], d[1], d[2], dx[0], y, 1.5, 0.5, alg=alg, plan=plan, workspace=ws[0])
+        torch.cuda.synchronize()
+        assert_close(y.cpu().numpy(), refs[0], scales[0], np.float64, f"alg {alg} after release")
         plan.destroy()
 
 
