@@ -266,6 +266,15 @@ class Plan:
         self.h = h
         self._keep = (row_ptr, col, val)  # keep alive
 
+    @classmethod
+    def adopt(cls, handle):
+        """A view of a plan made through the C-ABI directly; destroying it stays with the caller."""
+        p = cls.__new__(cls)
+        p.h = handle
+        p._keep = ()
+        p._owned = False
+        return p
+
     def block_stats(self):
         n, f = C.c_int64(0), C.c_double(0.0)
         _check(lib().asx_plan_block_stats(self.h, C.byref(n), C.byref(f)), "asx_plan_block_stats")
@@ -320,9 +329,9 @@ class Plan:
         return bool(lib().asx_plan_holds_values(self.h))
 
     def destroy(self):
-        if self.h:
+        if self.h and getattr(self, "_owned", True):
             lib().asx_plan_destroy(self.h)
-            self.h = None
+        self.h = None
 
     def __del__(self):
         try:

@@ -5,6 +5,8 @@ with tol = 1e-12 (fp64) / 1e-5 (fp32): the bound for a pure reordering of the ro
 import numpy as np
 import pytest
 
+import plan_check
+
 from conftest import analysis_shapes, csr_from_lengths, row_ptr_from_lengths
 
 pytestmark = pytest.mark.gpu
@@ -605,6 +607,7 @@ def test_spmv_sliced_kernel_shapes(torch, capi, oracle, dtype):
         d = [dev(torch, a) for a in (rp, col, val, x)]
         plan = capi.Plan(False, capi.SPMV_SLICED, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
         assert plan.alg == capi.SPMV_SLICED and plan.holds_values
+        plan_check.check_plan(plan, capi, rp, col, n, np.dtype(dtype).itemsize)
         for alpha, beta in ((1.5, 0.5), (1.0, 0.0), (-2.0, 1.0)):
             ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 2)
             scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
@@ -695,6 +698,7 @@ def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
         d = [dev(torch, a) for a in (rp, col, val, x)]
         plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
         assert plan.alg == capi.SPMV_WINDOW and plan.holds_values
+        plan_check.check_plan(plan, capi, rp, col, n, np.dtype(dtype).itemsize)
         assert plan.workspace_bytes == plan.info("carry_pass") * plan.info("tiles") * np.dtype(dtype).itemsize
         assert plan.info("bands") == 1 and plan.info("rows_per_block") % 256 == 0 and plan.info("tiles") > 0
         if name == "windows moving backwards":
@@ -740,6 +744,7 @@ def test_spmv_sliced_wide_steps(torch, capi, oracle):
         y0 = rng.uniform(-1, 1, m).astype(dtype)
         d = [dev(torch, a) for a in (rp, col, val, x)]
         plan = capi.Plan(False, capi.SPMV_SLICED, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
+        plan_check.check_plan(plan, capi, rp, col, n, np.dtype(dtype).itemsize)
         nrb = -(-m // plan.info("rows_per_wave"))
         mean_range = plan.info("partial_sums") / (nrb * plan.info("slices"))
         assert mean_range >= want, (mean_range, plan.info("rows_per_wave"), plan.info("slices"))
@@ -822,6 +827,7 @@ def test_spmv_window_kernel_bands_of_diagonals(torch, capi, oracle, dtype):
         d = [dev(torch, a) for a in (rp, col, val, x)]
         plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
         assert plan.alg == capi.SPMV_WINDOW and plan.holds_values
+        plan_check.check_plan(plan, capi, rp, col, n, np.dtype(dtype).itemsize)
         assert plan.workspace_bytes == plan.info("carry_pass") * plan.info("tiles") * np.dtype(dtype).itemsize
         assert 2 <= plan.info("bands") <= 4 and plan.info("slices") == -1, (name, plan.info("bands"))
         if name in ("stencil 7 points", "long rows"):  # rows of at most 16 are never cut by tiles
@@ -997,6 +1003,7 @@ def test_spmv_random_shapes_all_kernels(torch, capi, oracle):
             d = [dev(torch, a) for a in (rp, col, val, x)]
             y = dev(torch, y0)
             plan = capi.Plan(False, capi.SPMV_SLICED, np.dtype(dtype), rp.size - 1, ncols, col.size, d[0], col=d[1], val=d[2])
+            plan_check.check_plan(plan, capi, rp, col, ncols, np.dtype(dtype).itemsize)
             capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_SLICED, plan=plan)
             torch.cuda.synchronize()
             assert_close(y.cpu().numpy(), ref, scale, dtype, f"case {case} kind {kind} sliced")
@@ -1008,6 +1015,7 @@ def test_spmv_random_shapes_all_kernels(torch, capi, oracle):
                                                  capi._ptr(d[2]), None)
             assert rc in (0, 6), rc
             if rc == 0:
+                plan_check.check_plan(capi.Plan.adopt(h), capi, rp, col, ncols, np.dtype(dtype).itemsize)
                 y = dev(torch, y0)
                 fn = capi.lib().asx_spmv_csr_f64 if dtype == np.float64 else capi.lib().asx_spmv_csr_f32
                 assert fn(h, capi.SPMV_WINDOW, rp.size - 1, ncols, col.size, alpha, capi._ptr(d[0]), capi._ptr(d[1]),

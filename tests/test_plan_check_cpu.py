@@ -1,0 +1,177 @@
+"""The host-side plan checks (tests/plan_check.py) on plans built on the host from their definition:
+they accept those, and reject copies corrupted by hand in the ways that matter (the GPU tests run
+the same checks on the plans the library builds)."""
+import numpy as np
+import pytest
+
+import plan_check as pc
+from conftest import csr_from_lengths
+
+
+def _scattered(seed=5, m=3000, n=70000):
+    rng = np.random.default_rng(seed)
+    lens = np.r_[np.minimum(rng.zipf(1.7, m - 3), 900), 0, 1500, 0]
+    rp, col, _ = csr_from_lengths(lens, n, seed + 1, np.float64)
+    return rp, col, n
+
+
+@pytest.mark.parametrize("itemsize,width", [(8, 16384), (4, 32768)])
+def test_sliced_plan_from_its_definition_passes(itemsize, width):
+    rp, col, n = _scattered()
+    plan = pc.sliced_plan_arrays(rp, col, n, width, 256, itemsize)
+    pc.check_sliced(plan, rp, col, n, width, 256, itemsize)
+
+
+def test_sliced_corruptions_are_rejected():
+    rp, col, n = _scattered()
+    good = pc.sliced_plan_arrays(rp, col, n, 16384, 256, 8)
+    nslices = -(-n // 16384)
+
+    def corrupt(name, fn):
+        bad = {k: v.copy() for k, v in good.items()}
+        fn(bad)
+        with pytest.raises(pc.PlanError):
+            pc.check_sliced(bad, rp, col, n, 16384, 256, 8)
+
+    def dup_perm(p):  # one stored element placed twice, another not at all
+        real = np.nonzero(p["perm"] >= 0)[0]
+        p["perm"][real[10]] = p["perm"][real[11]]
+    corrupt("perm", dup_perm)
+
+    def swap_perm(p):  # still a permutation, but not the stable order
+        real = np.nonzero(p["perm"] >= 0)[0]
+        p["perm"][real[[20, 21]]] = p["perm"][real[[21, 20]]]
+    corrupt("order", swap_perm)
+
+    def range_off_by_one(p):
+        r = p["ranges"].reshape(-1, nslices)
+        b = int(np.nonzero(r[1:, 0] > r[:-1, 0])[0][1]) + 1
+        r[b, 0] += 1
+    corrupt("ranges", range_off_by_one)
+
+    def step_base(p):
+        p["steps"].reshape(-1, 4)[3, 0] += 1
+    corrupt("steps", step_base)
+
+    def step_count(p):  # a step that counts one entry fewer: a partial sum is never added
+        st = p["steps"].reshape(-1, 4)
+        j = int(np.nonzero((st[:, 3] >> 16) > 1)[0][0])
+        st[j, 3] -= 1 << 16
+    corrupt("step entries", step_count)
+
+    def flag(p):
+        p["cf"][5] ^= 0x8000
+    corrupt("run flag", flag)
+
+    def column(p):
+        p["cf"][7] ^= 1
+    corrupt("column", column)
+
+    def tile_base(p):
+        p["tile_words"][2] += 1
+    corrupt("tile_base", tile_base)
+
+    def partial_row(p):
+        p["partial_rows"][4] ^= 3
+    corrupt("partial row", partial_row)
+
+    def workgroups(p):  # a tile no workgroup of pass 1 multiplies
+        p["workgroups"].reshape(-1, 4)[0, 2] -= 1
+    corrupt("workgroups", workgroups)
+
+
+def _banded(seed, m, n, half, dens, cut_rows=True):
+    rng = np.random.default_rng(seed)
+    rows, cols = [], []
+    for r in range(m):
+        c = r * (n - 1) // max(m - 1, 1)
+        lo, hi = max(0, c - half), min(n, c + half + 1)
+        k = 0 if rng.random() < 0.1 else max(1, rng.binomial(hi - lo, dens))
+        if cut_rows and r % 97 == 0:
+            k = hi - lo
+        cs = np.sort(rng.choice(np.arange(lo, hi), size=min(k, hi - lo), replace=False))
+        rows.append(cs.size)
+        cols.append(cs)
+    rp = np.zeros(m + 1, np.int32)
+    np.cumsum(rows, out=rp[1:])
+    return rp, np.concatenate(cols).astype(np.int32)
+
+
+def _windows_moving_backwards(m=2048):
+    """Block b's columns lie below block b-1's: a chain may not continue into such a block."""
+    rng = np.random.default_rng(3)
+    R, per = 256, 5
+    rp = np.arange(m + 1, dtype=np.int32) * per
+    base = (m // R - 1 - np.arange(m) // R) * 1000  # later blocks reach lower columns
+    col = np.sort(base[:, None] + rng.integers(0, 900, (m, per)), axis=1).reshape(-1).astype(np.int32)
+    return rp, col, int(col.max()) + 1
+
+
+@pytest.mark.parametrize("itemsize", [8, 4])
+def test_window_plan_from_its_definition_passes(itemsize):
+    rp, col = _banded(11, 3000, 3000, 150, 0.05)
+    for tiles_per_chain in (1 << 30, 40):
+        plan = pc.window_plan_arrays(rp, col, 3000, 256, itemsize, tiles_per_chain)
+        assert (plan["tile_words"].reshape(-1, 2)[:, 0] < 0).any(), "the matrix should have rows cut by tile starts"
+        pc.check_window(plan, rp, col, 3000, 256, 1, itemsize)
+    rp, col, n = _windows_moving_backwards()
+    plan = pc.window_plan_arrays(rp, col, n, 256, itemsize)
+    assert plan["workgroups"].size // 2 == 8, "every block must have begun a chain of its own"
+    pc.check_window(plan, rp, col, n, 256, 1, itemsize)
+
+
+def test_window_corruptions_are_rejected():
+    # a chain that runs on into a block whose window starts below what the chain has fetched: the
+    # block's columns were never put into the ring
+    rp, col, n = _windows_moving_backwards()
+    bad = pc.window_plan_arrays(rp, col, n, 256, 8, fresh_check=False)
+    assert bad["workgroups"].size // 2 == 1
+    with pytest.raises(pc.PlanError, match="holds column"):
+        pc.check_window(bad, rp, col, n, 256, 1, 8)
+
+    rp, col = _banded(13, 3000, 3000, 150, 0.05)
+    good = pc.window_plan_arrays(rp, col, 3000, 256, 8, 40)
+
+    def corrupt(fn, match=None):
+        p = {k: v.copy() for k, v in good.items()}
+        fn(p)
+        with pytest.raises(pc.PlanError, match=match):
+            pc.check_window(p, rp, col, 3000, 256, 1, 8)
+
+    def dup_perm(p):
+        real = np.nonzero(p["perm"] >= 0)[0]
+        p["perm"][real[10]] = p["perm"][real[11]]
+    corrupt(dup_perm, "placed")
+
+    def first_piece_above(p):  # the first fetch of the second chain starts 64 columns late
+        ch = p["workgroups"].reshape(-1, 2)
+        b = int(ch[1, 0])
+        pcs = p["pieces"].reshape(-1, 4)
+        pcs[p["blocks"].reshape(-1, 4)[b, 2], 0] += 64
+    corrupt(first_piece_above, "holds column")
+
+    def lds_slot(p):
+        real = np.nonzero(pc.logical_order(p["perm"], 8) >= 0)[0]
+        p["cf"][real[100]] ^= 2
+    corrupt(lds_slot, "holds column")
+
+    def flag(p):
+        real = np.nonzero(pc.logical_order(p["perm"], 8) >= 0)[0]
+        p["cf"][real[100]] ^= 0x8000
+    corrupt(flag, "flag")
+
+    def tile_rows(p):  # a tile that claims one row fewer: that row would never be written
+        p["tile_words"].reshape(-1, 2)[3, 1] -= 1
+    corrupt(tile_rows)
+
+    def tile_first_row(p):
+        p["tile_words"].reshape(-1, 2)[3, 0] += 1
+    corrupt(tile_first_row)
+
+    def chain_gap(p):
+        p["workgroups"].reshape(-1, 2)[1, 0] += 1
+    corrupt(chain_gap, "chains")
+
+    def block_tiles(p):
+        p["blocks"].reshape(-1, 4)[2, 1] -= 1
+    corrupt(block_tiles)
