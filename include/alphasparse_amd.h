@@ -52,7 +52,8 @@ enum {
     ASX_SPMV_FLAT = 15,   /* tiles of 1024 stored elements, register walk + ordered carry fix-up */
     ASX_SPMV_SLICED = 101, /* not a reference id: stored elements regrouped by column slice, each slice of x
                              held in LDS; one partial sum per (row, slice), added per row by a second pass
-                             (needs a plan from asx_spmv_plan_create) */
+                             (needs a plan from asx_spmv_plan_create; NOT_SUPPORTED beyond 1024 slices of
+                             128 KiB of x: 16.7 M columns in fp64, 33.5 M in fp32) */
     ASX_SPMV_WINDOW = 102 /* not a reference id: chains of blocks of consecutive rows with a sliding window of x
                              in LDS and 16-bit columns, for matrices whose rows reach only nearby columns
                              (needs a plan from asx_spmv_plan_create; NOT_SUPPORTED when some 256 rows reach

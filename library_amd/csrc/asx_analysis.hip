@@ -244,6 +244,21 @@ __global__ __launch_bounds__(256) void k_copy16(const u32x4 *__restrict__ src, u
     for (; i < n16; i += stride) dst[i] = src[i];
 }
 
+// out[t * tile + i] = src[t * stride + i]: `samples` tiles of `tile` ints, one workgroup each
+__global__ __launch_bounds__(kBlock) void k_sample_tiles(const int32_t *__restrict__ src, int64_t stride, int32_t tile,
+                                                         int32_t *__restrict__ out)
+{
+    const int32_t *from = src + (int64_t)blockIdx.x * stride;
+    for (int32_t i = threadIdx.x; i < tile; i += blockDim.x) out[(int64_t)blockIdx.x * tile + i] = from[i];
+}
+int launch_sample_tiles(const int32_t *d_src, int64_t stride, int32_t tile, int32_t samples, int32_t *d_out,
+                        hipStream_t s)
+{
+    if (samples <= 0) return ASX_STATUS_SUCCESS;
+    hipLaunchKernelGGL(k_sample_tiles, dim3((unsigned)samples), dim3(kBlock), 0, s, d_src, stride, tile, d_out);
+    return check_launch();
+}
+
 int launch_copy_bytes(const void *d_src, void *d_dst, size_t bytes, hipStream_t s)
 {
     size_t n16 = bytes / 16;

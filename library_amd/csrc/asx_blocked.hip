@@ -15,7 +15,8 @@
 // The zero fill of a block is multiplied with real rows of B: a non-finite value in a row of B
 // that some row of the block does not reference reaches that row of C as NaN (0 * Inf), where a
 // row-wise kernel would not have read it.  As for any padded block format, B must be finite.
-#include <hipcub/hipcub.hpp>
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
 
 #include "asx_internal.hpp"
 
@@ -153,14 +154,14 @@ int build_blocked(int32_t m, int32_t k, int32_t nnz, const int32_t *row_ptr, con
         ASX_TRY(hipMalloc((void **)&idx2, sizeof(int32_t) * (size_t)nnz));
         ASX_TRY(hipMalloc((void **)&head, sizeof(int32_t) * (size_t)nnz));
         ASX_TRY(hipMalloc((void **)&block_of, sizeof(int32_t) * (size_t)nnz));
-        ASX_TRY(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_sort, keys, keys2, idx, idx2, nnz, 0, 64, s));
-        ASX_TRY(hipcub::DeviceScan::InclusiveSum(nullptr, tmp_scan, head, block_of, nnz, s));
+        ASX_TRY(rocprim::radix_sort_pairs(nullptr, tmp_sort, keys, keys2, idx, idx2, (size_t)nnz, 0u, (unsigned)64, s));
+        ASX_TRY(rocprim::inclusive_scan(nullptr, tmp_scan, head, block_of, (size_t)nnz, rocprim::plus<int32_t>(), s));
         tmp_bytes = tmp_sort > tmp_scan ? tmp_sort : tmp_scan;
         ASX_TRY(hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1));
         hipLaunchKernelGGL(k_block_keys, dim3(g_nnz), dim3(kBlock), 0, s, row_ptr, col, m, nnz, keys, idx);
-        ASX_TRY(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_sort, keys, keys2, idx, idx2, nnz, 0, 64, s));
+        ASX_TRY(rocprim::radix_sort_pairs(tmp, tmp_sort, keys, keys2, idx, idx2, (size_t)nnz, 0u, (unsigned)64, s));
         hipLaunchKernelGGL(k_block_heads, dim3(g_nnz), dim3(kBlock), 0, s, keys2, nnz, head);
-        ASX_TRY(hipcub::DeviceScan::InclusiveSum(tmp, tmp_scan, head, block_of, nnz, s));
+        ASX_TRY(rocprim::inclusive_scan(tmp, tmp_scan, head, block_of, (size_t)nnz, rocprim::plus<int32_t>(), s));
         ASX_TRY(hipMemcpyAsync(&nblocks, block_of + (nnz - 1), sizeof(int32_t), hipMemcpyDeviceToHost, s));
         ASX_TRY(hipStreamSynchronize(s));
     }

@@ -91,11 +91,14 @@ double sampled_line_spread(const int32_t *d_col, int32_t nnz, size_t sv, hipStre
     const int samples = (int)std::min<int64_t>(64, tiles);
     const int64_t stride = tiles / samples;
     std::vector<int32_t> h((size_t)samples * kFlatTile);
-    const size_t row_bytes = (size_t)kFlatTile * sizeof(int32_t);
-    if (hipMemcpy2DAsync(h.data(), row_bytes, d_col, (size_t)stride * row_bytes, row_bytes, (size_t)samples,
-                         hipMemcpyDeviceToHost, s) != hipSuccess ||
-        hipStreamSynchronize(s) != hipSuccess)
-        return 0.0;
+    // the sampled tiles, gathered on the device into one piece, then one plain copy
+    int32_t *d_sample = nullptr;
+    if (hipMalloc((void **)&d_sample, h.size() * sizeof(int32_t)) != hipSuccess) return 0.0;
+    const bool ok = launch_sample_tiles(d_col, stride * kFlatTile, kFlatTile, samples, d_sample, s) == ASX_STATUS_SUCCESS &&
+                    hipMemcpyAsync(h.data(), d_sample, h.size() * sizeof(int32_t), hipMemcpyDeviceToHost, s) == hipSuccess &&
+                    hipStreamSynchronize(s) == hipSuccess;
+    (void)hipFree(d_sample);
+    if (!ok) return 0.0;
     const int shift = sv == 8 ? 4 : 5;  // columns per 128-byte line of x
     int64_t distinct = 0;
     for (int t = 0; t < samples; ++t) {
@@ -588,6 +591,7 @@ static bool sliced_pays(const int64_t hist[33], int32_t m, int32_t n, int32_t nn
     const double row_bytes = (double)nnz * (sv + 4) + (double)n * sv + (double)m * (sv + 4);
     const double t_rows = std::max((double)nnz / gather_rate, row_bytes / 5e12);
     const int32_t nslices = (int32_t)ceil_div64((int64_t)n * (int64_t)sv, kSliceBytes);
+    if (nslices > kSlicedMaxSlices) return false;  // the plan build handles no more
     const double partials = sliced_expected_partials(hist, nslices);
     const double sl_bytes = (double)nnz * (sv + 2) + partials * (2.0 * sv + 2) + (double)n * sv + 2.0 * (double)m * sv;
     const double t_sliced = 12e-6 + sl_bytes / 4.7e12;

@@ -6,7 +6,7 @@
 //   asx_dense_transpose out[c][r] = in[r][c] for a strided dense matrix (column-major B and C of
 //                       SpMM; the reference: hip/format/transpose_dn_mat.h:4-35, one element per
 //                       thread with uncoalesced writes).
-#include <hipcub/hipcub.hpp>
+#include <rocprim/device/device_radix_sort.hpp>
 
 #include "asx_internal.hpp"
 
@@ -109,10 +109,10 @@ int csr_transpose(int32_t m, int32_t n, int32_t nnz, int32_t base, const int32_t
     ASX_TRY(hipMalloc((void **)&idx, sizeof(int32_t) * (size_t)nnz));
     ASX_TRY(hipMalloc((void **)&idx2, sizeof(int32_t) * (size_t)nnz));
     ASX_TRY(hipMalloc((void **)&trow, sizeof(int32_t) * (size_t)nnz));
-    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, keys, keys2, idx, idx2, nnz, 0, end_bit, s));
+    ASX_TRY(rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys, keys2, idx, idx2, (size_t)nnz, 0u, (unsigned)end_bit, s));
     ASX_TRY(hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1));
     hipLaunchKernelGGL(k_transpose_keys, dim3(grid), dim3(kBlock), 0, s, row_ptr, col, m, nnz, base, keys, idx);
-    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, keys, keys2, idx, idx2, nnz, 0, end_bit, s));
+    ASX_TRY(rocprim::radix_sort_pairs(tmp, tmp_bytes, keys, keys2, idx, idx2, (size_t)nnz, 0u, (unsigned)end_bit, s));
     hipLaunchKernelGGL((k_transpose_apply<T>), dim3(grid), dim3(kBlock), 0, s, keys2, idx2, val, nnz, trow, col_t,
                        val_t);
     hipLaunchKernelGGL(k_offsets_from_sorted, dim3((unsigned)ceil_div64((int64_t)n + 1, kBlock)), dim3(kBlock), 0, s,

@@ -1,7 +1,7 @@
 // COO -> CSR on the device: row offsets from sorted row indices, and the (row, column) sort
 // that callers run before it.  The reference does the first through hipSPARSE
 // (hip/format/coo2csr.h:7-16) and the second on the host with qsort (hip/format/coo_order.h:24-43).
-#include <hipcub/hipcub.hpp>
+#include <rocprim/device/device_radix_sort.hpp>
 
 #include "asx_internal.hpp"
 
@@ -69,10 +69,10 @@ int coo_sort(int32_t *row, int32_t *col, T *val, int32_t nnz, hipStream_t s)
     ASX_TRY(hipMalloc((void **)&idx, sizeof(int32_t) * (size_t)nnz));
     ASX_TRY(hipMalloc((void **)&idx2, sizeof(int32_t) * (size_t)nnz));
     ASX_TRY(hipMalloc((void **)&val2, sizeof(T) * (size_t)nnz));
-    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, keys, keys2, idx, idx2, nnz, 0, 64, s));
+    ASX_TRY(rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys, keys2, idx, idx2, (size_t)nnz, 0u, (unsigned)64, s));
     ASX_TRY(hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 1));
     hipLaunchKernelGGL(k_coo_keys, dim3(grid), dim3(kBlock), 0, s, row, col, nnz, keys, idx);
-    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, keys, keys2, idx, idx2, nnz, 0, 64, s));
+    ASX_TRY(rocprim::radix_sort_pairs(tmp, tmp_bytes, keys, keys2, idx, idx2, (size_t)nnz, 0u, (unsigned)64, s));
     ASX_TRY(hipMemcpyAsync(val2, val, sizeof(T) * (size_t)nnz, hipMemcpyDeviceToDevice, s));
     hipLaunchKernelGGL((k_coo_apply<T>), dim3(grid), dim3(kBlock), 0, s, keys2, idx2, val2, nnz, row, col, val);
     ASX_TRY(hipGetLastError());

@@ -52,6 +52,8 @@ int launch_loadbalance_partition(const int32_t *d_row_ptr, int32_t m, int32_t nn
 int launch_stream_row_blocks(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t *d_blocks,
                              hipStream_t s);
 int launch_copy_bytes(const void *d_src, void *d_dst, size_t bytes, hipStream_t s);
+int launch_sample_tiles(const int32_t *d_src, int64_t stride, int32_t tile, int32_t samples, int32_t *d_out,
+                        hipStream_t s);
 int launch_gather_lines(const void *d_buf, size_t bytes, int group_lanes, int per_lane, void *d_out, int *nthreads,
                         hipStream_t s);
 
@@ -123,6 +125,7 @@ int launch_offsets_from_sorted(const int32_t *sorted, int32_t count, int32_t n, 
 // its rows, slice after slice, into LDS accumulators and writes y.  The partial sums of one row
 // block inside one slice are a contiguous range (`chunk_lo`).
 constexpr int kSlicedTile = 256;  // stored elements per wave and step: 4 per lane
+constexpr int kSlicedMaxSlices = 1024;  // the plan build ranks stored elements by slice in LDS
 struct SlicedMatrix {
     int32_t width;          // columns per slice
     int32_t nslices;

@@ -24,14 +24,11 @@
 //
 // No global atomics; results are bit-reproducible.  The reference has no counterpart (its CSR
 // kernels gather x from global memory: hip/kernel/level2/alphasparse_spmv_csr_vector.h:99-126).
-#include <hipcub/hipcub.hpp>
-
-#include <rocprim/rocprim.hpp>
-
 #include <algorithm>
 #include <vector>
 
 #include "asx_internal.hpp"
+#include "asx_scan.hpp"
 #include "asx_tiles.hpp"
 
 namespace asx {
@@ -40,122 +37,322 @@ namespace {
 
 constexpr int32_t kPadRow = 0x7fffffff;
 
-__global__ __launch_bounds__(kBlock) void k_sliced_keys(const int32_t *__restrict__ col, int32_t nnz, int32_t width,
-                                                        int32_t *__restrict__ keys, int32_t *__restrict__ idx)
+// ---- plan build ---------------------------------------------------------------------------
+// The regrouping is a stable counting sort by slice, written for this purpose: the stored
+// elements are cut into blocks of kSortElems consecutive ones; a first kernel counts each block's
+// elements per slice; an exclusive scan over (slice, block) gives every block its place inside
+// every slice; a second kernel ranks the elements of a block inside their slices (stable: row
+// order, then column order, survives inside a slice), orders them by slice in LDS and writes
+// column, value, source index and row of each straight to its slot, in runs of consecutive slots.
+constexpr int kSortThreads = 512;
+constexpr int kSortWaves = kSortThreads / kWave;
+constexpr int kSortElems = 4096;  // per block
+constexpr int kSortPerLane = kSortElems / kSortThreads;
+constexpr int kSortWaveElems = kSortElems / kSortWaves;
+
+__global__ __launch_bounds__(kSortThreads) void k_sliced_count(const int32_t *__restrict__ col, int32_t nnz,
+                                                                int32_t width, int32_t nslices, int32_t nblocks,
+                                                                int32_t *__restrict__ counts)
 {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= nnz) return;
-    keys[i] = col[i] / width;
-    idx[i] = (int32_t)i;
+    __shared__ int32_t hist[kSlicedMaxSlices];
+    for (int s = threadIdx.x; s < nslices; s += kSortThreads) hist[s] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * kSortElems;
+#pragma unroll
+    for (int k = 0; k < kSortPerLane; ++k) {
+        const int64_t i = base + k * kSortThreads + threadIdx.x;
+        if (i < nnz) atomicAdd(&hist[col[i] / width], 1);  // integer counts: the order does not matter
+    }
+    __syncthreads();
+    for (int s = threadIdx.x; s < nslices; s += kSortThreads) counts[(int64_t)s * nblocks + blockIdx.x] = hist[s];
+    if (blockIdx.x == 0 && threadIdx.x == 0) counts[(int64_t)nslices * nblocks] = 0;
 }
 
-// srow[p] = row of A that holds stored element sidx[p]
-__global__ __launch_bounds__(kBlock) void k_sliced_rows(const int32_t *__restrict__ sidx, int32_t nnz,
-                                                        const int32_t *__restrict__ row_ptr, int32_t m,
-                                                        int32_t *__restrict__ srow)
+// pstart[s] = stored elements in slices before s (s = nslices: all of them)
+__global__ __launch_bounds__(kBlock) void k_sliced_slice_starts(const int32_t *__restrict__ offs, int32_t nslices,
+                                                                 int32_t nblocks, int32_t *__restrict__ pstart)
 {
-    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (p >= nnz) return;
-    const int32_t src = sidx[p];
-    int32_t lo = 0, hi = m;  // largest r with row_ptr[r] <= src
+    const int32_t s = (int32_t)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (s <= nslices) pstart[s] = offs[(int64_t)s * nblocks];
+}
+
+// largest r in [lo, hi] with row_ptr[r] <= i
+__device__ __forceinline__ int32_t row_holding(const int32_t *__restrict__ row_ptr, int32_t lo, int32_t hi, int32_t i)
+{
     while (lo < hi) {
         const int32_t mid = lo + (hi - lo + 1) / 2;
-        if (row_ptr[mid] <= src)
+        if (row_ptr[mid] <= i)
             lo = mid;
         else
             hi = mid - 1;
     }
-    srow[p] = lo;
+    return lo;
 }
 
-// Every slot of the padded element space starts as a pad: a run of its own with value 0 whose
-// partial sum no row block reads.
-template <typename T>
-__global__ __launch_bounds__(kBlock) void k_sliced_fill_pads(int64_t slots, int32_t *__restrict__ lrow,
-                                                             int32_t *__restrict__ lhead, uint16_t *__restrict__ cf,
-                                                             T *__restrict__ val, int32_t *__restrict__ perm)
+// in-place exclusive sum of a[0 .. n), n <= 2 * kSortThreads, by the whole workgroup (barriers inside)
+__device__ __forceinline__ void block_exclusive_sum(int32_t *a, int n, int32_t *wave_tot)
 {
-    const int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (d >= slots) return;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int32_t v0 = 2 * tid < n ? a[2 * tid] : 0, v1 = 2 * tid + 1 < n ? a[2 * tid + 1] : 0;
+    int32_t incl = v0 + v1;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int32_t t = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += t;
+    }
+    if (lane == kWave - 1) wave_tot[wave] = incl;
+    __syncthreads();
+    int32_t before = 0;
+    for (int w = 0; w < wave; ++w) before += wave_tot[w];
+    const int32_t excl = before + incl - (v0 + v1);
+    if (2 * tid < n) a[2 * tid] = excl;
+    if (2 * tid + 1 < n) a[2 * tid + 1] = excl + v0;
+    __syncthreads();
+}
+
+template <typename T>
+__device__ __forceinline__ int64_t slot_val_pos(int64_t d)
+{
+    return d / kSlicedTile * kSlicedTile + tile_val_pos<T>((int)(d % kSlicedTile));
+}
+
+// Run-start flags are not known here (they need the neighbours in slice order): cf gets the column
+// inside the slice, k_sliced_emit adds bit 15.
+template <typename T, int MAXS>
+__global__ __launch_bounds__(kSortThreads) void k_sliced_scatter(
+    const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col, const T *__restrict__ val,
+    const int32_t *__restrict__ seg_row, int32_t m, int32_t nnz, int32_t width, int32_t nslices, int32_t nbits,
+    int32_t nblocks, const int32_t *__restrict__ offs, const int32_t *__restrict__ tile_off, int32_t *__restrict__ lrow,
+    uint16_t *__restrict__ cf, T *__restrict__ val_out, int32_t *__restrict__ perm)
+{
+    __shared__ int32_t cnt[kSortWaves * MAXS];  // per wave and slice: count, then first rank of the wave's elements
+    __shared__ int32_t lofs[MAXS];              // per slice: the block's count, then its first position in slice order
+    __shared__ int32_t gbase[MAXS];             // per slice: slot of the block's first element of the slice
+    __shared__ int32_t wave_tot[kSortWaves];
+    __shared__ int32_t dest[kSortElems];        // slot of the element at each position of the block in slice order
+    __shared__ __align__(16) unsigned char stage_raw[kSortElems * 10];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    // consecutive blocks write neighbouring slots of every slice: keep them on one XCD, whose L2
+    // then merges their pieces of a cache line (the grid is a multiple of kXcds workgroups)
+    const int32_t per_xcd = (int32_t)gridDim.x / kXcds;
+    const int32_t b = ((int32_t)blockIdx.x % kXcds) * per_xcd + (int32_t)blockIdx.x / kXcds;
+    if (b >= nblocks) return;  // the whole workgroup leaves
+    for (int i = tid; i < kSortWaves * nslices; i += kSortThreads) cnt[i] = 0;
+    __syncthreads();
+    int32_t *mycnt = cnt + wave * nslices;
+    const int64_t wbase = (int64_t)b * kSortElems + (int64_t)wave * kSortWaveElems;
+    int32_t c[kSortPerLane], rk[kSortPerLane];
+#pragma unroll
+    for (int k = 0; k < kSortPerLane; ++k) {
+        const int64_t i = wbase + k * kWave + lane;
+        c[k] = i < nnz ? col[i] : 0;
+    }
+    // rank of every element among the wave's elements of its slice, in element order: the wave
+    // takes its elements 64 at a time; inside a step the lanes of one slice find each other by
+    // ballots over the bits of the slice number
+#pragma unroll
+    for (int k = 0; k < kSortPerLane; ++k) {
+        const bool valid = wbase + k * kWave + lane < nnz;
+        const int32_t key = c[k] / width;
+        unsigned long long same = __ballot(valid);
+        for (int bit = 0; bit < nbits; ++bit) {
+            const bool one = (key >> bit) & 1;
+            const unsigned long long bal = __ballot(one);
+            same &= one ? bal : ~bal;
+        }
+        const int below = lanes_below(same);  // lanes of this slice before this one
+        const int32_t prev = valid ? mycnt[key] : 0;
+        rk[k] = prev + below;
+        if (valid && below == 0) mycnt[key] = prev + __popcll(same);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+    for (int s = tid; s < nslices; s += kSortThreads) {
+        int32_t run = 0;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; ++w) {
+            const int32_t t = cnt[w * nslices + s];
+            cnt[w * nslices + s] = run;
+            run += t;
+        }
+        lofs[s] = run;
+        gbase[s] = tile_off[s] * kSlicedTile + offs[(int64_t)s * nblocks + b] - offs[(int64_t)s * nblocks];
+    }
+    __syncthreads();
+    block_exclusive_sum(lofs, nslices, wave_tot);
+    // rows: the wave's 512 elements lie in rows seg_row[g] .. seg_row[g + 1]
+    const int64_t g = wbase / kSortWaveElems;
+    int32_t r_lo = 0, r_hi = m - 1;
+    if (wbase < nnz) {
+        r_lo = seg_row[g];
+        r_hi = seg_row[g + 1];
+        r_hi = r_hi > m - 1 ? m - 1 : r_hi;
+    }
+    int32_t *row_s = reinterpret_cast<int32_t *>(stage_raw), *src_s = row_s + kSortElems;
+#pragma unroll
+    for (int k = 0; k < kSortPerLane; ++k) {
+        const int64_t i = wbase + k * kWave + lane;
+        if (i < nnz) {
+            const int32_t key = c[k] / width;
+            const int32_t in_slice = mycnt[key] + rk[k];
+            const int32_t p = lofs[key] + in_slice;
+            rk[k] = p;
+            dest[p] = gbase[key] + in_slice;
+            row_s[p] = row_holding(row_ptr, r_lo, r_hi, (int32_t)i);
+            src_s[p] = (int32_t)i;
+        }
+    }
+    __syncthreads();
+    const int64_t left = (int64_t)nnz - (int64_t)b * kSortElems;
+    const int32_t count = left < kSortElems ? (int32_t)left : kSortElems;
+    for (int j = tid; j < count; j += kSortThreads) {
+        const int64_t d = dest[j];
+        lrow[d] = row_s[j];
+        perm[slot_val_pos<T>(d)] = src_s[j];
+    }
+    __syncthreads();
+    T *val_s = reinterpret_cast<T *>(stage_raw);
+    uint16_t *cf_s = reinterpret_cast<uint16_t *>(stage_raw + (size_t)kSortElems * 8);
+    T v[kSortPerLane];
+#pragma unroll
+    for (int k = 0; k < kSortPerLane; ++k) {
+        const int64_t i = wbase + k * kWave + lane;
+        v[k] = i < nnz ? val[i] : T(0);
+    }
+#pragma unroll
+    for (int k = 0; k < kSortPerLane; ++k) {
+        if (wbase + k * kWave + lane < nnz) {
+            val_s[rk[k]] = v[k];
+            cf_s[rk[k]] = (uint16_t)(c[k] % width);
+        }
+    }
+    __syncthreads();
+    for (int j = tid; j < count; j += kSortThreads) {
+        const int64_t d = dest[j];
+        val_out[slot_val_pos<T>(d)] = val_s[j];
+        cf[d] = cf_s[j];
+    }
+}
+
+// The slots behind a slice's last stored element, up to the end of its last tile, are pads: runs
+// of their own with value 0 whose partial sums no row block reads.  One workgroup per slice.
+template <typename T>
+__global__ __launch_bounds__(kSlicedTile) void k_sliced_pads(const int32_t *__restrict__ pstart,
+                                                              const int32_t *__restrict__ tile_off,
+                                                              int32_t *__restrict__ lrow, uint16_t *__restrict__ cf,
+                                                              T *__restrict__ val, int32_t *__restrict__ perm)
+{
+    const int32_t s = blockIdx.x;
+    const int64_t d = (int64_t)tile_off[s] * kSlicedTile + (pstart[s + 1] - pstart[s]) + threadIdx.x;
+    if (d >= (int64_t)tile_off[s + 1] * kSlicedTile) return;
     lrow[d] = kPadRow;
-    lhead[d] = 1;
     cf[d] = 0x8000u;
-    val[d] = T(0);
-    perm[d] = -1;
+    val[slot_val_pos<T>(d)] = T(0);
+    perm[slot_val_pos<T>(d)] = -1;
 }
 
-template <typename T>
-__global__ __launch_bounds__(kBlock) void k_sliced_place(const int32_t *__restrict__ skey, const int32_t *__restrict__ sidx,
-                                                         const int32_t *__restrict__ srow, int32_t nnz, int32_t width,
-                                                         const int32_t *__restrict__ pstart,
-                                                         const int32_t *__restrict__ tile_off,
-                                                         const int32_t *__restrict__ col, const T *__restrict__ val,
-                                                         int32_t *__restrict__ lrow, int32_t *__restrict__ lhead,
-                                                         uint16_t *__restrict__ cf, T *__restrict__ val_out,
-                                                         int32_t *__restrict__ perm)
+// Run starts of a tile (one wave per tile, 4 consecutive slots per lane): a slot starts a run if
+// it is the tile's first, if its row differs from the slot before it, or if it is a pad.
+struct TileRuns {
+    int32_t r[4];
+    bool h[4];
+    int before;  // run starts in the lanes below
+    int total;
+    __device__ __forceinline__ void load(const int32_t *__restrict__ lrow, int64_t t, int lane)
+    {
+        const int4 q = reinterpret_cast<const int4 *>(lrow + t * kSlicedTile)[lane];
+        r[0] = q.x, r[1] = q.y, r[2] = q.z, r[3] = q.w;
+        const int32_t prev = __shfl_up(q.w, 1, kWave);
+        h[0] = lane == 0 || r[0] != prev || r[0] == kPadRow;
+#pragma unroll
+        for (int j = 1; j < 4; ++j) h[j] = r[j] != r[j - 1] || r[j] == kPadRow;
+        const unsigned long long m0 = __ballot(h[0]), m1 = __ballot(h[1]), m2 = __ballot(h[2]), m3 = __ballot(h[3]);
+        before = lanes_below(m0) + lanes_below(m1) + lanes_below(m2) + lanes_below(m3);
+        total = __popcll(m0) + __popcll(m1) + __popcll(m2) + __popcll(m3);
+    }
+};
+
+__global__ __launch_bounds__(kBlock) void k_sliced_tile_runs(const int32_t *__restrict__ lrow, int32_t ntiles,
+                                                              int32_t *__restrict__ tile_cnt)
 {
-    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (p >= nnz) return;
-    const int32_t sl = skey[p];
-    const int32_t q = (int32_t)(p - pstart[sl]);
-    const int64_t d = (int64_t)tile_off[sl] * kSlicedTile + q;
-    const int32_t src = sidx[p];
-    const int32_t row = srow[p];
-    const bool head = (q % kSlicedTile) == 0 || srow[p - 1] != row;
-    lrow[d] = row;
-    lhead[d] = head ? 1 : 0;
-    cf[d] = (uint16_t)((col[src] - sl * width) | (head ? 0x8000 : 0));
-    const int64_t t = d / kSlicedTile;
-    const int64_t phys = t * kSlicedTile + tile_val_pos<T>((int)(d % kSlicedTile));
-    val_out[phys] = val[src];
-    perm[phys] = src;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t t = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+    if (t >= ntiles) return;  // whole waves leave
+    TileRuns tr;
+    tr.load(lrow, t, lane);
+    if (lane == 0) tile_cnt[t] = tr.total;
+    if (t == 0 && lane == 0) tile_cnt[ntiles] = 0;
 }
 
-__global__ __launch_bounds__(kBlock) void k_sliced_tile_base(const int32_t *__restrict__ hscan, int32_t ntiles,
-                                                             int32_t *__restrict__ tile_base)
+// Per run: its row inside the row block (prow); per slot: the run-start bit of cf; per (row
+// block, slice): the first partial sum of the block in the slice (chunk_lo), written by the run
+// that is the first at or past the block's first row - and, behind a slice's last stored element,
+// for all the blocks that follow.
+__global__ __launch_bounds__(kBlock) void k_sliced_emit(const int32_t *__restrict__ lrow,
+                                                         const int32_t *__restrict__ tile_base,
+                                                         const int32_t *__restrict__ tile_off, int32_t ntiles,
+                                                         int32_t nslices, int32_t rpw, int32_t nrb,
+                                                         uint16_t *__restrict__ cf, uint16_t *__restrict__ prow,
+                                                         int32_t *__restrict__ chunk_lo)
 {
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t > ntiles) return;
-    tile_base[t] = t < ntiles ? hscan[t * kSlicedTile] - 1 : hscan[(int64_t)ntiles * kSlicedTile - 1];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t t = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+    if (t >= ntiles) return;  // whole waves leave
+    int32_t lo = 0, hi = nslices - 1;  // slice of tile t: largest s with tile_off[s] <= t (uniform)
+    while (lo < hi) {
+        const int32_t mid = lo + (hi - lo + 1) / 2;
+        if (tile_off[mid] <= t)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    const int32_t s = lo;
+    const bool first_tile = t == tile_off[s], last_tile = t + 1 == tile_off[s + 1];
+    TileRuns tr;
+    tr.load(lrow, t, lane);
+    const int32_t base = tile_base[t];
+    // row of the slot before the lane's first one (-1: none in this slice)
+    int32_t prev = __shfl_up(tr.r[3], 1, kWave);
+    if (lane == 0) prev = first_tile ? -1 : lrow[t * kSlicedTile - 1];
+    // row of the slot behind the lane's last one (a pad, if the slice ends there)
+    int32_t next = __shfl_down(tr.r[0], 1, kWave);
+    if (lane == kWave - 1) next = last_tile ? kPadRow : lrow[(t + 1) * kSlicedTile];
+    typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+    u16x4 *cfp = reinterpret_cast<u16x4 *>(cf + t * kSlicedTile) + lane;
+    u16x4 w = *cfp;
+    int id = base + tr.before - 1;  // run the slot before the lane's first one belongs to
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int32_t r = tr.r[j];
+        const int32_t before = j == 0 ? prev : tr.r[j - 1];
+        const int32_t after = j == 3 ? next : tr.r[j + 1];
+        if (tr.h[j]) {
+            ++id;
+            w[j] |= 0x8000u;
+            // bit 15: may continue the row of the partial sum before it (a run cut at a tile start)
+            const bool cont = lane == 0 && j == 0 && before == r && r != kPadRow;
+            prow[id] = (uint16_t)((r % rpw) | (cont ? 0x8000 : 0));
+            if (r != kPadRow) {
+                const int32_t rb = r / rpw;
+                for (int32_t q = before < 0 ? 0 : before / rpw + 1; q <= rb; ++q) chunk_lo[(int64_t)q * nslices + s] = id;
+            }
+        }
+        if (r != kPadRow && after == kPadRow)  // the slice's last stored element
+            for (int32_t q = r / rpw + 1; q <= nrb; ++q) chunk_lo[(int64_t)q * nslices + s] = id + 1;
+    }
+    *cfp = w;
 }
 
-__global__ __launch_bounds__(kBlock) void k_sliced_partial_rows(const int32_t *__restrict__ lrow,
-                                                                const int32_t *__restrict__ lhead,
-                                                                const int32_t *__restrict__ hscan, int64_t slots,
-                                                                int32_t rows_per_wave, int32_t *__restrict__ prow_full,
-                                                                uint16_t *__restrict__ prow)
-{
-    const int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (d >= slots || !lhead[d]) return;
-    const int32_t id = hscan[d] - 1;
-    const int32_t r = lrow[d];
-    prow_full[id] = r;
-    // bit 15: this partial sum may belong to the same row as the one before it (a run cut at a tile
-    // start); pass 2 must not add the two with one read-modify-write
-    const bool cont = d > 0 && d % kSlicedTile == 0 && lrow[d - 1] == r;
-    prow[id] = (uint16_t)((r % rows_per_wave) | (cont ? 0x8000 : 0));
-}
-
-// chunk_lo[b * nslices + s] = first partial sum of slice s whose row is >= b * rows_per_wave
-__global__ __launch_bounds__(kBlock) void k_sliced_chunks(const int32_t *__restrict__ prow_full,
-                                                          const int32_t *__restrict__ tile_base,
-                                                          const int32_t *__restrict__ tile_off, int32_t nslices,
-                                                          int32_t nrb, int32_t rows_per_wave,
-                                                          int32_t *__restrict__ chunk_lo)
+// slices without stored elements: every row block's range is empty
+__global__ __launch_bounds__(kBlock) void k_sliced_empty_slices(const int32_t *__restrict__ tile_base,
+                                                                 const int32_t *__restrict__ tile_off, int32_t nslices,
+                                                                 int32_t nrb, int32_t *__restrict__ chunk_lo)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= ((int64_t)nrb + 1) * nslices) return;
-    const int32_t b = (int32_t)(i / nslices), sl = (int32_t)(i % nslices);
-    const int64_t target = (int64_t)b * rows_per_wave;
-    int32_t lo = tile_base[tile_off[sl]], hi = tile_base[tile_off[sl + 1]];
-    while (lo < hi) {
-        const int32_t mid = lo + (hi - lo) / 2;
-        if ((int64_t)prow_full[mid] < target)
-            lo = mid + 1;
-        else
-            hi = mid;
-    }
-    chunk_lo[i] = lo;
+    const int32_t s = (int32_t)(i % nslices);
+    if (tile_off[s] == tile_off[s + 1]) chunk_lo[i] = tile_base[tile_off[s]];
 }
 
 template <typename T>
@@ -167,6 +364,7 @@ __global__ __launch_bounds__(kBlock) void k_sliced_regather(const int32_t *__res
     const int32_t src = perm[d];
     val_out[d] = src >= 0 ? val[src] : T(0);
 }
+
 
 // ---- pass 1 ------------------------------------------------------------------------------
 // A run's sum goes, at the run's rank, into the wave's staging area in LDS; the tile's sums then
@@ -240,41 +438,56 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const 
 constexpr int kPieces = 3;
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 
-// One thread per row block walks the block's ranges; `psteps == nullptr`: only count.
+// One wave per row block walks the block's ranges (loaded 64 slices at a time, then read lane by
+// lane: the walk itself is serial); `psteps == nullptr`: only count.
 __global__ __launch_bounds__(kBlock) void k_sliced_pack(const int32_t *__restrict__ chunk_lo, int32_t nrb,
                                                          int32_t nslices, const int32_t *__restrict__ pstep_ptr,
                                                          int32_t *__restrict__ count, i32x4 *__restrict__ psteps)
 {
-    const int32_t b = (int32_t)(blockIdx.x * blockDim.x + threadIdx.x);
-    if (b >= nrb) return;
-    const int32_t *lo_row = chunk_lo + (int64_t)b * nslices, *hi_row = lo_row + nslices;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t b = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+    if (b >= nrb) return;  // whole waves leave
+    const int32_t *lo_row = chunk_lo + b * nslices, *hi_row = lo_row + nslices;
     i32x4 *out = psteps ? psteps + pstep_ptr[b] : nullptr;
     int32_t nsteps = 0, fill = 0, pieces = 0;
-    int32_t base[kPieces] = {0, 0, 0}, first[kPieces] = {0, kWave, kWave};
-    for (int32_t sl = 0; sl < nslices; ++sl) {
-        int32_t lo = lo_row[sl], len = hi_row[sl] - lo;
-        while (len > 0) {
-            if (pieces == kPieces || fill == kWave) {
-                if (out) out[nsteps] = i32x4{base[0], base[1], base[2], first[1] | first[2] << 8 | fill << 16};
-                ++nsteps;
-                fill = pieces = 0;
-                first[1] = first[2] = kWave;
+    int32_t base0 = 0, base1 = 0, base2 = 0, first1 = kWave, first2 = kWave;
+    for (int32_t s0 = 0; s0 < nslices; s0 += kWave) {
+        const int32_t ns = nslices - s0 < kWave ? nslices - s0 : kWave;
+        const int32_t lo_v = lane < ns ? lo_row[s0 + lane] : 0;
+        const int32_t len_v = lane < ns ? hi_row[s0 + lane] - lo_v : 0;
+        unsigned long long todo = __ballot(len_v > 0);
+        while (todo) {  // uniform
+            const int j = __builtin_ctzll(todo);
+            todo &= todo - 1;
+            int32_t lo = __builtin_amdgcn_readlane(lo_v, j), len = __builtin_amdgcn_readlane(len_v, j);
+            while (len > 0) {
+                if (pieces == kPieces || fill == kWave) {
+                    if (out && lane == 0) out[nsteps] = i32x4{base0, base1, base2, first1 | first2 << 8 | fill << 16};
+                    ++nsteps;
+                    fill = pieces = 0;
+                    first1 = first2 = kWave;
+                }
+                const int32_t take = len < kWave - fill ? len : kWave - fill;
+                if (pieces == 0)
+                    base0 = lo - fill;
+                else if (pieces == 1)
+                    base1 = lo - fill, first1 = fill;
+                else
+                    base2 = lo - fill, first2 = fill;
+                ++pieces;
+                fill += take;
+                lo += take;
+                len -= take;
             }
-            const int32_t take = len < kWave - fill ? len : kWave - fill;
-            base[pieces] = lo - fill;
-            first[pieces] = fill;
-            ++pieces;
-            fill += take;
-            lo += take;
-            len -= take;
         }
     }
     if (fill > 0) {
-        if (out) out[nsteps] = i32x4{base[0], base[1], base[2], first[1] | first[2] << 8 | fill << 16};
+        if (out && lane == 0) out[nsteps] = i32x4{base0, base1, base2, first1 | first2 << 8 | fill << 16};
         ++nsteps;
     }
-    if (!psteps) count[b] = nsteps;
+    if (!psteps && lane == 0) count[b] = nsteps;
 }
+
 
 // U steps whose loads are issued together.
 template <typename T, int U>
@@ -413,41 +626,35 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
 {
     SlicedMatrix sm{};
     if (m <= 0 || nnz <= 0 || n <= 0) return ASX_STATUS_INVALID_SIZE;
-    if (width < 1 || width > 32768 || rows_per_wave < 1 || rows_per_wave > 65536 || target_wgs < 1)
+    if (width < 1 || width > 32768 || rows_per_wave < 1 || rows_per_wave > 32767 || target_wgs < 1)
         return ASX_STATUS_INVALID_VALUE;
     sm.width = width;
     sm.nslices = (int32_t)ceil_div64(n, width);
+    if (sm.nslices > kSlicedMaxSlices) return ASX_STATUS_NOT_SUPPORTED;
     sm.rows_per_wave = rows_per_wave;
     sm.nrb = (int32_t)ceil_div64(m, rows_per_wave);
-    int key_bits = 1;
-    while ((1 << key_bits) < sm.nslices) ++key_bits;
+    int nbits = 0;
+    while ((1 << nbits) < sm.nslices) ++nbits;
+    const int32_t nblocks = (int32_t)ceil_div64(nnz, kSortElems);
+    const int32_t nseg = (int32_t)ceil_div64(nnz, kSortWaveElems);
+    const int64_t ncount = (int64_t)sm.nslices * nblocks + 1;
+    const int64_t cap64 = (int64_t)nnz + (int64_t)(kSlicedTile - 1) * sm.nslices;  // the most slots there can be
+    const int64_t ncells = ((int64_t)sm.nrb + 1) * sm.nslices;
+    if (cap64 > 0x7fffffff || ncount > 0x7fffffff || ncells > 0x7fffffff) return ASX_STATUS_INVALID_SIZE;
 
     int st = ASX_STATUS_SUCCESS;
-    // Scratch of the build, in one allocation (every hipMalloc / hipFree of this size costs a
-    // fraction of a millisecond): five arrays of `cap` ints, cap = the most slots there can be
-    // (every slice padded to whole tiles), used in turn as
-    //   a: sort keys in, then row of each sorted element, then (after the placing) the scan of run starts
-    //   b: sorted keys = slice of each sorted element, then (after the placing) the row of each partial sum
-    //   c: sort values in, then row of each slot
-    //   d: sorted values = position in A of each sorted element
-    //   e: run-start flag of each slot
-    // followed by the slice offsets (elements, tiles) and the sort / scan workspace.
-    int32_t *arena = nullptr;
-    int32_t *a = nullptr, *b = nullptr, *c = nullptr, *d = nullptr, *e = nullptr;
-    int32_t *lrow = nullptr, *lhead = nullptr, *hscan = nullptr, *prow_full = nullptr;
-    int32_t *d_pstart = nullptr, *d_tile_off = nullptr;
-    void *tmp = nullptr;
-    int32_t *pack_tmp = nullptr;
-    void *pack_scan_tmp = nullptr;
-    size_t tmp_sort = 0, tmp_scan = 0, tmp_bytes = 0;
+    // Scratch of the build in one allocation: per-(slice, block) counts and their scan, the row
+    // holding every 512th stored element, slice offsets (elements, tiles), the row of every slot,
+    // per-tile and per-row-block counts, the scans' block sums.
+    char *arena = nullptr;
+    int32_t *counts = nullptr, *offs = nullptr, *seg_row = nullptr, *d_pstart = nullptr, *d_tile_off = nullptr;
+    int32_t *lrow = nullptr, *tile_cnt = nullptr, *step_cnt = nullptr;
+    int32_t *tmp = nullptr;
     std::vector<int32_t> pstart((size_t)sm.nslices + 1), tile_off((size_t)sm.nslices + 1, 0);
     std::vector<int32_t> tab;
     int64_t slots = 0;
-    const unsigned grid = (unsigned)ceil_div64(nnz, kBlock);
-    const int64_t cap64 = (int64_t)nnz + (int64_t)(kSlicedTile - 1) * sm.nslices;
-    if (cap64 > 0x7fffffff) return ASX_STATUS_INVALID_SIZE;
-    const size_t cap = ((size_t)cap64 + 63) & ~(size_t)63;
-    const size_t noff = ((size_t)sm.nslices + 1 + 63) & ~(size_t)63;
+    bool empty_slice = false;
+    const size_t max_tiles = (size_t)ceil_div64(cap64, kSlicedTile);
 #define ASX_TRY(expr)         \
     do {                      \
         st = status_of(expr); \
@@ -458,88 +665,94 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
         st = (expr);       \
         if (st) goto done; \
     } while (0)
-    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_sort, a, b, c, d, nnz, 0, key_bits, s));
-    ASX_TRY(hipcub::DeviceScan::InclusiveSum(nullptr, tmp_scan, lhead, hscan, (int)cap64, s));
-    tmp_bytes = std::max<size_t>(std::max(tmp_sort, tmp_scan), 256);
-    ASX_TRY(hipMalloc((void **)&arena, sizeof(int32_t) * (5 * cap + 2 * noff) + tmp_bytes));
-    a = arena, b = a + cap, c = b + cap, d = c + cap, e = d + cap;
-    d_pstart = e + cap;
-    d_tile_off = d_pstart + noff;
-    tmp = d_tile_off + noff;
+    {
+        size_t off = 0;
+        const auto take = [&off](size_t count) {
+            const size_t at = off;
+            off += align_up(count * sizeof(int32_t), 256);
+            return at;
+        };
+        const size_t o_counts = take((size_t)ncount), o_offs = take((size_t)ncount), o_seg = take((size_t)nseg + 1);
+        const size_t o_pstart = take((size_t)sm.nslices + 1), o_toff = take((size_t)sm.nslices + 1);
+        const size_t o_lrow = take((size_t)cap64), o_tcnt = take(max_tiles + 1), o_scnt = take((size_t)sm.nrb + 1);
+        const size_t o_tmp = take(scan_scratch_ints(std::max<int64_t>(ncount, (int64_t)max_tiles + 1)));
+        ASX_TRY(hipMalloc((void **)&arena, off));
+        counts = (int32_t *)(arena + o_counts), offs = (int32_t *)(arena + o_offs), seg_row = (int32_t *)(arena + o_seg);
+        d_pstart = (int32_t *)(arena + o_pstart), d_tile_off = (int32_t *)(arena + o_toff);
+        lrow = (int32_t *)(arena + o_lrow), tile_cnt = (int32_t *)(arena + o_tcnt), step_cnt = (int32_t *)(arena + o_scnt);
+        tmp = (int32_t *)(arena + o_tmp);
+    }
 
-    // 1. stored elements by slice (stable: row order, then column order, survives inside a slice)
-    hipLaunchKernelGGL(k_sliced_keys, dim3(grid), dim3(kBlock), 0, s, col, nnz, width, a, c);
-    ASX_TRY(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, a, b, c, d, nnz, 0, key_bits, s));
-    // b = slice of each sorted element, d = its position in A; a = its row
-    hipLaunchKernelGGL(k_sliced_rows, dim3(grid), dim3(kBlock), 0, s, d, nnz, row_ptr, m, a);
-    ASX_TRY_ST(launch_offsets_from_sorted(b, nnz, sm.nslices, d_pstart, s));
+    // 1. every block's stored elements per slice, and from their scan the block's place in each slice
+    hipLaunchKernelGGL(k_sliced_count, dim3((unsigned)nblocks), dim3(kSortThreads), 0, s, col, nnz, width, sm.nslices,
+                       nblocks, counts);
+    ASX_TRY_ST(launch_exclusive_scan_i32(counts, offs, ncount, tmp, s));
+    hipLaunchKernelGGL(k_sliced_slice_starts, dim3((unsigned)ceil_div64((int64_t)sm.nslices + 1, kBlock)), dim3(kBlock), 0, s,
+                       offs, sm.nslices, nblocks, d_pstart);
     ASX_TRY(hipMemcpyAsync(pstart.data(), d_pstart, sizeof(int32_t) * pstart.size(), hipMemcpyDeviceToHost, s));
+    ASX_TRY_ST(launch_nnz_split_rows(row_ptr, m, nnz, kSortWaveElems, seg_row, s));  // runs while the host waits
     ASX_TRY(hipStreamSynchronize(s));
 
     // 2. tiles: every slice starts a new tile
-    for (int32_t sl = 0; sl < sm.nslices; ++sl)
+    for (int32_t sl = 0; sl < sm.nslices; ++sl) {
         tile_off[sl + 1] = tile_off[sl] + (int32_t)ceil_div64(pstart[sl + 1] - pstart[sl], kSlicedTile);
+        empty_slice |= pstart[sl + 1] == pstart[sl];
+    }
     sm.ntiles = tile_off[sm.nslices];
     slots = (int64_t)sm.ntiles * kSlicedTile;
-    if (slots > 0x7fffffff) {
-        st = ASX_STATUS_INVALID_SIZE;
-        goto done;
-    }
     ASX_TRY(hipMemcpyAsync(d_tile_off, tile_off.data(), sizeof(int32_t) * tile_off.size(), hipMemcpyHostToDevice, s));
     ASX_TRY(hipMalloc(&sm.val, sizeof(T) * (size_t)slots));
     ASX_TRY(hipMalloc((void **)&sm.cf, sizeof(uint16_t) * (size_t)slots));
     ASX_TRY(hipMalloc((void **)&sm.perm, sizeof(int32_t) * (size_t)slots));
-    lrow = c;   // the sort's input values are spent
-    lhead = e;
+    // 3. every stored element to its slot; the pads behind every slice
     {
-        const unsigned sgrid = (unsigned)ceil_div64(slots, kBlock);
-        hipLaunchKernelGGL((k_sliced_fill_pads<T>), dim3(sgrid), dim3(kBlock), 0, s, slots, lrow, lhead, sm.cf,
-                           (T *)sm.val, sm.perm);
-        hipLaunchKernelGGL((k_sliced_place<T>), dim3(grid), dim3(kBlock), 0, s, b, d, a, nnz, width, d_pstart, d_tile_off,
-                           col, val, lrow, lhead, sm.cf, (T *)sm.val, sm.perm);
-        // 3. partial sums: one per run start
-        hscan = a;      // the placing has read the rows, slices and positions of the sorted elements:
-        prow_full = b;  // their arrays are free (kernels run in stream order)
-        ASX_TRY(hipcub::DeviceScan::InclusiveSum(tmp, tmp_bytes, lhead, hscan, (int)slots, s));
-        ASX_TRY(hipMemcpyAsync(&sm.npartials, hscan + (slots - 1), sizeof(int32_t), hipMemcpyDeviceToHost, s));
-        ASX_TRY(hipStreamSynchronize(s));
-        ASX_TRY(hipMalloc((void **)&sm.tile_base, sizeof(int32_t) * ((size_t)sm.ntiles + 1)));
-        ASX_TRY(hipMalloc((void **)&sm.prow, sizeof(uint16_t) * ((size_t)sm.npartials + kSlicedReducePad)));
-        ASX_TRY(hipMemsetAsync(sm.prow, 0, sizeof(uint16_t) * ((size_t)sm.npartials + kSlicedReducePad), s));
-        ASX_TRY(hipMalloc(&sm.partial, sizeof(T) * ((size_t)sm.npartials + kSlicedReducePad)));
-        ASX_TRY(hipMemsetAsync(sm.partial, 0, sizeof(T) * ((size_t)sm.npartials + kSlicedReducePad), s));
-        ASX_TRY(hipMalloc((void **)&sm.chunk_lo, sizeof(int32_t) * ((size_t)sm.nrb + 1) * (size_t)sm.nslices));
-        hipLaunchKernelGGL(k_sliced_tile_base, dim3((unsigned)ceil_div64((int64_t)sm.ntiles + 1, kBlock)), dim3(kBlock),
-                           0, s, hscan, sm.ntiles, sm.tile_base);
-        hipLaunchKernelGGL(k_sliced_partial_rows, dim3(sgrid), dim3(kBlock), 0, s, lrow, lhead, hscan, slots,
-                           rows_per_wave, prow_full, sm.prow);
-        // 4. where each row block starts inside each slice's partial sums
-        const int64_t nchunks = ((int64_t)sm.nrb + 1) * sm.nslices;
-        hipLaunchKernelGGL(k_sliced_chunks, dim3((unsigned)ceil_div64(nchunks, kBlock)), dim3(kBlock), 0, s, prow_full,
-                           sm.tile_base, d_tile_off, sm.nslices, sm.nrb, rows_per_wave, sm.chunk_lo);
+        const unsigned sgrid = (unsigned)(ceil_div64(nblocks, kXcds) * kXcds);
+#define ASX_SCATTER(MAXS)                                                                                              \
+    hipLaunchKernelGGL((k_sliced_scatter<T, MAXS>), dim3(sgrid), dim3(kSortThreads), 0, s, row_ptr, col, val, seg_row, m, \
+                       nnz, width, sm.nslices, nbits, nblocks, offs, d_tile_off, lrow, sm.cf, (T *)sm.val, sm.perm)
+        if (sm.nslices <= 256)
+            ASX_SCATTER(256);
+        else
+            ASX_SCATTER(kSlicedMaxSlices);
+#undef ASX_SCATTER
+        hipLaunchKernelGGL((k_sliced_pads<T>), dim3((unsigned)sm.nslices), dim3(kSlicedTile), 0, s, d_pstart, d_tile_off, lrow,
+                           sm.cf, (T *)sm.val, sm.perm);
     }
-    // 4b. the steps in which pass 2 reads each row block's ranges
+    // 4. partial sums: one per run start; tile_base = the run starts before each tile
     {
-        size_t scan_bytes = 0;
-        int32_t *cnt = nullptr;
-        ASX_TRY(hipMalloc((void **)&pack_tmp, sizeof(int32_t) * ((size_t)sm.nrb + 1)));
-        cnt = pack_tmp;
+        const unsigned wgrid = (unsigned)ceil_div64((int64_t)sm.ntiles * kWave, kBlock);
+        ASX_TRY(hipMalloc((void **)&sm.tile_base, sizeof(int32_t) * ((size_t)sm.ntiles + 1)));
+        hipLaunchKernelGGL(k_sliced_tile_runs, dim3(wgrid), dim3(kBlock), 0, s, lrow, sm.ntiles, tile_cnt);
+        ASX_TRY_ST(launch_exclusive_scan_i32(tile_cnt, sm.tile_base, (int64_t)sm.ntiles + 1, tmp, s));
+        ASX_TRY(hipMemcpyAsync(&sm.npartials, sm.tile_base + sm.ntiles, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+        ASX_TRY(hipMalloc((void **)&sm.chunk_lo, sizeof(int32_t) * (size_t)ncells));  // while the kernels run
         ASX_TRY(hipMalloc((void **)&sm.pstep_ptr, sizeof(int32_t) * ((size_t)sm.nrb + 1)));
-        ASX_TRY(hipMemsetAsync(cnt, 0, sizeof(int32_t) * ((size_t)sm.nrb + 1), s));
-        ASX_TRY(rocprim::exclusive_scan(nullptr, scan_bytes, cnt, sm.pstep_ptr, 0, (size_t)sm.nrb + 1, rocprim::plus<int32_t>(), s));
-        ASX_TRY(hipMalloc(&pack_scan_tmp, std::max<size_t>(scan_bytes, 256)));
-        const unsigned pgrid = (unsigned)ceil_div64(sm.nrb, kBlock);
-        hipLaunchKernelGGL(k_sliced_pack, dim3(pgrid), dim3(kBlock), 0, s, sm.chunk_lo, sm.nrb, sm.nslices, nullptr, cnt,
+        ASX_TRY(hipStreamSynchronize(s));
+        ASX_TRY(hipMalloc((void **)&sm.prow, sizeof(uint16_t) * ((size_t)sm.npartials + kSlicedReducePad)));
+        ASX_TRY(hipMemsetAsync(sm.prow + sm.npartials, 0, sizeof(uint16_t) * kSlicedReducePad, s));
+        // 5. rows of the partial sums, run-start bits, and where each row block starts inside each slice
+        hipLaunchKernelGGL(k_sliced_emit, dim3(wgrid), dim3(kBlock), 0, s, lrow, sm.tile_base, d_tile_off, sm.ntiles,
+                           sm.nslices, rows_per_wave, sm.nrb, sm.cf, sm.prow, sm.chunk_lo);
+        if (empty_slice)
+            hipLaunchKernelGGL(k_sliced_empty_slices, dim3((unsigned)ceil_div64(ncells, kBlock)), dim3(kBlock), 0, s,
+                               sm.tile_base, d_tile_off, sm.nslices, sm.nrb, sm.chunk_lo);
+    }
+    // 6. the steps in which pass 2 reads each row block's ranges
+    {
+        const unsigned pgrid = (unsigned)ceil_div64((int64_t)sm.nrb * kWave, kBlock);
+        ASX_TRY(hipMemsetAsync(step_cnt + sm.nrb, 0, sizeof(int32_t), s));
+        hipLaunchKernelGGL(k_sliced_pack, dim3(pgrid), dim3(kBlock), 0, s, sm.chunk_lo, sm.nrb, sm.nslices, nullptr, step_cnt,
                            nullptr);
-        ASX_TRY(rocprim::exclusive_scan(pack_scan_tmp, scan_bytes, cnt, sm.pstep_ptr, 0, (size_t)sm.nrb + 1, rocprim::plus<int32_t>(), s));
+        ASX_TRY_ST(launch_exclusive_scan_i32(step_cnt, sm.pstep_ptr, (int64_t)sm.nrb + 1, tmp, s));
         ASX_TRY(hipMemcpyAsync(&sm.npsteps, sm.pstep_ptr + sm.nrb, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+        ASX_TRY(hipMalloc(&sm.partial, sizeof(T) * ((size_t)sm.npartials + kSlicedReducePad)));  // while the kernels run
         ASX_TRY(hipStreamSynchronize(s));
         ASX_TRY(hipMalloc((void **)&sm.psteps, sizeof(int32_t) * 4 * ((size_t)sm.npsteps + kSlicedStepPad)));
-        ASX_TRY(hipMemsetAsync(sm.psteps, 0, sizeof(int32_t) * 4 * ((size_t)sm.npsteps + kSlicedStepPad), s));
+        ASX_TRY(hipMemsetAsync(sm.psteps + 4 * (size_t)sm.npsteps, 0, sizeof(int32_t) * 4 * kSlicedStepPad, s));
         hipLaunchKernelGGL(k_sliced_pack, dim3(pgrid), dim3(kBlock), 0, s, sm.chunk_lo, sm.nrb, sm.nslices, sm.pstep_ptr,
                            nullptr, reinterpret_cast<i32x4 *>(sm.psteps));
     }
-    // 5. workgroups of pass 1: every slice gets its share of about `target_wgs` workgroups (at
+    // 7. workgroups of pass 1: every slice gets its share of about `target_wgs` workgroups (at
     //    least one, and no workgroup smaller than 32 tiles unless the slice is), its tiles in equal
     //    pieces
     {
@@ -578,8 +791,6 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
 #undef ASX_TRY_ST
 done:
     if (arena) (void)hipFree(arena);
-    if (pack_tmp) (void)hipFree(pack_tmp);
-    if (pack_scan_tmp) (void)hipFree(pack_scan_tmp);
     if (st) {
         free_sliced(&sm);
         return st;
@@ -587,6 +798,7 @@ done:
     *out = sm;
     return ASX_STATUS_SUCCESS;
 }
+
 
 template <typename T>
 int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s)

@@ -22,12 +22,11 @@
 //
 // The reference has no counterpart (its CSR kernels read 32-bit columns and gather x from global
 // memory: hip/kernel/level2/alphasparse_spmv_csr_vector.h:99-126).
-#include <hipcub/hipcub.hpp>
-
 #include <algorithm>
 #include <vector>
 
 #include "asx_internal.hpp"
+#include "asx_scan.hpp"
 #include "asx_tiles.hpp"
 
 namespace asx {
@@ -545,8 +544,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     int32_t *arena = nullptr;
     int32_t *cmin = nullptr, *cmax = nullptr, *row_start = nullptr;  // m each
     int32_t *bmin = nullptr, *bmax = nullptr, *btiles = nullptr, *tile_off = nullptr, *d_small = nullptr;
-    void *tmp = nullptr;
-    size_t tmp_bytes = 0;
+    int32_t *tmp = nullptr;
     std::vector<int32_t> h_bmin, h_bmax, h_off, blk, pcs, chains;
     std::vector<uint32_t> h_bits;
     uint32_t *d_bits = nullptr;
@@ -562,11 +560,10 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
         if (st) goto done;    \
     } while (0)
     // the scratch of the build in one allocation: three arrays of m ints, four of max_nb + 1, two
-    // counters, the scan's workspace
-    ASX_TRY(hipcub::DeviceScan::ExclusiveSum(nullptr, tmp_bytes, btiles, tile_off, max_nb + 1, s));
+    // counters, the scan's block sums
     {
         const size_t per_row = ((size_t)m + 63) & ~(size_t)63, per_block = ((size_t)max_nb + 1 + 63) & ~(size_t)63;
-        ASX_TRY(hipMalloc((void **)&arena, sizeof(int32_t) * (3 * per_row + 4 * per_block + 64) + std::max<size_t>(tmp_bytes, 256)));
+        ASX_TRY(hipMalloc((void **)&arena, sizeof(int32_t) * (3 * per_row + 4 * per_block + 64 + scan_scratch_ints((int64_t)max_nb + 1))));
         cmin = arena, cmax = cmin + per_row, row_start = cmax + per_row;
         bmin = row_start + per_row, bmax = bmin + per_block, btiles = bmax + per_block, tile_off = btiles + per_block;
         d_small = tile_off + per_block;
@@ -663,7 +660,8 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     hipLaunchKernelGGL(k_window_row_starts, dim3((unsigned)ceil_div64((int64_t)wm.nblocks * kWave, kBlock)), dim3(kBlock), 0, s, row_ptr, m,
                        wm.rows_per_block, wm.nblocks, row_start, btiles);
     ASX_TRY(hipMemsetAsync(btiles + wm.nblocks, 0, sizeof(int32_t), s));
-    ASX_TRY(hipcub::DeviceScan::ExclusiveSum(tmp, tmp_bytes, btiles, tile_off, wm.nblocks + 1, s));
+    st = launch_exclusive_scan_i32(btiles, tile_off, (int64_t)wm.nblocks + 1, tmp, s);
+    if (st) goto done;
     h_bmin.resize((size_t)wm.nblocks);
     h_bmax.resize((size_t)wm.nblocks);
     h_off.resize((size_t)wm.nblocks + 1);
