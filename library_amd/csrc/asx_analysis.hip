@@ -29,12 +29,29 @@ __global__ __launch_bounds__(256) void k_row_histogram(const int32_t *__restrict
     if (threadIdx.x == 0) s_max = 0;
     __syncthreads();
     int local_max = 0;
-    for (int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; r < m;
-         r += (int64_t)gridDim.x * blockDim.x) {
-        int len = row_ptr[r + 1] - row_ptr[r];
-        int bin = len <= 0 ? 0 : 32 - __clz(len);
-        atomicAdd(&s_hist[bin], 1u);
-        atomicAdd(&s_bins[len < 2 ? 0 : (len < 1024 ? 1 : 2)], 1u);
+    const int lane = threadIdx.x & (kWave - 1);
+    for (int64_t r0 = (int64_t)blockIdx.x * blockDim.x; r0 < m; r0 += (int64_t)gridDim.x * blockDim.x) {  // uniform
+        const int64_t r = r0 + threadIdx.x;
+        const bool valid = r < m;
+        const int len = valid ? row_ptr[r + 1] - row_ptr[r] : 0;
+        const int bin = len <= 0 ? 0 : 32 - __clz(len);
+        // one LDS atomic per distinct bin among the wave's 64 rows (rows of one length would
+        // otherwise serialise 64 atomics on one address)
+        unsigned long long todo = __ballot(valid);
+        while (todo) {  // uniform
+            const int first = __builtin_ctzll(todo);
+            const int b = __builtin_amdgcn_readlane(bin, first);
+            const unsigned long long same = __ballot(valid && bin == b);
+            if (lane == first) atomicAdd(&s_hist[b], (unsigned int)__popcll(same));
+            todo &= ~same;
+        }
+        const unsigned int c0 = __popcll(__ballot(valid && len < 2)), c1 = __popcll(__ballot(valid && len >= 2 && len < 1024));
+        const unsigned int c2 = __popcll(__ballot(valid && len >= 1024));
+        if (lane == 0) {
+            if (c0) atomicAdd(&s_bins[0], c0);
+            if (c1) atomicAdd(&s_bins[1], c1);
+            if (c2) atomicAdd(&s_bins[2], c2);
+        }
         local_max = len > local_max ? len : local_max;
     }
     atomicMax(&s_max, local_max);
@@ -244,18 +261,52 @@ __global__ __launch_bounds__(256) void k_copy16(const u32x4 *__restrict__ src, u
     for (; i < n16; i += stride) dst[i] = src[i];
 }
 
-// out[t * tile + i] = src[t * stride + i]: `samples` tiles of `tile` ints, one workgroup each
-__global__ __launch_bounds__(kBlock) void k_sample_tiles(const int32_t *__restrict__ src, int64_t stride, int32_t tile,
-                                                         int32_t *__restrict__ out)
+// out[t] = number of distinct values of src[t * stride + i] >> shift, i in [0, 1024): one workgroup
+// per sampled tile, the values entered into a hash table in LDS (4096 slots, linear probing)
+__global__ __launch_bounds__(kBlock) void k_sample_distinct(const int32_t *__restrict__ src, int64_t stride, int shift,
+                                                            int32_t *__restrict__ out)
 {
+    constexpr int kSlots = 4096;
+    __shared__ int32_t table[kSlots];
+    __shared__ int32_t count;
+    for (int i = threadIdx.x; i < kSlots; i += kBlock) table[i] = -1;
+    if (threadIdx.x == 0) count = 0;
+    __syncthreads();
     const int32_t *from = src + (int64_t)blockIdx.x * stride;
-    for (int32_t i = threadIdx.x; i < tile; i += blockDim.x) out[(int64_t)blockIdx.x * tile + i] = from[i];
+    int32_t mine = 0;
+    for (int i = threadIdx.x; i < kFlatTile; i += kBlock) {
+        const int32_t v = from[i] >> shift;
+        uint32_t h = ((uint32_t)v * 2654435761u) >> 20;
+        for (;;) {
+            const int32_t old = atomicCAS(&table[h], -1, v);
+            if (old == -1) {
+                ++mine;
+                break;
+            }
+            if (old == v) break;
+            h = (h + 1) & (kSlots - 1);
+        }
+    }
+    if (mine) atomicAdd(&count, mine);
+    __syncthreads();
+    if (threadIdx.x == 0) out[blockIdx.x] = count;
 }
-int launch_sample_tiles(const int32_t *d_src, int64_t stride, int32_t tile, int32_t samples, int32_t *d_out,
-                        hipStream_t s)
+int launch_sample_distinct(const int32_t *d_src, int64_t stride, int shift, int32_t samples, int32_t *d_out, hipStream_t s)
 {
     if (samples <= 0) return ASX_STATUS_SUCCESS;
-    hipLaunchKernelGGL(k_sample_tiles, dim3((unsigned)samples), dim3(kBlock), 0, s, d_src, stride, tile, d_out);
+    hipLaunchKernelGGL(k_sample_distinct, dim3((unsigned)samples), dim3(kBlock), 0, s, d_src, stride, shift, d_out);
+    return check_launch();
+}
+
+__global__ __launch_bounds__(kBlock) void k_fill_i32(int32_t *__restrict__ p, int64_t n, int32_t v)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+int launch_fill_i32(int32_t *d_dst, int64_t n, int32_t value, hipStream_t s)
+{
+    if (n <= 0) return ASX_STATUS_SUCCESS;
+    hipLaunchKernelGGL(k_fill_i32, dim3((unsigned)ceil_div64(n, kBlock)), dim3(kBlock), 0, s, d_dst, n, value);
     return check_launch();
 }
 

@@ -82,31 +82,23 @@ SpmmLayout spmm_merge_layout(int32_t m, int32_t nnz, int32_t ncols, size_t sv, b
 
 // How scattered the columns are: the number of distinct 128-byte lines of x that the columns of a
 // tile of 1024 consecutive stored elements touch, divided by 1024, averaged over up to 64 tiles
-// spread over the matrix (copied to the host; 256 KiB).  Random columns give about 1, a 5-point
+// spread over the matrix (counted on the device).  Random columns give about 1, a 5-point
 // stencil 0.04, a band matrix 0.01.  Regrouping by column slice only pays for scattered columns.
-double sampled_line_spread(const int32_t *d_col, int32_t nnz, size_t sv, hipStream_t s)
+double sampled_line_spread(const int32_t *d_col, int32_t nnz, size_t sv, int32_t *d_scratch, hipStream_t s)
 {
     const int64_t tiles = nnz / kFlatTile;
     if (tiles < 1) return 0.0;
     const int samples = (int)std::min<int64_t>(64, tiles);
     const int64_t stride = tiles / samples;
-    std::vector<int32_t> h((size_t)samples * kFlatTile);
-    // the sampled tiles, gathered on the device into one piece, then one plain copy
-    int32_t *d_sample = nullptr;
-    if (hipMalloc((void **)&d_sample, h.size() * sizeof(int32_t)) != hipSuccess) return 0.0;
-    const bool ok = launch_sample_tiles(d_col, stride * kFlatTile, kFlatTile, samples, d_sample, s) == ASX_STATUS_SUCCESS &&
-                    hipMemcpyAsync(h.data(), d_sample, h.size() * sizeof(int32_t), hipMemcpyDeviceToHost, s) == hipSuccess &&
-                    hipStreamSynchronize(s) == hipSuccess;
-    (void)hipFree(d_sample);
-    if (!ok) return 0.0;
+    // the distinct lines of every sampled tile are counted on the device (d_scratch: 64 ints)
+    int32_t h[64];
     const int shift = sv == 8 ? 4 : 5;  // columns per 128-byte line of x
+    if (launch_sample_distinct(d_col, stride * kFlatTile, shift, samples, d_scratch, s) != ASX_STATUS_SUCCESS ||
+        hipMemcpyAsync(h, d_scratch, sizeof(int32_t) * (size_t)samples, hipMemcpyDeviceToHost, s) != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess)
+        return 0.0;
     int64_t distinct = 0;
-    for (int t = 0; t < samples; ++t) {
-        int32_t *p = h.data() + (size_t)t * kFlatTile;
-        for (int i = 0; i < kFlatTile; ++i) p[i] >>= shift;
-        std::sort(p, p + kFlatTile);
-        distinct += std::unique(p, p + kFlatTile) - p;
-    }
+    for (int t = 0; t < samples; ++t) distinct += h[t];
     return (double)distinct / ((double)samples * kFlatTile);
 }
 constexpr double kScatteredMinSpread = 0.5;
@@ -359,65 +351,57 @@ int asx_loadbalance_partition(const int32_t *d_row_ptr, int32_t m, int32_t nnz, 
 }
 
 // ---------------------------------------------------------------- plans
-int asx_plan_create(asx_plan **out, int is_spmm, int alg, int value_type, int32_t m, int32_t n,
-                    int32_t nnz, const int32_t *d_row_ptr, int32_t ncols_dense, void *stream)
+}  // extern "C"
+
+namespace {
+
+// A plan with sizes and the row-length histogram, no kernel chosen yet.  The counters on the device
+// stay with the plan (33 histogram bins, 4 stats, spare words for what else the build reads back):
+// freeing them here would cost more than the build's kernels.
+int plan_begin(asx_plan **out, int is_spmm, int value_type, int32_t m, int32_t n, int32_t nnz, const int32_t *d_row_ptr,
+               int32_t ncols_dense, hipStream_t s)
 {
-    if (!out) return ASX_STATUS_INVALID_POINTER;
-    *out = nullptr;
-    if (m < 0 || n < 0 || nnz < 0 || ncols_dense < 1) return ASX_STATUS_INVALID_SIZE;
-    if (value_type != ASX_R_32F && value_type != ASX_R_64F) return ASX_STATUS_NOT_SUPPORTED;
-    if (m > 0 && !d_row_ptr) return ASX_STATUS_INVALID_POINTER;
-    hipStream_t s = (hipStream_t)stream;
     asx_plan *p = new (std::nothrow) asx_plan();
     if (!p) return ASX_STATUS_ALLOC_FAILED;
     std::memset(p, 0, sizeof(*p));
     p->is_spmm = is_spmm ? 1 : 0;
+    p->alg = -1;
     p->value_type = value_type;
     p->m = m;
     p->n = n;
     p->nnz = nnz;
     p->ncols = is_spmm ? ncols_dense : 1;
     p->row_ptr = d_row_ptr;
-
-    // histogram (always: it is cheap and callers may ask for it)
-    int64_t *d_cnt = nullptr;
-    int st = status_of(hipMalloc((void **)&d_cnt, 37 * sizeof(int64_t)));
-    if (st) {
-        delete p;
-        return st;
-    }
-    st = launch_row_histogram(d_row_ptr, m, d_cnt, d_cnt + 33, s);
-    if (!st) st = status_of(hipMemcpyAsync(p->hist, d_cnt, 33 * sizeof(int64_t), hipMemcpyDeviceToHost, s));
-    if (!st) st = status_of(hipMemcpyAsync(p->stats, d_cnt + 33, 4 * sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    int st = status_of(hipMalloc((void **)&p->d_counters, kPlanCounters * sizeof(int64_t)));
+    if (!st) st = launch_row_histogram(d_row_ptr, m, p->d_counters, p->d_counters + 33, s);
+    if (!st) st = status_of(hipMemcpyAsync(p->hist, p->d_counters, 33 * sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    if (!st) st = status_of(hipMemcpyAsync(p->stats, p->d_counters + 33, 4 * sizeof(int64_t), hipMemcpyDeviceToHost, s));
     if (!st) st = status_of(hipStreamSynchronize(s));
-    (void)hipFree(d_cnt);
     if (st) {
-        delete p;
+        asx_plan_destroy(p);
         return st;
     }
+    *out = p;
+    return ASX_STATUS_SUCCESS;
+}
 
-    const size_t sv = vsize(value_type);
-    if (!is_spmm) {
-        int kernel = alg;
-        if (alg == ASX_SPMV_DEFAULT)
-            kernel = choose_spmv_from_stats(p->hist, p->stats, m, nnz);
-        else
-            kernel = asx_spmv_resolve_alg(alg, m, nnz);
-        if (kernel < 0) {
-            delete p;
-            return ASX_STATUS_NOT_SUPPORTED;
-        }
-        p->alg = kernel;
-        if (m == 0) {
-            // nothing to analyse (and no row_ptr to read): calls with m == 0 return before any launch
-            p->workspace_bytes = 0;
-        } else if (kernel == ASX_SPMV_STREAM) {
+// Split points of a row-ordered kernel onto a plan from plan_begin.
+int plan_row_ordered(asx_plan *p, int kernel, hipStream_t s)
+{
+    const int32_t m = p->m, nnz = p->nnz;
+    const int32_t *d_row_ptr = p->row_ptr;
+    const size_t sv = vsize(p->value_type);
+    int st = ASX_STATUS_SUCCESS;
+    p->alg = kernel;
+    p->workspace_bytes = 0;
+    if (m == 0) return ASX_STATUS_SUCCESS;  // nothing to analyse: calls with m == 0 return before any launch
+    if (!p->is_spmm) {
+        if (kernel == ASX_SPMV_STREAM) {
             int32_t nb = std::max(stream_blocks(nnz), 1);
             p->nunits = nb;
             p->meta_bytes = ((size_t)nb + 1) * 8;
             st = status_of(hipMalloc((void **)&p->d_meta, p->meta_bytes));
             if (!st) st = launch_stream_row_blocks(d_row_ptr, m, nnz, p->d_meta, s);
-            p->workspace_bytes = 0;
         } else if (kernel == ASX_SPMV_FLAT) {
             const size_t nt = (size_t)flat_tiles(nnz);
             p->nunits = (int32_t)nt;
@@ -427,60 +411,66 @@ int asx_plan_create(asx_plan **out, int is_spmm, int alg, int value_type, int32_
             p->workspace_bytes = spmv_flat_layout(nnz, sv, false).bytes;
             p->carry_pass = 1;
             if (!st) {  // is any row cut by a tile boundary?  (one int read back; creation syncs anyway)
-                int32_t *d_flag = nullptr, h_flag = 1;
-                st = status_of(hipMalloc((void **)&d_flag, sizeof(int32_t)));
-                if (!st) {
-                    st = status_of(hipMemsetAsync(d_flag, 0, sizeof(int32_t), s));
-                    if (!st) st = launch_flat_has_carry(d_row_ptr, m, nnz, p->d_meta, d_flag, s);
-                    if (!st) st = status_of(hipMemcpyAsync(&h_flag, d_flag, sizeof(int32_t), hipMemcpyDeviceToHost, s));
-                    if (!st) st = status_of(hipStreamSynchronize(s));
-                    (void)hipFree(d_flag);
-                    if (!st) p->carry_pass = h_flag != 0;
-                }
+                int32_t *d_flag = reinterpret_cast<int32_t *>(p->d_counters + 40), h_flag = 1;
+                st = launch_fill_i32(d_flag, 1, 0, s);
+                if (!st) st = launch_flat_has_carry(d_row_ptr, m, nnz, p->d_meta, d_flag, s);
+                if (!st) st = status_of(hipMemcpyAsync(&h_flag, d_flag, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+                if (!st) st = status_of(hipStreamSynchronize(s));
+                if (!st) p->carry_pass = h_flag != 0;
             }
         } else if (kernel == ASX_SPMV_MERGE) {
             const size_t nt = (size_t)merge_tiles(m, nnz);
             p->nunits = (int32_t)nt;
             p->meta_bytes = 2 * (nt + 1) * 4;
             st = status_of(hipMalloc((void **)&p->d_meta, p->meta_bytes));
-            if (!st)
-                st = launch_merge_path_search(d_row_ptr, m, nnz, kMergeTile, p->d_meta,
-                                              p->d_meta + (nt + 1), s);
+            if (!st) st = launch_merge_path_search(d_row_ptr, m, nnz, kMergeTile, p->d_meta, p->d_meta + (nt + 1), s);
             p->workspace_bytes = spmv_merge_layout(m, nnz, sv, false).bytes;
-        } else {
-            p->workspace_bytes = 0;
         }
-    } else {
-        int kernel = asx_spmm_resolve_alg(alg, m, nnz, ncols_dense);
-        if (kernel < 0 || kernel == ASX_SPMM_BLOCKED) {  // blocked plans need col and val too
-            delete p;
-            return ASX_STATUS_NOT_SUPPORTED;
-        }
-        p->alg = kernel;
-        if (m == 0) {
-            p->workspace_bytes = 0;
-        } else if (kernel == ASX_SPMM_MERGE) {
-            const size_t ns = (size_t)spmm_segments(m, nnz);
-            p->nunits = (int32_t)ns;
-            p->meta_bytes = 2 * (ns + 1) * 4;
-            int32_t *raw = nullptr;  // the merge-path points, then snapped to short-row ends
-            st = status_of(hipMalloc((void **)&p->d_meta, p->meta_bytes));
-            if (!st) st = status_of(hipMalloc((void **)&raw, p->meta_bytes));
-            if (!st) st = launch_merge_path_search(d_row_ptr, m, nnz, kSpmmSegment, raw, raw + (ns + 1), s);
-            if (!st)
-                st = launch_spmm_snap_splits(m, nnz, d_row_ptr, raw, raw + (ns + 1), p->d_meta,
-                                             p->d_meta + (ns + 1), s);
-            if (!st) st = status_of(hipStreamSynchronize(s));
-            if (raw) (void)hipFree(raw);
-            p->workspace_bytes = spmm_merge_layout(m, nnz, ncols_dense, sv, false).bytes;
-        } else {
-            p->workspace_bytes = 0;
-        }
+    } else if (kernel == ASX_SPMM_MERGE) {
+        const size_t ns = (size_t)spmm_segments(m, nnz);
+        p->nunits = (int32_t)ns;
+        p->meta_bytes = 2 * (ns + 1) * 4;
+        int32_t *raw = nullptr;  // the merge-path points, then snapped to short-row ends
+        st = status_of(hipMalloc((void **)&p->d_meta, p->meta_bytes));
+        if (!st) st = status_of(hipMalloc((void **)&raw, p->meta_bytes));
+        if (!st) st = launch_merge_path_search(d_row_ptr, m, nnz, kSpmmSegment, raw, raw + (ns + 1), s);
+        if (!st) st = launch_spmm_snap_splits(m, nnz, d_row_ptr, raw, raw + (ns + 1), p->d_meta, p->d_meta + (ns + 1), s);
+        if (!st) st = status_of(hipStreamSynchronize(s));
+        if (raw) (void)hipFree(raw);
+        p->workspace_bytes = spmm_merge_layout(m, nnz, p->ncols, sv, false).bytes;
     }
     if (!st) st = status_of(hipStreamSynchronize(s));
+    return st;
+}
+
+}  // namespace
+
+extern "C" {
+
+int asx_plan_create(asx_plan **out, int is_spmm, int alg, int value_type, int32_t m, int32_t n,
+                    int32_t nnz, const int32_t *d_row_ptr, int32_t ncols_dense, void *stream)
+{
+    if (!out) return ASX_STATUS_INVALID_POINTER;
+    *out = nullptr;
+    if (m < 0 || n < 0 || nnz < 0 || ncols_dense < 1) return ASX_STATUS_INVALID_SIZE;
+    if (value_type != ASX_R_32F && value_type != ASX_R_64F) return ASX_STATUS_NOT_SUPPORTED;
+    if (m > 0 && !d_row_ptr) return ASX_STATUS_INVALID_POINTER;
+    hipStream_t s = (hipStream_t)stream;
+    asx_plan *p = nullptr;
+    int st = plan_begin(&p, is_spmm, value_type, m, n, nnz, d_row_ptr, ncols_dense, s);
+    if (st) return st;
+    int kernel;
+    if (!is_spmm)
+        kernel = alg == ASX_SPMV_DEFAULT ? choose_spmv_from_stats(p->hist, p->stats, m, nnz) : asx_spmv_resolve_alg(alg, m, nnz);
+    else
+        kernel = asx_spmm_resolve_alg(alg, m, nnz, ncols_dense);
+    if (kernel < 0 || (is_spmm && kernel == ASX_SPMM_BLOCKED)) {  // blocked plans need col and val too
+        asx_plan_destroy(p);
+        return ASX_STATUS_NOT_SUPPORTED;
+    }
+    st = plan_row_ordered(p, kernel, s);
     if (st) {
-        if (p->d_meta) (void)hipFree(p->d_meta);
-        delete p;
+        asx_plan_destroy(p);
         return st;
     }
     *out = p;
@@ -492,6 +482,7 @@ int asx_plan_destroy(asx_plan *plan)
     if (!plan) return ASX_STATUS_SUCCESS;
     int st = ASX_STATUS_SUCCESS;
     if (plan->d_meta) st = status_of(hipFree(plan->d_meta));
+    if (plan->d_counters) (void)hipFree(plan->d_counters);
     free_blocked(&plan->blocked);
     free_sliced(&plan->sliced);
     free_window(&plan->window);
@@ -515,9 +506,14 @@ int asx_spmm_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     const bool want_blocked = kernel == ASX_SPMM_BLOCKED;
     // scattered columns (a sample of tiles of 1024 stored elements touches mostly distinct
     // 128-byte lines) cannot fill 16x4 blocks: the blocks are not even built then
-    const bool probe_blocked = alg == ASX_SPMM_DEFAULT && nnz > 0 && nnz <= kBlockedProbeMaxNnz && d_col &&
-                               (value_type == ASX_R_32F || value_type == ASX_R_64F) &&
-                               sampled_line_spread(d_col, nnz, vsize(value_type), (hipStream_t)stream) < kScatteredMinSpread;
+    bool probe_blocked = alg == ASX_SPMM_DEFAULT && nnz > 0 && nnz <= kBlockedProbeMaxNnz && d_col &&
+                         (value_type == ASX_R_32F || value_type == ASX_R_64F);
+    if (probe_blocked) {
+        int32_t *d_scratch = nullptr;
+        if (hipMalloc((void **)&d_scratch, 64 * sizeof(int32_t)) != hipSuccess) return ASX_STATUS_ALLOC_FAILED;
+        probe_blocked = sampled_line_spread(d_col, nnz, vsize(value_type), d_scratch, (hipStream_t)stream) < kScatteredMinSpread;
+        (void)hipFree(d_scratch);
+    }
     if (!want_blocked && !probe_blocked)
         return asx_plan_create(out, 1, alg, value_type, m, k, nnz, d_row_ptr, ncols, stream);
     if (m < 0 || k < 0 || nnz < 0 || ncols < 1) return ASX_STATUS_INVALID_SIZE;
@@ -654,6 +650,17 @@ int plan_add_window(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
     return ASX_STATUS_SUCCESS;
 }
 
+// DEFAULT tries the row-block copy for matrices the flat or merge-path kernel would take, without
+// rows past the carry pass's limit, and with few empty rows: the copy gives every empty row a
+// slot of its own (a value, a column word and a source index, read in every call), so a matrix
+// with more empty rows than a quarter of its stored elements stays with the merge-path kernel,
+// which streams row offsets only.
+static bool window_may_pay(const asx_plan *p, int row_kernel)
+{
+    return p->stats[0] <= kWindowMaxRow && (row_kernel == ASX_SPMV_FLAT || row_kernel == ASX_SPMV_MERGE) &&
+           p->hist[0] <= (int64_t)p->nnz / 4;
+}
+
 extern "C" {
 
 int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
@@ -663,43 +670,53 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     *out = nullptr;
     if (m < 0 || n < 0 || nnz < 0) return ASX_STATUS_INVALID_SIZE;
     if (value_type != ASX_R_32F && value_type != ASX_R_64F) return ASX_STATUS_NOT_SUPPORTED;
+    if (m > 0 && !d_row_ptr) return ASX_STATUS_INVALID_POINTER;
     const bool want = alg == ASX_SPMV_SLICED || alg == ASX_SPMV_WINDOW;
     if (want && (m == 0 || nnz == 0 || n == 0)) return ASX_STATUS_INVALID_SIZE;
     if (want && (!d_row_ptr || !d_col || !d_val)) return ASX_STATUS_INVALID_POINTER;
-    hipStream_t s = (hipStream_t)stream;
-    // histogram, sizes and (for DEFAULT) the row-ordered kernel the histogram picks
-    asx_plan *p = nullptr;
-    int st = asx_plan_create(&p, 0, want ? ASX_SPMV_VECTOR : alg, value_type, m, n, nnz, d_row_ptr, 1, stream);
-    if (st) return st;
-    if (alg == ASX_SPMV_WINDOW) {
-        st = value_type == ASX_R_64F ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
-                                     : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
-        if (st) {
-            asx_plan_destroy(p);
-            return st;
-        }
-        *out = p;
-        return ASX_STATUS_SUCCESS;
+    int row_kernel = -1;  // the row-ordered kernel to fall back to
+    if (alg != ASX_SPMV_DEFAULT && !want) {
+        row_kernel = asx_spmv_resolve_alg(alg, m, nnz);
+        if (row_kernel < 0) return ASX_STATUS_NOT_SUPPORTED;
     }
-    bool slices = alg == ASX_SPMV_SLICED;
-    if (alg == ASX_SPMV_DEFAULT && d_col && d_val && sliced_pays(p->hist, m, n, nnz, vsize(value_type)))
-        slices = sampled_line_spread(d_col, nnz, vsize(value_type), s) >= kScatteredMinSpread;
-    if (slices) {
-        st = value_type == ASX_R_64F ? plan_add_slices<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
-                                     : plan_add_slices<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
-        if (st && alg == ASX_SPMV_SLICED) {
-            asx_plan_destroy(p);
-            return st;
+    hipStream_t s = (hipStream_t)stream;
+    asx_plan *p = nullptr;
+    int st = plan_begin(&p, 0, value_type, m, n, nnz, d_row_ptr, 1, s);
+    if (st) return st;
+    if (alg == ASX_SPMV_DEFAULT) row_kernel = choose_spmv_from_stats(p->hist, p->stats, m, nnz);
+    const bool f64 = value_type == ASX_R_64F;
+    const bool can_regroup = alg == ASX_SPMV_DEFAULT && d_col && d_val && m > 0 && n > 0 && nnz >= kSlicedMinNnz;
+    bool done = false;
+    if (alg == ASX_SPMV_WINDOW) {
+        st = f64 ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
+                 : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
+        done = true;
+    } else if (alg == ASX_SPMV_SLICED) {
+        st = f64 ? plan_add_slices<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
+                 : plan_add_slices<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
+        done = true;
+    } else if (can_regroup) {
+        // DEFAULT: a regrouped copy where it pays; a build that fails (out of memory, a matrix the
+        // kernel does not take) is not an error: the row-ordered plan stands
+        bool slices = false;
+        if (sliced_pays(p->hist, m, n, nnz, vsize(value_type)))
+            slices = sampled_line_spread(d_col, nnz, vsize(value_type), reinterpret_cast<int32_t *>(p->d_counters + 64), s) >=
+                     kScatteredMinSpread;
+        if (slices) {
+            done = (f64 ? plan_add_slices<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
+                        : plan_add_slices<float>(p, d_row_ptr, d_col, (const float *)d_val, s)) == ASX_STATUS_SUCCESS;
+        } else if (window_may_pay(p, row_kernel)) {
+            // rows that reach only nearby columns: row blocks with a sliding window of x in LDS (measured
+            // 23 % faster than the flat kernel on the 5-point stencil, 20 % on a band of 19); the build
+            // reports NOT_SUPPORTED when some 256 rows reach further than a window
+            done = (f64 ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
+                        : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, s)) == ASX_STATUS_SUCCESS;
         }
-        // DEFAULT: no slices (out of memory, ...) is not an error; the row-ordered plan stands
-    } else if (alg == ASX_SPMV_DEFAULT && d_col && d_val && nnz >= kSlicedMinNnz && p->stats[0] <= kWindowMaxRow &&
-               (p->alg == ASX_SPMV_FLAT || p->alg == ASX_SPMV_MERGE)) {
-        // rows that reach only nearby columns: row blocks with a sliding window of x in LDS (measured
-        // 23 % faster than the flat kernel on the 5-point stencil, 20 % on a band of 19); the build
-        // reports NOT_SUPPORTED when some 256 rows reach further than a window, and then, as after
-        // any other failure, the row-ordered plan stands
-        (void)(value_type == ASX_R_64F ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
-                                       : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, s));
+    }
+    if (!done) st = plan_row_ordered(p, row_kernel, s);
+    if (st) {
+        asx_plan_destroy(p);
+        return st;
     }
     *out = p;
     return ASX_STATUS_SUCCESS;

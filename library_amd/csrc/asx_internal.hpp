@@ -52,8 +52,9 @@ int launch_loadbalance_partition(const int32_t *d_row_ptr, int32_t m, int32_t nn
 int launch_stream_row_blocks(const int32_t *d_row_ptr, int32_t m, int32_t nnz, int32_t *d_blocks,
                              hipStream_t s);
 int launch_copy_bytes(const void *d_src, void *d_dst, size_t bytes, hipStream_t s);
-int launch_sample_tiles(const int32_t *d_src, int64_t stride, int32_t tile, int32_t samples, int32_t *d_out,
-                        hipStream_t s);
+int launch_fill_i32(int32_t *d_dst, int64_t n, int32_t value, hipStream_t s);
+int launch_sample_distinct(const int32_t *d_src, int64_t stride, int shift, int32_t samples, int32_t *d_out,
+                           hipStream_t s);
 int launch_gather_lines(const void *d_buf, size_t bytes, int group_lanes, int per_lane, void *d_out, int *nthreads,
                         hipStream_t s);
 
@@ -134,6 +135,7 @@ struct SlicedMatrix {
     int32_t nwg;            // workgroups of pass 1
     int32_t rows_per_wave;  // pass 2
     int32_t nrb;            // ceil(m / rows_per_wave)
+    void *store;            // one allocation: val, perm, cf, tile_base, wg_tab, chunk_lo, pstep_ptr
     void *val;              // ntiles * kSlicedTile values (a copy of A's, in slice order; pads are 0)
     void *partial;          // npartials + kSlicedReducePad values: the partial sums of one call, for callers
                             // that bring no buffer of their own (null once released)
@@ -175,6 +177,8 @@ struct WindowMatrix {
     int32_t ntiles;
     int32_t nbands;          // 1: one window per block; 2..kWindowBands: bands of diagonals
     int has_carry;           // some tile starts inside a row: the ordered carry pass is needed
+    void *store;             // one allocation: val, perm, cf, tile_info
+    void *tables;            // one allocation: blocks, pieces, chains
     void *val;               // ntiles * kSlicedTile values (a copy of A's; pads are 0)
     void *carry;             // ntiles values: the carries of one call, for callers that bring no buffer (null once released)
     uint16_t *cf;            // ntiles * kSlicedTile: LDS slot of the column, bit 15 = first slot of a row (or tile)
@@ -202,6 +206,7 @@ inline int32_t spmm_segments(int32_t m, int32_t nnz) { return (int32_t)ceil_div6
 
 }  // namespace asx
 
+constexpr int kPlanCounters = 128;
 // Plan: analysis results kept on the device across calls.
 struct asx_plan {
     int is_spmm;
@@ -209,6 +214,7 @@ struct asx_plan {
     int value_type;
     int32_t m, n, nnz, ncols;
     const int32_t *row_ptr;  // the device array the plan was built from (identity check only)
+    int64_t *d_counters;     // kPlanCounters words on the device: histogram (33), stats (4), a flag (40), 64 sample counts (64..95)
     int32_t *d_meta;         // split points / row blocks (layout depends on alg)
     size_t meta_bytes;
     int32_t nunits;  // tiles / row blocks / segments

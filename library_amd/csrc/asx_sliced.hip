@@ -612,10 +612,9 @@ __global__ __launch_bounds__(kWave) void k_sliced_reduce(int32_t m, int32_t nrb,
 
 void free_sliced(SlicedMatrix *p)
 {
-    for (void *q : {p->val, p->partial, (void *)p->cf, (void *)p->perm, (void *)p->tile_base, (void *)p->wg_tab,
-                    (void *)p->prow, (void *)p->chunk_lo, (void *)p->pstep_ptr, (void *)p->psteps})
+    for (void *q : {p->store, p->partial, (void *)p->prow, (void *)p->psteps})
         if (q) (void)hipFree(q);
-    p->val = p->partial = nullptr;
+    p->store = p->val = p->partial = nullptr;
     p->cf = p->prow = nullptr;
     p->perm = p->tile_base = p->wg_tab = p->chunk_lo = p->pstep_ptr = p->psteps = nullptr;
 }
@@ -701,58 +700,7 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
     sm.ntiles = tile_off[sm.nslices];
     slots = (int64_t)sm.ntiles * kSlicedTile;
     ASX_TRY(hipMemcpyAsync(d_tile_off, tile_off.data(), sizeof(int32_t) * tile_off.size(), hipMemcpyHostToDevice, s));
-    ASX_TRY(hipMalloc(&sm.val, sizeof(T) * (size_t)slots));
-    ASX_TRY(hipMalloc((void **)&sm.cf, sizeof(uint16_t) * (size_t)slots));
-    ASX_TRY(hipMalloc((void **)&sm.perm, sizeof(int32_t) * (size_t)slots));
-    // 3. every stored element to its slot; the pads behind every slice
-    {
-        const unsigned sgrid = (unsigned)(ceil_div64(nblocks, kXcds) * kXcds);
-#define ASX_SCATTER(MAXS)                                                                                              \
-    hipLaunchKernelGGL((k_sliced_scatter<T, MAXS>), dim3(sgrid), dim3(kSortThreads), 0, s, row_ptr, col, val, seg_row, m, \
-                       nnz, width, sm.nslices, nbits, nblocks, offs, d_tile_off, lrow, sm.cf, (T *)sm.val, sm.perm)
-        if (sm.nslices <= 256)
-            ASX_SCATTER(256);
-        else
-            ASX_SCATTER(kSlicedMaxSlices);
-#undef ASX_SCATTER
-        hipLaunchKernelGGL((k_sliced_pads<T>), dim3((unsigned)sm.nslices), dim3(kSlicedTile), 0, s, d_pstart, d_tile_off, lrow,
-                           sm.cf, (T *)sm.val, sm.perm);
-    }
-    // 4. partial sums: one per run start; tile_base = the run starts before each tile
-    {
-        const unsigned wgrid = (unsigned)ceil_div64((int64_t)sm.ntiles * kWave, kBlock);
-        ASX_TRY(hipMalloc((void **)&sm.tile_base, sizeof(int32_t) * ((size_t)sm.ntiles + 1)));
-        hipLaunchKernelGGL(k_sliced_tile_runs, dim3(wgrid), dim3(kBlock), 0, s, lrow, sm.ntiles, tile_cnt);
-        ASX_TRY_ST(launch_exclusive_scan_i32(tile_cnt, sm.tile_base, (int64_t)sm.ntiles + 1, tmp, s));
-        ASX_TRY(hipMemcpyAsync(&sm.npartials, sm.tile_base + sm.ntiles, sizeof(int32_t), hipMemcpyDeviceToHost, s));
-        ASX_TRY(hipMalloc((void **)&sm.chunk_lo, sizeof(int32_t) * (size_t)ncells));  // while the kernels run
-        ASX_TRY(hipMalloc((void **)&sm.pstep_ptr, sizeof(int32_t) * ((size_t)sm.nrb + 1)));
-        ASX_TRY(hipStreamSynchronize(s));
-        ASX_TRY(hipMalloc((void **)&sm.prow, sizeof(uint16_t) * ((size_t)sm.npartials + kSlicedReducePad)));
-        ASX_TRY(hipMemsetAsync(sm.prow + sm.npartials, 0, sizeof(uint16_t) * kSlicedReducePad, s));
-        // 5. rows of the partial sums, run-start bits, and where each row block starts inside each slice
-        hipLaunchKernelGGL(k_sliced_emit, dim3(wgrid), dim3(kBlock), 0, s, lrow, sm.tile_base, d_tile_off, sm.ntiles,
-                           sm.nslices, rows_per_wave, sm.nrb, sm.cf, sm.prow, sm.chunk_lo);
-        if (empty_slice)
-            hipLaunchKernelGGL(k_sliced_empty_slices, dim3((unsigned)ceil_div64(ncells, kBlock)), dim3(kBlock), 0, s,
-                               sm.tile_base, d_tile_off, sm.nslices, sm.nrb, sm.chunk_lo);
-    }
-    // 6. the steps in which pass 2 reads each row block's ranges
-    {
-        const unsigned pgrid = (unsigned)ceil_div64((int64_t)sm.nrb * kWave, kBlock);
-        ASX_TRY(hipMemsetAsync(step_cnt + sm.nrb, 0, sizeof(int32_t), s));
-        hipLaunchKernelGGL(k_sliced_pack, dim3(pgrid), dim3(kBlock), 0, s, sm.chunk_lo, sm.nrb, sm.nslices, nullptr, step_cnt,
-                           nullptr);
-        ASX_TRY_ST(launch_exclusive_scan_i32(step_cnt, sm.pstep_ptr, (int64_t)sm.nrb + 1, tmp, s));
-        ASX_TRY(hipMemcpyAsync(&sm.npsteps, sm.pstep_ptr + sm.nrb, sizeof(int32_t), hipMemcpyDeviceToHost, s));
-        ASX_TRY(hipMalloc(&sm.partial, sizeof(T) * ((size_t)sm.npartials + kSlicedReducePad)));  // while the kernels run
-        ASX_TRY(hipStreamSynchronize(s));
-        ASX_TRY(hipMalloc((void **)&sm.psteps, sizeof(int32_t) * 4 * ((size_t)sm.npsteps + kSlicedStepPad)));
-        ASX_TRY(hipMemsetAsync(sm.psteps + 4 * (size_t)sm.npsteps, 0, sizeof(int32_t) * 4 * kSlicedStepPad, s));
-        hipLaunchKernelGGL(k_sliced_pack, dim3(pgrid), dim3(kBlock), 0, s, sm.chunk_lo, sm.nrb, sm.nslices, sm.pstep_ptr,
-                           nullptr, reinterpret_cast<i32x4 *>(sm.psteps));
-    }
-    // 7. workgroups of pass 1: every slice gets its share of about `target_wgs` workgroups (at
+    //    workgroups of pass 1: every slice gets its share of about `target_wgs` workgroups (at
     //    least one, and no workgroup smaller than 32 tiles unless the slice is), its tiles in equal
     //    pieces
     {
@@ -782,8 +730,69 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
             }
             tab.swap(placed);
         }
-        ASX_TRY(hipMalloc((void **)&sm.wg_tab, sizeof(int32_t) * std::max<size_t>(tab.size(), 4)));
+    }
+    {   // what the plan keeps and whose size is known by now, in one allocation
+        size_t off = 0;
+        const auto take = [&off](size_t bytes) {
+            const size_t at = off;
+            off += align_up(bytes, 256);
+            return at;
+        };
+        const size_t o_val = take(sizeof(T) * (size_t)slots), o_perm = take(sizeof(int32_t) * (size_t)slots);
+        const size_t o_cf = take(sizeof(uint16_t) * (size_t)slots), o_tb = take(sizeof(int32_t) * ((size_t)sm.ntiles + 1));
+        const size_t o_wg = take(sizeof(int32_t) * std::max<size_t>(tab.size(), 4));
+        const size_t o_cl = take(sizeof(int32_t) * (size_t)ncells), o_sp = take(sizeof(int32_t) * ((size_t)sm.nrb + 1));
+        ASX_TRY(hipMalloc(&sm.store, off));
+        char *base = static_cast<char *>(sm.store);
+        sm.val = base + o_val, sm.perm = (int32_t *)(base + o_perm), sm.cf = (uint16_t *)(base + o_cf);
+        sm.tile_base = (int32_t *)(base + o_tb), sm.wg_tab = (int32_t *)(base + o_wg);
+        sm.chunk_lo = (int32_t *)(base + o_cl), sm.pstep_ptr = (int32_t *)(base + o_sp);
         ASX_TRY(hipMemcpyAsync(sm.wg_tab, tab.data(), sizeof(int32_t) * tab.size(), hipMemcpyHostToDevice, s));
+    }
+    // 3. every stored element to its slot; the pads behind every slice
+    {
+        const unsigned sgrid = (unsigned)(ceil_div64(nblocks, kXcds) * kXcds);
+#define ASX_SCATTER(MAXS)                                                                                              \
+    hipLaunchKernelGGL((k_sliced_scatter<T, MAXS>), dim3(sgrid), dim3(kSortThreads), 0, s, row_ptr, col, val, seg_row, m, \
+                       nnz, width, sm.nslices, nbits, nblocks, offs, d_tile_off, lrow, sm.cf, (T *)sm.val, sm.perm)
+        if (sm.nslices <= 256)
+            ASX_SCATTER(256);
+        else
+            ASX_SCATTER(kSlicedMaxSlices);
+#undef ASX_SCATTER
+        hipLaunchKernelGGL((k_sliced_pads<T>), dim3((unsigned)sm.nslices), dim3(kSlicedTile), 0, s, d_pstart, d_tile_off, lrow,
+                           sm.cf, (T *)sm.val, sm.perm);
+    }
+    // 4. partial sums: one per run start; tile_base = the run starts before each tile
+    {
+        const unsigned wgrid = (unsigned)ceil_div64((int64_t)sm.ntiles * kWave, kBlock);
+        hipLaunchKernelGGL(k_sliced_tile_runs, dim3(wgrid), dim3(kBlock), 0, s, lrow, sm.ntiles, tile_cnt);
+        ASX_TRY_ST(launch_exclusive_scan_i32(tile_cnt, sm.tile_base, (int64_t)sm.ntiles + 1, tmp, s));
+        ASX_TRY(hipMemcpyAsync(&sm.npartials, sm.tile_base + sm.ntiles, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+        ASX_TRY(hipStreamSynchronize(s));
+        ASX_TRY(hipMalloc((void **)&sm.prow, sizeof(uint16_t) * ((size_t)sm.npartials + kSlicedReducePad)));
+        ASX_TRY(hipMemsetAsync(sm.prow + sm.npartials, 0, sizeof(uint16_t) * kSlicedReducePad, s));
+        // 5. rows of the partial sums, run-start bits, and where each row block starts inside each slice
+        hipLaunchKernelGGL(k_sliced_emit, dim3(wgrid), dim3(kBlock), 0, s, lrow, sm.tile_base, d_tile_off, sm.ntiles,
+                           sm.nslices, rows_per_wave, sm.nrb, sm.cf, sm.prow, sm.chunk_lo);
+        if (empty_slice)
+            hipLaunchKernelGGL(k_sliced_empty_slices, dim3((unsigned)ceil_div64(ncells, kBlock)), dim3(kBlock), 0, s,
+                               sm.tile_base, d_tile_off, sm.nslices, sm.nrb, sm.chunk_lo);
+    }
+    // 6. the steps in which pass 2 reads each row block's ranges
+    {
+        const unsigned pgrid = (unsigned)ceil_div64((int64_t)sm.nrb * kWave, kBlock);
+        ASX_TRY(hipMemsetAsync(step_cnt + sm.nrb, 0, sizeof(int32_t), s));
+        hipLaunchKernelGGL(k_sliced_pack, dim3(pgrid), dim3(kBlock), 0, s, sm.chunk_lo, sm.nrb, sm.nslices, nullptr, step_cnt,
+                           nullptr);
+        ASX_TRY_ST(launch_exclusive_scan_i32(step_cnt, sm.pstep_ptr, (int64_t)sm.nrb + 1, tmp, s));
+        ASX_TRY(hipMemcpyAsync(&sm.npsteps, sm.pstep_ptr + sm.nrb, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+        ASX_TRY(hipMalloc(&sm.partial, sizeof(T) * ((size_t)sm.npartials + kSlicedReducePad)));  // while the kernels run
+        ASX_TRY(hipStreamSynchronize(s));
+        ASX_TRY(hipMalloc((void **)&sm.psteps, sizeof(int32_t) * 4 * ((size_t)sm.npsteps + kSlicedStepPad)));
+        ASX_TRY(hipMemsetAsync(sm.psteps + 4 * (size_t)sm.npsteps, 0, sizeof(int32_t) * 4 * kSlicedStepPad, s));
+        hipLaunchKernelGGL(k_sliced_pack, dim3(pgrid), dim3(kBlock), 0, s, sm.chunk_lo, sm.nrb, sm.nslices, sm.pstep_ptr,
+                           nullptr, reinterpret_cast<i32x4 *>(sm.psteps));
     }
     ASX_TRY(hipStreamSynchronize(s));
     ASX_TRY(hipGetLastError());

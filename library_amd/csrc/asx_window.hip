@@ -39,55 +39,64 @@ constexpr int kWindowSlack = 8;       // a block's window is kept this much narr
 constexpr int kWindowWaves = 16;
 constexpr int32_t kAlignRowLen = 16;  // rows up to this length are not cut by tile starts
 
-// first and last column of every row (cmin = kNoCol, cmax = -1 for an empty row)
-__global__ __launch_bounds__(kBlock) void k_window_row_span(const int32_t *__restrict__ row_ptr,
-                                                            const int32_t *__restrict__ col, int32_t m,
-                                                            int32_t *__restrict__ cmin, int32_t *__restrict__ cmax)
-{
-    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (r >= m) return;
-    int32_t lo = kNoCol, hi = -1;
-    for (int32_t k = row_ptr[r]; k < row_ptr[r + 1]; ++k) {
-        const int32_t c = col[k];
-        lo = c < lo ? c : lo;
-        hi = c > hi ? c : hi;
-    }
-    cmin[r] = lo;
-    cmax[r] = hi;
-}
+constexpr int kSpanGroup = 128;  // rows per group of the column-span table; every block size is a multiple
 
-// bmin / bmax of every block of `rows` rows (bmin preset to kNoCol, bmax to -1)
-__global__ __launch_bounds__(kBlock) void k_window_block_span(const int32_t *__restrict__ cmin,
-                                                              const int32_t *__restrict__ cmax, int32_t m,
-                                                              int32_t rows, int32_t *__restrict__ bmin,
-                                                              int32_t *__restrict__ bmax)
+// first and last column of every group of kSpanGroup consecutive rows (gmin = kNoCol, gmax = -1 for
+// a group without stored elements); one wave per group, two rows per lane
+__global__ __launch_bounds__(kBlock) void k_window_group_span(const int32_t *__restrict__ row_ptr,
+                                                              const int32_t *__restrict__ col, int32_t m,
+                                                              int32_t ngroups, int32_t *__restrict__ gmin,
+                                                              int32_t *__restrict__ gmax)
 {
-    // `rows` is a multiple of 256, so the 64 rows of a wave lie in one block: one pair of atomics a wave
-    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t g = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+    if (g >= ngroups) return;  // whole waves leave
     int32_t lo = kNoCol, hi = -1;
-    if (r < m && cmax[r] >= 0) lo = cmin[r], hi = cmax[r];
+#pragma unroll
+    for (int h = 0; h < kSpanGroup / kWave; ++h) {
+        const int64_t r = g * kSpanGroup + h * kWave + lane;
+        if (r < m)
+            for (int32_t k = row_ptr[r]; k < row_ptr[r + 1]; ++k) {
+                const int32_t c = col[k];
+                lo = c < lo ? c : lo;
+                hi = c > hi ? c : hi;
+            }
+    }
 #pragma unroll
     for (int d = 1; d < kWave; d <<= 1) {
         lo = min(lo, __shfl_xor(lo, d, kWave));
         hi = max(hi, __shfl_xor(hi, d, kWave));
     }
-    if (__lane_id() != 0 || hi < 0) return;
-    atomicMin(bmin + r / rows, lo);
-    atomicMax(bmax + r / rows, hi);
+    if (lane == 0) {
+        gmin[g] = lo;
+        gmax[g] = hi;
+    }
+}
+// Column span of every block of `per` groups; bmin / bmax are written when given; *widest receives
+// (atomic max; preset to 0) the widest window a block needs once its start is rounded down to a
+// multiple of 4 columns.
+__global__ __launch_bounds__(kBlock) void k_window_block_span(const int32_t *__restrict__ gmin,
+                                                              const int32_t *__restrict__ gmax, int32_t ngroups,
+                                                              int32_t per, int32_t nblocks, int32_t *__restrict__ bmin,
+                                                              int32_t *__restrict__ bmax, int32_t *__restrict__ widest)
+{
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    int32_t lo = kNoCol, hi = -1;
+    for (int64_t g = b * per; g < (b + 1) * per && g < ngroups; ++g) {
+        lo = min(lo, gmin[g]);
+        hi = max(hi, gmax[g]);
+    }
+    if (bmin) {
+        bmin[b] = lo;
+        bmax[b] = hi;
+    }
+    if (hi >= 0) atomicMax(widest, hi - (lo & ~3) + 1);
 }
 __global__ __launch_bounds__(kBlock) void k_window_fill_i32(int32_t *p, int64_t n, int32_t v)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
-}
-// widest window any block needs once its start is rounded down to a multiple of 4 columns
-__global__ __launch_bounds__(kBlock) void k_window_max_span(const int32_t *__restrict__ bmin,
-                                                            const int32_t *__restrict__ bmax, int32_t nblocks,
-                                                            int32_t *__restrict__ out)
-{
-    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (b >= nblocks || bmax[b] < 0) return;
-    atomicMax(out, bmax[b] - (bmin[b] & ~3) + 1);
 }
 
 // Slot (from the start of its block) at which every row starts, and the tiles of every block.  A
@@ -140,15 +149,31 @@ __global__ __launch_bounds__(kBlock) void k_window_row_starts(const int32_t *__r
     if (lane == 0) block_tiles[b] = (pos + kSlicedTile - 1) / kSlicedTile;
 }
 
+// The slots that hold no stored element: the slot of an empty row, the slots between a row's end
+// and the start of the next one where that row was moved to a tile start, and the tail of a
+// block's last tile.  Each is a zero that points at the zero behind the rings and opens a run of
+// its own.  One thread per row fills what follows its own stored elements.
 template <typename T>
-__global__ __launch_bounds__(kBlock) void k_window_fill_pads(int64_t slots, uint16_t pad, uint16_t *__restrict__ cf,
-                                                             T *__restrict__ val, int32_t *__restrict__ perm)
+__global__ __launch_bounds__(kBlock) void k_window_pads(const int32_t *__restrict__ row_ptr, int32_t m, int32_t rows,
+                                                        const int32_t *__restrict__ row_start,
+                                                        const int32_t *__restrict__ tile_off, uint16_t pad,
+                                                        uint16_t *__restrict__ cf, T *__restrict__ val,
+                                                        int32_t *__restrict__ perm)
 {
-    const int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (d >= slots) return;
-    cf[d] = pad;
-    val[d] = T(0);
-    perm[d] = -1;
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= m) return;
+    const int64_t b = r / rows;
+    const int64_t last = (b + 1) * rows < m ? (b + 1) * rows : m;  // one past the block's last row
+    const int32_t from = row_start[r] + (row_ptr[r + 1] - row_ptr[r]);
+    const int32_t to = r + 1 < last ? row_start[r + 1] : (tile_off[b + 1] - tile_off[b]) * kSlicedTile;
+    const int64_t base = (int64_t)tile_off[b] * kSlicedTile;
+    for (int32_t o = from; o < to; ++o) {
+        const int64_t d = base + o;
+        const int64_t phys = d / kSlicedTile * kSlicedTile + tile_val_pos<T>((int)(d % kSlicedTile));
+        cf[d] = pad;
+        val[phys] = T(0);
+        perm[phys] = -1;
+    }
 }
 
 // Where the columns of x live in LDS.  One band (nbands = 1): column c at c mod kWindowCols.
@@ -182,13 +207,17 @@ template <typename T>
 __global__ __launch_bounds__(kBlock) void k_window_place(const int32_t *__restrict__ row_ptr,
                                                          const int32_t *__restrict__ col, const T *__restrict__ val,
                                                          int32_t m, int32_t n, int32_t nnz, int32_t rows, BandTable bands,
+                                                         const int32_t *__restrict__ seg_row,
                                                          const int32_t *__restrict__ row_start,
                                                          const int32_t *__restrict__ tile_off, uint16_t *__restrict__ cf,
                                                          T *__restrict__ val_out, int32_t *__restrict__ perm)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= nnz) return;
-    int32_t lo = 0, hi = m;  // row holding stored element i: largest r with row_ptr[r] <= i
+    // row holding stored element i: largest r with row_ptr[r] <= i; the workgroup's kBlock elements
+    // lie in rows seg_row[blockIdx.x] .. seg_row[blockIdx.x + 1]
+    int32_t lo = seg_row[blockIdx.x], hi = seg_row[blockIdx.x + 1];
+    hi = hi > m - 1 ? m - 1 : hi;
     while (lo < hi) {
         const int32_t mid = lo + (hi - lo + 1) / 2;
         if (row_ptr[mid] <= i)
@@ -525,10 +554,9 @@ __global__ __launch_bounds__(kBlock) void k_window_fixup(int32_t ntiles, T alpha
 
 void free_window(WindowMatrix *p)
 {
-    for (void *q : {p->val, p->carry, (void *)p->cf, (void *)p->perm, (void *)p->tile_info, (void *)p->blocks,
-                    (void *)p->pieces, (void *)p->chains})
+    for (void *q : {p->store, p->tables, p->carry})
         if (q) (void)hipFree(q);
-    p->val = p->carry = nullptr;
+    p->store = p->tables = p->val = p->carry = nullptr;
     p->cf = nullptr;
     p->perm = p->tile_info = p->blocks = p->pieces = p->chains = nullptr;
 }
@@ -542,7 +570,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     if (target_wgs < 1) return ASX_STATUS_INVALID_VALUE;
     int st = ASX_STATUS_SUCCESS;
     int32_t *arena = nullptr;
-    int32_t *cmin = nullptr, *cmax = nullptr, *row_start = nullptr;  // m each
+    int32_t *gmin = nullptr, *gmax = nullptr, *row_start = nullptr, *seg_row = nullptr;
     int32_t *bmin = nullptr, *bmax = nullptr, *btiles = nullptr, *tile_off = nullptr, *d_small = nullptr;
     int32_t *tmp = nullptr;
     std::vector<int32_t> h_bmin, h_bmax, h_off, blk, pcs, chains;
@@ -550,44 +578,60 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     uint32_t *d_bits = nullptr;
     BandTable bands{};
     int64_t slots = 0;
-    int32_t h_small[2] = {0, 0};
+    constexpr int kCandidates = 11;
+    static const int32_t kBlockRows[kCandidates] = {8192, 6144, 4096, 3072, 2048, 1536, 1024, 768, 512, 384, 256};
+    int32_t h_small[16] = {0};
     const unsigned mgrid = (unsigned)ceil_div64(m, kBlock);
     const int32_t min_blocks = 4 * target_wgs;  // larger blocks only while at least this many blocks remain
     const int32_t max_nb = (int32_t)ceil_div64(m, 256);
+    const int32_t ngroups = (int32_t)ceil_div64(m, kSpanGroup);
+    const int32_t nseg = (int32_t)ceil_div64(nnz, kBlock);
 #define ASX_TRY(expr)         \
     do {                      \
         st = status_of(expr); \
         if (st) goto done;    \
     } while (0)
-    // the scratch of the build in one allocation: three arrays of m ints, four of max_nb + 1, two
-    // counters, the scan's block sums
+    // the scratch of the build in one allocation: the span of every group of rows (two arrays), where
+    // every row starts, the row holding every 256th stored element, four arrays of max_nb + 1, a
+    // few counters, the scan's block sums
     {
-        const size_t per_row = ((size_t)m + 63) & ~(size_t)63, per_block = ((size_t)max_nb + 1 + 63) & ~(size_t)63;
-        ASX_TRY(hipMalloc((void **)&arena, sizeof(int32_t) * (3 * per_row + 4 * per_block + 64 + scan_scratch_ints((int64_t)max_nb + 1))));
-        cmin = arena, cmax = cmin + per_row, row_start = cmax + per_row;
-        bmin = row_start + per_row, bmax = bmin + per_block, btiles = bmax + per_block, tile_off = btiles + per_block;
+        const auto pad64 = [](size_t v) { return (v + 63) & ~(size_t)63; };
+        const size_t per_group = pad64((size_t)ngroups), per_row = pad64((size_t)m), per_seg = pad64((size_t)nseg + 1);
+        const size_t per_block = pad64((size_t)max_nb + 1);
+        ASX_TRY(hipMalloc((void **)&arena, sizeof(int32_t) * (2 * per_group + per_row + per_seg + 4 * per_block + 64 +
+                                                              scan_scratch_ints((int64_t)max_nb + 1))));
+        gmin = arena, gmax = gmin + per_group, row_start = gmax + per_group, seg_row = row_start + per_row;
+        bmin = seg_row + per_seg, bmax = bmin + per_block, btiles = bmax + per_block, tile_off = btiles + per_block;
         d_small = tile_off + per_block;
         tmp = d_small + 64;
     }
 
-    // 1. column span of every row
-    hipLaunchKernelGGL(k_window_row_span, dim3(mgrid), dim3(kBlock), 0, s, row_ptr, col, m, cmin, cmax);
-    // 2. the largest block of rows (a multiple of 256) whose widest window fits the ring
-    wm.rows_per_block = 0;
-    for (int32_t rows : {8192, 6144, 4096, 3072, 2048, 1536, 1024, 768, 512, 384, 256}) {
+    // 1. column span of every group of rows
+    hipLaunchKernelGGL(k_window_group_span, dim3((unsigned)ceil_div64((int64_t)ngroups * kWave, kBlock)), dim3(kBlock), 0, s,
+                       row_ptr, col, m, ngroups, gmin, gmax);
+    // 2. the largest block of rows whose widest window fits the ring: the widest window of every
+    //    candidate size, all read back at once
+    hipLaunchKernelGGL(k_window_fill_i32, dim3(1), dim3(kBlock), 0, s, d_small, (int64_t)16, 0);
+    for (int k = 0; k < kCandidates; ++k) {
+        const int32_t rows = kBlockRows[k];
         if (rows > 256 && ceil_div64(m, rows) < min_blocks) continue;  // too few blocks to share out
         const int32_t nb = (int32_t)ceil_div64(m, rows);
-        const unsigned bgrid = (unsigned)ceil_div64(nb, kBlock);
-        hipLaunchKernelGGL(k_window_fill_i32, dim3(bgrid), dim3(kBlock), 0, s, bmin, (int64_t)nb, kNoCol);
-        hipLaunchKernelGGL(k_window_fill_i32, dim3(bgrid), dim3(kBlock), 0, s, bmax, (int64_t)nb, -1);
-        ASX_TRY(hipMemsetAsync(d_small, 0, sizeof(int32_t) * 2, s));
-        hipLaunchKernelGGL(k_window_block_span, dim3(mgrid), dim3(kBlock), 0, s, cmin, cmax, m, rows, bmin, bmax);
-        hipLaunchKernelGGL(k_window_max_span, dim3(bgrid), dim3(kBlock), 0, s, bmin, bmax, nb, d_small);
-        ASX_TRY(hipMemcpyAsync(h_small, d_small, sizeof(int32_t), hipMemcpyDeviceToHost, s));
-        ASX_TRY(hipStreamSynchronize(s));
-        if (h_small[0] <= kWindowCols - kWindowSlack) {
+        hipLaunchKernelGGL(k_window_block_span, dim3((unsigned)ceil_div64(nb, kBlock)), dim3(kBlock), 0, s, gmin, gmax, ngroups,
+                           rows / kSpanGroup, nb, (int32_t *)nullptr, (int32_t *)nullptr, d_small + k);
+    }
+    st = launch_nnz_split_rows(row_ptr, m, nnz, kBlock, seg_row, s);  // for step 4; runs while the host waits
+    if (st) goto done;
+    ASX_TRY(hipMemcpyAsync(h_small, d_small, sizeof(int32_t) * kCandidates, hipMemcpyDeviceToHost, s));
+    ASX_TRY(hipStreamSynchronize(s));
+    wm.rows_per_block = 0;
+    for (int k = 0; k < kCandidates; ++k) {
+        const int32_t rows = kBlockRows[k];
+        if (rows > 256 && ceil_div64(m, rows) < min_blocks) continue;
+        if (h_small[k] <= kWindowCols - kWindowSlack) {
             wm.rows_per_block = rows;
-            wm.nblocks = nb;
+            wm.nblocks = (int32_t)ceil_div64(m, rows);
+            hipLaunchKernelGGL(k_window_block_span, dim3((unsigned)ceil_div64(wm.nblocks, kBlock)), dim3(kBlock), 0, s, gmin,
+                               gmax, ngroups, rows / kSpanGroup, wm.nblocks, bmin, bmax, d_small + 15);
             break;
         }
     }
@@ -677,20 +721,24 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
         st = ASX_STATUS_INVALID_SIZE;
         goto done;
     }
-    ASX_TRY(hipMalloc(&wm.val, sizeof(T) * (size_t)slots));
-    ASX_TRY(hipMalloc((void **)&wm.cf, sizeof(uint16_t) * (size_t)slots));
-    ASX_TRY(hipMalloc((void **)&wm.perm, sizeof(int32_t) * (size_t)slots));
-    ASX_TRY(hipMalloc((void **)&wm.tile_info, sizeof(int2) * (size_t)wm.ntiles));
+    {   // the regrouped copy in one allocation
+        const size_t o_val = 0, o_perm = align_up(sizeof(T) * (size_t)slots, 256);
+        const size_t o_cf = o_perm + align_up(sizeof(int32_t) * (size_t)slots, 256);
+        const size_t o_info = o_cf + align_up(sizeof(uint16_t) * (size_t)slots, 256);
+        ASX_TRY(hipMalloc(&wm.store, o_info + sizeof(int2) * (size_t)wm.ntiles));
+        char *base = static_cast<char *>(wm.store);
+        wm.val = base + o_val, wm.perm = (int32_t *)(base + o_perm), wm.cf = (uint16_t *)(base + o_cf);
+        wm.tile_info = (int32_t *)(base + o_info);
+    }
     ASX_TRY(hipMalloc(&wm.carry, sizeof(T) * (size_t)wm.ntiles));
-    ASX_TRY(hipMemsetAsync(wm.carry, 0, sizeof(T) * (size_t)wm.ntiles, s));
-    // 4. every slot starts as a zero that points at the zero behind the ring and opens a run of its
-    //    own (the slots of empty rows and the padding stay that way)
-    hipLaunchKernelGGL((k_window_fill_pads<T>), dim3((unsigned)ceil_div64(slots, kBlock)), dim3(kBlock), 0, s, slots,
-                       (uint16_t)(0x8000 | kWindowCols), wm.cf, (T *)wm.val, wm.perm);
+    // 4. every stored element to its slot; every other slot becomes a zero that points at the zero
+    //    behind the rings and opens a run of its own
     hipLaunchKernelGGL((k_window_place<T>), dim3((unsigned)ceil_div64(nnz, kBlock)), dim3(kBlock), 0, s, row_ptr, col, val,
-                       m, n, nnz, wm.rows_per_block, bands, row_start, tile_off, wm.cf, (T *)wm.val, wm.perm);
+                       m, n, nnz, wm.rows_per_block, bands, seg_row, row_start, tile_off, wm.cf, (T *)wm.val, wm.perm);
+    hipLaunchKernelGGL((k_window_pads<T>), dim3(mgrid), dim3(kBlock), 0, s, row_ptr, m, wm.rows_per_block, row_start, tile_off,
+                       (uint16_t)(0x8000 | kWindowCols), wm.cf, (T *)wm.val, wm.perm);
     // 5. first row and number of rows of every tile
-    ASX_TRY(hipMemsetAsync(d_small, 0, sizeof(int32_t) * 2, s));
+    hipLaunchKernelGGL(k_window_fill_i32, dim3(1), dim3(kBlock), 0, s, d_small, (int64_t)2, 0);
     hipLaunchKernelGGL(k_window_tile_info, dim3((unsigned)ceil_div64(wm.ntiles, kBlock)), dim3(kBlock), 0, s, row_start, m,
                        wm.rows_per_block, wm.nblocks, tile_off, wm.ntiles, (int2 *)wm.tile_info, d_small);
     ASX_TRY(hipMemcpyAsync(h_small, d_small, sizeof(int32_t), hipMemcpyDeviceToHost, s));
@@ -766,10 +814,14 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
         wm.nchains = (int32_t)(chains.size() / 2);
         wm.npieces = (int32_t)(pcs.size() / 4);
     }
-    ASX_TRY(hipMalloc((void **)&wm.pieces, sizeof(int32_t) * pcs.size()));
+    {   // the tables of the blocks in one allocation (16-byte entries first)
+        const size_t o_pieces = align_up(sizeof(int32_t) * blk.size(), 256);
+        const size_t o_chains = o_pieces + align_up(sizeof(int32_t) * pcs.size(), 256);
+        ASX_TRY(hipMalloc(&wm.tables, o_chains + sizeof(int32_t) * chains.size()));
+        char *base = static_cast<char *>(wm.tables);
+        wm.blocks = (int32_t *)base, wm.pieces = (int32_t *)(base + o_pieces), wm.chains = (int32_t *)(base + o_chains);
+    }
     ASX_TRY(hipMemcpyAsync(wm.pieces, pcs.data(), sizeof(int32_t) * pcs.size(), hipMemcpyHostToDevice, s));
-    ASX_TRY(hipMalloc((void **)&wm.blocks, sizeof(int32_t) * blk.size()));
-    ASX_TRY(hipMalloc((void **)&wm.chains, sizeof(int32_t) * chains.size()));
     ASX_TRY(hipMemcpyAsync(wm.blocks, blk.data(), sizeof(int32_t) * blk.size(), hipMemcpyHostToDevice, s));
     ASX_TRY(hipMemcpyAsync(wm.chains, chains.data(), sizeof(int32_t) * chains.size(), hipMemcpyHostToDevice, s));
     ASX_TRY(hipStreamSynchronize(s));
