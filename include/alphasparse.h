@@ -413,6 +413,12 @@ alphasparseStatus_t alphasparse_spmv(alphasparseHandle_t handle, alphasparseOper
                                      alphasparse_dcu_spmv_alg_t alg, size_t *buffer_size,
                                      void *temp_buffer);
 
+// Not in the reference: the kernel the analysis kept on matA for (opA, algorithm, and for SpMM the
+// number of dense columns) runs as, e.g. "sliced", "window", "flat", "merge" - or "none" when no
+// analysis is kept (the call then picks a row-ordered kernel and recomputes its split points).
+const char *alphasparseAmdKeptKernel(alphasparseSpMatDescr_t matA, alphasparseOperation_t opA, int is_spmm, int alg,
+                                     int ncols);
+
 // ---- generic SpMM (include/alphasparse/spapi.h:6963-6974,7004-7028) ------------------------------
 alphasparseStatus_t alphasparseSpMM(alphasparseHandle_t handle, alphasparseOperation_t opA,
                                     alphasparseOperation_t opB, const void *alpha,

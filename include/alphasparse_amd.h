@@ -216,6 +216,9 @@ int asx_plan_holds_values(const asx_plan *plan);
 /* Number of 16x4 blocks and their fill of a blocked plan. */
 int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill);
 int asx_plan_destroy(asx_plan *plan);
+/* Short name of a kernel id (ASX_SPMV_* / ASX_SPMM_* value): "vector", "stream", "merge", "flat",
+ * "sliced", "window"; "row", "merge", "blocked"; "?" for anything else. */
+const char *asx_kernel_name(int is_spmm, int kernel);
 /* Kernel the plan resolved to, and bytes of per-call workspace its launches need (carries; for a
  * sliced plan the partial sums of a call, for a window plan with cut rows its carries).  A sliced
  * or window plan also keeps a buffer of that size of its own, used by calls whose workspace is

@@ -99,7 +99,8 @@ def build_library(verbose=False):
     spilling = sorted(n for n, r in resources.items() if r.get("ScratchSize", 0))
     if spilling:
         raise RuntimeError("kernels that spill registers to scratch memory: " + ", ".join(spilling))
-    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--version-script=" + os.path.join(CSRC, "exports.map"),
+          "-o", LIB, *objs])
     return LIB
 
 

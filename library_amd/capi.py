@@ -28,7 +28,7 @@ EXPORTS = [
     "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_coo2csr", "asx_coo_sort", "asx_csr_transpose", "asx_csr_rebase",
     "asx_dense_transpose", "asx_mtx_read", "asx_host_free", "asx_spmv_plan_create",
     "asx_plan_update_values", "asx_plan_holds_values", "asx_plan_info", "asx_plan_create",
-    "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_plan_workspace_bytes", "asx_plan_histogram",
+    "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_kernel_name", "asx_plan_workspace_bytes", "asx_plan_histogram",
     "asx_plan_release_scratch", "asx_plan_own_scratch_bytes", "asx_plan_export",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
     "asx_spmv_csr_f64_noalloc", "asx_spmv_noalloc_max_workspace",
@@ -80,6 +80,8 @@ def lib():
     L.asx_plan_block_stats.argtypes = [vp, C.POINTER(i64), C.POINTER(C.c_double)]
     L.asx_plan_destroy.argtypes = [vp]
     L.asx_plan_alg.argtypes = [vp]
+    L.asx_kernel_name.argtypes = [C.c_int, C.c_int]
+    L.asx_kernel_name.restype = C.c_char_p
     L.asx_plan_workspace_bytes.argtypes = [vp]
     L.asx_plan_workspace_bytes.restype = sz
     L.asx_plan_histogram.argtypes = [vp, vp, vp]

@@ -20,7 +20,9 @@
 #include <algorithm>
 #include <cstddef>
 #include <cstdlib>
+#include <mutex>
 #include <new>
+#include <unordered_set>
 #include <vector>
 
 #include "../../include/alphasparse.h"
@@ -115,6 +117,7 @@ struct KeptPlan {
     int value_type;
     int ncols;
     asx_plan *plan;
+    bool reads_callers_values_only;  // made by analysis on first use: never a regrouped copy of A's values
 };
 // A zero-based and/or transposed device copy of a caller's CSR matrix.
 struct DerivedCsr {
@@ -127,7 +130,6 @@ struct DerivedCsr {
     int *row_ptr, *col;
     void *val;  // owned only when transposed (otherwise the caller's values)
 };
-constexpr uint64_t kInfoMagic = 0x415358494e464f31ull;  // "ASXINFO1"
 // What alphasparseSpMV_bufferSize last reported for (matrix, algorithm): the size the caller's
 // externalBuffer is taken to have (its size is not part of alphasparseSpMV's signature).
 struct PromisedBuffer {
@@ -137,7 +139,6 @@ struct PromisedBuffer {
 struct MatInfoExt {
     _alphasparse_mat_info info;
     _alphasparse_csrmv_info csrmv;
-    uint64_t magic;
     alphasparseHandle_t owner;  // null once that handle is gone
     std::vector<KeptPlan> plans;
     std::vector<PromisedBuffer> promised;
@@ -151,10 +152,25 @@ HandleRegistry *registry_of(alphasparseHandle_t h, bool create)
     if (!h->pflat_analysis_data && create) h->pflat_analysis_data = new (std::nothrow) HandleRegistry();
     return (HandleRegistry *)h->pflat_analysis_data;
 }
+// The objects this library has put behind a matA->info, by address: a pointer found there is
+// only taken for one of them after it was looked up here (a caller compiled against the
+// reference's header may have put its own, smaller _alphasparse_mat_info there, which must not
+// be read past its end).
+struct LiveInfos {
+    std::mutex lock;
+    std::unordered_set<const void *> set;
+};
+LiveInfos &live_infos()
+{
+    static LiveInfos *l = new LiveInfos();  // never destroyed: descriptors may outlive static destructors
+    return *l;
+}
 MatInfoExt *ext_of(const _alphasparseSpMatDescr *A)
 {
-    MatInfoExt *e = (MatInfoExt *)A->info;
-    return e && e->magic == kInfoMagic ? e : nullptr;
+    if (!A->info) return nullptr;
+    LiveInfos &l = live_infos();
+    std::lock_guard<std::mutex> g(l.lock);
+    return l.set.count(A->info) ? (MatInfoExt *)A->info : nullptr;
 }
 // The matrix's store, made on first use (a foreign object already behind matA->info is left alone:
 // analysis then reports NOT_SUPPORTED).
@@ -177,8 +193,12 @@ MatInfoExt *ext_create(alphasparseHandle_t h, _alphasparseSpMatDescr *A)
     e->info = _alphasparse_mat_info{};
     e->csrmv = _alphasparse_csrmv_info{};
     e->info.csrmv_info = &e->csrmv;
-    e->magic = kInfoMagic;
     e->owner = h;
+    {
+        LiveInfos &l = live_infos();
+        std::lock_guard<std::mutex> g(l.lock);
+        l.set.insert(&e->info);
+    }
     reg->mats.push_back(e);
     A->info = &e->info;
     return e;
@@ -218,6 +238,24 @@ size_t promised_bytes(const _alphasparseSpMatDescr *A, int alg)
         for (const PromisedBuffer &p : e->promised)
             if (p.alg == alg) return p.bytes;
     return 0;
+}
+bool kept_is_restricted(const _alphasparseSpMatDescr *A, const asx_plan *plan)
+{
+    if (MatInfoExt *e = ext_of(A))
+        for (const KeptPlan &k : e->plans)
+            if (k.plan == plan) return k.reads_callers_values_only;
+    return false;
+}
+void drop_one_plan(const _alphasparseSpMatDescr *A, asx_plan *plan)
+{
+    MatInfoExt *e = ext_of(A);
+    if (!e) return;
+    for (size_t i = 0; i < e->plans.size(); ++i)
+        if (e->plans[i].plan == plan) {
+            asx_plan_destroy(plan);
+            e->plans.erase(e->plans.begin() + (long)i);
+            return;
+        }
 }
 void drop_plans(alphasparseHandle_t h, bool spmm, int alg, bool all)
 {
@@ -654,7 +692,11 @@ alphasparseStatus_t alphasparseDestroySpMat(alphasparseSpMatDescr_t descr)
                         reg->mats.erase(reg->mats.begin() + (long)i);
                         break;
                     }
-        e->magic = 0;
+        {
+            LiveInfos &l = live_infos();
+            std::lock_guard<std::mutex> g(l.lock);
+            l.set.erase(&e->info);
+        }
         delete e;
         descr->info = nullptr;
     }
@@ -711,22 +753,42 @@ alphasparseStatus_t alphasparseSpMV_bufferSize(alphasparseHandle_t handle, alpha
 
 // Analysis on first use, for callers written against the reference, where alphasparseSpMV_analysis
 // and alphasparseSpMM_preprocess are stubs or cheap and therefore often never called
-// (hip/kernel/level2/alphasparse_spmv.hip:229-256): with ALPHASPARSE_AMD_AUTO_ANALYSIS=1 in the
-// environment the first alphasparseSpMV / alphasparseSpMM on a descriptor runs the analysis itself
-// (allocates and synchronises once; later calls are kernels only).  Off by default, because kept
-// analysis may hold a copy of A's values that a caller who updates them in place would not know
-// to refresh.  Read once per process.
-static bool auto_analysis()
+// (hip/kernel/level2/alphasparse_spmv.hip:229-256; its own test loops go from _bufferSize straight to
+// the timed alphasparseSpMV, hip/test/level2/spmv_csr_r_f64_test.hip:183-198): the first
+// alphasparseSpMV / alphasparseSpMM on a descriptor runs an analysis itself (allocates and
+// synchronises once; later calls are kernels only).  ALPHASPARSE_AMD_AUTO_ANALYSIS selects how far
+// it goes; read once per process:
+//   unset, "structure"  only analysis that reads the caller's values in every call (split points
+//                       of the row-ordered kernels): sound whenever the row offsets and columns
+//                       behind a descriptor stay as they are, which holds for a caller who
+//                       changes values in place.  Not done for opA = TRANSPOSE (the kept copy of
+//                       the transposed matrix would hold values).
+//   "1", "values"       the full analysis, which may keep a regrouped copy of A's values: for callers
+//                       who do not change values in place without calling the analysis again
+//   "0", "off"          none: every call recomputes its split points, as the reference does
+enum AutoAnalysis { kAutoOff = 0, kAutoStructure = 1, kAutoValues = 2 };
+static AutoAnalysis auto_analysis()
 {
-    static const bool on = [] {
+    static const AutoAnalysis mode = [] {
         const char *e = std::getenv("ALPHASPARSE_AMD_AUTO_ANALYSIS");
-        return e && e[0] && e[0] != '0';
+        if (!e || !e[0] || e[0] == 's' || e[0] == 'S') return kAutoStructure;
+        if (e[0] == '0' || e[0] == 'o' || e[0] == 'O' || e[0] == 'n' || e[0] == 'N') return kAutoOff;
+        return kAutoValues;
     }();
-    return on;
+    return mode;
 }
+
+static alphasparseStatus_t spmv_analysis(alphasparseHandle_t handle, alphasparseOperation_t opA, alphasparseSpMatDescr_t matA,
+                                         alphasparseSpMVAlg_t alg, bool callers_values_only);
 
 alphasparseStatus_t alphasparseSpMV_analysis(alphasparseHandle_t handle, alphasparseOperation_t opA,
                                              alphasparseSpMatDescr_t matA, alphasparseSpMVAlg_t alg)
+{
+    return spmv_analysis(handle, opA, matA, alg, false);
+}
+
+static alphasparseStatus_t spmv_analysis(alphasparseHandle_t handle, alphasparseOperation_t opA, alphasparseSpMatDescr_t matA,
+                                         alphasparseSpMVAlg_t alg, bool callers_values_only)
 {
     if (!handle) return ALPHA_SPARSE_STATUS_INVALID_HANDLE;
     if (!matA) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
@@ -742,19 +804,24 @@ alphasparseStatus_t alphasparseSpMV_analysis(alphasparseHandle_t handle, alphasp
     const _alphasparseSpMatDescr *A = &eff.d;
     if (asx_plan *have = find_plan(matA, false, (int)alg, A, 1)) {
         // analysed before: the sparsity pattern is taken to be the same (alphasparseSpMV_clear first
-        // if it is not); a plan that holds a copy of the values picks up the current ones
-        return st(asx_plan_update_values(have, A->val_data, (void *)handle->stream));
+        // if it is not); a plan that holds a copy of the values picks up the current ones.  What
+        // analysis on first use left there makes way for the caller's own, full analysis.
+        if (callers_values_only || !kept_is_restricted(matA, have))
+            return st(asx_plan_update_values(have, A->val_data, (void *)handle->stream));
+        (void)hipStreamSynchronize(handle->stream);
+        drop_one_plan(matA, have);
     }
     MatInfoExt *x = ext_create(handle, matA);
     if (!x) return matA->info ? ALPHA_SPARSE_STATUS_NOT_SUPPORTED : ALPHA_SPARSE_STATUS_ALLOC_FAILED;
     asx_plan *plan = nullptr;
-    // may keep a regrouped copy of A's columns and values (column slices): call again after
-    // changing the values
+    // may keep a regrouped copy of A's columns and values (column slices, row blocks): call again
+    // after changing the values.  Without the columns and values the plan stays row-ordered.
     int rc = asx_spmv_plan_create(&plan, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
-                                  (int32_t)A->nnz, A->row_data, A->col_data, A->val_data, (void *)handle->stream);
+                                  (int32_t)A->nnz, A->row_data, callers_values_only ? nullptr : A->col_data,
+                                  callers_values_only ? nullptr : A->val_data, (void *)handle->stream);
     if (rc) return st(rc);
     x->plans.push_back(KeptPlan{false, (int)alg, A->row_data, A->col_data, A->val_data, A->rows, A->cols, A->nnz,
-                                (int)A->data_type, 1, plan});
+                                (int)A->data_type, 1, plan, callers_values_only});
     // the reference's own record of what was analysed (include/alphasparse/handle.h:190-197)
     x->csrmv.trans = opA;
     x->csrmv.m = (int)matA->rows;
@@ -791,9 +858,10 @@ alphasparseStatus_t alphasparseSpMV(alphasparseHandle_t handle, alphasparseOpera
     const _alphasparseSpMatDescr *A = &eff.d;
     const int32_t m = (int32_t)A->rows, n = (int32_t)A->cols, nnz = (int32_t)A->nnz;
     const asx_plan *plan = find_plan(matA, false, (int)alg, A, 1);
-    if (!plan && auto_analysis()) {
+    const AutoAnalysis mode = auto_analysis();
+    if (!plan && (mode == kAutoValues || (mode == kAutoStructure && !is_transpose(opA))) && (!matA->info || ext_of(matA))) {
         release_effective(handle, &eff);
-        s = alphasparseSpMV_analysis(handle, opA, matA, alg);
+        s = spmv_analysis(handle, opA, matA, alg, mode == kAutoStructure);
         if (s) return s;
         s = make_effective(handle, matA, opA, &eff);
         if (s) return s;
@@ -857,6 +925,13 @@ alphasparseStatus_t alphasparse_spmv(alphasparseHandle_t handle, alphasparseOper
     return alphasparseSpMV(handle, trans, alpha, mat, x, beta, y, ct, a, temp_buffer);
 }
 
+const char *alphasparseAmdKeptKernel(alphasparseSpMatDescr_t matA, alphasparseOperation_t opA, int is_spmm, int alg, int ncols)
+{
+    if (!matA) return "none";
+    const asx_plan *plan = kept_plan(matA, opA, is_spmm != 0, alg, is_spmm ? ncols : 1);
+    return plan ? asx_kernel_name(is_spmm, asx_plan_alg(plan)) : "none";
+}
+
 // ------------------------------------------------------------------------------------ SpMM
 alphasparseStatus_t alphasparseSpMM_bufferSize(alphasparseHandle_t handle, alphasparseOperation_t opA,
                                                alphasparseOperation_t opB, const void *alpha,
@@ -885,6 +960,11 @@ alphasparseStatus_t alphasparseSpMM_bufferSize(alphasparseHandle_t handle, alpha
 // blocked copy of A for the MFMA kernel, which holds A's values: call again after changing them.
 // *bufferSize, when given, receives the workspace a later alphasparseSpMM call needs (never more
 // than alphasparseSpMM_bufferSize reports).
+static alphasparseStatus_t spmm_preprocess(alphasparseHandle_t handle, alphasparseOperation_t opA, alphasparseOperation_t opB,
+                                           const void *alpha, alphasparseSpMatDescr_t matA, alphasparseDnMatDescr_t matB,
+                                           const void *beta, alphasparseDnMatDescr_t matC, alphasparseDataType computeType,
+                                           alphasparseSpMMAlg_t alg, size_t *bufferSize, bool callers_values_only);
+
 alphasparseStatus_t alphasparseSpMM_preprocess(alphasparseHandle_t handle, alphasparseOperation_t opA,
                                                alphasparseOperation_t opB, const void *alpha,
                                                alphasparseSpMatDescr_t matA,
@@ -892,6 +972,14 @@ alphasparseStatus_t alphasparseSpMM_preprocess(alphasparseHandle_t handle, alpha
                                                alphasparseDnMatDescr_t matC,
                                                alphasparseDataType computeType,
                                                alphasparseSpMMAlg_t alg, size_t *bufferSize)
+{
+    return spmm_preprocess(handle, opA, opB, alpha, matA, matB, beta, matC, computeType, alg, bufferSize, false);
+}
+
+static alphasparseStatus_t spmm_preprocess(alphasparseHandle_t handle, alphasparseOperation_t opA, alphasparseOperation_t opB,
+                                           const void *alpha, alphasparseSpMatDescr_t matA, alphasparseDnMatDescr_t matB,
+                                           const void *beta, alphasparseDnMatDescr_t matC, alphasparseDataType computeType,
+                                           alphasparseSpMMAlg_t alg, size_t *bufferSize, bool callers_values_only)
 {
     alphasparseStatus_t s = check_spmm(handle, opA, opB, alpha, matA, matB, beta, matC, computeType);
     if (s) return s;
@@ -906,6 +994,12 @@ alphasparseStatus_t alphasparseSpMM_preprocess(alphasparseHandle_t handle, alpha
     if (s) return s;
     const _alphasparseSpMatDescr *A = &eff.d;
     asx_plan *have = find_plan(matA, true, (int)alg, A, ncols);
+    if (have && !callers_values_only && kept_is_restricted(matA, have)) {
+        // what analysis on first use left there makes way for the caller's own, full preprocessing
+        (void)hipStreamSynchronize(handle->stream);
+        drop_one_plan(matA, have);
+        have = nullptr;
+    }
     if (have) {
         // preprocessed before: a plan that holds a copy of A's values picks up the current ones
         int rc = asx_plan_update_values(have, A->val_data, (void *)handle->stream);
@@ -914,12 +1008,16 @@ alphasparseStatus_t alphasparseSpMM_preprocess(alphasparseHandle_t handle, alpha
         MatInfoExt *x = ext_create(handle, matA);
         if (!x) return matA->info ? ALPHA_SPARSE_STATUS_NOT_SUPPORTED : ALPHA_SPARSE_STATUS_ALLOC_FAILED;
         asx_plan *plan = nullptr;
-        int rc = asx_spmm_plan_create(&plan, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
-                                      (int32_t)A->nnz, A->row_data, A->col_data, A->val_data, ncols,
-                                      (void *)handle->stream);
+        // without the columns and values: split points only, never the blocked copy of A's values
+        int rc = callers_values_only
+                     ? asx_plan_create(&plan, 1, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
+                                       (int32_t)A->nnz, A->row_data, ncols, (void *)handle->stream)
+                     : asx_spmm_plan_create(&plan, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
+                                            (int32_t)A->nnz, A->row_data, A->col_data, A->val_data, ncols,
+                                            (void *)handle->stream);
         if (rc) return st(rc);
         x->plans.push_back(KeptPlan{true, (int)alg, A->row_data, A->col_data, A->val_data, A->rows, A->cols, A->nnz,
-                                    (int)A->data_type, ncols, plan});
+                                    (int)A->data_type, ncols, plan, callers_values_only});
         have = plan;
         matA->analysed = true;
     }
@@ -950,11 +1048,13 @@ alphasparseStatus_t alphasparseSpMM(alphasparseHandle_t handle, alphasparseOpera
     const int32_t m = (int32_t)A->rows, k = (int32_t)A->cols, nnz = (int32_t)A->nnz;
     const int vt = (int)A->data_type;
     const asx_plan *plan = find_plan(matA, true, (int)alg, A, ncols);
-    if (!plan && auto_analysis()) {
+    const AutoAnalysis mode = auto_analysis();
+    if (!plan && (mode == kAutoValues || (mode == kAutoStructure && !is_transpose(opA))) && (!matA->info || ext_of(matA))) {
         release_effective(handle, &eff);
         size_t unused = 0;
-        s = alphasparseSpMM_preprocess(handle, opA, opB, alpha, matA, matB, beta, matC, computeType, alg, &unused);
-        if (s) return s;
+        s = spmm_preprocess(handle, opA, opB, alpha, matA, matB, beta, matC, computeType, alg, &unused, mode == kAutoStructure);
+        // the blocked algorithm has no analysis without A's values: the call goes on without one
+        if (s && !(mode == kAutoStructure && s == ALPHA_SPARSE_STATUS_NOT_SUPPORTED)) return s;
         s = make_effective(handle, matA, opA, &eff);
         if (s) return s;
         plan = find_plan(matA, true, (int)alg, A, ncols);

@@ -833,6 +833,26 @@ int asx_plan_export(const asx_plan *plan, int what, void *h_dst, size_t cap, siz
 }
 
 int asx_plan_alg(const asx_plan *plan) { return plan ? plan->alg : -1; }
+const char *asx_kernel_name(int is_spmm, int kernel)
+{
+    if (is_spmm) {
+        switch (kernel) {
+        case ASX_SPMM_ROW: return "row";
+        case ASX_SPMM_MERGE: return "merge";
+        case ASX_SPMM_BLOCKED: return "blocked";
+        default: return "?";
+        }
+    }
+    switch (kernel) {
+    case ASX_SPMV_VECTOR: return "vector";
+    case ASX_SPMV_STREAM: return "stream";
+    case ASX_SPMV_MERGE: return "merge";
+    case ASX_SPMV_FLAT: return "flat";
+    case ASX_SPMV_SLICED: return "sliced";
+    case ASX_SPMV_WINDOW: return "window";
+    default: return "?";
+    }
+}
 size_t asx_plan_workspace_bytes(const asx_plan *plan) { return plan ? plan->workspace_bytes : 0; }
 int64_t asx_plan_info(const asx_plan *plan, int what)
 {

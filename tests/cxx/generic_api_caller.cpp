@@ -101,12 +101,15 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
             s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
         }
-        // analysis on first use (ALPHASPARSE_AMD_AUTO_ANALYSIS=1): the calls above must have left
-        // kept analysis on the descriptor although alphasparseSpMV_analysis was never called
         if (!analysis) {
+            // analysis on first use: unless ALPHASPARSE_AMD_AUTO_ANALYSIS=0, the calls above left kept
+            // analysis on the descriptor although alphasparseSpMV_analysis was never called ("1": the
+            // full one, which may regroup A; unset: only what reads the caller's values in every call)
             const char *e = std::getenv("ALPHASPARSE_AMD_AUTO_ANALYSIS");
-            if ((e && e[0] == '1') != A->analysed) return 12;
+            const bool off = e && e[0] == '0';
+            if (!v.trans_a && off == A->analysed) return 12;
         }
+        std::printf("kernel %s\n", alphasparseAmdKeptKernel(A, opA, 0, alg, 1));
         if (analysis == 2) {
             // the caller changes A's values in place (same pattern) and says so by calling the
             // analysis again; the next product must use the new values
@@ -215,10 +218,12 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
             s = alphasparseSpMM(handle, opA, opB, &alpha, A, B, &beta, C, dt, (alphasparseSpMMAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
         }
-        if (!analysis) {
+        if (!analysis && alg != 10) {
             const char *e = std::getenv("ALPHASPARSE_AMD_AUTO_ANALYSIS");
-            if ((e && e[0] == '1') != A->analysed) return 12;
+            const bool off = e && e[0] == '0';
+            if (!v.trans_a && off == A->analysed) return 12;
         }
+        std::printf("kernel %s\n", alphasparseAmdKeptKernel(A, opA, 1, alg, (int)ncols));
         if (analysis == 2) {  // new values in place, preprocess again, multiply again
             auto val2 = read_bin<T>(dir + "/val2.bin", nnz);
             HIP_OK(hipStreamSynchronize(handle->stream));
@@ -347,6 +352,26 @@ static int selftest()
     HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
     EXPECT(y[0] == 42.5 && y[1] == 65.0);
     EXPECT(alphasparseSpMV_clear(h, ALPHA_SPARSE_SPMV_ALG_DEFAULT) == 0);
+    // an object of the caller's own behind matA->info (the reference's 176-byte struct) is left
+    // alone: no analysis is kept there, and products still work
+    {
+        _alphasparse_mat_info *foreign = new _alphasparse_mat_info();
+        alphasparseSpMatDescr_t F;
+        EXPECT(alphasparseCreateCsr(&F, 2, 2, 3, d_rp, d_col, d_val, ALPHA_SPARSE_INDEXTYPE_I32, ALPHA_SPARSE_INDEXTYPE_I32,
+                                    ALPHA_SPARSE_INDEX_BASE_ZERO, ALPHA_R_64F) == 0);
+        F->info = foreign;
+        EXPECT(alphasparseSpMV_analysis(h, N, F, ALPHA_SPARSE_SPMV_ALG_DEFAULT) == ALPHA_SPARSE_STATUS_NOT_SUPPORTED);
+        EXPECT(alphasparseSpMV_bufferSize(h, N, &alpha, F, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, &bytes) == 0);
+        EXPECT(F->info == foreign && !F->analysed);
+        HIP_OK(hipMemcpy(d_y, x.data(), sizeof(double) * 2, hipMemcpyHostToDevice));
+        EXPECT(alphasparseSpMV(h, N, &alpha, F, X, &beta, Y, ALPHA_R_64F, ALPHA_SPARSE_SPMV_ALG_DEFAULT, nullptr) == 0);
+        HIP_OK(hipDeviceSynchronize());
+        HIP_OK(hipMemcpy(y.data(), d_y, sizeof(double) * 2, hipMemcpyDeviceToHost));
+        EXPECT(y[0] == 42.5 && y[1] == 65.0);
+        F->info = nullptr;
+        alphasparseDestroySpMat(F);
+        delete foreign;
+    }
     // two-phase form: size query, then compute
     {
         size_t need = 0;

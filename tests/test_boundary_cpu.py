@@ -56,6 +56,23 @@ def test_generic_api_mangled_names(lib):
         assert name in exported, name
 
 
+def test_nothing_else_is_exported(lib):
+    """The drop-in library exports the C-ABI, the generic API's C++ names (those a caller compiled
+    against the reference's headers links to, plus what the alphasparseCreateCsr<T> template and
+    the descriptor destructors resolve to) and nothing else: no launcher, no helper, no kernel stub."""
+    out = subprocess.run(["nm", "-D", "--defined-only", capi.LIB_PATH], check=True, capture_output=True, text=True).stdout
+    exported = {line.split()[-1] for line in out.splitlines() if line.strip()}
+    also = {
+        "_Z27alphasparseCreateCsrUntypedPP22_alphasparseSpMatDescrlllPiS2_Pv22alphasparseIndexType_tS4_22alphasparseIndexBase_t19alphasparseDataType",
+        "_Z23alphasparseDestroySpMatP22_alphasparseSpMatDescr",
+        "_Z23alphasparseDestroyDnVecP24_alphasparse_dnvec_descr",
+        "_Z23alphasparseDestroyDnMatP24_alphasparse_dnmat_descr",
+        "_Z24alphasparseAmdKeptKernelP22_alphasparseSpMatDescr22alphasparseOperation_tiii",  # alphasparseAmdKeptKernel (no counterpart in the reference)
+    }
+    extra = exported - set(capi.EXPORTS) - set(MANGLED) - also
+    assert not extra, sorted(extra)
+
+
 def test_struct_layouts_match_the_reference_fixture(tmp_path):
     """tests/golden/layout.json holds sizeof / offsetof of the boundary structs as the reference's
     own headers give them (written by tests/golden/make_layout.py in the build container).  The

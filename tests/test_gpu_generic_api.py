@@ -15,7 +15,7 @@ EXE = os.path.join(ROOT, "tests", "cxx", "generic_api_caller")
 
 
 def _run_case(tmp_path, op, dtype, rp, col, val, x, y, ncols, alg, alpha, beta, analysis, variant=(0, 0, 0, 0, 0),
-              n=None, val2=None, env=None, x2=None, tag=""):
+              n=None, val2=None, env=None, x2=None, tag="", said=None):
     """variant = (trans_a, idx_base, col_major_b, col_major_c, trans_b); n = columns of A."""
     d = tmp_path / f"{op}_{np.dtype(dtype).name}_{alg}_{analysis}_{''.join(map(str, variant))}{'_env' if env else ''}{tag}"
     d.mkdir()
@@ -33,6 +33,8 @@ def _run_case(tmp_path, op, dtype, rp, col, val, x, y, ncols, alg, alpha, beta, 
     r = subprocess.run([EXE, str(d)], capture_output=True, text=True, timeout=120,
                        env=dict(os.environ, **env) if env else None)
     assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
+    if said is not None:
+        said.append(r.stdout)
     return np.fromfile(d / "out.bin", dtype=dtype)
 
 
@@ -254,29 +256,39 @@ def test_two_streams_share_one_analysed_descriptor(tmp_path, oracle):
 
 
 def test_analysis_on_first_use(tmp_path, oracle):
-    """ALPHASPARSE_AMD_AUTO_ANALYSIS=1: a caller that never calls alphasparseSpMV_analysis /
-    alphasparseSpMM_preprocess (the reference's own test loops do not) gets kept analysis from its
-    first call on; the caller program checks that the descriptor ends up analysed, and without the
-    variable does not."""
+    """A caller that never calls alphasparseSpMV_analysis / alphasparseSpMM_preprocess (the reference's
+    own test loops do not) gets kept analysis from its first call on: by default only analysis that
+    reads the caller's values in every call (a row-ordered kernel's split points), with
+    ALPHASPARSE_AMD_AUTO_ANALYSIS=1 the full one (column slices on this matrix), with =0 none.  The
+    caller program prints the kept kernel and checks that the descriptor ends up analysed or not."""
     from library_amd import workloads as W
     rp, col, val = W.csr_zipf(1 << 20, 1 << 20, 20, 1.0, 5000, 0.01, np.float64, 5)
     n = 1 << 20
     rng = np.random.default_rng(71)
     x = rng.uniform(-1, 1, n)
     y0 = rng.uniform(-1, 1, rp.size - 1)
-    got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, 2.1, 3.2, 0,
-                    env={"ALPHASPARSE_AMD_AUTO_ANALYSIS": "1"})
-    assert_close(got, oracle.spmv(rp, col, val, x, 2.1, 3.2, y0, 8), spmv_scale(rp, col, val, x, 2.1, 3.2, y0),
-                 np.float64, "SpMV, analysis on first use")
+    ref, scale = oracle.spmv(rp, col, val, x, 2.1, 3.2, y0, 8), spmv_scale(rp, col, val, x, 2.1, 3.2, y0)
+    for env, kernels in ((None, ("kernel flat", "kernel merge")), ({"ALPHASPARSE_AMD_AUTO_ANALYSIS": "1"}, ("kernel sliced",)),
+                         ({"ALPHASPARSE_AMD_AUTO_ANALYSIS": "0"}, ("kernel none",))):
+        said = []
+        if env is None and "ALPHASPARSE_AMD_AUTO_ANALYSIS" in os.environ:
+            env = {"ALPHASPARSE_AMD_AUTO_ANALYSIS": "structure"}
+        got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, 2.1, 3.2, 0, env=env, said=said,
+                        tag="" if env is None else "_" + list(env.values())[0])
+        assert_close(got, ref, scale, np.float64, f"SpMV, analysis on first use, {env}")
+        assert any(k in said[0] for k in kernels), (env, said[0])
     from test_gpu_parity import _block_structured
     m, k, nc = 700, 640, 64
     rp, col, val = _block_structured(rng, m, k, np.float32)
     B = rng.uniform(-1, 1, k * nc).astype(np.float32)
     C0 = rng.uniform(-1, 1, m * nc).astype(np.float32)
-    got = _run_case(tmp_path, "spmm", np.float32, rp, col, val, B, C0, nc, 0, 2.0, 3.0, 0,
-                    env={"ALPHASPARSE_AMD_AUTO_ANALYSIS": "1"})
-    assert_close(got, oracle.spmm(rp, col, val, B, nc, 2.0, 3.0, C0, 4), spmm_scale(rp, col, val, B, nc, 2.0, 3.0, C0),
-                 np.float32, "SpMM, analysis on first use")
+    ref, scale = oracle.spmm(rp, col, val, B, nc, 2.0, 3.0, C0, 4), spmm_scale(rp, col, val, B, nc, 2.0, 3.0, C0)
+    for env, kernel in ((None, "kernel merge"), ({"ALPHASPARSE_AMD_AUTO_ANALYSIS": "1"}, "kernel blocked")):
+        said = []
+        got = _run_case(tmp_path, "spmm", np.float32, rp, col, val, B, C0, nc, 0, 2.0, 3.0, 0, env=env, said=said,
+                        tag="" if env is None else "_full")
+        assert_close(got, ref, scale, np.float32, f"SpMM, analysis on first use, {env}")
+        assert kernel in said[0], (env, said[0])
 
 
 def test_spmm_blocked_values_changed_after_preprocess(tmp_path, oracle):
