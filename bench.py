@@ -34,9 +34,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
-ORDER = ["banded_f64", "uniform16_f32", "powerlaw_f64", "stencil5_f64", "spmm_zipf_f32"]
-# not BASELINE configurations: a dense-block matrix for the MFMA SpMM variant; config 2's matrix in fp64
-EXTRA = ["spmm_banded_f32", "uniform16_f64"]
+# the five BASELINE configurations, and config 2's matrix in fp64 (the "uniform fp64" case the target names)
+ORDER = ["banded_f64", "uniform16_f32", "uniform16_f64", "powerlaw_f64", "stencil5_f64", "spmm_zipf_f32"]
+# not a BASELINE configuration: a dense-block matrix for the MFMA SpMM variant
+EXTRA = ["spmm_banded_f32"]
 KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "k_spmv_flat",
                 101: "k_sliced_products+k_sliced_reduce", 102: "k_spmv_window", 5: "k_spmm_row", 7: "k_spmm_merge", 10: "k_spmm_blocked"}
 
@@ -69,6 +70,9 @@ def parse():
     ap.add_argument("--calibrate-gather", action="store_true",
                     help="only run the random-line gather kernel (lines per second the memory system delivers "
                          "past the L2s: the bound of a gather without reuse)")
+    ap.add_argument("--selection-audit", action="store_true",
+                    help="only time, over families of matrices, the plan DEFAULT picks against every kernel that "
+                         "accepts the matrix; prints a markdown table and one JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run the plain copy kernel on 1 GiB (known traffic, for scaling profiler counters)")
     return ap.parse_args()
@@ -393,6 +397,13 @@ def main():
         return
     if a.calibrate_copy:
         print(json.dumps(copy_calibration(a.steps)))
+        return
+    if a.selection_audit:
+        from library_amd import selection_audit
+        load_plan_kernels()
+        rows = selection_audit.run()
+        print(selection_audit.markdown(rows))
+        print(json.dumps({"selection_audit": rows, "worst_ratio": max(r["ratio"] for r in rows)}))
         return
     names = [a.workload] if (a.only or a.workload in EXTRA) else ORDER
     first_use_ms = load_plan_kernels()

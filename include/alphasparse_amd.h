@@ -305,11 +305,13 @@ int asx_spmv_csr_f32(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_
  * carries that asx_spmv_csr_f64 puts into the caller's workspace live in an array inside the
  * library, one copy per GPU, asx_spmv_noalloc_max_workspace() bytes (4 MiB) large: a call whose
  * asx_spmv_workspace_bytes(alg, ASX_R_64F, m, nnz) exceeds that returns ASX_STATUS_INVALID_SIZE
- * and launches nothing (the flat kernel, alg 0, needs 12 bytes per 1024 stored elements: about
- * 350 million stored elements fit).  The call allocates nothing and frees nothing.  Every call on
+ * and launches nothing (sized for the kernel the call runs; the flat kernel, alg 0, needs 12 bytes
+ * per 1024 stored elements: about 350 million stored elements fit).  The call allocates nothing and frees nothing.  Every call on
  * a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads)
  * race; calls on one stream are safe.  Same kernels, same results as asx_spmv_csr_f64 with the
- * same `alg`. */
+ * same `alg`.  The array's device address is looked up once per device, by asx_device_info or by
+ * the first call on that device (a host-side lookup that may load the library's code): before
+ * capturing a call into a HIP graph, call asx_device_info or make one call eagerly. */
 int asx_spmv_csr_f64_noalloc(int alg, int32_t m, int32_t n, int32_t nnz, double alpha,
                              const int32_t *d_row_ptr, const int32_t *d_col, const double *d_val,
                              const double *d_x, double beta, double *d_y, void *stream);

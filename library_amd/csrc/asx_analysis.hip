@@ -261,21 +261,28 @@ __global__ __launch_bounds__(256) void k_copy16(const u32x4 *__restrict__ src, u
     for (; i < n16; i += stride) dst[i] = src[i];
 }
 
-// out[t] = number of distinct values of src[t * stride + i] >> shift, i in [0, 1024): one workgroup
-// per sampled tile, the values entered into a hash table in LDS (4096 slots, linear probing)
-__global__ __launch_bounds__(kBlock) void k_sample_distinct(const int32_t *__restrict__ src, int64_t stride, int shift,
-                                                            int32_t *__restrict__ out)
+// A sample of the columns: `samples` tiles of 1024 consecutive stored elements, `stride` elements
+// apart, one workgroup each.  out[t] = number of distinct 128-byte lines of x the tile's columns
+// touch (col >> shift entered into a hash table in LDS: 4096 slots, linear probing).  With
+// row_ptr given also out[64 + t] = number of (row, slice) pairs among the tile's elements, slices
+// of `width` columns: an element opens a pair when it is the first of its row (or of the tile) or
+// lies in another slice than the element before it (columns ascend inside a row).
+__global__ __launch_bounds__(kBlock) void k_sample_columns(const int32_t *__restrict__ col, int64_t stride, int shift,
+                                                           const int32_t *__restrict__ row_ptr, int32_t m, int32_t width,
+                                                           int32_t *__restrict__ out)
 {
     constexpr int kSlots = 4096;
     __shared__ int32_t table[kSlots];
-    __shared__ int32_t count;
+    __shared__ int32_t count, pairs;
     for (int i = threadIdx.x; i < kSlots; i += kBlock) table[i] = -1;
-    if (threadIdx.x == 0) count = 0;
+    if (threadIdx.x == 0) count = 0, pairs = 0;
     __syncthreads();
-    const int32_t *from = src + (int64_t)blockIdx.x * stride;
-    int32_t mine = 0;
+    const int64_t first = (int64_t)blockIdx.x * stride;
+    const int32_t *from = col + first;
+    int32_t mine = 0, mine_pairs = 0;
     for (int i = threadIdx.x; i < kFlatTile; i += kBlock) {
-        const int32_t v = from[i] >> shift;
+        const int32_t c = from[i];
+        const int32_t v = c >> shift;
         uint32_t h = ((uint32_t)v * 2654435761u) >> 20;
         for (;;) {
             const int32_t old = atomicCAS(&table[h], -1, v);
@@ -286,15 +293,37 @@ __global__ __launch_bounds__(kBlock) void k_sample_distinct(const int32_t *__res
             if (old == v) break;
             h = (h + 1) & (kSlots - 1);
         }
+        if (row_ptr) {
+            bool opens = i == 0 || c / width != from[i - 1] / width;
+            if (!opens) {  // first element of its row?
+                const int64_t e = first + i;
+                int32_t lo = 0, hi = m;  // largest r with row_ptr[r] <= e
+                while (lo < hi) {
+                    const int32_t mid = lo + (hi - lo + 1) / 2;
+                    if ((int64_t)row_ptr[mid] <= e)
+                        lo = mid;
+                    else
+                        hi = mid - 1;
+                }
+                opens = row_ptr[lo] == e;
+            }
+            mine_pairs += opens;
+        }
     }
     if (mine) atomicAdd(&count, mine);
+    if (mine_pairs) atomicAdd(&pairs, mine_pairs);
     __syncthreads();
-    if (threadIdx.x == 0) out[blockIdx.x] = count;
+    if (threadIdx.x == 0) {
+        out[blockIdx.x] = count;
+        if (row_ptr) out[64 + blockIdx.x] = pairs;
+    }
 }
-int launch_sample_distinct(const int32_t *d_src, int64_t stride, int shift, int32_t samples, int32_t *d_out, hipStream_t s)
+int launch_sample_columns(const int32_t *d_col, int64_t stride, int shift, const int32_t *d_row_ptr, int32_t m,
+                          int32_t width, int32_t samples, int32_t *d_out, hipStream_t s)
 {
-    if (samples <= 0) return ASX_STATUS_SUCCESS;
-    hipLaunchKernelGGL(k_sample_distinct, dim3((unsigned)samples), dim3(kBlock), 0, s, d_src, stride, shift, d_out);
+    if (samples <= 0 || samples > 64) return samples > 64 ? ASX_STATUS_INVALID_VALUE : ASX_STATUS_SUCCESS;
+    hipLaunchKernelGGL(k_sample_columns, dim3((unsigned)samples), dim3(kBlock), 0, s, d_col, stride, shift, d_row_ptr, m, width,
+                       d_out);
     return check_launch();
 }
 

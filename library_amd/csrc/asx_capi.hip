@@ -80,26 +80,39 @@ SpmmLayout spmm_merge_layout(int32_t m, int32_t nnz, int32_t ncols, size_t sv, b
     return L;
 }
 
-// How scattered the columns are: the number of distinct 128-byte lines of x that the columns of a
-// tile of 1024 consecutive stored elements touch, divided by 1024, averaged over up to 64 tiles
-// spread over the matrix (counted on the device).  Random columns give about 1, a 5-point
-// stencil 0.04, a band matrix 0.01.  Regrouping by column slice only pays for scattered columns.
-double sampled_line_spread(const int32_t *d_col, int32_t nnz, size_t sv, int32_t *d_scratch, hipStream_t s)
+// What a sample of the columns says (up to 64 tiles of 1024 consecutive stored elements spread over
+// the matrix, counted on the device):
+//   spread  distinct 128-byte lines of x a tile's columns touch, per stored element.  Random
+//           columns give about 1, a 5-point stencil 0.04, a band matrix 0.01.
+//   pairs   (row, slice) pairs per stored element, for column slices of 128 KiB of x: the partial
+//           sums the column-sliced kernel would carry through memory.  16 random columns per row
+//           over 32 slices give 0.8, a band matrix about 1 / (row length).
+struct ColumnSample {
+    bool ok;
+    double spread, pairs;
+};
+constexpr int32_t kSliceBytes = 131072;  // of x per slice: one workgroup of 16 waves per compute unit
+ColumnSample sample_columns(const int32_t *d_row_ptr, int32_t m, const int32_t *d_col, int32_t nnz, size_t sv,
+                            int32_t *d_scratch /* 128 ints */, hipStream_t s)
 {
+    ColumnSample cs{false, 0.0, 1.0};
     const int64_t tiles = nnz / kFlatTile;
-    if (tiles < 1) return 0.0;
+    if (tiles < 1) return cs;
     const int samples = (int)std::min<int64_t>(64, tiles);
     const int64_t stride = tiles / samples;
-    // the distinct lines of every sampled tile are counted on the device (d_scratch: 64 ints)
-    int32_t h[64];
+    int32_t h[128];
     const int shift = sv == 8 ? 4 : 5;  // columns per 128-byte line of x
-    if (launch_sample_distinct(d_col, stride * kFlatTile, shift, samples, d_scratch, s) != ASX_STATUS_SUCCESS ||
-        hipMemcpyAsync(h, d_scratch, sizeof(int32_t) * (size_t)samples, hipMemcpyDeviceToHost, s) != hipSuccess ||
+    if (launch_sample_columns(d_col, stride * kFlatTile, shift, d_row_ptr, m, (int32_t)(kSliceBytes / sv), samples, d_scratch,
+                              s) != ASX_STATUS_SUCCESS ||
+        hipMemcpyAsync(h, d_scratch, sizeof(h), hipMemcpyDeviceToHost, s) != hipSuccess ||
         hipStreamSynchronize(s) != hipSuccess)
-        return 0.0;
-    int64_t distinct = 0;
-    for (int t = 0; t < samples; ++t) distinct += h[t];
-    return (double)distinct / ((double)samples * kFlatTile);
+        return cs;
+    int64_t distinct = 0, pairs = 0;
+    for (int t = 0; t < samples; ++t) distinct += h[t], pairs += h[64 + t];
+    cs.ok = true;
+    cs.spread = (double)distinct / ((double)samples * kFlatTile);
+    cs.pairs = d_row_ptr ? (double)pairs / ((double)samples * kFlatTile) : 1.0;
+    return cs;
 }
 constexpr double kScatteredMinSpread = 0.5;
 
@@ -274,6 +287,8 @@ int spmm_impl(const asx_plan *plan, int alg, int32_t m, int32_t k, int32_t nnz, 
 
 }  // namespace
 
+static int noalloc_scratch(void **out);
+
 extern "C" {
 
 const char *asx_version(void) { return "0.1"; }
@@ -290,6 +305,10 @@ int asx_device_info(int *compute_units, int *wavefront_size)
     if (e != hipSuccess) return status_of(e);
     if (compute_units) *compute_units = cu;
     if (wavefront_size) *wavefront_size = wf;
+    // the address of this device's scratch array of asx_spmv_csr_f64_noalloc, so that its calls are
+    // stream work only from the first one on (the lookup may load the library's code onto the device)
+    void *unused = nullptr;
+    (void)noalloc_scratch(&unused);
     return ASX_STATUS_SUCCESS;
 }
 
@@ -510,8 +529,9 @@ int asx_spmm_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
                          (value_type == ASX_R_32F || value_type == ASX_R_64F);
     if (probe_blocked) {
         int32_t *d_scratch = nullptr;
-        if (hipMalloc((void **)&d_scratch, 64 * sizeof(int32_t)) != hipSuccess) return ASX_STATUS_ALLOC_FAILED;
-        probe_blocked = sampled_line_spread(d_col, nnz, vsize(value_type), d_scratch, (hipStream_t)stream) < kScatteredMinSpread;
+        if (hipMalloc((void **)&d_scratch, 128 * sizeof(int32_t)) != hipSuccess) return ASX_STATUS_ALLOC_FAILED;
+        const ColumnSample cs = sample_columns(nullptr, m, d_col, nnz, vsize(value_type), d_scratch, (hipStream_t)stream);
+        probe_blocked = cs.ok && cs.spread < kScatteredMinSpread;
         (void)hipFree(d_scratch);
     }
     if (!want_blocked && !probe_blocked)
@@ -553,63 +573,64 @@ int asx_spmm_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
 
 }  // extern "C"
 
-// ---- the column-sliced kernel as DEFAULT's choice ------------------------------------------
-// Decided from figures that do not change from one plan build to the next: the row-length
-// histogram, the sizes, and the column sample.  Model (fitted to measurements on MI355X):
-//   row-ordered kernels   t = nnz / g(x bytes), g = 180 G gathers/s while x fits an L2 (<= 3 MiB),
-//                         62 G/s once it does not (>= 6 MiB), linear in between, and never less
-//                         than their bytes at 5 TB/s;
-//   column-sliced kernel  t = 12 us + bytes / 4.7 TB/s with
-//                         bytes = nnz (sv + 2) + P (2 sv + 2) + n sv + 2 m sv,
-//                         P = expected number of (row, slice) pairs = sum over rows of
-//                         S (1 - (1 - 1/S)^len), S = number of slices, from the histogram.
-// Sliced is chosen when its estimate is at least 10 % lower.
+// ---- what DEFAULT picks when it may regroup A --------------------------------------------
+// Decided from figures that do not change from one plan build to the next (the row-length
+// histogram, the sizes, the column sample), never from timings: two analyses of one matrix keep the
+// same kernel.  Estimated times (rates fitted to measurements on MI355X over families of matrices:
+// uniform and power-law rows, bands, stencils, clustered columns):
+//   row-ordered kernels   5 us + max(nnz spread' / g, bytes / 4.0 TB/s); g = gathers of x an L2
+//                         serves per second: 180 G while x fits one (<= 3 MiB), 62 G once it does
+//                         not (>= 6 MiB), linear in between; spread' = the sample's spread, at least
+//                         0.05 (neighbouring columns share a line); bytes = nnz (sv + 4) + n sv + m (sv + 4)
+//   column-sliced kernel  8 us + bytes / 6.0 TB/s, bytes = nnz (sv + 2) + P (2 sv + 2) + n sv + 2 m sv,
+//                         P = nnz times the sample's pairs per stored element
+//   row-block kernel      8 us + bytes / 5.0 TB/s (3.7 TB/s when rows longer than 16 are cut by
+//                         tiles), bytes = (nnz + empty rows) (sv + 2) + n sv + 2 m sv; only for
+//                         columns that are not scattered, and whether every block's columns fit a
+//                         window is known once its build was tried
+// A regrouped kernel is taken when its estimate is at least 3 % below the row-ordered one; of the
+// two, the sliced one unless the row-block one is estimated more than 5 % faster.
 constexpr int32_t kSlicedMinNnz = 1 << 21;
-constexpr int32_t kSliceBytes = 131072;  // of x per slice: one workgroup of 16 waves per compute unit
-static double sliced_expected_partials(const int64_t hist[33], int32_t nslices)
+struct KernelEstimates {
+    double rows, sliced, window;  // seconds; infinity where the kernel does not apply
+};
+static KernelEstimates estimate_kernels(const asx_plan *p, size_t sv, const ColumnSample &cs, bool window_ok)
 {
-    double p = 0.0;
-    const double q = nslices > 1 ? std::log1p(-1.0 / (double)nslices) : 0.0;
-    for (int b = 1; b <= 32; ++b) {
-        if (!hist[b]) continue;
-        const double len = b == 1 ? 1.0 : 0.75 * std::ldexp(1.0, b);  // middle of [2^(b-1), 2^b)
-        p += (double)hist[b] * (nslices > 1 ? (double)nslices * -std::expm1(len * q) : 1.0);
-    }
-    return p;
-}
-static bool sliced_pays(const int64_t hist[33], int32_t m, int32_t n, int32_t nnz, size_t sv)
-{
-    if (nnz < kSlicedMinNnz || m <= 0 || n <= 0) return false;
-    const double xbytes = (double)n * (double)sv;
+    const double inf = 1e30;
+    const double nnz = (double)p->nnz, m = (double)p->m, n = (double)p->n, dsv = (double)sv;
+    const double xbytes = n * dsv;
     const double lo = 3.0 * 1048576.0, hi = 6.0 * 1048576.0;
     const double f = xbytes <= lo ? 0.0 : xbytes >= hi ? 1.0 : (xbytes - lo) / (hi - lo);
     const double gather_rate = 180e9 + f * (62e9 - 180e9);
-    const double row_bytes = (double)nnz * (sv + 4) + (double)n * sv + (double)m * (sv + 4);
-    const double t_rows = std::max((double)nnz / gather_rate, row_bytes / 5e12);
-    const int32_t nslices = (int32_t)ceil_div64((int64_t)n * (int64_t)sv, kSliceBytes);
-    if (nslices > kSlicedMaxSlices) return false;  // the plan build handles no more
-    const double partials = sliced_expected_partials(hist, nslices);
-    const double sl_bytes = (double)nnz * (sv + 2) + partials * (2.0 * sv + 2) + (double)n * sv + 2.0 * (double)m * sv;
-    const double t_sliced = 12e-6 + sl_bytes / 4.7e12;
-    return t_sliced < 0.9 * t_rows;
+    KernelEstimates e;
+    e.rows = 5e-6 + std::max(nnz * std::max(cs.spread, 0.05) / gather_rate, (nnz * (dsv + 4) + n * dsv + m * (dsv + 4)) / 4.0e12);
+    const int64_t nslices = ceil_div64((int64_t)p->n * (int64_t)sv, kSliceBytes);
+    e.sliced = nslices > kSlicedMaxSlices
+                   ? inf
+                   : 8e-6 + (nnz * (dsv + 2) + cs.pairs * nnz * (2 * dsv + 2) + n * dsv + 2 * m * dsv) / 6.0e12;
+    e.window = !window_ok ? inf
+                          : 8e-6 + ((nnz + (double)p->hist[0]) * (dsv + 2) + n * dsv + 2 * m * dsv) /
+                                       (p->stats[0] <= 16 ? 5.0e12 : 3.7e12);
+    return e;
 }
 
 // Builds the sliced copy onto a plan that already holds the histogram (`p` takes the slices over;
 // its own split points are dropped).
 template <typename T>
-int plan_add_slices(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, hipStream_t s)
+int plan_add_slices(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, double pairs_per_element,
+                    hipStream_t s)
 {
     int cus = 256;
     (void)asx_device_info(&cus, nullptr);
     // pass 2: one wave per block of rows, its accumulators (8 bytes a row) in LDS.  Blocks of 256
     // rows, doubled up to 1024 while that leaves more than 8 waves per compute unit and the block's
-    // partial sums inside one slice (expected from the row-length histogram) are fewer than 12: a
+    // partial sums inside one slice (expected from the column sample) are fewer than 12: a
     // step of pass 2 takes its 64 entries from at most three ranges.  Small blocks mean many waves
     // in flight.  Measured: the power-law matrix (4 per range at 256 rows) 50 / 34.5 / 36.6 us with
     // 512 / 1024 / 2048 rows; 16 per row over 32 slices (100 per range at 256 rows) 17.5 / 20 us
     // with 256 / 512 rows; the same in fp64 over 64 slices 26.5 / 27.5 / 36.8 us with 256 / 512 / 1024.
     const int32_t nslices = (int32_t)ceil_div64((int64_t)p->n * (int64_t)sizeof(T), kSliceBytes);
-    const double per_row_slice = sliced_expected_partials(p->hist, nslices) / ((double)p->m * (double)nslices);
+    const double per_row_slice = pairs_per_element * (double)p->nnz / ((double)p->m * (double)nslices);
     int32_t rpw = 256;
     while (rpw < 1024 && (int64_t)rpw * cus * 8 < p->m && per_row_slice * rpw < 12.0) rpw *= 2;
     SlicedMatrix sm{};
@@ -655,6 +676,19 @@ int plan_add_window(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
 // slot of its own (a value, a column word and a source index, read in every call), so a matrix
 // with more empty rows than a quarter of its stored elements stays with the merge-path kernel,
 // which streams row offsets only.
+// A regrouped copy roughly doubles what the matrix takes on the device (per stored element: the
+// value, 2 bytes of column, 4 bytes of source index; the sliced kernel also keeps a buffer for the
+// partial sums of a call), and its build needs about 4 bytes per stored element more for a while.
+// DEFAULT only makes one while twice that is free: a caller who sized the device for one copy of A
+// is not pushed to the edge by an analysis call.
+static bool regrouped_copy_fits(const asx_plan *p, size_t sv)
+{
+    size_t free_b = 0, total_b = 0;
+    if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) return false;
+    const double copy = (double)p->nnz * (double)(sv + 6) + (double)p->nnz * (double)(sv + 2) + (double)p->nnz * 4.0;
+    return (double)free_b >= 2.0 * copy;
+}
+
 static bool window_may_pay(const asx_plan *p, int row_kernel)
 {
     return p->stats[0] <= kWindowMaxRow && (row_kernel == ASX_SPMV_FLAT || row_kernel == ASX_SPMV_MERGE) &&
@@ -685,32 +719,39 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     if (st) return st;
     if (alg == ASX_SPMV_DEFAULT) row_kernel = choose_spmv_from_stats(p->hist, p->stats, m, nnz);
     const bool f64 = value_type == ASX_R_64F;
-    const bool can_regroup = alg == ASX_SPMV_DEFAULT && d_col && d_val && m > 0 && n > 0 && nnz >= kSlicedMinNnz;
+    const size_t sv = vsize(value_type);
+    int32_t *d_sample = reinterpret_cast<int32_t *>(p->d_counters + 64);  // 128 ints
+    const auto add_slices = [&](double pairs) {
+        return f64 ? plan_add_slices<double>(p, d_row_ptr, d_col, (const double *)d_val, pairs, s)
+                   : plan_add_slices<float>(p, d_row_ptr, d_col, (const float *)d_val, pairs, s);
+    };
+    const auto add_window = [&]() {
+        return f64 ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
+                   : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
+    };
+    const bool can_regroup = alg == ASX_SPMV_DEFAULT && d_col && d_val && m > 0 && n > 0 && nnz >= kSlicedMinNnz &&
+                             regrouped_copy_fits(p, sv);
     bool done = false;
     if (alg == ASX_SPMV_WINDOW) {
-        st = f64 ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
-                 : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
+        st = add_window();
         done = true;
     } else if (alg == ASX_SPMV_SLICED) {
-        st = f64 ? plan_add_slices<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
-                 : plan_add_slices<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
+        const ColumnSample cs = sample_columns(d_row_ptr, m, d_col, nnz, sv, d_sample, s);  // sizes the row blocks of pass 2
+        st = add_slices(cs.pairs);
         done = true;
     } else if (can_regroup) {
-        // DEFAULT: a regrouped copy where it pays; a build that fails (out of memory, a matrix the
-        // kernel does not take) is not an error: the row-ordered plan stands
-        bool slices = false;
-        if (sliced_pays(p->hist, m, n, nnz, vsize(value_type)))
-            slices = sampled_line_spread(d_col, nnz, vsize(value_type), reinterpret_cast<int32_t *>(p->d_counters + 64), s) >=
-                     kScatteredMinSpread;
-        if (slices) {
-            done = (f64 ? plan_add_slices<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
-                        : plan_add_slices<float>(p, d_row_ptr, d_col, (const float *)d_val, s)) == ASX_STATUS_SUCCESS;
-        } else if (window_may_pay(p, row_kernel)) {
-            // rows that reach only nearby columns: row blocks with a sliding window of x in LDS (measured
-            // 23 % faster than the flat kernel on the 5-point stencil, 20 % on a band of 19); the build
-            // reports NOT_SUPPORTED when some 256 rows reach further than a window
-            done = (f64 ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
-                        : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, s)) == ASX_STATUS_SUCCESS;
+        // DEFAULT: a regrouped copy where it is estimated to pay; a build that fails (out of memory,
+        // a matrix the kernel does not take) is not an error: the next choice stands
+        const ColumnSample cs = sample_columns(d_row_ptr, m, d_col, nnz, sv, d_sample, s);
+        if (cs.ok) {
+            // the row-block kernel needs columns near each other; whether they fit its windows the
+            // build finds out (NOT_SUPPORTED when some 256 rows reach further)
+            const bool window_ok = window_may_pay(p, row_kernel) && cs.spread < kScatteredMinSpread;
+            const KernelEstimates e = estimate_kernels(p, sv, cs, window_ok);
+            const bool sliced_pays = e.sliced < 0.97 * e.rows, window_pays = e.window < 0.97 * e.rows;
+            if (window_pays && e.window < e.sliced / 1.05) done = add_window() == ASX_STATUS_SUCCESS;
+            if (!done && sliced_pays) done = add_slices(cs.pairs) == ASX_STATUS_SUCCESS;
+            if (!done && window_pays && !(e.window < e.sliced / 1.05)) done = add_window() == ASX_STATUS_SUCCESS;
         }
     }
     if (!done) st = plan_row_ordered(p, row_kernel, s);
@@ -988,8 +1029,9 @@ int asx_spmv_csr_f64_noalloc(int alg, int32_t m, int32_t n, int32_t nnz, double 
 {
     if (m < 0 || n < 0 || nnz < 0) return ASX_STATUS_INVALID_SIZE;
     if (asx_spmv_resolve_alg(alg, m, nnz) < 0) return ASX_STATUS_NOT_SUPPORTED;
-    // what asx_spmv_csr_f64 would ask of a caller's buffer for this call must fit the array
-    const size_t need = asx_spmv_workspace_bytes(alg, ASX_R_64F, m, nnz);
+    // what the kernel this call runs would ask of a caller's buffer must fit the array (for DEFAULT
+    // that is the flat kernel: without a plan nothing else is chosen)
+    const size_t need = asx_spmv_workspace_bytes(asx_spmv_resolve_alg(alg, m, nnz), ASX_R_64F, m, nnz);
     if (need > kNoAllocScratchBytes) return ASX_STATUS_INVALID_SIZE;
     void *ws = nullptr;
     const int st = noalloc_scratch(&ws);

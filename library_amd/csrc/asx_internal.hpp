@@ -53,8 +53,8 @@ int launch_stream_row_blocks(const int32_t *d_row_ptr, int32_t m, int32_t nnz, i
                              hipStream_t s);
 int launch_copy_bytes(const void *d_src, void *d_dst, size_t bytes, hipStream_t s);
 int launch_fill_i32(int32_t *d_dst, int64_t n, int32_t value, hipStream_t s);
-int launch_sample_distinct(const int32_t *d_src, int64_t stride, int shift, int32_t samples, int32_t *d_out,
-                           hipStream_t s);
+int launch_sample_columns(const int32_t *d_col, int64_t stride, int shift, const int32_t *d_row_ptr, int32_t m,
+                          int32_t width, int32_t samples, int32_t *d_out, hipStream_t s);
 int launch_gather_lines(const void *d_buf, size_t bytes, int group_lanes, int per_lane, void *d_out, int *nthreads,
                         hipStream_t s);
 

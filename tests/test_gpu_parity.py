@@ -850,6 +850,39 @@ def test_spmv_window_kernel_bands_of_diagonals(torch, capi, oracle, dtype):
     assert not h.value
 
 
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_regrouped_kernels_with_x_off_a_16_byte_boundary(torch, capi, oracle, dtype):
+    """x passed as a view that starts one element into an allocation (a sub-vector behind
+    vecX->values): its address is no multiple of 16, so the kernels that copy x into LDS take their
+    element-by-element fetch; and matrices with 1 to 3 columns, shorter than one 16-byte unit.
+    Window plans with one band and with bands of diagonals, and a sliced plan."""
+    rng = np.random.default_rng(211)
+    cases = [("band", capi.SPMV_WINDOW, _banded_random(rng, 9000, 9000, 300, 0.05, dtype, longrow=700), 9000),
+             ("two bands", capi.SPMV_WINDOW, _diagonal_bands(rng, 50000, 70001, [(-30000, -29990), (-5, 40)], 0.5, dtype), 70001),
+             ("scattered", capi.SPMV_SLICED, csr_from_lengths(np.minimum(rng.zipf(1.6, 30000), 2000), 70001, 3, dtype), 70001)]
+    for n in (1, 2, 3):
+        lens = rng.integers(0, n + 1, 5000)
+        cases.append((f"{n} columns", capi.SPMV_WINDOW, csr_from_lengths(lens, n, 5, dtype), n))
+        cases.append((f"{n} columns", capi.SPMV_SLICED, csr_from_lengths(lens, n, 5, dtype), n))
+    for name, alg, (rp, col, val), n in cases:
+        m = rp.size - 1
+        x = rng.uniform(-1, 1, n).astype(dtype)
+        y0 = rng.uniform(-1, 1, m).astype(dtype)
+        d = [dev(torch, a) for a in (rp, col, val)]
+        xbuf = dev(torch, np.r_[dtype(7.0), x, dtype(9.0)])
+        xv = xbuf[1:1 + n]
+        assert xv.data_ptr() % 16 != 0 and xv.data_ptr() == xbuf.data_ptr() + np.dtype(dtype).itemsize
+        plan = capi.Plan(False, alg, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
+        plan_check.check_plan(plan, capi, rp, col, n, np.dtype(dtype).itemsize)
+        ref = oracle.spmv(rp, col, val, x, dtype(1.5), dtype(0.5), y0, 2)
+        for xin, tag in ((xv, "offset x"), (dev(torch, x), "aligned x")):
+            y = dev(torch, y0)
+            capi.spmv(d[0], d[1], d[2], xin, y, 1.5, 0.5, alg=alg, plan=plan, n=n)
+            torch.cuda.synchronize()
+            assert_close(y.cpu().numpy(), ref, spmv_scale(rp, col, val, x, 1.5, 0.5, y0), dtype, f"{name} alg {alg} {tag}")
+        plan.destroy()
+
+
 def test_sliced_and_window_calls_replay_in_a_hip_graph(torch, capi, oracle):
     """A call with a sliced or window plan is kernels only (no allocation, copy, memset or
     synchronisation): captured once in a HIP graph it must give the eager result on every replay,
