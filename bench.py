@@ -47,12 +47,13 @@ KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "
 # WRITE_SIZE all of them).  The Infinity Cache serves part of it: the counters read the same with
 # warm and with cold caches.
 MEASURED_TRAFFIC_BYTES = {
-    "banded_f64": 458_340,             # profiles/spmv_vector_banded_f64.md
-    "uniform16_f32": 248_827_868,      # profiles/spmv_sliced_uniform16_f32.md
-    "powerlaw_f64": 719_680_994,       # profiles/spmv_sliced_powerlaw_f64.md
-    "stencil5_f64": 1_135_144_526,     # profiles/spmv_window_stencil5_f64.md
-    "spmm_zipf_f32": 4_964_375_542,    # profiles/spmm_merge_spmm_zipf_f32.md
-    "spmm_banded_f32": 1_868_453_131,  # profiles/spmm_blocked_spmm_banded_f32.md
+    "banded_f64": 458_624,  # profiles/spmv_vector_banded_f64.md
+    "uniform16_f32": 256_450_608,  # profiles/spmv_sliced_uniform16_f32.md
+    "uniform16_f64": 477_788_284,  # profiles/spmv_sliced_uniform16_f64.md
+    "powerlaw_f64": 728_906_293,  # profiles/spmv_sliced_powerlaw_f64.md
+    "stencil5_f64": 1_135_136_745,  # profiles/spmv_window_stencil5_f64.md
+    "spmm_zipf_f32": 4_965_331_333,  # profiles/spmm_merge_spmm_zipf_f32.md
+    "spmm_banded_f32": 1_870_263_890,  # profiles/spmm_blocked_spmm_banded_f32.md
 }
 
 

@@ -287,11 +287,16 @@ __global__ __launch_bounds__(kBlock) void k_spmm_merge(int32_t m, int32_t nnz, i
     if (lane == 0 && blockIdx.y == 0) carry_row[seg] = has_tail ? x1 : -1;
 }
 
-// One thread per segment looks for the first segment of a run of segments that left carries for
-// the same row; each such run is then summed by the whole wave (lanes = columns): the run length
+// Every wave looks at kFixupSegs consecutive segments (one lane each) for the first segment of a run
+// of segments that left carries for the same row; each such run is then summed by the whole wave
+// (lanes = columns), one after the other: few segments per wave, because a run costs three or four
+// dependent memory round trips and the runs of a wave are taken in turn (64 segments per wave left
+// the pass with 2000 waves, each with five runs in a row: 22 us on the Zipf matrix, 19 us with 8; what
+// remains is the longest rows, whose hundreds of carry rows one wave adds 64 at a time).  The run length
 // comes from ballots over carry_row (64 segments per step), the carry rows are added in segment
 // order with a counted, unrolled loop (many independent loads in flight; a loop that tests
 // carry_row before every add would pay one memory round trip per segment).
+constexpr int kFixupSegs = 8;
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_spmm_merge_fixup(int32_t m, int32_t nseg, int32_t ncols,
                                                              T alpha, const T *__restrict__ carry,
@@ -299,10 +304,11 @@ __global__ __launch_bounds__(kBlock) void k_spmm_merge_fixup(int32_t m, int32_t 
                                                              T *__restrict__ C, int64_t ldc)
 {
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t wave = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+    const int64_t t = wave * kFixupSegs + lane;
     int32_t my_row = -1;
     bool head = false;
-    if (t < nseg) {
+    if (lane < kFixupSegs && t < nseg) {
         my_row = carry_row[t];
         head = my_row >= 0 && my_row < m && (t == 0 || carry_row[t - 1] != my_row);
     }
@@ -357,7 +363,8 @@ int launch_spmm_merge(int32_t m, int32_t nnz, int32_t ncols, T alpha, const int3
     dim3 grid((unsigned)ceil_div64(nseg, kBlock / kWave), (unsigned)ceil_div64(ncols, kWave));
     hipLaunchKernelGGL((k_spmm_merge<T>), grid, dim3(kBlock), 0, s, m, nnz, nseg, ncols, alpha, row_ptr,
                        col, val, B, ldb, beta, C, ldc, xs, ys, carry, carry_row);
-    hipLaunchKernelGGL((k_spmm_merge_fixup<T>), dim3((unsigned)ceil_div64(nseg, kBlock)), dim3(kBlock), 0, s, m,
+    hipLaunchKernelGGL((k_spmm_merge_fixup<T>), dim3((unsigned)ceil_div64(ceil_div64(nseg, kFixupSegs), kBlock / kWave)),
+                       dim3(kBlock), 0, s, m,
                        nseg, ncols, alpha, carry, carry_row, C, ldc);
     return check_launch();
 }

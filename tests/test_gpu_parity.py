@@ -966,6 +966,37 @@ def test_one_plan_two_streams_two_workspaces(torch, capi, oracle):
         plan.destroy()
 
 
+def test_default_keeps_the_row_block_copy_off_matrices_of_mostly_empty_rows(torch, capi, oracle):
+    """The window format gives every empty row a slot of its own (value, column word, source index,
+    read in every call): for a matrix with far more rows than stored elements that is more traffic
+    than the row offsets the other kernels stream.  Three quarters of 9 M rows empty, the rest
+    with one element next to the diagonal (columns as local as they get): DEFAULT must not pick the
+    window kernel, the forced window plan still works, and both give the oracle's result."""
+    rng = np.random.default_rng(171)
+    m = n = 9 << 20
+    rows = np.nonzero(rng.random(m) < 0.25)[0]
+    col = np.clip(rows + rng.integers(-100, 101, rows.size), 0, n - 1).astype(np.int32)
+    rp = np.zeros(m + 1, np.int32)
+    np.cumsum(np.bincount(rows, minlength=m), out=rp[1:])
+    assert col.size >= 1 << 21
+    val = rng.uniform(-1, 1, col.size)
+    x = rng.uniform(-1, 1, n)
+    y0 = rng.uniform(-1, 1, m)
+    ref = oracle.spmv(rp, col, val, x, 1.5, 0.5, y0, 8)
+    scale = spmv_scale(rp, col, val, x, 1.5, 0.5, y0)
+    d = [dev(torch, a) for a in (rp, col, val, x)]
+    plan = capi.Plan(False, capi.SPMV_DEFAULT, val.dtype, m, n, col.size, d[0], col=d[1], val=d[2])
+    assert plan.alg != capi.SPMV_WINDOW, plan.alg
+    forced = capi.Plan(False, capi.SPMV_WINDOW, val.dtype, m, n, col.size, d[0], col=d[1], val=d[2])
+    assert forced.info("tiles") * 256 >= m, "a slot per row, empty or not"
+    for p in (plan, forced):
+        y = dev(torch, y0)
+        capi.spmv(d[0], d[1], d[2], d[3], y, 1.5, 0.5, plan=p)
+        torch.cuda.synchronize()
+        assert_close(y.cpu().numpy(), ref, scale, np.float64, f"kernel {p.alg}")
+        p.destroy()
+
+
 def test_default_workspace_covers_every_choice(torch, capi, oracle):
     """alphasparseSpMV_bufferSize(DEFAULT) is asx_spmv_workspace_bytes(DEFAULT): whatever kernel a
     DEFAULT plan settles on must fit in it.  Hypersparse (the plan takes the merge-path kernel,
