@@ -242,7 +242,9 @@ enum {
     ASX_PLAN_INFO_STEPS = 9,          /* steps of pass 2, each up to 64 partial sums (sliced) */
     ASX_PLAN_INFO_WIDTH = 10,         /* columns per slice (sliced), columns the rings hold together (window) */
     ASX_PLAN_INFO_WORKGROUPS = 11,    /* workgroups of pass 1 (sliced), chains (window) */
-    ASX_PLAN_INFO_PIECES = 12         /* pieces of x fetched over all blocks (window) */
+    ASX_PLAN_INFO_PIECES = 12,        /* pieces of x fetched over all blocks (window) */
+    ASX_PLAN_INFO_STACKED_ROWS = 13   /* rows of a plane when the three bands share rotating regions of LDS and the
+                                         blocks are stored plane above plane (window; 0 otherwise) */
 };
 int64_t asx_plan_info(const asx_plan *plan, int what);
 /* Frees the buffer a sliced or window plan keeps for the partial sums / carries of a call.  Calls

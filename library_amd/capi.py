@@ -301,7 +301,8 @@ class Plan:
         self._keep = (self._keep[0], self._keep[1], val)
 
     INFO = {"tiles": 0, "slices": 1, "partial_sums": 2, "rows_per_wave": 3, "rows_per_block": 4, "bands": 5,
-            "chains": 6, "carry_pass": 7, "row_blocks": 8, "steps": 9, "width": 10, "workgroups": 11, "pieces": 12}
+            "chains": 6, "carry_pass": 7, "row_blocks": 8, "steps": 9, "width": 10, "workgroups": 11, "pieces": 12,
+            "stacked_rows": 13}
     # asx_plan_export: name -> (id, element type; "value" = the plan's value type)
     ARRAYS = {"val": (0, "value"), "cf": (1, np.uint16), "perm": (2, np.int32), "tile_words": (3, np.int32),
               "workgroups": (4, np.int32), "partial_rows": (5, np.uint16), "ranges": (6, np.int32),

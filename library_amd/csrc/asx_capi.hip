@@ -913,6 +913,7 @@ int64_t asx_plan_info(const asx_plan *plan, int what)
     case ASX_PLAN_INFO_WIDTH: return sliced ? plan->sliced.width : window ? 16384 : -1;
     case ASX_PLAN_INFO_WORKGROUPS: return sliced ? plan->sliced.nwg : window ? plan->window.nchains : -1;
     case ASX_PLAN_INFO_PIECES: return window ? plan->window.npieces : -1;
+    case ASX_PLAN_INFO_STACKED_ROWS: return window ? plan->window.stack_rows : -1;
     default: return -1;
     }
 }

@@ -176,6 +176,7 @@ struct WindowMatrix {
     int32_t npieces;         // entries of `pieces`
     int32_t ntiles;
     int32_t nbands;          // 1: one window per block; 2..kWindowBands: bands of diagonals
+    int32_t stack_rows;      // > 0: three bands on stacked planes of this many rows, the blocks stored column by column
     int has_carry;           // some tile starts inside a row: the ordered carry pass is needed
     void *store;             // one allocation: val, perm, cf, tile_info
     void *tables;            // one allocation: blocks, pieces, chains

@@ -373,7 +373,10 @@ constexpr int kStageRuns = kSlicedTile;  // every run of a tile
 template <typename T>
 struct StageRun {
     T *stage;
-    __device__ __forceinline__ void operator()(int rank, T v) const { stage[rank] = v; }
+    __device__ __forceinline__ void operator()(bool wanted, int rank, T v) const
+    {
+        if (wanted) stage[rank] = v;
+    }
 };
 template <typename T>
 __device__ __forceinline__ void store_staged(const T *stage, int lane, int total, T *__restrict__ out)

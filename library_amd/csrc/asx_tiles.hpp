@@ -65,10 +65,13 @@ __device__ __forceinline__ void tile_load(Tile<T> &tl, int32_t t, int lane, cons
     tl.base = tile_word[t];
 }
 
-// Products, running sums and wave scan of one tile; `emit(rank, sum)` is called once for every run
-// of the tile, rank = position of the run in the tile (a tile starts with a run start); returns the
-// number of runs.  Lane l
-// holds elements 4l .. 4l+3; a run start closes the run before it; lane 63 closes the last one.
+// Products, running sums and wave scan of one tile; `emit(wanted, rank, sum)` is called five times
+// by every lane, `wanted` on the lanes that close a run: rank = position of the run in the tile (a
+// tile starts with a run start; meaningless where not wanted).  Whether an emitter branches on
+// `wanted` or stores to a spare place instead is its own choice: a branch that depends on the lane
+// makes the compiler restructure the loops around it, and with them what it knows about which
+// loads are still in flight.  Returns the number of runs.  Lane l holds elements 4l .. 4l+3; a run
+// start closes the run before it; lane 63 closes the last one.
 template <typename T, typename Emit>
 __device__ __forceinline__ int tile_reduce(const Tile<T> &tl, int lane, const T *xs, Emit emit)
 {
@@ -88,14 +91,14 @@ __device__ __forceinline__ int tile_reduce(const Tile<T> &tl, int lane, const T 
     const T open = wave_segsum_dpp<T>(r3, nh != 0);
     const T cin = wave_shift_up1<T>(open);  // what earlier lanes hold of the run open at this lane's start
     int hb = before;
-    if (f0 && hb > 0) emit(hb - 1, cin);
+    emit(f0 && hb > 0, hb - 1, cin);
     hb += f0;
-    if (f1) emit(hb - 1, f0 ? r0 : cin + r0);
+    emit(f1, hb - 1, f0 ? r0 : cin + r0);
     hb += f1;
-    if (f2) emit(hb - 1, (f0 | f1) ? r1 : cin + r1);
+    emit(f2, hb - 1, (f0 | f1) ? r1 : cin + r1);
     hb += f2;
-    if (f3) emit(hb - 1, (f0 | f1 | f2) ? r2 : cin + r2);
-    if (lane == kWave - 1) emit(total - 1, open);
+    emit(f3, hb - 1, (f0 | f1 | f2) ? r2 : cin + r2);
+    emit(lane == kWave - 1, total - 1, open);
     return total;
 }
 

@@ -11,11 +11,14 @@
 // still being multiplied - and x crosses the L2 once.  Where no such window exists but the
 // stored elements lie on at most kWindowBands bands of diagonals (column minus row inside a few
 // narrow intervals: the planes of a 7- or 27-point stencil), every band gets a ring of its own in
-// LDS and a block fetches the new columns of every band (x then crosses the L2 once per band).
+// LDS and a block fetches the new columns of every band (x then crosses the L2 once per band);
+// three bands a whole number of planes apart share three regions of LDS that take turns, the
+// blocks of a chain climb the planes, and x crosses the L2 about once (see BandTable).
 // The block's stored elements stream as tiles of 256 with a 16-bit LDS slot and a "first element
 // of a row" flag per element (10 instead of 12.8 bytes per stored element in fp64; no row offsets
-// are read).  Every row owns at least one slot (an empty row gets a zero that points at a zero in
-// LDS), so the runs of a tile are consecutive rows and a run's sum goes straight to y.  Rows of up
+// are read).  Every row owns at least two slots (what its stored elements leave free holds zeros
+// that point at a zero in LDS), so the runs of a tile are consecutive rows, at most 128 of them,
+// and a run's sum goes straight to y.  Rows of up
 // to 16 stored elements are never cut by a tile start (the tile is padded instead); a longer row
 // that is cut leaves its later pieces in carry slots, which an ordered pass adds to y afterwards
 // (no atomics; results are bit-reproducible).
@@ -26,7 +29,6 @@
 #include <vector>
 
 #include "asx_internal.hpp"
-#include "asx_scan.hpp"
 #include "asx_tiles.hpp"
 
 namespace asx {
@@ -38,7 +40,15 @@ constexpr int kWindowCols = 16384;    // ring size in columns: 128 KiB of fp64, 
 constexpr int kWindowSlack = 8;       // a block's window is kept this much narrower (aligned fetches)
 constexpr int kWindowWaves = 16;
 constexpr int32_t kAlignRowLen = 16;  // rows up to this length are not cut by tile starts
+constexpr int32_t kMinRowSlots = 2;   // slots a row takes at least
 
+// Tiles in flight per wave: as many as the 128 registers a lane of a 1024-thread workgroup may use
+// hold beside the columns of x on their way to LDS (the compiler spills those first)
+template <typename T>
+constexpr int window_depth(int rings, bool beta)
+{
+    return rings > 1 ? 2 : sizeof(T) == 8 ? 2 : 3;
+}
 constexpr int kSpanGroup = 128;  // rows per group of the column-span table; every block size is a multiple
 
 // first and last column of every group of kSpanGroup consecutive rows (gmin = kNoCol, gmax = -1 for
@@ -100,8 +110,9 @@ __global__ __launch_bounds__(kBlock) void k_window_fill_i32(int32_t *p, int64_t 
 }
 
 // Slot (from the start of its block) at which every row starts, and the tiles of every block.  A
-// row takes max(1, length) slots; a row of at most kAlignRowLen slots that would cross a tile
-// start begins at that tile start instead.  One wave walks one block's rows in order, 64 at a time:
+// row takes max(kMinRowSlots, length) slots (a tile of 256 slots then holds at most 128 rows, which
+// is what a wave stages and stores per tile); a row of at most kAlignRowLen slots that would cross
+// a tile start begins at that tile start instead.  One wave walks one block's rows in order, 64 at a time:
 // starts from a scan of the lengths; at the first row of the 64 that has to move to the next tile
 // the walk restarts behind that row (the rows after it shift).
 __global__ __launch_bounds__(kBlock) void k_window_row_starts(const int32_t *__restrict__ row_ptr, int32_t m,
@@ -121,7 +132,7 @@ __global__ __launch_bounds__(kBlock) void k_window_row_starts(const int32_t *__r
         int32_t len = 0;
         if (rr < r1) {
             len = row_ptr[rr + 1] - row_ptr[rr];
-            len = len > 0 ? len : 1;
+            len = len > kMinRowSlots ? len : kMinRowSlots;
         }
         int32_t incl = len;
 #pragma unroll
@@ -149,14 +160,17 @@ __global__ __launch_bounds__(kBlock) void k_window_row_starts(const int32_t *__r
     if (lane == 0) block_tiles[b] = (pos + kSlicedTile - 1) / kSlicedTile;
 }
 
-// The slots that hold no stored element: the slot of an empty row, the slots between a row's end
-// and the start of the next one where that row was moved to a tile start, and the tail of a
-// block's last tile.  Each is a zero that points at the zero behind the rings and opens a run of
-// its own.  One thread per row fills what follows its own stored elements.
+// The slots that hold no stored element: the slots of an empty row, the second slot of a row with
+// one stored element, the slots between a row's end and the start of the next one where that row
+// was moved to a tile start, and the tail of a block's last tile.  Each is a zero that points at the
+// zero behind the rings; the first slot of an empty row opens the row's run, a slot that makes a row
+// up to kMinRowSlots belongs to that run, every other one opens a run of its own.  One thread per
+// row fills what follows its own stored elements.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_window_pads(const int32_t *__restrict__ row_ptr, int32_t m, int32_t rows,
                                                         const int32_t *__restrict__ row_start,
-                                                        const int32_t *__restrict__ tile_off, uint16_t pad,
+                                                        const int32_t *__restrict__ tile_off,
+                                                        const int32_t *__restrict__ block_tiles, uint16_t pad,
                                                         uint16_t *__restrict__ cf, T *__restrict__ val,
                                                         int32_t *__restrict__ perm)
 {
@@ -164,13 +178,15 @@ __global__ __launch_bounds__(kBlock) void k_window_pads(const int32_t *__restric
     if (r >= m) return;
     const int64_t b = r / rows;
     const int64_t last = (b + 1) * rows < m ? (b + 1) * rows : m;  // one past the block's last row
-    const int32_t from = row_start[r] + (row_ptr[r + 1] - row_ptr[r]);
-    const int32_t to = r + 1 < last ? row_start[r + 1] : (tile_off[b + 1] - tile_off[b]) * kSlicedTile;
+    const int32_t len = row_ptr[r + 1] - row_ptr[r];
+    const int32_t from = row_start[r] + len;
+    const int32_t own = row_start[r] + (len > kMinRowSlots ? len : kMinRowSlots);  // end of the row's own slots
+    const int32_t to = r + 1 < last ? row_start[r + 1] : block_tiles[b] * kSlicedTile;
     const int64_t base = (int64_t)tile_off[b] * kSlicedTile;
     for (int32_t o = from; o < to; ++o) {
         const int64_t d = base + o;
         const int64_t phys = d / kSlicedTile * kSlicedTile + tile_val_pos<T>((int)(d % kSlicedTile));
-        cf[d] = pad;
+        cf[d] = o < own && o > row_start[r] ? (uint16_t)(pad & 0x7fff) : pad;
         val[phys] = T(0);
         perm[phys] = -1;
     }
@@ -179,9 +195,16 @@ __global__ __launch_bounds__(kBlock) void k_window_pads(const int32_t *__restric
 // Where the columns of x live in LDS.  One band (nbands = 1): column c at c mod kWindowCols.
 // Several: the stored elements whose offset from the diagonal, c - floor(r n / m), lies in
 // [dlo[k], dhi[k]] use ring k: column c at base[k] + c mod width[k].
+// Stacked planes (stack_rows = P > 0; three bands whose centres lie -P, 0 and +P from the diagonal, as
+// in a stencil on a three-dimensional grid whose planes hold P points): the blocks of a chain are P
+// rows apart, and what block (plane p) fetched as its +P band is what the chain's next block
+// (plane p + 1) needs as its centre band and the one after as its -P band.  The three bands
+// therefore share three regions of stack_size slots that take turns: the columns around row r + d P,
+// d = -1, 0, 1, live in region (r / P + d) mod 3, column c at c mod stack_size inside it.
 struct BandTable {
     int32_t nbands;
     int32_t dlo[kWindowBands], dhi[kWindowBands], base[kWindowBands], width[kWindowBands];
+    int32_t stack_rows, stack_size;
 };
 __host__ __device__ __forceinline__ int64_t band_centre(int64_t r, int64_t m, int64_t n) { return r * n / m; }
 
@@ -236,7 +259,13 @@ __global__ __launch_bounds__(kBlock) void k_window_place(const int32_t *__restri
         for (int j = 1; j < kWindowBands; ++j)
             if (j < bands.nbands && off >= bands.dlo[j]) k = j;  // bands ascend and cover every offset
     }
-    const int32_t slot = bands.base[k] + c % bands.width[k];
+    int32_t slot;
+    if (bands.stack_rows > 0) {
+        const int32_t q = r / bands.stack_rows + (k - 1);  // -1 .. number of planes
+        slot = ((q % 3 + 3) % 3) * bands.stack_size + c % bands.stack_size;
+    } else {
+        slot = bands.base[k] + c % bands.width[k];
+    }
     cf[d] = (uint16_t)(slot | (head ? 0x8000 : 0));
     const int64_t phys = d / kSlicedTile * kSlicedTile + tile_val_pos<T>((int)(d % kSlicedTile));
     val_out[phys] = val[i];
@@ -244,26 +273,30 @@ __global__ __launch_bounds__(kBlock) void k_window_place(const int32_t *__restri
 }
 
 // per tile: x = the row its first slot belongs to, bit 31 set when the tile starts inside that
-// row; y = the number of runs of the tile that are rows (the slots behind them are padding)
+// row; y = the number of runs of the tile that are rows (the slots behind them are padding).
+// The blocks are stored in the order the chains walk them: stored_off[i] = first tile of the i-th
+// stored block, which holds the rows of block order[i] (of block i without an order).
 __global__ __launch_bounds__(kBlock) void k_window_tile_info(const int32_t *__restrict__ row_start, int32_t m,
                                                              int32_t rows, int32_t nblocks,
-                                                             const int32_t *__restrict__ tile_off, int32_t ntiles,
+                                                             const int32_t *__restrict__ stored_off,
+                                                             const int32_t *__restrict__ order, int32_t ntiles,
                                                              int2 *__restrict__ tile_info, int32_t *__restrict__ any_cont)
 {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= ntiles) return;
-    int32_t lo = 0, hi = nblocks - 1;  // block of tile t: largest b with tile_off[b] <= t
+    int32_t lo = 0, hi = nblocks - 1;  // stored block of tile t: largest i with stored_off[i] <= t
     while (lo < hi) {
         const int32_t mid = lo + (hi - lo + 1) / 2;
-        if (tile_off[mid] <= t)
+        if (stored_off[mid] <= t)
             lo = mid;
         else
             hi = mid - 1;
     }
-    const int32_t b = lo, r0 = b * rows;
-    const int32_t r1 = (int64_t)r0 + rows < m ? r0 + rows : m;
-    const int32_t o = (int32_t)(t - tile_off[b]) * kSlicedTile;
-    int32_t a = r0, z = r1 - 1;  // largest row whose start is <= o
+    const int32_t b = order ? order[lo] : lo;
+    const int64_t r0 = (int64_t)b * rows;
+    const int32_t r1 = r0 + rows < m ? (int32_t)(r0 + rows) : m;
+    const int32_t o = (int32_t)(t - stored_off[lo]) * kSlicedTile;
+    int32_t a = (int32_t)r0, z = r1 - 1;  // largest row whose start is <= o
     while (a < z) {
         const int32_t mid = a + (z - a + 1) / 2;
         if (row_start[mid] <= o)
@@ -295,94 +328,185 @@ __global__ __launch_bounds__(kBlock) void k_window_regather(const int32_t *__res
 }
 
 // ---- the kernel ----------------------------------------------------------------------------
-// Run k of a tile is row (first row of the tile) + k, for the `limit` runs that are rows; the
-// first sum of a tile that starts inside a row goes to the tile's carry slot.  The sums of the
-// first kStageRows rows of a tile pass through a staging area of the wave in LDS and leave as
-// stores of consecutive lanes to consecutive rows: stored straight from the lanes that close the
-// runs (4 or 5 masked stores a tile, 8 bytes every 32 to 40), the same 134 MB of y cost 66 us of
-// the 5-point stencil's 220; staged, a third of that.  Rows past kStageRows (a tile of rows shorter
-// than 2 on average) are stored directly.
+// Run k of a tile is row (first row of the tile) + k, for the `limit` runs that are rows (at most
+// kStageRows: a row takes at least two slots); the first sum of a tile that starts inside a row
+// goes to the tile's carry slot.  The sums pass through a staging area of the wave in LDS and
+// leave as stores of consecutive lanes to consecutive rows: stored straight from the lanes that
+// close the runs (4 or 5 masked stores a tile, 8 bytes every 32 to 40), the same 134 MB of y cost
+// 66 us of the 5-point stencil's 220; staged, a third of that.
+//
+// Memory operations of a wave complete in the order they were issued, and a wait for one of them
+// names how many younger ones may still be in flight.  A tile's loads are issued D steps before
+// the tile is multiplied; for them to stay in flight that long, every wait of the steady state
+// must be for something at least as old, and the compiler must be able to count, on every path
+// through the loop, what was issued in between.  Hence:
+//  * with beta != 0 (BETA) what y holds in a tile's rows is loaded together with the tile, D steps
+//    ahead, not when the rows are written: a wait for a load issued then would also wait for every
+//    tile on its way;
+//  * nothing inside a step branches on the lane: sums nobody wants go to a spare place in LDS,
+//    rows a lane does not own are cut off by the range check of a buffer store.  Branches that
+//    depend on the lane make the compiler rebuild the loops around them with flags, and across
+//    those it assumes the worst: that a tile is multiplied right after it was requested;
+//  * the loop over a wave's tiles of one block is a loop of its own, unrolled D times, once for
+//    every buffer the block can start with; the start of a block, which waits for the columns of
+//    x it stores, separates them.
 constexpr int kStageRows = 128;
+constexpr int kStageSlots = kStageRows + kWave;  // + one place per lane for the sums nobody wants
+constexpr uint32_t kOutOfRange = 0xfffffff0u;     // a byte offset past any range of rows
+
+// y in rows row0 .. row0 + rows - 1 as a buffer: loads past the range return 0, stores are dropped
 template <typename T>
-struct StoreRows {
-    T *y, *carry_slot, *stage;
-    int32_t row0, limit;
-    bool cont;
-    T alpha, beta;
-    __device__ __forceinline__ void operator()(int rank, T v) const
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_of_y(T *y, int32_t row0, int32_t rows)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(y + row0, 0, rows * (int32_t)sizeof(T), 0x00020000);
+}
+template <typename T>
+struct RowIO;
+template <>
+struct RowIO<double> {
+    typedef int bits_t __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ double load(__amdgpu_buffer_rsrc_t r, uint32_t off)
     {
-        if (rank == 0 && cont) {
-            *carry_slot = v;
-            return;
-        }
-        if (rank < kStageRows) {
-            stage[rank] = v;  // ranks at or past `limit` are written too and never read
-        } else if (rank < limit) {
-            const int64_t r = (int64_t)row0 + rank;
-            y[r] = beta == T(0) ? alpha * v : fma_t<T>(alpha, v, beta * y[r]);
-        }
+        return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0));
     }
-    // after the tile's runs are staged: the wave's LDS writes and reads execute in order
-    __device__ __forceinline__ void flush(int lane) const
+    static __device__ __forceinline__ void store(double v, __amdgpu_buffer_rsrc_t r, uint32_t off)
     {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        const int32_t first = cont ? 1 : 0, end = limit < kStageRows ? limit : kStageRows;
-#pragma unroll
-        for (int k = 0; k < kStageRows / kWave; ++k) {
-            const int32_t i = k * kWave + lane;
-            if (k * kWave < end) {  // uniform
-                if (i >= first && i < end) {
-                    const int64_t r = (int64_t)row0 + i;
-                    const T v = stage[i];
-                    y[r] = beta == T(0) ? alpha * v : fma_t<T>(alpha, v, beta * y[r]);
-                }
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(bits_t, v), r, off, 0, 0);
+    }
+};
+template <>
+struct RowIO<float> {
+    static __device__ __forceinline__ float load(__amdgpu_buffer_rsrc_t r, uint32_t off)
+    {
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
+    }
+    static __device__ __forceinline__ void store(float v, __amdgpu_buffer_rsrc_t r, uint32_t off)
+    {
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, off, 0, 0);
     }
 };
 
-template <typename T>
+template <typename T, bool BETA>
 struct WindowTile : Tile<T> {
-    int32_t limit;
+    int32_t limit;             // base, limit: the tile's two words, uniform
+    T yv[kStageRows / kWave];  // BETA: y in rows (first row) + lane + 64 k
 };
-template <typename T>
-__device__ __forceinline__ void window_tile_load(WindowTile<T> &tl, int32_t t, int lane, const uint16_t *__restrict__ cf,
-                                                 const T *__restrict__ val, const int2 *__restrict__ tile_info)
+// the loads of tile t, whose words are `info`
+template <typename T, bool BETA>
+__device__ __forceinline__ void window_tile_load(WindowTile<T, BETA> &tl, int32_t t, int2 info, int lane,
+                                                 const uint16_t *__restrict__ cf, const T *__restrict__ val, T *y)
 {
     typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
     const u32x2 cw = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(cf + (int64_t)t * kSlicedTile) + lane);
     tl.c01 = cw.x;
     tl.c23 = cw.y;
     TileValues<T>::load(val + (int64_t)t * kSlicedTile, lane, tl.v);
-    const int2 info = tile_info[t];
     tl.base = info.x;
     tl.limit = info.y;
+    if (BETA) {
+        const __amdgpu_buffer_rsrc_t rows = rows_of_y<T>(y, info.x & 0x7fffffff, info.y);
+#pragma unroll
+        for (int k = 0; k < kStageRows / kWave; ++k) tl.yv[k] = RowIO<T>::load(rows, (uint32_t)((k * kWave + lane) * sizeof(T)));
+    }
+}
+
+template <typename T>
+struct StageRows {
+    T *stage;
+    int lane;
+    __device__ __forceinline__ void operator()(bool wanted, int rank, T v) const
+    {
+        stage[wanted && rank < kStageRows ? rank : kStageRows + lane] = v;  // runs past the rows are padding
+    }
+};
+
+// Everything a step needs beside its tile.
+template <typename T>
+struct WindowStep {
+    const uint16_t *__restrict__ cf;
+    const T *__restrict__ val;
+    const int2 *__restrict__ tile_info;
+    T *y, *carry;
+    const T *xs;
+    T *stage;
+    T alpha, beta;
+    int32_t chain_last;
+    int lane;
+    int2 info_next;  // the words of the tile the next step will request
+};
+// One tile: its rows' sums into the staging area and from there to y, then the loads of the tile
+// `ahead` tiles further on (past the end of the chain: the last tile again) into the registers this
+// one has just left, and the words of the tile after that.
+template <typename T, bool BETA>
+__device__ __forceinline__ void window_step(WindowTile<T, BETA> &tl, int32_t t, int32_t ahead, int32_t stride, WindowStep<T> &w)
+{
+    tile_reduce<T>(tl, w.lane, w.xs, StageRows<T>{w.stage, w.lane});
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the wave's LDS writes and reads execute in order
+    __builtin_amdgcn_wave_barrier();
+    const int32_t row0 = tl.base & 0x7fffffff, limit = tl.limit;
+    const bool cont = tl.base < 0;
+    const __amdgpu_buffer_rsrc_t rows = rows_of_y<T>(w.y, row0, limit);
+#pragma unroll
+    for (int k = 0; k < kStageRows / kWave; ++k) {
+        if (k * kWave < limit) {  // uniform
+            const int32_t i = k * kWave + w.lane;
+            const T v = w.stage[i];
+            const T out = BETA ? fma_t<T>(w.alpha, v, w.beta * tl.yv[k]) : w.alpha * v;
+            // the first sum of a tile that starts inside a row is no row's
+            RowIO<T>::store(out, rows, k == 0 && cont && i == 0 ? kOutOfRange : (uint32_t)(i * sizeof(T)));
+        }
+    }
+    if (cont) w.carry[t] = w.stage[0];  // uniform; every lane stores the same value
+    __builtin_amdgcn_wave_barrier();
+    const int32_t t1 = t + ahead < w.chain_last ? t + ahead : w.chain_last;
+    window_tile_load<T, BETA>(tl, t1, w.info_next, w.lane, w.cf, w.val, w.y);
+    const int32_t t2 = t + ahead + stride < w.chain_last ? t + ahead + stride : w.chain_last;
+    w.info_next = w.tile_info[t2];
+}
+// `cnt` tiles of one wave in turn, the first in buffer P; a loop of its own for every P, with one
+// way out (a loop left from the middle is rebuilt with flags too), so that on every path through
+// it a buffer is used D - 1 steps after it was requested
+template <typename T, bool BETA, int D, int NW, int P>
+__device__ __forceinline__ void window_steps(WindowTile<T, BETA> (&tl)[D], int32_t &t, int32_t cnt, WindowStep<T> &w)
+{
+    for (int32_t i = cnt / D; i > 0; --i) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            window_step<T, BETA>(tl[(P + j) % D], t, D * NW, NW, w);
+            t += NW;
+        }
+    }
+    const int32_t rest = cnt % D;
+#pragma unroll
+    for (int j = 0; j + 1 < D; ++j) {
+        if (j < rest) {
+            window_step<T, BETA>(tl[(P + j) % D], t, D * NW, NW, w);
+            t += NW;
+        }
+    }
 }
 
 // The pieces of x a block needs before it is multiplied (at most kWindowBands ranges of columns
-// [from, to), from a multiple of 4, together at most kWindowCols columns; ring of piece q: slots
-// base .. base + width) into registers, one 16-byte unit per thread and step, and later from the
-// registers into the rings.  Columns at or past n read as 0.  Every register is written by one
-// load instruction only (predicated, after a zero fill), never by two alternative ones: with
-// alternatives the compiler orders them with a full s_waitcnt between the steps and the fetch
-// takes one memory round trip per step.  VEC (x on a 16-byte boundary, n at least one unit): one
-// 16-byte load per unit; the unit that straddles the end of x is read from the last whole unit
-// inside x (an unaligned address) and shifted into place when it is stored.  Otherwise element by
-// element.  NB = 1: one piece, ring of kWindowCols slots from slot 0 (no piece search, constant modulus).
-template <typename T, int THREADS, bool VEC, int NB>
+// [from, to), from and to multiples of 4; ring of piece q: slots base .. base + width) into
+// registers, one 16-byte unit per thread and step, and later from the registers into the rings.
+// x is read as a buffer whose range ends with x: what lies past the last column reads as 0, word
+// by word, so a unit may straddle the end, and x needs no more than the alignment of its elements.
+// With several pieces (NB > 1) every piece starts at a multiple of 64 units: the 64 lanes of a wave
+// then work on one piece, and which one is found with scalar compares; the builder keeps the
+// pieces of a block, each rounded up to 64 units, within what the registers hold (kWindowCols
+// columns).  NB = 1: one piece, ring of kWindowCols slots from slot 0 (constant modulus).
+template <typename T, int THREADS, int NB>
 struct XFetch {
     static constexpr int V = 16 / sizeof(T);
     static constexpr int PER = kWindowCols / (THREADS * V);
     typedef T vec_t __attribute__((ext_vector_type(V)));
-    typedef vec_t vec_u __attribute__((aligned(sizeof(T))));
+    typedef uint32_t bits_t __attribute__((ext_vector_type(4)));
     vec_t buf[PER];
-    // the pending fetch (uniform values): its pieces, the first unit of each and the ring slot of
-    // its first column
-    int32_t from[NB], to[NB], base[NB], width[NB], ustart[NB], fslot[NB];
+    // the pending fetch (uniform values): its pieces, the first unit of each, the ring slot of its
+    // first column and how many of its columns lie inside x
+    int32_t from[NB], len[NB], inside[NB], base[NB], width[NB], ustart[NB], fslot[NB];
 
-    __device__ __forceinline__ void set(const int4 *__restrict__ pieces, int32_t lo, int32_t hi)
+    __device__ __forceinline__ void set(const int4 *__restrict__ pieces, int32_t lo, int32_t hi, int32_t n)
     {
         int32_t u = 0;
 #pragma unroll
@@ -390,147 +514,119 @@ struct XFetch {
             int4 pc = make_int4(0, 0, 0, 4);
             if (lo + q < hi) pc = pieces[lo + q];  // uniform
             from[q] = __builtin_amdgcn_readfirstlane(pc.x);
-            to[q] = __builtin_amdgcn_readfirstlane(pc.y);
+            len[q] = __builtin_amdgcn_readfirstlane(pc.y) - from[q];
+            const int32_t left = n - from[q];
+            inside[q] = left < 0 ? 0 : left < len[q] ? left : len[q];
             base[q] = NB == 1 ? 0 : __builtin_amdgcn_readfirstlane(pc.z);
             width[q] = NB == 1 ? kWindowCols : __builtin_amdgcn_readfirstlane(pc.w);
             fslot[q] = (int32_t)((uint32_t)from[q] % (uint32_t)width[q]);
             ustart[q] = u;
-            u += (to[q] - from[q] + V - 1) / V;
+            u += (len[q] + V - 1) / V;
+            if (NB > 1) u = (u + kWave - 1) & ~(kWave - 1);
         }
     }
-    // unit u: first column, end of its piece, LDS slot (a unit past the last piece lands at or past
-    // `to` of the last one).  A piece is no longer than its ring, so one wrap suffices.
-    __device__ __forceinline__ void locate(int32_t u, int32_t &c, int32_t &c_to, int32_t &slot) const
+    // the piece the 64 units from `first_unit` on belong to (all values uniform)
+    struct Piece {
+        int32_t from, len, inside, base, width, ustart, fslot;
+    };
+    __device__ __forceinline__ Piece piece_of(int32_t first_unit) const
     {
-        int32_t f = from[0], s = 0, fs = fslot[0], b = base[0], w = width[0];
-        c_to = to[0];
+        Piece p{from[0], len[0], inside[0], base[0], width[0], ustart[0], fslot[0]};
 #pragma unroll
-        for (int q = 1; q < NB; ++q) {
-            const bool in = u >= ustart[q];
-            f = in ? from[q] : f;
-            s = in ? ustart[q] : s;
-            fs = in ? fslot[q] : fs;
-            b = in ? base[q] : b;
-            w = in ? width[q] : w;
-            c_to = in ? to[q] : c_to;
+        for (int j = 1; j < NB; ++j) {
+            const bool in = first_unit >= ustart[j];
+            p.from = in ? from[j] : p.from;
+            p.len = in ? len[j] : p.len;
+            p.inside = in ? inside[j] : p.inside;
+            p.base = in ? base[j] : p.base;
+            p.width = in ? width[j] : p.width;
+            p.ustart = in ? ustart[j] : p.ustart;
+            p.fslot = in ? fslot[j] : p.fslot;
         }
-        const int32_t off = (u - s) * V;
-        c = f + off;
-        const int32_t sl = fs + off;
-        slot = b + (sl >= w ? sl - w : sl);
+        return p;
     }
-    __device__ __forceinline__ void load(const T *__restrict__ x, int32_t n)
-    {
-#pragma unroll
-        for (int k = 0; k < PER; ++k) {
-            int32_t c, c_to, slot;
-            locate(k * THREADS + (int)threadIdx.x, c, c_to, slot);
-            buf[k] = vec_t(T(0));
-            if (VEC) {
-                if (c < c_to && c < n) buf[k] = *reinterpret_cast<const vec_u *>(x + (n - c >= V ? (int64_t)c : (int64_t)n - V));
-            } else {
-#pragma unroll
-                for (int e = 0; e < V; ++e)
-                    if (c_to - c > e && n - c > e) buf[k][e] = x[(int64_t)c + e];
-            }
-        }
-    }
-    __device__ __forceinline__ void store(T *xs, int32_t n) const
+    __device__ __forceinline__ void load(const T *__restrict__ x, int wave)
     {
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
-            int32_t c, c_to, slot;
-            locate(k * THREADS + (int)threadIdx.x, c, c_to, slot);
-            if (c < c_to) {
-                vec_t v = buf[k];
-                if (VEC && c < n && n - c < V) {
-                    // holds x[n - V .. n): the columns c .. n - 1 move to the front, zeros behind them
-                    const int cnt = n - c;
-                    vec_t w = vec_t(T(0));
+            const Piece p = piece_of(k * THREADS + wave * kWave);
+            const int32_t u = k * THREADS + (int)threadIdx.x - p.ustart;  // unit inside the piece
+            const __amdgpu_buffer_rsrc_t cols =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(x) + p.from, 0, p.inside * (int32_t)sizeof(T), 0x00020000);
+            buf[k] = __builtin_bit_cast(vec_t, __builtin_amdgcn_raw_buffer_load_b128(cols, (uint32_t)u * 16u, 0, 0));
+        }
+    }
+    __device__ __forceinline__ void store(T *xs, int wave) const
+    {
 #pragma unroll
-                    for (int e = 0; e < V - 1; ++e)
-#pragma unroll
-                        for (int j = 1; j < V; ++j)
-                            if (e < cnt && j == V - cnt + e) w[e] = v[j];
-                    v = w;
-                }
-                *reinterpret_cast<vec_t *>(xs + slot) = v;
+        for (int k = 0; k < PER; ++k) {
+            const Piece p = piece_of(k * THREADS + wave * kWave);
+            const int32_t e = (k * THREADS + (int)threadIdx.x - p.ustart) * V;  // column inside the piece
+            if (e < p.len) {
+                const int32_t sl = p.fslot + e;  // a piece is no longer than its ring: one wrap at most
+                *reinterpret_cast<vec_t *>(xs + p.base + (sl >= p.width ? sl - p.width : sl)) = buf[k];
             }
         }
     }
 };
 
-template <typename T, int NW, bool VEC, int NB, int D>
+template <typename T, int NW, int NB, int D, bool BETA>
 __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T beta, const int2 *__restrict__ chains,
                                                            const int4 *__restrict__ blocks,
                                                            const int4 *__restrict__ pieces,
                                                            const uint16_t *__restrict__ cf, const T *__restrict__ val,
                                                            const int2 *__restrict__ tile_info,
-                                                           const T *__restrict__ x, T *__restrict__ y,
-                                                           T *__restrict__ carry)
+                                                           const T *__restrict__ x, T *y, T *__restrict__ carry)
 {
+    static_assert(D >= 1 && D <= 3, "one loop per starting buffer is written out for up to three buffers");
     // the rings over the columns of x, then the zero the pads point at
     __shared__ __align__(16) T xs[kWindowCols + 16 / sizeof(T)];
-    __shared__ T stage_all[NW * kStageRows];
+    __shared__ T stage_all[NW * kStageSlots];
     const int2 chain = chains[blockIdx.x];  // first block, end block
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    T *stage = stage_all + wave * kStageRows;
-    const int32_t chain_last = blocks[chain.y - 1].y - 1;  // last tile of the chain
+    // the wave's number as a scalar: the tile counters and every loop condition below are uniform
+    const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    WindowStep<T> w{cf, val, tile_info, y, carry, xs, stage_all + wave * kStageSlots, alpha, beta,
+                    blocks[chain.y - 1].y - 1, lane, make_int2(0, 0)};
     // this wave's tiles are those congruent to its number, across the blocks of the chain; D are
-    // in flight (loaded D steps ahead; past the end of the chain the last tile is re-read)
-    WindowTile<T> tl[D];
+    // in flight (requested D steps ahead; past the end of the chain the last tile is re-read)
+    WindowTile<T, BETA> tl[D];
     int32_t t = blocks[chain.x].x + wave;
 #pragma unroll
-    for (int d = 0; d < D; ++d)
-        window_tile_load<T>(tl[d], t + d * NW < chain_last ? t + d * NW : chain_last, lane, cf, val, tile_info);
+    for (int d = 0; d < D; ++d) {
+        const int32_t td = t + d * NW < w.chain_last ? t + d * NW : w.chain_last;
+        window_tile_load<T, BETA>(tl[d], td, tile_info[td], lane, cf, val, y);
+    }
+    w.info_next = tile_info[t + D * NW < w.chain_last ? t + D * NW : w.chain_last];
     if (threadIdx.x == 0) xs[kWindowCols] = T(0);
-    XFetch<T, NW * kWave, VEC, NB> xf;
+    XFetch<T, NW * kWave, NB> xf;
     int4 blk = blocks[chain.x];  // first tile, end tile, pieces of x to fetch before the block: first, end
-    xf.set(pieces, blk.z, blk.w);
-    xf.load(x, n);
-    int32_t b = chain.x, tile_hi;
-    // Start of block b: the columns fetched for it go into the ring once every wave is done with
-    // the block before; the next block's new columns are fetched while this one is multiplied.
-#define ASX_BLOCK_BEGIN()                      \
-    {                                          \
-        __syncthreads();                       \
-        xf.store(xs, n);                       \
-        __syncthreads();                       \
-        tile_hi = blk.y;                       \
-        if (b + 1 < chain.y) {                 \
-            blk = blocks[b + 1];               \
-            xf.set(pieces, blk.z, blk.w);      \
-            xf.load(x, n);                     \
-        }                                      \
-    }
-#define ASX_NEXT(TL, TT) window_tile_load<T>(TL, (TT) < chain_last ? (TT) : chain_last, lane, cf, val, tile_info)
-    // one tile: its rows' sums into the staging area, the loads of the tile D steps ahead (into
-    // the registers this one has just left), then the staged sums to y
-#define ASX_STEP(TL, TT)                                                                                          \
-    {                                                                                                             \
-        const StoreRows<T> out{y, carry + (TT), stage, TL.base & 0x7fffffff, TL.limit, TL.base < 0, alpha, beta}; \
-        tile_reduce<T>(TL, lane, xs, out);                                                                        \
-        ASX_NEXT(TL, (TT) + D * NW);                                                                              \
-        out.flush(lane);                                                                                          \
-    }
+    xf.set(pieces, blk.z, blk.w, n);
+    xf.load(x, wave);
+    int32_t first = 0;  // the buffer that holds the wave's next tile
     // Every wave passes the start of every block of the chain (the barriers count all waves),
-    // whether it has tiles in the block or not.  The D tile buffers take turns without changing
-    // places (the loop over them is unrolled).
-    ASX_BLOCK_BEGIN()
-    for (;;) {  // all conditions are uniform over the wave
-#pragma unroll
-        for (int d = 0; d < D; ++d) {
-            while (t >= tile_hi) {
-                if (++b >= chain.y) return;
-                ASX_BLOCK_BEGIN()
-            }
-            ASX_STEP(tl[d], t);
-            t += NW;
+    // whether it has tiles in the block or not.  All conditions are uniform over the wave.
+    for (int32_t b = chain.x; b < chain.y; ++b) {
+        // the columns fetched for the block go into the ring once every wave is done with the block
+        // before; the next block's new columns are fetched while this one is multiplied
+        __syncthreads();
+        xf.store(xs, wave);
+        __syncthreads();
+        const int32_t tile_hi = blk.y;
+        if (b + 1 < chain.y) {
+            blk = blocks[b + 1];
+            xf.set(pieces, blk.z, blk.w, n);
+            xf.load(x, wave);
         }
+        const int32_t cnt = t < tile_hi ? (tile_hi - t + NW - 1) / NW : 0;  // this wave's tiles in the block
+        // the D tile buffers take turns without changing places
+        if (D == 1 || first == 0)
+            window_steps<T, BETA, D, NW, 0>(tl, t, cnt, w);
+        else if (D == 2 || first == 1)
+            window_steps<T, BETA, D, NW, 1 % D>(tl, t, cnt, w);
+        else
+            window_steps<T, BETA, D, NW, 2 % D>(tl, t, cnt, w);
+        first = (first + cnt) % D;
     }
-#undef ASX_BLOCK_BEGIN
-#undef ASX_STEP
-#undef ASX_NEXT
 }
 
 // Adds the carries to their rows, in tile order: the thread of the first tile of a run of tiles
@@ -572,8 +668,9 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     int32_t *arena = nullptr;
     int32_t *gmin = nullptr, *gmax = nullptr, *row_start = nullptr, *seg_row = nullptr;
     int32_t *bmin = nullptr, *bmax = nullptr, *btiles = nullptr, *tile_off = nullptr, *d_small = nullptr;
-    int32_t *tmp = nullptr;
-    std::vector<int32_t> h_bmin, h_bmax, h_off, blk, pcs, chains;
+    std::vector<int32_t> h_bmin, h_bmax, h_bt, h_off, h_soff, h_order, blk, pcs, chains;
+    int64_t stack_ulo = 0, stack_uhi = 0;
+    bool stacked = false;
     std::vector<uint32_t> h_bits;
     uint32_t *d_bits = nullptr;
     BandTable bands{};
@@ -593,17 +690,15 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     } while (0)
     // the scratch of the build in one allocation: the span of every group of rows (two arrays), where
     // every row starts, the row holding every 256th stored element, four arrays of max_nb + 1, a
-    // few counters, the scan's block sums
+    // few counters
     {
         const auto pad64 = [](size_t v) { return (v + 63) & ~(size_t)63; };
         const size_t per_group = pad64((size_t)ngroups), per_row = pad64((size_t)m), per_seg = pad64((size_t)nseg + 1);
         const size_t per_block = pad64((size_t)max_nb + 1);
-        ASX_TRY(hipMalloc((void **)&arena, sizeof(int32_t) * (2 * per_group + per_row + per_seg + 4 * per_block + 64 +
-                                                              scan_scratch_ints((int64_t)max_nb + 1))));
+        ASX_TRY(hipMalloc((void **)&arena, sizeof(int32_t) * (2 * per_group + per_row + per_seg + 4 * per_block + 64)));
         gmin = arena, gmax = gmin + per_group, row_start = gmax + per_group, seg_row = row_start + per_row;
         bmin = seg_row + per_seg, bmax = bmin + per_block, btiles = bmax + per_block, tile_off = btiles + per_block;
         d_small = tile_off + per_block;
-        tmp = d_small + 64;
     }
 
     // 1. column span of every group of rows
@@ -643,6 +738,12 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
         //     c - centre(r) occur (a bit per 64 of them), the runs of occupied offsets, and the
         //     largest block whose bands (block's advance along the diagonal + width of the run) fit
         //     the LDS together.  More runs than rings: the closest runs are joined.
+        // a ring holds a multiple of 64 16-byte units: a block's pieces, each rounded up to 64 units
+        // (one wave's worth) as the kernel fetches them, then fit the registers the fetch passes through
+        const auto ring_size = [](int64_t columns) {
+            constexpr int64_t unit = kWave * (16 / (int64_t)sizeof(T));
+            return (columns + unit - 1) / unit * unit;
+        };
         const int64_t nbins = (2 * (int64_t)n >> 6) + 2;
         const size_t words = (size_t)(nbins + 31) / 32;
         ASX_TRY(hipMalloc((void **)&d_bits, sizeof(uint32_t) * words));
@@ -659,37 +760,91 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
             else
                 runs.emplace_back(b, b);
         }
-        while ((int)runs.size() > kWindowBands) {  // join the two runs with the smallest gap
-            size_t best = 0;
-            for (size_t i = 1; i + 1 < runs.size(); ++i)
-                if (runs[i + 1].first - runs[i].second < runs[best + 1].first - runs[best].second) best = i;
-            runs[best].second = runs[best + 1].second;
-            runs.erase(runs.begin() + (long)best + 1);
+        const auto join_runs = [&runs](size_t keep) {  // join the two runs with the smallest gap until `keep` are left
+            while (runs.size() > keep) {
+                size_t best = 0;
+                for (size_t i = 1; i + 1 < runs.size(); ++i)
+                    if (runs[i + 1].first - runs[i].second < runs[best + 1].first - runs[best].second) best = i;
+                runs[best].second = runs[best + 1].second;
+                runs.erase(runs.begin() + (long)best + 1);
+            }
+        };
+        const auto set_bands = [&runs, &bands, n]() {
+            bands.nbands = (int32_t)runs.size();
+            for (int k = 0; k < bands.nbands; ++k) {
+                bands.dlo[k] = (int32_t)std::max<int64_t>((runs[(size_t)k].first << 6) - n, -(int64_t)n);
+                bands.dhi[k] = (int32_t)std::min<int64_t>(((runs[(size_t)k].second + 1) << 6) - 1 - n, n);
+            }
+        };
+        // Stacked planes first (see BandTable): a square matrix whose runs, joined into three bands,
+        // lie a whole number of planes apart.  P = the divisor of m nearest to half the distance
+        // between the outer bands (any P is correct; one off the true distance only widens what the
+        // regions must hold); U = the offsets all three bands span once band k is shifted back by
+        // (k - 1) P; R = P / d rows per block: the largest that leaves enough blocks, else the
+        // smallest whose three regions fit.
+        if (runs.size() >= 3 && m == n) {
+            const std::vector<std::pair<int64_t, int64_t>> all_runs = runs;
+            join_runs(3);
+            set_bands();
+            const int64_t p0 = (((int64_t)bands.dlo[2] + bands.dhi[2]) - ((int64_t)bands.dlo[0] + bands.dhi[0])) / 4;
+            int64_t P = 0;
+            for (int64_t e = 0; e <= 64 && !P; ++e)
+                for (int64_t cand : {p0 - e, p0 + e})
+                    if (cand >= 256 && cand < m && m % cand == 0) {
+                        P = cand;
+                        break;
+                    }
+            if (P) {
+                int64_t ulo = INT64_MAX, uhi = INT64_MIN;
+                for (int k = 0; k < 3; ++k) {
+                    ulo = std::min<int64_t>(ulo, bands.dlo[k] - (k - 1) * P);
+                    uhi = std::max<int64_t>(uhi, bands.dhi[k] - (k - 1) * P);
+                }
+                int64_t pick = 0, size = 0;
+                for (int64_t d = 1; P / d >= 256; ++d) {
+                    if (P % d) continue;
+                    const int64_t rows = P / d;
+                    const int64_t sz = ring_size(rows + (uhi - ulo) + kWindowSlack + 3 + 3);
+                    if (rows > 8192 || 3 * sz > kWindowCols) continue;
+                    pick = rows, size = sz;
+                    if (m / rows >= min_blocks) break;
+                }
+                if (pick) {
+                    wm.rows_per_block = (int32_t)pick;
+                    wm.nblocks = (int32_t)(m / pick);
+                    bands.stack_rows = (int32_t)P;
+                    bands.stack_size = (int32_t)size;
+                    stack_ulo = ulo, stack_uhi = uhi;
+                    for (int k = 0; k < 3; ++k) bands.base[k] = 0, bands.width[k] = (int32_t)size;  // not used to place
+                }
+            }
+            if (!wm.rows_per_block) runs = all_runs;
         }
-        // one run of offsets: the rows fill a band too wide for the single window tried above
-        // (the one-ring kernel places column c at c mod kWindowCols; it is not built from here)
-        if (runs.size() < 2) {
-            st = ASX_STATUS_NOT_SUPPORTED;
-            goto done;
-        }
-        bands.nbands = (int32_t)runs.size();
-        for (int k = 0; k < bands.nbands; ++k) {
-            bands.dlo[k] = (int32_t)std::max<int64_t>((runs[(size_t)k].first << 6) - n, -(int64_t)n);
-            bands.dhi[k] = (int32_t)std::min<int64_t>(((runs[(size_t)k].second + 1) << 6) - 1 - n, n);
+        if (!wm.rows_per_block) {
+            // a ring per band; more runs than rings: the closest runs are joined
+            join_runs(kWindowBands);
+            // one run of offsets: the rows fill a band too wide for the single window tried above
+            // (the one-ring kernel places column c at c mod kWindowCols; it is not built from here)
+            if (runs.size() < 2) {
+                st = ASX_STATUS_NOT_SUPPORTED;
+                goto done;
+            }
+            set_bands();
         }
         for (int32_t rows : {8192, 7168, 6144, 5120, 4608, 4096, 3584, 3072, 2560, 2048, 1792, 1536, 1280, 1024, 768, 512, 384, 256}) {
+            if (wm.rows_per_block) break;  // stacked planes
             if (rows > 256 && ceil_div64(m, rows) < min_blocks) continue;
             const int64_t advance = ceil_div64((int64_t)rows * n, m) + 1;  // of the centre over a block
             int64_t total = 0;
             for (int k = 0; k < bands.nbands; ++k)
-                total += (advance + ((int64_t)bands.dhi[k] - bands.dlo[k]) + 1 + kWindowSlack + 3 + 3) & ~(int64_t)3;
+                total += ring_size(advance + ((int64_t)bands.dhi[k] - bands.dlo[k]) + 1 + kWindowSlack + 3 + 3);
             if (total > kWindowCols) continue;
             wm.rows_per_block = rows;
             wm.nblocks = (int32_t)ceil_div64(m, rows);
             int32_t at = 0;
             for (int k = 0; k < bands.nbands; ++k) {
                 bands.base[k] = at;
-                bands.width[k] = (int32_t)((advance + ((int64_t)bands.dhi[k] - bands.dlo[k]) + 1 + kWindowSlack + 3 + 3) & ~(int64_t)3);
+                bands.width[k] = (int32_t)ring_size(advance + ((int64_t)bands.dhi[k] - bands.dlo[k]) + 1 + kWindowSlack + 3 + 3);
                 at += bands.width[k];
             }
             break;
@@ -700,26 +855,55 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
         }
     }
     wm.nbands = bands.nbands;
-    // 3. where every row starts inside its block; tiles of every block
+    stacked = bands.stack_rows > 0;
+    wm.stack_rows = bands.stack_rows;
+    // 3. where every row starts inside its block; tiles of every block; the order the blocks are
+    //    stored in (the order the chains walk them) and the first tile of each
     hipLaunchKernelGGL(k_window_row_starts, dim3((unsigned)ceil_div64((int64_t)wm.nblocks * kWave, kBlock)), dim3(kBlock), 0, s, row_ptr, m,
                        wm.rows_per_block, wm.nblocks, row_start, btiles);
-    ASX_TRY(hipMemsetAsync(btiles + wm.nblocks, 0, sizeof(int32_t), s));
-    st = launch_exclusive_scan_i32(btiles, tile_off, (int64_t)wm.nblocks + 1, tmp, s);
-    if (st) goto done;
     h_bmin.resize((size_t)wm.nblocks);
     h_bmax.resize((size_t)wm.nblocks);
+    h_bt.resize((size_t)wm.nblocks);
     h_off.resize((size_t)wm.nblocks + 1);
     if (bands.nbands == 1) {
         ASX_TRY(hipMemcpyAsync(h_bmin.data(), bmin, sizeof(int32_t) * h_bmin.size(), hipMemcpyDeviceToHost, s));
         ASX_TRY(hipMemcpyAsync(h_bmax.data(), bmax, sizeof(int32_t) * h_bmax.size(), hipMemcpyDeviceToHost, s));
     }
-    ASX_TRY(hipMemcpyAsync(h_off.data(), tile_off, sizeof(int32_t) * h_off.size(), hipMemcpyDeviceToHost, s));
+    ASX_TRY(hipMemcpyAsync(h_bt.data(), btiles, sizeof(int32_t) * h_bt.size(), hipMemcpyDeviceToHost, s));
     ASX_TRY(hipStreamSynchronize(s));
-    wm.ntiles = h_off[(size_t)wm.nblocks];
-    slots = (int64_t)wm.ntiles * kSlicedTile;
+    if (stacked) {
+        // column j of blocks (the j-th R rows of every plane), plane after plane, then column j + 1
+        const int32_t per_plane = bands.stack_rows / wm.rows_per_block, nplanes = m / bands.stack_rows;
+        h_order.resize((size_t)wm.nblocks);
+        h_soff.resize((size_t)wm.nblocks + 1);
+        int64_t at = 0;
+        for (int32_t i = 0; i < wm.nblocks; ++i) {
+            const int32_t b = (i % nplanes) * per_plane + i / nplanes;
+            h_order[(size_t)i] = b;
+            h_soff[(size_t)i] = (int32_t)at;
+            h_off[(size_t)b] = (int32_t)at;
+            at += h_bt[(size_t)b];
+        }
+        slots = at * kSlicedTile;
+        h_soff[(size_t)wm.nblocks] = h_off[(size_t)wm.nblocks] = (int32_t)std::min<int64_t>(at, 0x7fffffff);
+    } else {
+        int64_t at = 0;
+        for (int32_t b = 0; b < wm.nblocks; ++b) {
+            h_off[(size_t)b] = (int32_t)at;
+            at += h_bt[(size_t)b];
+        }
+        slots = at * kSlicedTile;
+        h_off[(size_t)wm.nblocks] = (int32_t)std::min<int64_t>(at, 0x7fffffff);
+    }
     if (slots > 0x7fffffff) {
         st = ASX_STATUS_INVALID_SIZE;
         goto done;
+    }
+    wm.ntiles = (int32_t)(slots / kSlicedTile);
+    ASX_TRY(hipMemcpyAsync(tile_off, h_off.data(), sizeof(int32_t) * h_off.size(), hipMemcpyHostToDevice, s));
+    if (stacked) {  // bmin and bmax are free: they serve single windows only
+        ASX_TRY(hipMemcpyAsync(bmin, h_soff.data(), sizeof(int32_t) * h_soff.size(), hipMemcpyHostToDevice, s));
+        ASX_TRY(hipMemcpyAsync(bmax, h_order.data(), sizeof(int32_t) * h_order.size(), hipMemcpyHostToDevice, s));
     }
     {   // the regrouped copy in one allocation
         const size_t o_val = 0, o_perm = align_up(sizeof(T) * (size_t)slots, 256);
@@ -736,19 +920,61 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     hipLaunchKernelGGL((k_window_place<T>), dim3((unsigned)ceil_div64(nnz, kBlock)), dim3(kBlock), 0, s, row_ptr, col, val,
                        m, n, nnz, wm.rows_per_block, bands, seg_row, row_start, tile_off, wm.cf, (T *)wm.val, wm.perm);
     hipLaunchKernelGGL((k_window_pads<T>), dim3(mgrid), dim3(kBlock), 0, s, row_ptr, m, wm.rows_per_block, row_start, tile_off,
-                       (uint16_t)(0x8000 | kWindowCols), wm.cf, (T *)wm.val, wm.perm);
+                       btiles, (uint16_t)(0x8000 | kWindowCols), wm.cf, (T *)wm.val, wm.perm);
     // 5. first row and number of rows of every tile
     hipLaunchKernelGGL(k_window_fill_i32, dim3(1), dim3(kBlock), 0, s, d_small, (int64_t)2, 0);
     hipLaunchKernelGGL(k_window_tile_info, dim3((unsigned)ceil_div64(wm.ntiles, kBlock)), dim3(kBlock), 0, s, row_start, m,
-                       wm.rows_per_block, wm.nblocks, tile_off, wm.ntiles, (int2 *)wm.tile_info, d_small);
+                       wm.rows_per_block, wm.nblocks, stacked ? bmin : tile_off, stacked ? bmax : (int32_t *)nullptr,
+                       wm.ntiles, (int2 *)wm.tile_info, d_small);
     ASX_TRY(hipMemcpyAsync(h_small, d_small, sizeof(int32_t), hipMemcpyDeviceToHost, s));
     // 6. chains of blocks, one per workgroup, of about equal numbers of tiles.  Inside a chain a
     //    block fetches, per band, only the columns behind those already in the band's ring; a block
     //    whose columns start before what a ring still holds begins a new chain (and fetches its
     //    whole windows).
     {
-        const int64_t per_chain = std::max<int64_t>(1, ceil_div64(wm.ntiles, target_wgs));
-        blk.resize((size_t)wm.nblocks * 4);
+    const int64_t per_chain = std::max<int64_t>(1, ceil_div64(wm.ntiles, target_wgs));
+    blk.resize((size_t)wm.nblocks * 4);
+    if (stacked) {
+        // A chain stays inside one column of blocks and climbs the planes.  Region g holds, for one
+        // q at a time, the columns around the rows of plane q of this column: block (plane p) needs
+        // q = p - 1, p, p + 1 and fetches those its chain has not left in place.
+        const int64_t P = bands.stack_rows, R = wm.rows_per_block, nplanes = m / P;
+        int64_t held[3] = {INT64_MIN, INT64_MIN, INT64_MIN};
+        int32_t chain_lo = 0;
+        int64_t chain_tiles = 0;
+        for (int32_t i = 0; i < wm.nblocks; ++i) {
+            const int64_t j = i / nplanes, p = i % nplanes;
+            if (i != chain_lo && (p == 0 || chain_tiles >= per_chain)) {
+                chains.push_back(chain_lo);
+                chains.push_back(i);
+                chain_lo = i;
+                chain_tiles = 0;
+                held[0] = held[1] = held[2] = INT64_MIN;
+            }
+            blk[(size_t)i * 4 + 0] = h_soff[(size_t)i];
+            blk[(size_t)i * 4 + 1] = h_soff[(size_t)i + 1];
+            blk[(size_t)i * 4 + 2] = (int32_t)(pcs.size() / 4);
+            for (int64_t q = p - 1; q <= p + 1; ++q) {
+                const int g = (int)(((q % 3) + 3) % 3);
+                int64_t from = 0, to = 0;
+                if (held[g] != q) {
+                    const int64_t a = std::min<int64_t>(std::max<int64_t>(q * P + j * R + stack_ulo, 0), n);
+                    const int64_t z = std::min<int64_t>(std::max<int64_t>(q * P + (j + 1) * R + stack_uhi, 0), n);
+                    from = a & ~(int64_t)3;
+                    to = z > a ? (z + 3) & ~(int64_t)3 : from;
+                    held[g] = q;
+                }
+                pcs.push_back((int32_t)from);
+                pcs.push_back((int32_t)to);
+                pcs.push_back(g * bands.stack_size);
+                pcs.push_back(bands.stack_size);
+            }
+            blk[(size_t)i * 4 + 3] = (int32_t)(pcs.size() / 4);
+            chain_tiles += h_soff[(size_t)i + 1] - h_soff[(size_t)i];
+        }
+        chains.push_back(chain_lo);
+        chains.push_back(wm.nblocks);
+    } else {
         int64_t have[kWindowBands];  // columns [low, have) were fetched in this chain (have = -1: nothing yet)
         int64_t low[kWindowBands];
         for (int k = 0; k < kWindowBands; ++k) have[k] = -1, low[k] = 0;
@@ -811,8 +1037,9 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
         }
         chains.push_back(chain_lo);
         chains.push_back(wm.nblocks);
-        wm.nchains = (int32_t)(chains.size() / 2);
-        wm.npieces = (int32_t)(pcs.size() / 4);
+    }
+    wm.nchains = (int32_t)(chains.size() / 2);
+    wm.npieces = (int32_t)(pcs.size() / 4);
     }
     {   // the tables of the blocks in one allocation (16-byte entries first)
         const size_t o_pieces = align_up(sizeof(int32_t) * blk.size(), 256);
@@ -855,15 +1082,13 @@ int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, co
 {
     if (m <= 0) return ASX_STATUS_SUCCESS;
     if (wm->has_carry && !carry) return ASX_STATUS_INVALID_POINTER;
-    // x on a 16-byte boundary (every allocation is) and at least one 16-byte unit long: 16-byte
-    // fetches; else element by element
-    const bool vec = ((uintptr_t)x % 16) == 0 && (size_t)n * sizeof(T) >= 16;
-    // tiles in flight per wave: three with one window (measured 1-2 % ahead of two); two with bands,
-    // where three no longer fit the 128 registers a lane of a 1024-thread workgroup may use
-    const auto kernel = wm->nbands == 1
-                            ? (vec ? k_spmv_window<T, kWindowWaves, true, 1, 3> : k_spmv_window<T, kWindowWaves, false, 1, 3>)
-                            : (vec ? k_spmv_window<T, kWindowWaves, true, kWindowBands, 2>
-                                   : k_spmv_window<T, kWindowWaves, false, kWindowBands, 2>);
+    // a kernel of its own for beta != 0, which loads y ahead with the tiles
+    const bool bands = wm->nbands != 1, b0 = beta == T(0);
+#define ASX_PICK(NB)                                                                 \
+    (b0 ? k_spmv_window<T, kWindowWaves, NB, window_depth<T>(NB, false), false>      \
+        : k_spmv_window<T, kWindowWaves, NB, window_depth<T>(NB, true), true>)
+    const auto kernel = bands ? ASX_PICK(kWindowBands) : ASX_PICK(1);
+#undef ASX_PICK
     hipLaunchKernelGGL(kernel, dim3((unsigned)wm->nchains), dim3(kWindowWaves * kWave), 0, s, n, alpha, beta,
                        reinterpret_cast<const int2 *>(wm->chains), reinterpret_cast<const int4 *>(wm->blocks),
                        reinterpret_cast<const int4 *>(wm->pieces), wm->cf, (const T *)wm->val,

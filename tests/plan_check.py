@@ -19,6 +19,8 @@ import numpy as np
 TILE = 256
 WINDOW_COLS = 16384
 PAD_ROW = 0x7FFFFFFF
+MIN_ROW_SLOTS = 2    # slots a row takes at least in a window plan
+MAX_TILE_ROWS = 128  # so a tile of 256 slots holds at most this many rows
 
 
 class PlanError(AssertionError):
@@ -256,8 +258,8 @@ def check_window(arrays, rp, col, n, rows_per_block, nbands, itemsize):
     nblocks = blocks.shape[0]
     _need(nblocks == -(-m // R), f"{nblocks} blocks for {m} rows in blocks of {R}")
     # blocks tile the tiles, chains tile the blocks, blocks' pieces are consecutive
-    _need(blocks[0, 0] == 0 and blocks[-1, 1] == ntiles and np.all(blocks[1:, 0] == blocks[:-1, 1]) and np.all(blocks[:, 1] >= blocks[:, 0]),
-          "the blocks' tile ranges must follow one another and cover every tile")
+    _need(blocks[0, 0] == 0 and blocks[-1, 1] == ntiles and np.all(blocks[1:, 0] == blocks[:-1, 1]) and np.all(blocks[:, 1] > blocks[:, 0]),
+          "the blocks' tile ranges must follow one another, cover every tile and hold at least one tile each")
     _need(blocks[0, 2] == 0 and blocks[-1, 3] == pieces.shape[0] and np.all(blocks[1:, 2] == blocks[:-1, 3]),
           "the blocks' piece ranges must follow one another")
     _need(np.all(blocks[:, 3] - blocks[:, 2] == nbands), f"every block lists one piece per band ({nbands})")
@@ -265,14 +267,23 @@ def check_window(arrays, rp, col, n, rows_per_block, nbands, itemsize):
           "the chains must follow one another and cover every block")
     _need(np.all(pieces[:, 0] % 4 == 0) and np.all(pieces[:, 2] % 4 == 0) and np.all(pieces[:, 3] % 4 == 0),
           "pieces start at, and rings are, multiples of 4 columns (16-byte units)")
+    _need(np.all(pieces[:, 0] >= 0) and np.all(pieces[:, 1] <= n + 3), "a piece leaves the columns of x")
     _need(np.all(pieces[:, 1] >= pieces[:, 0]) and np.all(pieces[:, 1] - pieces[:, 0] <= pieces[:, 3]), "a piece is longer than its ring")
     if nbands == 1:
         _need(np.all(pieces[:, 2] == 0) and np.all(pieces[:, 3] == WINDOW_COLS), "one band: the ring is the whole window")
-    ring = pieces[: nbands, 2:4]
-    _need(np.all(pieces[:, 2:4].reshape(-1, nbands, 2) == ring[None]), "every block must use the same rings")
+    # the rings (in any order within a block: stacked planes rotate them) are the same for every
+    # block, apart and inside the window; what a block fetches fits the fetch registers (one window)
+    rings = pieces[:, 2:4].reshape(-1, nbands, 2)
+    rings = np.take_along_axis(rings, np.argsort(rings[:, :, 0], axis=1)[:, :, None], axis=1)
+    ring = rings[0]
+    _need(np.all(rings == ring[None]), "every block must use the same rings")
     _need(np.all(ring[1:, 0] >= ring[:-1, 0] + ring[:-1, 1]) and ring[-1, 0] + ring[-1, 1] <= WINDOW_COLS, "rings overlap or leave the LDS window")
+    unit = 16 // itemsize * (64 if nbands > 1 else 1)  # several pieces: each starts a wave's 64 units
+    fetched = (-(-(pieces[:, 1] - pieces[:, 0]) // unit) * unit).reshape(-1, nbands).sum(axis=1)
+    _need(np.all(fetched <= WINDOW_COLS), "a block fetches more columns than the fetch registers hold")
 
-    # stored elements: each placed once, in order
+    # stored elements: each placed once; the blocks may be stored in another order than their rows'
+    # (block i of the tables holds the rows of row block order[i]), the elements of one block in order
     slots = ntiles * TILE
     perm = np.asarray(arrays["perm"], np.int64)
     _need(perm.size == slots, f"perm holds {perm.size} slots for {ntiles} tiles")
@@ -280,27 +291,47 @@ def check_window(arrays, rp, col, n, rows_per_block, nbands, itemsize):
     cf = np.asarray(arrays["cf"], np.int64)
     real = np.nonzero(perm >= 0)[0]
     src = perm[real]
-    if src.size != nnz or not np.array_equal(src, np.arange(nnz)):
+    if src.size != nnz or not np.array_equal(np.sort(src), np.arange(nnz)):
         u, c = np.unique(src, return_counts=True)
         dup = u[c > 1]
-        raise PlanError(f"stored elements are not placed once each in order: {src.size} placed of {nnz}"
+        raise PlanError(f"stored elements are not placed once each: {src.size} placed of {nnz}"
                         + (f", element {int(dup[0])} placed {int(c[c > 1][0])} times" if dup.size else ""))
-    erow = rows_of(rp, nnz)
+    erow = rows_of(rp, nnz)[src]  # row of the stored element in every occupied slot
     tile_of = real // TILE
     blk_of_tile = np.searchsorted(blocks[:, 1], np.arange(ntiles), side="right")
-    _need(np.array_equal(blk_of_tile[tile_of], erow // R), "a stored element sits in a tile of another block than its row's")
-    # flags: first slot of a row, first slot of a tile; pads open runs of their own and point at the zero
+    order = (info[blocks[:, 0], 0] & 0x7FFFFFFF) // R
+    _need(np.array_equal(np.sort(order), np.arange(nblocks)), "the stored blocks do not hold every block of rows once")
+    _need(np.array_equal(order[blk_of_tile[tile_of]], erow // R), "a stored element sits in a tile of another block than its row's")
+    same_block = blk_of_tile[tile_of][1:] == blk_of_tile[tile_of][:-1]
+    _need(np.all(src[1:][same_block] > src[:-1][same_block]), "the stored elements of a block are out of order")
+    # flags: first slot of a row, first slot of a tile; pads point at the zero and open runs of their
+    # own, except the one that makes a row of fewer than MIN_ROW_SLOTS stored elements up to that many
+    # slots (a tile then holds at most MAX_TILE_ROWS rows, all the kernel stages per tile)
     flag = cf >> 15
-    want_flag = np.ones(slots, np.int64)
-    want_flag[real] = ((src == rp[erow]) | (real % TILE == 0)).astype(np.int64)
-    bad = np.nonzero(flag != want_flag)[0]
-    _need(bad.size == 0, f"slot {int(bad[0]) if bad.size else -1}: run-start flag {int(flag[bad[0]]) if bad.size else 0} is wrong")
     pad = perm < 0
     _need(np.all((cf[pad] & 0x7FFF) == WINDOW_COLS), "a pad does not point at the zero behind the rings")
-    # tile words: run k of tile t is row first(t) + k for k < limit(t); later runs are padding
     first = info[:, 0] & 0x7FFFFFFF
     cont = (info[:, 0] >> 31) & 1
     limit = info[:, 1]
+    _need(np.all(limit <= MAX_TILE_ROWS) and np.all(limit >= 0), f"a tile holds more than {MAX_TILE_ROWS} rows")
+    row_of_element = rows_of(rp, nnz)
+    want_flag = np.ones(slots, np.int64)
+    want_flag[real] = ((src == rp[erow]) | (real % TILE == 0)).astype(np.int64)
+    # where every row starts, from the tile words and the flags as they are: run k of a tile is row
+    # first + k; the slot behind the start of a row of 0 or 1 stored elements continues its run
+    hd0 = np.nonzero(flag)[0]
+    ht0 = hd0 // TILE
+    k0 = np.arange(hd0.size) - np.searchsorted(ht0, ht0, side="left")
+    starts = (k0 < limit[ht0]) & ~((k0 == 0) & (cont[ht0] == 1))
+    short = starts & (first[ht0] + k0 < m)
+    short[short] = (rp[(first[ht0] + k0)[short] + 1] - rp[(first[ht0] + k0)[short]]) < MIN_ROW_SLOTS
+    ext = hd0[short] + 1
+    _need(np.all(ext % TILE != 0) and np.all(ext < slots), "a row of fewer than two stored elements starts in the last slot of a tile")
+    _need(np.all(pad[ext]), "the slot behind a row of fewer than two stored elements holds a stored element")
+    want_flag[ext] = 0
+    bad = np.nonzero(flag != want_flag)[0]
+    _need(bad.size == 0, f"slot {int(bad[0]) if bad.size else -1}: run-start flag {int(flag[bad[0]]) if bad.size else 0} is wrong")
+    # tile words: run k of tile t is row first(t) + k for k < limit(t); later runs are padding
     hd = np.nonzero(flag)[0]
     ht = hd // TILE
     k = np.arange(hd.size) - np.searchsorted(ht, ht, side="left")
@@ -312,7 +343,7 @@ def check_window(arrays, rp, col, n, rows_per_block, nbands, itemsize):
     empty = rp[hr + 1] == rp[hr]
     _need(np.all(perm[hs[empty]] < 0), "the slot of an empty row holds a stored element")
     ne = ~empty
-    _need(np.all(perm[hs[ne]] >= 0) and np.array_equal(erow[perm[hs[ne]]], hr[ne]), "run k of a tile is not row (first row + k)")
+    _need(np.all(perm[hs[ne]] >= 0) and np.array_equal(row_of_element[perm[hs[ne]]], hr[ne]), "run k of a tile is not row (first row + k)")
     starts_row = perm[hs[ne]] == rp[hr[ne]]
     kk, tt = k[is_row][ne], ht[is_row][ne]
     _need(np.all(starts_row | ((kk == 0) & (cont[tt] == 1))), "a run that continues a row must be the first of a tile marked so")
@@ -327,7 +358,7 @@ def check_window(arrays, rp, col, n, rows_per_block, nbands, itemsize):
     # columns: replay every chain's fetches on a model of the rings
     lds = cf & 0x7FFF
     ecol = np.full(slots, -1, np.int64)
-    ecol[real] = col
+    ecol[real] = col[src]
     for c0, c1 in chains:
         held = np.full(WINDOW_COLS, -1, np.int64)
         for b in range(int(c0), int(c1)):
@@ -343,10 +374,15 @@ def check_window(arrays, rp, col, n, rows_per_block, nbands, itemsize):
                                 f"{int(ecol[d])}, which holds column {int(held[lds[d]])} when the block is multiplied")
 
 
-def window_plan_arrays(rp, col, n, rows_per_block, itemsize, tiles_per_chain=1 << 30, fresh_check=True):
-    """A one-band window plan built on the host from its definition, in the layout Plan.export
-    gives.  fresh_check=False leaves out the rule that a block whose columns start below what its
-    chain has fetched begins a new chain (the mistake a replay of the rings must catch)."""
+def window_plan_arrays(rp, col, n, rows_per_block, itemsize, tiles_per_chain=1 << 30, fresh_check=True, stack=None,
+                       rotate=0):
+    """A window plan built on the host from its definition, in the layout Plan.export gives: one
+    band, or, with stack = (P, lowest, highest offset from the diagonal once the bands P below
+    and above it are shifted onto it), three bands on stacked planes of P rows (square matrix, P a
+    multiple of rows_per_block and a divisor of the number of rows).  fresh_check=False leaves out
+    the rule that a block whose columns start below what its chain has fetched begins a new chain,
+    rotate != 0 turns the regions of stacked planes the wrong way (the mistakes a replay of the
+    rings must catch)."""
     rp = np.asarray(rp, np.int64)
     col = np.asarray(col, np.int64)
     m, nnz, R = rp.size - 1, col.size, rows_per_block
@@ -356,14 +392,26 @@ def window_plan_arrays(rp, col, n, rows_per_block, itemsize, tiles_per_chain=1 <
     for b in range(nblocks):
         pos = 0
         for r in range(b * R, min(m, (b + 1) * R)):
-            ln = max(1, int(rp[r + 1] - rp[r]))
+            ln = max(MIN_ROW_SLOTS, int(rp[r + 1] - rp[r]))
             if ln <= 16 and pos % TILE + ln > TILE:
                 pos = (pos // TILE + 1) * TILE
             row_start[r] = pos
             pos += ln
         btiles[b] = -(-pos // TILE)
-    tile_off = np.r_[0, np.cumsum(btiles)]
-    ntiles = int(tile_off[-1])
+    if stack:
+        P, ulo, uhi = stack
+        assert m == n and m % P == 0 and P % R == 0
+        per_plane, nplanes = P // R, m // P
+        order = np.array([(i % nplanes) * per_plane + i // nplanes for i in range(nblocks)])
+        unit = 64 * (16 // itemsize)
+        size = -(-(R + (uhi - ulo) + 8 + 6) // unit) * unit
+        assert 3 * size <= WINDOW_COLS
+    else:
+        order = np.arange(nblocks)
+    stored_off = np.r_[0, np.cumsum(btiles[order])]
+    tile_off = np.zeros(nblocks + 1, np.int64)
+    tile_off[order] = stored_off[:-1]
+    ntiles = int(stored_off[-1])
     slots = ntiles * TILE
     erow = rows_of(rp, nnz)
     o = row_start[erow] + (np.arange(nnz) - rp[erow])
@@ -371,43 +419,73 @@ def window_plan_arrays(rp, col, n, rows_per_block, itemsize, tiles_per_chain=1 <
     perm = np.full(slots, -1, np.int64)
     perm[d] = np.arange(nnz)
     cf = np.full(slots, 0x8000 | WINDOW_COLS, np.int64)
+    lens = rp[1:] - rp[:-1]
+    short_rows = np.nonzero(lens < MIN_ROW_SLOTS)[0]
+    cf[tile_off[short_rows // R] * TILE + row_start[short_rows] + 1] = WINDOW_COLS  # continues the row's run
     head = (np.arange(nnz) == rp[erow]) | (o % TILE == 0)
-    cf[d] = (col % WINDOW_COLS) | (head.astype(np.int64) << 15)
+    if stack:
+        off = col - erow
+        band = np.where(off < ulo, 0, np.where(off > uhi, 2, 1))  # the bands lie P apart, further than they are wide
+        q = erow // P + band - 1
+        cf[d] = (((q + rotate) % 3) * size + col % size) | (head.astype(np.int64) << 15)
+    else:
+        cf[d] = (col % WINDOW_COLS) | (head.astype(np.int64) << 15)
     info = np.zeros((ntiles, 2), np.int64)
     for b in range(nblocks):
         r0, r1 = b * R, min(m, (b + 1) * R)
         rs = row_start[r0:r1]
-        for t in range(int(tile_off[b]), int(tile_off[b + 1])):
+        for t in range(int(tile_off[b]), int(tile_off[b] + btiles[b])):
             off = (t - tile_off[b]) * TILE
             a = r0 + int(np.searchsorted(rs, off, side="right")) - 1
             u = r0 + int(np.searchsorted(rs, off + TILE, side="left"))
             info[t] = (a | ((1 << 31) if row_start[a] != off else 0), u - a)
     blocks, pieces, chains = [], [], []
-    have, low, chain_lo, chain_tiles = -1, 0, 0, 0
-    for b in range(nblocks):
-        e0, e1 = int(rp[b * R]), int(rp[min(m, (b + 1) * R)])
-        lo = hi = 0
-        if e1 > e0:
-            lo, hi = int(col[e0:e1].min()) & ~3, (int(col[e0:e1].max()) + 4) & ~3
-        fresh = False
-        if b != chain_lo:
-            if fresh_check and hi > lo and have >= 0 and (lo < low or lo < max(have, hi) - WINDOW_COLS + 8):
-                fresh = True
-            if chain_tiles >= tiles_per_chain:
-                fresh = True
-        if fresh:
-            chains.append([chain_lo, b])
-            chain_lo, chain_tiles, have, low = b, 0, -1, 0
-        fr = to = lo
-        if hi > lo:
-            if have < 0 or lo >= have:
-                fr, to, low = lo, hi, lo
-            else:
-                fr, to = have, max(have, hi)
-            have = to
-        blocks.append([tile_off[b], tile_off[b + 1], len(pieces), len(pieces) + 1])
-        pieces.append([fr, to, 0, WINDOW_COLS])
-        chain_tiles += int(btiles[b])
+    chain_lo, chain_tiles = 0, 0
+    if stack:
+        held = [None, None, None]
+        for i in range(nblocks):
+            j, p = i // nplanes, i % nplanes
+            if i != chain_lo and (p == 0 or chain_tiles >= tiles_per_chain):
+                chains.append([chain_lo, i])
+                chain_lo, chain_tiles, held = i, 0, [None, None, None]
+            blocks.append([stored_off[i], stored_off[i + 1], len(pieces), len(pieces) + 3])
+            for qq in (p - 1, p, p + 1):
+                g = qq % 3
+                fr = to = 0
+                if held[g] != qq:
+                    a = min(max(qq * P + j * R + ulo, 0), n)
+                    z = min(max(qq * P + (j + 1) * R + uhi, 0), n)
+                    fr = a & ~3
+                    to = (z + 3) & ~3 if z > a else fr
+                    held[g] = qq
+                pieces.append([fr, to, g * size, size])
+            chain_tiles += int(btiles[order[i]])
+    else:
+        have, low = -1, 0
+        for b in range(nblocks):
+            e0, e1 = int(rp[b * R]), int(rp[min(m, (b + 1) * R)])
+            lo = hi = 0
+            if e1 > e0:
+                lo, hi = int(col[e0:e1].min()) & ~3, (int(col[e0:e1].max()) + 4) & ~3
+            fresh = False
+            if b != chain_lo:
+                if fresh_check and hi > lo and have >= 0 and (lo < low or lo < max(have, hi) - WINDOW_COLS + 8):
+                    fresh = True
+                if chain_tiles >= tiles_per_chain:
+                    fresh = True
+            if fresh:
+                chains.append([chain_lo, b])
+                chain_lo, chain_tiles, have, low = b, 0, -1, 0
+            fr = to = lo
+            if hi > lo:
+                if have < 0 or lo >= have:
+                    fr, to, low = lo, hi, lo
+                else:
+                    fr, to = have, max(have, hi)
+                have = to
+            blocks.append([stored_off[b], stored_off[b + 1], len(pieces), len(pieces) + 1])
+            pieces.append([fr, to, 0, WINDOW_COLS])
+            chain_tiles += int(btiles[b])
     chains.append([chain_lo, nblocks])
     perm_phys = np.empty_like(perm).reshape(-1, TILE)
     perm_phys[:, val_pos(itemsize)] = perm.reshape(-1, TILE)

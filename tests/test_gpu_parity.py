@@ -789,7 +789,8 @@ def _diagonal_bands(rng, m, n, bands, dens, dtype, empty=0.05):
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_spmv_window_kernel_bands_of_diagonals(torch, capi, oracle, dtype):
     """Matrices no single window holds but a few bands of diagonals do (the planes of a stencil on
-    a three-dimensional grid): a 7-point and a 27-point stencil on 96 x 96 x 12, random bands on a
+    a three-dimensional grid): a 7-point and a 27-point stencil on 96 x 96 x 12 and a 7-point one on
+    95 x 95 x 14 (stacked planes), three bands that are no planes, random bands on a
     rectangular matrix with an odd number of columns, five bands (the two closest are joined), long
     rows that tiles cut (carry pass); and NOT_SUPPORTED where the bands are too wide for the LDS."""
     rng = np.random.default_rng(131)
@@ -797,7 +798,8 @@ def test_spmv_window_kernel_bands_of_diagonals(torch, capi, oracle, dtype):
     plane = nx * ny
     cases = []
 
-    def stencil3d(points):
+    def stencil3d(points, nx=nx, ny=ny, nz=nz):
+        plane = nx * ny
         idx = np.arange(nx * ny * nz, dtype=np.int64)
         i, j, k = idx % nx, (idx // nx) % ny, idx // plane
         rng3 = (-1, 0, 1)
@@ -815,6 +817,10 @@ def test_spmv_window_kernel_bands_of_diagonals(torch, capi, oracle, dtype):
 
     for pts in (7, 27):
         cases.append((f"stencil {pts} points", stencil3d(pts), nx * ny * nz))
+    # planes of 9025 points (no multiple of 64, nor of the 16-byte units x is fetched in), blocks of 361 rows
+    cases.append(("stencil 7 points, planes of 9025", stencil3d(7, 95, 95, 14), 9025 * 14))
+    # three bands whose distance does not divide the rows: a ring per band
+    cases.append(("three bands", _diagonal_bands(rng, 50000, 50000, [(-9501, -9499), (-2, 2), (9499, 9501)], 0.9, dtype), 50000))
     cases.append(("two far bands, rectangular", _diagonal_bands(rng, 50000, 70001, [(-30000, -29990), (-5, 40)], 0.5, dtype), 70001))
     cases.append(("five bands", _diagonal_bands(rng, 40000, 40000, [(-20000, -20000), (-9000, -8990), (0, 0), (300, 310), (15000, 15001)],
                                                 0.9, dtype), 40000))
@@ -830,6 +836,16 @@ def test_spmv_window_kernel_bands_of_diagonals(torch, capi, oracle, dtype):
         plan_check.check_plan(plan, capi, rp, col, n, np.dtype(dtype).itemsize)
         assert plan.workspace_bytes == plan.info("carry_pass") * plan.info("tiles") * np.dtype(dtype).itemsize
         assert 2 <= plan.info("bands") <= 4 and plan.info("slices") == -1, (name, plan.info("bands"))
+        # the stencils' three bands lie whole planes apart: their blocks are stored plane above plane
+        # and x is fetched about once (a ring per band: three times)
+        want_planes = {"stencil 7 points": plane, "stencil 27 points": plane, "stencil 7 points, planes of 9025": 9025}.get(name, 0)
+        assert plan.info("stacked_rows") == want_planes, (name, plan.info("stacked_rows"))
+        if want_planes:  # past the first block of a chain a block fetches the plane above it only
+            pcs = plan.export("pieces").reshape(-1, 3, 4)
+            fetches = (pcs[:, :, 1] > pcs[:, :, 0]).sum(axis=1)
+            first = np.zeros(fetches.size, bool)
+            first[plan.export("workgroups").reshape(-1, 2)[:, 0]] = True
+            assert np.all(fetches[~first] <= 1) and np.all(fetches[first] >= 2), name
         if name in ("stencil 7 points", "long rows"):  # rows of at most 16 are never cut by tiles
             assert plan.info("carry_pass") == (1 if name == "long rows" else 0), name
         for alpha, beta in ((1.5, 0.5), (1.0, 0.0)):

@@ -158,7 +158,7 @@ def test_window_corruptions_are_rejected():
     def flag(p):
         real = np.nonzero(pc.logical_order(p["perm"], 8) >= 0)[0]
         p["cf"][real[100]] ^= 0x8000
-    corrupt(flag, "flag")
+    corrupt(flag, "flag|fewer than two stored elements")
 
     def tile_rows(p):  # a tile that claims one row fewer: that row would never be written
         p["tile_words"].reshape(-1, 2)[3, 1] -= 1
@@ -175,3 +175,79 @@ def test_window_corruptions_are_rejected():
     def block_tiles(p):
         p["blocks"].reshape(-1, 4)[2, 1] -= 1
     corrupt(block_tiles)
+
+
+def _stencil3d(nx, ny, nz, points=7):
+    idx = np.arange(nx * ny * nz, dtype=np.int64)
+    i, j, k = idx % nx, (idx // nx) % ny, idx // (nx * ny)
+    keys = []
+    for dk in (-1, 0, 1):
+        for dj in (-1, 0, 1):
+            for di in (-1, 0, 1):
+                if points != 27 and abs(di) + abs(dj) + abs(dk) > 1:
+                    continue
+                ii, jj, kk = i + di, j + dj, k + dk
+                ok = (ii >= 0) & (ii < nx) & (jj >= 0) & (jj < ny) & (kk >= 0) & (kk < nz)
+                keys.append(idx[ok] * idx.size + (ii + nx * (jj + ny * kk))[ok])
+    keys = np.unique(np.concatenate(keys))
+    rp = np.zeros(idx.size + 1, np.int64)
+    np.cumsum(np.bincount(keys // idx.size, minlength=idx.size), out=rp[1:])
+    return rp.astype(np.int32), (keys % idx.size).astype(np.int32)
+
+
+@pytest.mark.parametrize("points", [7, 27])
+def test_stacked_planes_plan_from_its_definition_passes(points):
+    # planes of 32 x 32 = 1024 points, 12 of them; blocks of 256 rows: four columns of blocks
+    rp, col = _stencil3d(32, 32, 12, points)
+    n = 32 * 32 * 12
+    reach = 33 if points == 27 else 32
+    for tiles_per_chain in (1 << 30, 30):
+        plan = pc.window_plan_arrays(rp, col, n, 256, 8, tiles_per_chain, stack=(1024, -reach, reach))
+        pc.check_window(plan, rp, col, n, 256, 3, 8)
+        ch = plan["workgroups"].reshape(-1, 2)
+        assert ch.shape[0] >= 4  # a chain never leaves its column of blocks
+    # inside a chain every block but the first fetches one region only
+    plan = pc.window_plan_arrays(rp, col, n, 256, 8, stack=(1024, -reach, reach))
+    pcs = plan["pieces"].reshape(-1, 3, 4)
+    fetched = (pcs[:, :, 1] > pcs[:, :, 0]).sum(axis=1)
+    first = np.zeros(fetched.size, bool)
+    first[plan["workgroups"].reshape(-1, 2)[:, 0]] = True
+    # the first block of a chain is plane 0 here: nothing, or a few columns at the start of x, below it
+    assert np.all(fetched[~first] <= 1) and np.all(fetched[first] >= 2)
+    x_columns = (pcs[:, :, 1] - pcs[:, :, 0]).sum()
+    assert x_columns < 1.5 * n  # x is fetched about once (rings per band: three times)
+
+
+def test_stacked_planes_corruptions_are_rejected():
+    rp, col = _stencil3d(32, 32, 12)
+    n = 32 * 32 * 12
+    bad = pc.window_plan_arrays(rp, col, n, 256, 8, stack=(1024, -32, 32), rotate=1)
+    with pytest.raises(pc.PlanError, match="holds column"):
+        pc.check_window(bad, rp, col, n, 256, 3, 8)
+    good = pc.window_plan_arrays(rp, col, n, 256, 8, 30, stack=(1024, -32, 32))
+
+    def corrupt(fn, match):
+        p = {k: v.copy() for k, v in good.items()}
+        fn(p)
+        with pytest.raises(pc.PlanError, match=match):
+            pc.check_window(p, rp, col, n, 256, 3, 8)
+
+    def skip_a_region(p):  # a block in the middle of a chain does not fetch its new plane
+        pcs = p["pieces"].reshape(-1, 3, 4)
+        ch = p["workgroups"].reshape(-1, 2)
+        b = int(ch[0, 0]) + 1
+        k = int(np.argmax(pcs[b, :, 1] > pcs[b, :, 0]))
+        pcs[b, k, 1] = pcs[b, k, 0]
+    corrupt(skip_a_region, "holds column")
+
+    def overlapping_regions(p):
+        pcs = p["pieces"].reshape(-1, 4)
+        pcs[pcs[:, 2] > 0, 2] -= 4
+    corrupt(overlapping_regions, "rings overlap|holds column")
+
+    def swap_two_blocks_tiles(p):  # the tables name another block's tiles
+        blk = p["blocks"].reshape(-1, 4)
+        info = p["tile_words"].reshape(-1, 2)
+        t0, t1 = int(blk[0, 0]), int(blk[1, 0])
+        info[t0, 0], info[t1, 0] = info[t1, 0], info[t0, 0]
+    corrupt(swap_two_blocks_tiles, "block")
