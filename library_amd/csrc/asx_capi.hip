@@ -592,7 +592,9 @@ int asx_spmm_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
 // two, the sliced one unless the row-block one is estimated more than 5 % faster.
 constexpr int32_t kSlicedMinNnz = 1 << 21;
 struct KernelEstimates {
-    double rows, sliced, window;  // seconds; infinity where the kernel does not apply
+    // seconds; infinity where the kernel does not apply.  window: with one ring of x per block;
+    // window_bands: with rings per band of diagonals, which only the build finds out
+    double rows, sliced, window, window_bands;
 };
 static KernelEstimates estimate_kernels(const asx_plan *p, size_t sv, const ColumnSample &cs, bool window_ok)
 {
@@ -608,9 +610,14 @@ static KernelEstimates estimate_kernels(const asx_plan *p, size_t sv, const Colu
     e.sliced = nslices > kSlicedMaxSlices
                    ? inf
                    : 8e-6 + (nnz * (dsv + 2) + cs.pairs * nnz * (2 * dsv + 2) + n * dsv + 2 * m * dsv) / 6.0e12;
-    e.window = !window_ok ? inf
-                          : 8e-6 + ((nnz + (double)p->hist[0]) * (dsv + 2) + n * dsv + 2 * m * dsv) /
-                                       (p->stats[0] <= 16 ? 5.0e12 : 3.7e12);
+    // The row-block copy gives every row at least two slots.  Rates measured over the audit's
+    // families (what the copy moves / (time - 8 us)): one ring 5.8e12 with rows the tiles do not cut
+    // (5-point stencil, band of 9), 5.0 and 4.6e12 with rows of 19 and 65; rings per band, x fetched
+    // about 1.5 times: 4.7e12 (7-point stencil) and 3.9e12 (27-point).
+    const double wslots = nnz + 2.0 * (double)p->hist[0] + (double)p->hist[1];
+    const bool uncut = p->stats[0] <= 16;
+    e.window = !window_ok ? inf : 8e-6 + (wslots * (dsv + 2) + n * dsv + 2 * m * dsv) / (uncut ? 5.6e12 : 4.8e12);
+    e.window_bands = !window_ok ? inf : 8e-6 + (wslots * (dsv + 2) + 1.5 * n * dsv + 2 * m * dsv) / (uncut ? 4.6e12 : 3.9e12);
     return e;
 }
 
@@ -672,10 +679,10 @@ int plan_add_window(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
 }
 
 // DEFAULT tries the row-block copy for matrices the flat or merge-path kernel would take, without
-// rows past the carry pass's limit, and with few empty rows: the copy gives every empty row a
-// slot of its own (a value, a column word and a source index, read in every call), so a matrix
-// with more empty rows than a quarter of its stored elements stays with the merge-path kernel,
-// which streams row offsets only.
+// rows past the carry pass's limit, and with few rows of fewer than two stored elements: the copy
+// gives every row at least two slots (a value, a column word and a source index each, read in every
+// call), so a matrix where that padding exceeds a quarter of its stored elements stays with the
+// other kernels.
 // A regrouped copy roughly doubles what the matrix takes on the device (per stored element: the
 // value, 2 bytes of column, 4 bytes of source index; the sliced kernel also keeps a buffer for the
 // partial sums of a call), and its build needs about 4 bytes per stored element more for a while.
@@ -692,7 +699,7 @@ static bool regrouped_copy_fits(const asx_plan *p, size_t sv)
 static bool window_may_pay(const asx_plan *p, int row_kernel)
 {
     return p->stats[0] <= kWindowMaxRow && (row_kernel == ASX_SPMV_FLAT || row_kernel == ASX_SPMV_MERGE) &&
-           p->hist[0] <= (int64_t)p->nnz / 4;
+           2 * p->hist[0] + p->hist[1] <= (int64_t)p->nnz / 4;
 }
 
 extern "C" {
@@ -750,6 +757,15 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
             const KernelEstimates e = estimate_kernels(p, sv, cs, window_ok);
             const bool sliced_pays = e.sliced < 0.97 * e.rows, window_pays = e.window < 0.97 * e.rows;
             if (window_pays && e.window < e.sliced / 1.05) done = add_window() == ASX_STATUS_SUCCESS;
+            if (done && p->window.nbands > 1 && sliced_pays && !(e.window_bands < e.sliced / 1.05)) {
+                // the build needed a ring per band of diagonals; with those the slices are ahead
+                WindowMatrix built = p->window;
+                p->window = WindowMatrix{};
+                if (add_slices(cs.pairs) == ASX_STATUS_SUCCESS)
+                    free_window(&built);
+                else
+                    p->window = built, p->alg = ASX_SPMV_WINDOW;
+            }
             if (!done && sliced_pays) done = add_slices(cs.pairs) == ASX_STATUS_SUCCESS;
             if (!done && window_pays && !(e.window < e.sliced / 1.05)) done = add_window() == ASX_STATUS_SUCCESS;
         }
