@@ -52,7 +52,7 @@ constexpr int window_depth(int rings, bool beta)
 constexpr int kSpanGroup = 128;  // rows per group of the column-span table; every block size is a multiple
 
 // first and last column of every group of kSpanGroup consecutive rows (gmin = kNoCol, gmax = -1 for
-// a group without stored elements); one wave per group, two rows per lane
+// a group without stored elements); one wave per group reads the group's columns in order
 __global__ __launch_bounds__(kBlock) void k_window_group_span(const int32_t *__restrict__ row_ptr,
                                                               const int32_t *__restrict__ col, int32_t m,
                                                               int32_t ngroups, int32_t *__restrict__ gmin,
@@ -62,15 +62,11 @@ __global__ __launch_bounds__(kBlock) void k_window_group_span(const int32_t *__r
     const int64_t g = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
     if (g >= ngroups) return;  // whole waves leave
     int32_t lo = kNoCol, hi = -1;
-#pragma unroll
-    for (int h = 0; h < kSpanGroup / kWave; ++h) {
-        const int64_t r = g * kSpanGroup + h * kWave + lane;
-        if (r < m)
-            for (int32_t k = row_ptr[r]; k < row_ptr[r + 1]; ++k) {
-                const int32_t c = col[k];
-                lo = c < lo ? c : lo;
-                hi = c > hi ? c : hi;
-            }
+    const int64_t r1 = (g + 1) * kSpanGroup < m ? (g + 1) * kSpanGroup : m;
+    for (int32_t k = row_ptr[g * kSpanGroup] + lane, end = row_ptr[r1]; k < end; k += kWave) {
+        const int32_t c = col[k];
+        lo = c < lo ? c : lo;
+        hi = c > hi ? c : hi;
     }
 #pragma unroll
     for (int d = 1; d < kWave; d <<= 1) {
@@ -208,21 +204,74 @@ struct BandTable {
 };
 __host__ __device__ __forceinline__ int64_t band_centre(int64_t r, int64_t m, int64_t n) { return r * n / m; }
 
-// bit b of `bits` set = some stored element has (c - centre(r) + n) / 64 == b
+// The row that holds stored element i: the largest r with row_ptr[r] <= i.  The kBlock elements of
+// a workgroup lie in rows seg_row[blockIdx.x] .. seg_row[blockIdx.x + 1]; their offsets are staged
+// in LDS (when they are at most kBlock + 1: no long run of empty rows) and searched there.  Every
+// thread of the workgroup calls this; *first_of_row receives row_ptr[r].
+__device__ __forceinline__ int32_t row_of_element(const int32_t *__restrict__ row_ptr, int32_t m,
+                                                  const int32_t *__restrict__ seg_row, int64_t i, int32_t *s_rp /* kBlock + 1 */,
+                                                  int32_t *first_of_row)
+{
+    const int32_t r_lo = seg_row[blockIdx.x];
+    int32_t r_hi = seg_row[blockIdx.x + 1];
+    r_hi = r_hi > m - 1 ? m - 1 : r_hi;
+    const int32_t cnt = r_hi - r_lo + 1;
+    const bool staged = cnt <= kBlock + 1;  // uniform
+    if (staged)
+        for (int32_t j = threadIdx.x; j < cnt; j += kBlock) s_rp[j] = row_ptr[r_lo + j];
+    __syncthreads();
+    int32_t lo = 0, hi = cnt - 1;
+    if (staged) {
+        while (lo < hi) {
+            const int32_t mid = lo + (hi - lo + 1) / 2;
+            if (s_rp[mid] <= i)
+                lo = mid;
+            else
+                hi = mid - 1;
+        }
+        *first_of_row = s_rp[lo];
+    } else {
+        while (lo < hi) {
+            const int32_t mid = lo + (hi - lo + 1) / 2;
+            if (row_ptr[r_lo + mid] <= i)
+                lo = mid;
+            else
+                hi = mid - 1;
+        }
+        *first_of_row = row_ptr[r_lo + lo];
+    }
+    return r_lo + lo;
+}
+
+// bit b of `bits` set = some stored element has (c - centre(r) + n) / 64 == b.  One thread per
+// stored element (the columns are read in order).  The workgroup collects its bits in LDS first (a
+// few words: its elements lie on a few bands) and ors into memory only the words that still miss
+// some of them: a hundred million atomics on the same fifty words would take milliseconds.
 __global__ __launch_bounds__(kBlock) void k_window_offset_bins(const int32_t *__restrict__ row_ptr,
                                                                const int32_t *__restrict__ col, int32_t m, int32_t n,
-                                                               uint32_t *__restrict__ bits)
+                                                               int32_t nnz, const int32_t *__restrict__ seg_row,
+                                                               uint32_t *bits)
 {
-    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (r >= m) return;
-    const int64_t shift = (int64_t)n - band_centre(r, m, n);
-    int64_t last = -1;
-    for (int32_t k = row_ptr[r]; k < row_ptr[r + 1]; ++k) {
-        const int64_t bin = ((int64_t)col[k] + shift) >> 6;
-        if (bin == last) continue;
-        last = bin;
-        const uint32_t mask = 1u << (bin & 31);
-        if (!(bits[bin >> 5] & mask)) atomicOr(bits + (bin >> 5), mask);  // mostly set already: few atomics
+    constexpr int kSlots = 64;  // words collected per workgroup, by word index modulo kSlots
+    __shared__ uint32_t s_word[kSlots], s_mask[kSlots];
+    __shared__ int32_t s_rp[kBlock + 1];
+    if (threadIdx.x < kSlots) s_word[threadIdx.x] = 0xffffffffu, s_mask[threadIdx.x] = 0;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int32_t first;
+    const int32_t r = row_of_element(row_ptr, m, seg_row, i < nnz ? i : nnz - 1, s_rp, &first);  // syncs
+    if (i < nnz) {
+        const int64_t bin = ((int64_t)col[i] + (int64_t)n - band_centre(r, m, n)) >> 6;
+        const uint32_t word = (uint32_t)(bin >> 5), mask = 1u << (bin & 31);
+        const uint32_t owner = atomicCAS(&s_word[word % kSlots], 0xffffffffu, word);
+        if (owner == 0xffffffffu || owner == word)
+            atomicOr(&s_mask[word % kSlots], mask);
+        else if (!(__atomic_load_n(bits + word, __ATOMIC_RELAXED) & mask))  // the slot serves another word
+            atomicOr(bits + word, mask);
+    }
+    __syncthreads();
+    if (threadIdx.x < kSlots && s_mask[threadIdx.x]) {
+        uint32_t *w = bits + s_word[threadIdx.x];
+        if ((__atomic_load_n(w, __ATOMIC_RELAXED) & s_mask[threadIdx.x]) != s_mask[threadIdx.x]) atomicOr(w, s_mask[threadIdx.x]);
     }
 }
 
@@ -235,23 +284,15 @@ __global__ __launch_bounds__(kBlock) void k_window_place(const int32_t *__restri
                                                          const int32_t *__restrict__ tile_off, uint16_t *__restrict__ cf,
                                                          T *__restrict__ val_out, int32_t *__restrict__ perm)
 {
+    __shared__ int32_t s_rp[kBlock + 1];
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int32_t first;
+    const int32_t r = row_of_element(row_ptr, m, seg_row, i < nnz ? i : nnz - 1, s_rp, &first);  // syncs
     if (i >= nnz) return;
-    // row holding stored element i: largest r with row_ptr[r] <= i; the workgroup's kBlock elements
-    // lie in rows seg_row[blockIdx.x] .. seg_row[blockIdx.x + 1]
-    int32_t lo = seg_row[blockIdx.x], hi = seg_row[blockIdx.x + 1];
-    hi = hi > m - 1 ? m - 1 : hi;
-    while (lo < hi) {
-        const int32_t mid = lo + (hi - lo + 1) / 2;
-        if (row_ptr[mid] <= i)
-            lo = mid;
-        else
-            hi = mid - 1;
-    }
-    const int32_t r = lo, b = r / rows;
-    const int32_t o = row_start[r] + (int32_t)(i - row_ptr[r]);
+    const int32_t b = r / rows;
+    const int32_t o = row_start[r] + (int32_t)(i - first);
     const int64_t d = (int64_t)tile_off[b] * kSlicedTile + o;
-    const bool head = i == row_ptr[r] || o % kSlicedTile == 0;
+    const bool head = i == first || o % kSlicedTile == 0;
     const int32_t c = col[i];
     int k = 0;
     if (bands.nbands > 1) {
@@ -748,7 +789,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
         const size_t words = (size_t)(nbins + 31) / 32;
         ASX_TRY(hipMalloc((void **)&d_bits, sizeof(uint32_t) * words));
         ASX_TRY(hipMemsetAsync(d_bits, 0, sizeof(uint32_t) * words, s));
-        hipLaunchKernelGGL(k_window_offset_bins, dim3(mgrid), dim3(kBlock), 0, s, row_ptr, col, m, n, d_bits);
+        hipLaunchKernelGGL(k_window_offset_bins, dim3((unsigned)nseg), dim3(kBlock), 0, s, row_ptr, col, m, n, nnz, seg_row, d_bits);
         h_bits.resize(words);
         ASX_TRY(hipMemcpyAsync(h_bits.data(), d_bits, sizeof(uint32_t) * words, hipMemcpyDeviceToHost, s));
         ASX_TRY(hipStreamSynchronize(s));
