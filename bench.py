@@ -36,8 +36,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 # the five BASELINE configurations, and config 2's matrix in fp64 (the "uniform fp64" case the target names)
 ORDER = ["banded_f64", "uniform16_f32", "uniform16_f64", "powerlaw_f64", "stencil5_f64", "spmm_zipf_f32"]
-# not a BASELINE configuration: a dense-block matrix for the MFMA SpMM variant
-EXTRA = ["spmm_banded_f32"]
+# not BASELINE configurations: a dense-block matrix for the MFMA SpMM variant, a 7-point stencil on 256^3
+EXTRA = ["spmm_banded_f32", "stencil7_f64"]
 KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "k_spmv_flat",
                 101: "k_sliced_products+k_sliced_reduce", 102: "k_spmv_window", 5: "k_spmm_row", 7: "k_spmm_merge", 10: "k_spmm_blocked"}
 
@@ -54,6 +54,7 @@ MEASURED_TRAFFIC_BYTES = {
     "stencil5_f64": 1_137_229_657,  # profiles/spmv_window_stencil5_f64.md
     "spmm_zipf_f32": 4_965_331_333,  # profiles/spmm_merge_spmm_zipf_f32.md
     "spmm_banded_f32": 1_870_263_890,  # profiles/spmm_blocked_spmm_banded_f32.md
+    "stencil7_f64": 1_622_985_065,  # profiles/spmv_window_stencil7_256_f64.md
 }
 
 

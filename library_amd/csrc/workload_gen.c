@@ -241,3 +241,31 @@ void wl_stencil5_fill_f64(int32_t nx, int32_t ny, const int32_t *row_ptr, int32_
         if (iy < ny - 1) { col[p] = (int32_t)(r + nx); val[p++] = -1.0; }
     }
 }
+
+/* ------------------------------------------------------------------ 7-point stencil on nx x ny x nz */
+int64_t wl_stencil7_row_ptr(int32_t nx, int32_t ny, int32_t nz, int32_t *row_ptr)
+{
+    int64_t plane = (int64_t)nx * ny, m = plane * nz;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < m; ++r) {
+        int32_t ix = (int32_t)(r % nx), iy = (int32_t)(r / nx % ny), iz = (int32_t)(r / plane);
+        row_ptr[r + 1] = 1 + (iz > 0) + (iy > 0) + (ix > 0) + (ix < nx - 1) + (iy < ny - 1) + (iz < nz - 1);
+    }
+    return prefix_in_place(row_ptr, m);
+}
+void wl_stencil7_fill_f64(int32_t nx, int32_t ny, int32_t nz, const int32_t *row_ptr, int32_t *col, double *val)
+{
+    int64_t plane = (int64_t)nx * ny, m = plane * nz;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < m; ++r) {
+        int32_t ix = (int32_t)(r % nx), iy = (int32_t)(r / nx % ny), iz = (int32_t)(r / plane);
+        int64_t p = row_ptr[r];
+        if (iz > 0) { col[p] = (int32_t)(r - plane); val[p++] = -1.0; }
+        if (iy > 0) { col[p] = (int32_t)(r - nx); val[p++] = -1.0; }
+        if (ix > 0) { col[p] = (int32_t)(r - 1); val[p++] = -1.0; }
+        col[p] = (int32_t)r; val[p++] = 6.0;
+        if (ix < nx - 1) { col[p] = (int32_t)(r + 1); val[p++] = -1.0; }
+        if (iy < ny - 1) { col[p] = (int32_t)(r + nx); val[p++] = -1.0; }
+        if (iz < nz - 1) { col[p] = (int32_t)(r + plane); val[p++] = -1.0; }
+    }
+}

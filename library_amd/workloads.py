@@ -42,8 +42,11 @@ def lib():
         L.wl_stencil5_row_ptr.argtypes = [C.c_int32, C.c_int32, i32p]
         L.wl_stencil5_row_ptr.restype = C.c_int64
         L.wl_stencil5_fill_f64.argtypes = [C.c_int32, C.c_int32, i32p, i32p, f64p]
+        L.wl_stencil7_row_ptr.argtypes = [C.c_int32, C.c_int32, C.c_int32, i32p]
+        L.wl_stencil7_row_ptr.restype = C.c_int64
+        L.wl_stencil7_fill_f64.argtypes = [C.c_int32, C.c_int32, C.c_int32, i32p, i32p, f64p]
         for f in (L.wl_fill_uniform_f64, L.wl_fill_uniform_f32, L.wl_banded_cols, L.wl_random_cols,
-                  L.wl_stencil5_fill_f64):
+                  L.wl_stencil5_fill_f64, L.wl_stencil7_fill_f64):
             f.restype = None
         _lib = L
     return _lib
@@ -136,6 +139,16 @@ def csr_stencil5(nx, ny):
     return row_ptr, col, val
 
 
+def csr_stencil7(nx, ny, nz):
+    m = nx * ny * nz
+    row_ptr = np.empty(m + 1, dtype=np.int32)
+    nnz = lib().wl_stencil7_row_ptr(nx, ny, nz, _p(row_ptr, C.c_int32))
+    col = np.empty(nnz, dtype=np.int32)
+    val = np.empty(nnz, dtype=np.float64)
+    lib().wl_stencil7_fill_f64(nx, ny, nz, _p(row_ptr, C.c_int32), _p(col, C.c_int32), _p(val, C.c_double))
+    return row_ptr, col, val
+
+
 # Scale applied to Zipf(2.2) draws so that the realised mean row length of the SpMM
 # configuration is 16.0 +- 0.1 after rounding and clipping to [1, 50000].
 SPMM_ZIPF_SCALE = 4.76
@@ -179,6 +192,13 @@ def stencil5_f64(nx=4096, ny=4096, seed=0):
     return _spmv("stencil5_f64", np.float64, rp, col, val, nx * ny, 1.0, 0.0, seed, xlo=0.0)
 
 
+def stencil7_f64(nx=256, ny=256, nz=256, seed=0):
+    """Not a BASELINE configuration: 3D 7-point Laplacian in natural order (planes of nx * ny points),
+    fp64, x ~ U(0,1), y = 1.5*A*x + 0.5*y."""
+    rp, col, val = csr_stencil7(nx, ny, nz)
+    return _spmv("stencil7_f64", np.float64, rp, col, val, nx * ny * nz, 1.5, 0.5, seed, xlo=0.0)
+
+
 def spmm_zipf_f32(m=1 << 20, ncols=64, max_len=50000, seed=0, scale=SPMM_ZIPF_SCALE):
     """Config 5: C = 1.0*A*B + 1.0*C, A m x m Zipf(2.2)-shaped rows (mean 16), B, C m x ncols fp32."""
     rp, col, val = csr_zipf(m, m, 22, scale, min(max_len, m), 0.0, np.float32, seed)
@@ -205,4 +225,5 @@ CONFIGS = {
     "spmm_zipf_f32": spmm_zipf_f32,
     "spmm_banded_f32": spmm_banded_f32,
     "uniform16_f64": uniform16_f64,
+    "stencil7_f64": stencil7_f64,
 }

@@ -336,8 +336,10 @@ def test_spmm_padded_leading_dimensions_and_integers(torch, capi, oracle):
 # ------------------------------------------------------------------ benchmark configurations at full size
 def test_benchmark_configs_full_size(torch, capi, oracle):
     from library_amd import workloads as W
-    for name in ("uniform16_f32", "uniform16_f64", "powerlaw_f64", "stencil5_f64"):
-        w = W.CONFIGS[name]()
+    # the BASELINE configurations 2-4, config 2's matrix in fp64, and a 7-point stencil on 160^3 (the
+    # bench extra at a size whose oracle run stays short: stacked planes, y read ahead for beta != 0)
+    for name in ("uniform16_f32", "uniform16_f64", "powerlaw_f64", "stencil5_f64", "stencil7_f64"):
+        w = W.CONFIGS[name](160, 160, 160) if name == "stencil7_f64" else W.CONFIGS[name]()
         ref = oracle.spmv(w.row_ptr, w.col, w.val, w.x, w.alpha, w.beta, w.y, 16)
         scale = spmv_scale(w.row_ptr, w.col, w.val, w.x, w.alpha, w.beta, w.y)
         d = [dev(torch, a) for a in (w.row_ptr, w.col, w.val, w.x)]
