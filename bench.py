@@ -20,6 +20,9 @@ Per workload, on the GPU:
   cold_ms         as event_ms, after a 1 GiB sweep that evicts the caches before every call
   noplan_ms       the call without kept analysis (split points recomputed inside every call, as
                   the reference does)
+  unchanged_caller_ms   SpMV: what a caller that never calls the analysis gets by default through the
+                  generic API: a plan made on first use that may hold a copy of the values, checked
+                  against the caller's values by checksum in every call (unchanged_caller_kernel)
 and on the host (unless --no-cpu), the reference's own CPU kernels (oracle/_ref, kind
 "reference") or their C restatement (kind "port") on the same inputs: all physical cores of the
 box's share, and one thread.
@@ -163,6 +166,30 @@ def measure(w, steps, warmup, alg):
     e1.record()
     torch.cuda.synchronize()
     noplan_ms = e0.elapsed_time(e1) / nrep
+    # (e) SpMV, what a caller written for the reference gets by default (no analysis call, values may
+    #     change in place): analysis on first use that may keep a copy of the values, and in every
+    #     call two checksums of the caller's values on the device with a refresh of the copy where
+    #     they differ.  DEFAULT's choice counts that read, so the kernel may be another one.
+    checked_ms, checked_kernel = None, None
+    if not spmm:
+        cplan = capi.Plan(False, alg, w.val.dtype, w.m, w.n, w.nnz, d_rp, col=d_col, val=d_val, checked=True)
+        checked_kernel = KERNEL_NAMES.get(cplan.alg, str(cplan.alg)) + (" + checksum" if cplan.checked else "")
+        ws3 = torch.empty(max(cplan.workspace_bytes, 256), dtype=torch.uint8, device="cuda")
+
+        def step_checked():
+            cplan.refresh_if_changed(d_val)
+            capi.spmv(d_rp, d_col, d_val, d_x, d_y, w.alpha, w.beta, plan=cplan, workspace=ws3)
+
+        for _ in range(3):
+            step_checked()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(nrep):
+            step_checked()
+        e1.record()
+        torch.cuda.synchronize()
+        checked_ms = e0.elapsed_time(e1) / nrep
+        cplan.destroy()
     nbytes = w.bytes_algorithmic()
     res = {
         "workload": w.name, "kind": w.kind, "dtype": "f64" if w.dtype.itemsize == 8 else "f32",
@@ -176,6 +203,7 @@ def measure(w, steps, warmup, alg):
         "event_ms_min": float(per_call.min()),
         "cold_ms_median": float(np.median(cold)),
         "noplan_ms": float(noplan_ms),
+        "unchanged_caller_ms": None if checked_ms is None else float(checked_ms), "unchanged_caller_kernel": checked_kernel,
     }
     res["gbs"] = nbytes / (wall_ms * 1e-3) / 1e9
     res["gflops"] = w.flops / (wall_ms * 1e-3) / 1e9

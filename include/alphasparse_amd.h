@@ -213,6 +213,25 @@ int asx_spmv_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, in
  * asx_plan_holds_values tells the two kinds apart.  No counterpart in the reference. */
 int asx_plan_update_values(asx_plan *plan, const void *d_val, void *stream);
 int asx_plan_holds_values(const asx_plan *plan);
+/* For callers who may change A's values in place without saying so (the reference's own callers:
+ * its alphasparseSpMV reads A's arrays in every call, hip/kernel/level2/alphasparse_spmv.hip:16-199,
+ * and its analysis keeps nothing).  asx_spmv_plan_create_checked is asx_spmv_plan_create, except
+ * that a plan which ends up holding a copy of the values also keeps two 64-bit checksums of
+ * them (position-dependent sums over their 32-bit words; a single changed word always changes
+ * them, several changes escape with probability 2^-128) and that DEFAULT's choice counts what
+ * checking costs.  d_val must lie on a 16-byte boundary for such a plan (otherwise the plan is made
+ * row-ordered).  asx_plan_refresh_if_changed, called before every SpMV through the plan with the
+ * values as they are now, takes their checksums (one read of the values: 42 us for 34 M fp64
+ * values) and brings the copy up to date where they differ from the kept ones; all on the device,
+ * asynchronous on `stream`, nothing is read back.  It does nothing for a plan that was made
+ * unchecked or that reads the caller's values anyway (asx_plan_is_checked = 0).  The sparsity
+ * pattern is taken to stay as it was.  Calls through one checked plan on several streams at once
+ * may refresh the copy more often than needed (they share the checksum words); results stay
+ * right.  No counterpart in the reference. */
+int asx_spmv_plan_create_checked(asx_plan **plan, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
+                                 const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, void *stream);
+int asx_plan_refresh_if_changed(asx_plan *plan, const void *d_val, void *stream);
+int asx_plan_is_checked(const asx_plan *plan);
 /* Number of 16x4 blocks and their fill of a blocked plan. */
 int asx_plan_block_stats(const asx_plan *plan, int64_t *nblocks, double *fill);
 int asx_plan_destroy(asx_plan *plan);

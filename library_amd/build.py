@@ -150,4 +150,5 @@ def build_all():
 
 if __name__ == "__main__":
     build_all()
+    build_cxx_example()
     sys.exit(0)

@@ -27,7 +27,8 @@ EXPORTS = [
     "asx_nnz_split_rows", "asx_merge_path_search", "asx_loadbalance_nwarps",
     "asx_loadbalance_partition", "asx_csr_adaptive_row_blocks", "asx_coo2csr", "asx_coo_sort", "asx_csr_transpose", "asx_csr_rebase",
     "asx_dense_transpose", "asx_mtx_read", "asx_host_free", "asx_spmv_plan_create",
-    "asx_plan_update_values", "asx_plan_holds_values", "asx_plan_info", "asx_plan_create",
+    "asx_plan_update_values", "asx_plan_holds_values", "asx_spmv_plan_create_checked", "asx_plan_refresh_if_changed",
+    "asx_plan_is_checked", "asx_plan_info", "asx_plan_create",
     "asx_spmm_plan_create", "asx_plan_block_stats", "asx_plan_destroy", "asx_plan_alg", "asx_kernel_name", "asx_plan_workspace_bytes", "asx_plan_histogram",
     "asx_plan_release_scratch", "asx_plan_own_scratch_bytes", "asx_plan_export",
     "asx_spmv_resolve_alg", "asx_spmv_workspace_bytes", "asx_spmv_csr_f64", "asx_spmv_csr_f32",
@@ -75,6 +76,9 @@ def lib():
     L.asx_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, C.c_int, i32, i32, i32, vp, i32, vp]
     L.asx_spmm_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, i32, i32, i32, vp, vp, vp, i32, vp]
     L.asx_spmv_plan_create.argtypes = [C.POINTER(vp), C.c_int, C.c_int, i32, i32, i32, vp, vp, vp, vp]
+    L.asx_spmv_plan_create_checked.argtypes = [C.POINTER(vp), C.c_int, C.c_int, i32, i32, i32, vp, vp, vp, vp]
+    L.asx_plan_refresh_if_changed.argtypes = [vp, vp, vp]
+    L.asx_plan_is_checked.argtypes = [vp]
     L.asx_plan_update_values.argtypes = [vp, vp, vp]
     L.asx_plan_holds_values.argtypes = [vp]
     L.asx_plan_block_stats.argtypes = [vp, C.POINTER(i64), C.POINTER(C.c_double)]
@@ -254,9 +258,12 @@ def csr_adaptive_row_blocks(row_ptr_host):
 
 # ------------------------------------------------------------------------------ plans
 class Plan:
-    def __init__(self, is_spmm, alg, dtype, m, n, nnz, row_ptr, ncols=1, col=None, val=None):
+    def __init__(self, is_spmm, alg, dtype, m, n, nnz, row_ptr, ncols=1, col=None, val=None, checked=False):
         h = C.c_void_p()
-        if is_spmm and col is not None and val is not None:
+        if checked:
+            _check(lib().asx_spmv_plan_create_checked(C.byref(h), alg, value_type(dtype), m, n, nnz, _ptr(row_ptr), _ptr(col),
+                                                      _ptr(val), _stream()), "asx_spmv_plan_create_checked")
+        elif is_spmm and col is not None and val is not None:
             _check(lib().asx_spmm_plan_create(C.byref(h), alg, value_type(dtype), m, n, nnz, _ptr(row_ptr), _ptr(col),
                                               _ptr(val), ncols, _stream()), "asx_spmm_plan_create")
         elif not is_spmm and col is not None and val is not None:
@@ -295,6 +302,14 @@ class Plan:
         stats = np.zeros(4, dtype=np.int64)
         _check(lib().asx_plan_histogram(self.h, hist.ctypes.data_as(C.c_void_p), stats.ctypes.data_as(C.c_void_p)), "asx_plan_histogram")
         return hist, stats
+
+    @property
+    def checked(self):
+        return bool(lib().asx_plan_is_checked(self.h))
+
+    def refresh_if_changed(self, val):
+        """asx_plan_refresh_if_changed: checksums of val, and the plan's copy refreshed on the device where they differ."""
+        _check(lib().asx_plan_refresh_if_changed(self.h, _ptr(val), _stream()), "asx_plan_refresh_if_changed")
 
     def update_values(self, val):
         _check(lib().asx_plan_update_values(self.h, _ptr(val), _stream()), "asx_plan_update_values")

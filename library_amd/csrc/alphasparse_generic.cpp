@@ -117,7 +117,7 @@ struct KeptPlan {
     int value_type;
     int ncols;
     asx_plan *plan;
-    bool reads_callers_values_only;  // made by analysis on first use: never a regrouped copy of A's values
+    bool reads_callers_values_only;  // made by analysis on first use: no copy of A's values, or one guarded by checksums
 };
 // A zero-based and/or transposed device copy of a caller's CSR matrix.
 struct DerivedCsr {
@@ -758,38 +758,49 @@ alphasparseStatus_t alphasparseSpMV_bufferSize(alphasparseHandle_t handle, alpha
 // alphasparseSpMV / alphasparseSpMM on a descriptor runs an analysis itself (allocates and
 // synchronises once; later calls are kernels only).  ALPHASPARSE_AMD_AUTO_ANALYSIS selects how far
 // it goes; read once per process:
-//   unset, "structure"  only analysis that reads the caller's values in every call (split points
+//   unset, "checked"    SpMV: the full analysis, which may keep a regrouped copy of A's values, guarded:
+//                       every call takes two 64-bit checksums of the caller's values (one read of them
+//                       on the device, counted when the kernel is chosen) and refreshes the copy where
+//                       they differ from the kept ones, so a caller who changes values in place is
+//                       served as by the reference.  SpMM, and SpMV with opA = TRANSPOSE: as "structure".
+//   "structure"         only analysis that reads the caller's values in every call (split points
 //                       of the row-ordered kernels): sound whenever the row offsets and columns
 //                       behind a descriptor stay as they are, which holds for a caller who
 //                       changes values in place.  Not done for opA = TRANSPOSE (the kept copy of
 //                       the transposed matrix would hold values).
-//   "1", "values"       the full analysis, which may keep a regrouped copy of A's values: for callers
-//                       who do not change values in place without calling the analysis again
+//   "1", "values"       the full analysis without the checksums: for callers who do not change
+//                       values in place without calling the analysis again
 //   "0", "off"          none: every call recomputes its split points, as the reference does
-enum AutoAnalysis { kAutoOff = 0, kAutoStructure = 1, kAutoValues = 2 };
+// In every mode the sparsity pattern behind a descriptor is taken to stay as it is.
+enum AutoAnalysis { kAutoOff = 0, kAutoStructure = 1, kAutoValues = 2, kAutoChecked = 3 };
 static AutoAnalysis auto_analysis()
 {
     static const AutoAnalysis mode = [] {
         const char *e = std::getenv("ALPHASPARSE_AMD_AUTO_ANALYSIS");
-        if (!e || !e[0] || e[0] == 's' || e[0] == 'S') return kAutoStructure;
+        if (!e || !e[0] || e[0] == 'c' || e[0] == 'C') return kAutoChecked;
+        if (e[0] == 's' || e[0] == 'S') return kAutoStructure;
         if (e[0] == '0' || e[0] == 'o' || e[0] == 'O' || e[0] == 'n' || e[0] == 'N') return kAutoOff;
         return kAutoValues;
     }();
     return mode;
 }
 
+// what an analysis may keep: anything (the caller's own analysis call), only what reads the
+// caller's values in every call, or a copy of the values guarded by checksums
+enum Keeps { kKeepsAnything = 0, kKeepsStructure = 1, kKeepsCheckedValues = 2 };
 static alphasparseStatus_t spmv_analysis(alphasparseHandle_t handle, alphasparseOperation_t opA, alphasparseSpMatDescr_t matA,
-                                         alphasparseSpMVAlg_t alg, bool callers_values_only);
+                                         alphasparseSpMVAlg_t alg, Keeps keeps);
 
 alphasparseStatus_t alphasparseSpMV_analysis(alphasparseHandle_t handle, alphasparseOperation_t opA,
                                              alphasparseSpMatDescr_t matA, alphasparseSpMVAlg_t alg)
 {
-    return spmv_analysis(handle, opA, matA, alg, false);
+    return spmv_analysis(handle, opA, matA, alg, kKeepsAnything);
 }
 
 static alphasparseStatus_t spmv_analysis(alphasparseHandle_t handle, alphasparseOperation_t opA, alphasparseSpMatDescr_t matA,
-                                         alphasparseSpMVAlg_t alg, bool callers_values_only)
+                                         alphasparseSpMVAlg_t alg, Keeps keeps)
 {
+    const bool callers_values_only = keeps != kKeepsAnything;  // made on first use: gives way to the caller's own analysis
     if (!handle) return ALPHA_SPARSE_STATUS_INVALID_HANDLE;
     if (!matA) return ALPHA_SPARSE_STATUS_INVALID_POINTER;
     alphasparseStatus_t s = check_csr(matA, opA);
@@ -816,9 +827,12 @@ static alphasparseStatus_t spmv_analysis(alphasparseHandle_t handle, alphasparse
     asx_plan *plan = nullptr;
     // may keep a regrouped copy of A's columns and values (column slices, row blocks): call again
     // after changing the values.  Without the columns and values the plan stays row-ordered.
-    int rc = asx_spmv_plan_create(&plan, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
-                                  (int32_t)A->nnz, A->row_data, callers_values_only ? nullptr : A->col_data,
-                                  callers_values_only ? nullptr : A->val_data, (void *)handle->stream);
+    int rc = keeps == kKeepsCheckedValues
+                 ? asx_spmv_plan_create_checked(&plan, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
+                                                (int32_t)A->nnz, A->row_data, A->col_data, A->val_data, (void *)handle->stream)
+                 : asx_spmv_plan_create(&plan, (int)alg, (int)A->data_type, (int32_t)A->rows, (int32_t)A->cols,
+                                        (int32_t)A->nnz, A->row_data, keeps == kKeepsStructure ? nullptr : A->col_data,
+                                        keeps == kKeepsStructure ? nullptr : A->val_data, (void *)handle->stream);
     if (rc) return st(rc);
     x->plans.push_back(KeptPlan{false, (int)alg, A->row_data, A->col_data, A->val_data, A->rows, A->cols, A->nnz,
                                 (int)A->data_type, 1, plan, callers_values_only});
@@ -859,9 +873,10 @@ alphasparseStatus_t alphasparseSpMV(alphasparseHandle_t handle, alphasparseOpera
     const int32_t m = (int32_t)A->rows, n = (int32_t)A->cols, nnz = (int32_t)A->nnz;
     const asx_plan *plan = find_plan(matA, false, (int)alg, A, 1);
     const AutoAnalysis mode = auto_analysis();
-    if (!plan && (mode == kAutoValues || (mode == kAutoStructure && !is_transpose(opA))) && (!matA->info || ext_of(matA))) {
+    if (!plan && (mode == kAutoValues || (mode != kAutoOff && !is_transpose(opA))) && (!matA->info || ext_of(matA))) {
         release_effective(handle, &eff);
-        s = spmv_analysis(handle, opA, matA, alg, mode == kAutoStructure);
+        s = spmv_analysis(handle, opA, matA, alg,
+                          mode == kAutoValues ? kKeepsAnything : mode == kAutoChecked ? kKeepsCheckedValues : kKeepsStructure);
         if (s) return s;
         s = make_effective(handle, matA, opA, &eff);
         if (s) return s;
@@ -888,7 +903,13 @@ alphasparseStatus_t alphasparseSpMV(alphasparseHandle_t handle, alphasparseOpera
             return ALPHA_SPARSE_STATUS_INVALID_POINTER;
         }
     }
-    int rc;
+    int rc = plan && asx_plan_is_checked(plan)
+                 ? asx_plan_refresh_if_changed(const_cast<asx_plan *>(plan), A->val_data, (void *)handle->stream)
+                 : ASX_STATUS_SUCCESS;
+    if (rc) {
+        release_effective(handle, &eff);
+        return st(rc);
+    }
     if (A->data_type == ALPHA_R_64F)
         rc = asx_spmv_csr_f64(plan, (int)alg, m, n, nnz, *(const double *)alpha, A->row_data, A->col_data,
                               (const double *)A->val_data, (const double *)vecX->values,
@@ -1049,12 +1070,13 @@ alphasparseStatus_t alphasparseSpMM(alphasparseHandle_t handle, alphasparseOpera
     const int vt = (int)A->data_type;
     const asx_plan *plan = find_plan(matA, true, (int)alg, A, ncols);
     const AutoAnalysis mode = auto_analysis();
-    if (!plan && (mode == kAutoValues || (mode == kAutoStructure && !is_transpose(opA))) && (!matA->info || ext_of(matA))) {
+    const bool structure_only = mode == kAutoStructure || mode == kAutoChecked;  // no checksums for SpMM plans
+    if (!plan && (mode == kAutoValues || (structure_only && !is_transpose(opA))) && (!matA->info || ext_of(matA))) {
         release_effective(handle, &eff);
         size_t unused = 0;
-        s = spmm_preprocess(handle, opA, opB, alpha, matA, matB, beta, matC, computeType, alg, &unused, mode == kAutoStructure);
+        s = spmm_preprocess(handle, opA, opB, alpha, matA, matB, beta, matC, computeType, alg, &unused, structure_only);
         // the blocked algorithm has no analysis without A's values: the call goes on without one
-        if (s && !(mode == kAutoStructure && s == ALPHA_SPARSE_STATUS_NOT_SUPPORTED)) return s;
+        if (s && !(structure_only && s == ALPHA_SPARSE_STATUS_NOT_SUPPORTED)) return s;
         s = make_effective(handle, matA, opA, &eff);
         if (s) return s;
         plan = find_plan(matA, true, (int)alg, A, ncols);

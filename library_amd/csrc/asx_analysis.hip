@@ -3,6 +3,8 @@
 // the reference functions cited at each launcher (and in include/alphasparse_amd.h).
 // One thread per output element; every search is a binary search over row_ptr in global
 // memory (row_ptr is small next to the matrix and stays in L2 across the searches).
+#include <algorithm>
+
 #include "asx_internal.hpp"
 
 namespace asx {
@@ -396,6 +398,99 @@ int launch_gather_lines(const void *d_buf, size_t bytes, int group_lanes, int pe
     } else {
         return ASX_STATUS_INVALID_VALUE;
     }
+    return check_launch();
+}
+
+
+// ---- a checksum of the caller's values ------------------------------------------------------
+// Two 64-bit sums over the 32-bit words of an array, each word mixed with its position (a
+// changed word always changes the first sum: its term is the product of two non-zero 32-bit
+// numbers; swapped words change it unless the mixed values collide).  Sums of terms: any order of
+// accumulation gives the same pair.  Every workgroup leaves its two sums in partials[2 * blockIdx.x]
+// (no atomics: thousands of them on one address take longer than reading the values).
+constexpr int kChecksumThreads = 256;
+__global__ __launch_bounds__(kChecksumThreads) void k_checksum_words(const uint32_t *__restrict__ data, int64_t nwords,
+                                                                     unsigned long long *__restrict__ partials)
+{
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    __shared__ unsigned long long s_sum[2 * kChecksumThreads / kWave];
+    unsigned long long h1 = 0, h2 = 0;
+    const int64_t nvec = nwords / 4;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const auto mix = [&](uint32_t w, int64_t j) {
+        const uint32_t jj = (uint32_t)j, a = w + 0x9E3779B9u * jj;
+        h1 += (unsigned long long)a * ((0x85EBCA6Bu ^ jj) | 1u) + (unsigned long long)(j >> 32);
+        h2 += (unsigned long long)(a ^ (a >> 15)) * (0xC2B2AE35u + 2u * jj + 1u);
+    };
+    for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += stride) {
+        const u32x4 q = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(data) + v);
+        mix(q.x, 4 * v);
+        mix(q.y, 4 * v + 1);
+        mix(q.z, 4 * v + 2);
+        mix(q.w, 4 * v + 3);
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (int)(nwords - 4 * nvec)) mix(data[4 * nvec + threadIdx.x], 4 * nvec + threadIdx.x);
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        h1 += __shfl_xor(h1, d, kWave);
+        h2 += __shfl_xor(h2, d, kWave);
+    }
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) s_sum[2 * wave] = h1, s_sum[2 * wave + 1] = h2;
+    __syncthreads();
+    if (threadIdx.x < 2) {
+        unsigned long long t = 0;
+        for (int k = 0; k < kChecksumThreads / kWave; ++k) t += s_sum[2 * k + threadIdx.x];
+        partials[2 * (int64_t)blockIdx.x + threadIdx.x] = t;
+    }
+}
+// now[0..1] = the sums over the workgroups' partial sums (one workgroup)
+__global__ __launch_bounds__(kChecksumThreads) void k_checksum_finish(const unsigned long long *__restrict__ partials,
+                                                                      int32_t nparts, unsigned long long *__restrict__ now)
+{
+    __shared__ unsigned long long s_sum[2 * kChecksumThreads / kWave];
+    unsigned long long h1 = 0, h2 = 0;
+    for (int32_t i = threadIdx.x; i < nparts; i += kChecksumThreads) h1 += partials[2 * i], h2 += partials[2 * i + 1];
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        h1 += __shfl_xor(h1, d, kWave);
+        h2 += __shfl_xor(h2, d, kWave);
+    }
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) s_sum[2 * wave] = h1, s_sum[2 * wave + 1] = h2;
+    __syncthreads();
+    if (threadIdx.x < 2) {
+        unsigned long long t = 0;
+        for (int k = 0; k < kChecksumThreads / kWave; ++k) t += s_sum[2 * k + threadIdx.x];
+        now[threadIdx.x] = t;
+    }
+}
+// kept = now (after the copy was brought up to the values the sums were taken from)
+__global__ void k_checksum_commit(const unsigned long long *now, unsigned long long *kept)
+{
+    if (threadIdx.x < 2 && blockIdx.x == 0) kept[threadIdx.x] = now[threadIdx.x];
+}
+
+int checksum_parts()
+{
+    int cus = 256;
+    (void)asx_device_info(&cus, nullptr);
+    return cus * 8;
+}
+int launch_checksum(const void *d_data, size_t bytes, unsigned long long *d_partials, unsigned long long *d_now, hipStream_t s)
+{
+    if (((uintptr_t)d_data % 16) != 0 || bytes % 4 != 0) return ASX_STATUS_INVALID_VALUE;
+    const int64_t nwords = (int64_t)(bytes / 4);
+    const int64_t want = ceil_div64(nwords / 4 + 1, kChecksumThreads * 4);  // about four 16-byte loads a thread
+    const int parts = (int)std::max<int64_t>(1, std::min<int64_t>(want, checksum_parts()));
+    hipLaunchKernelGGL(k_checksum_words, dim3((unsigned)parts), dim3(kChecksumThreads), 0, s, (const uint32_t *)d_data, nwords,
+                       d_partials);
+    hipLaunchKernelGGL(k_checksum_finish, dim3(1), dim3(kChecksumThreads), 0, s, d_partials, parts, d_now);
+    return check_launch();
+}
+int launch_checksum_commit(const unsigned long long *d_now, unsigned long long *d_kept, hipStream_t s)
+{
+    hipLaunchKernelGGL(k_checksum_commit, dim3(1), dim3(64), 0, s, d_now, d_kept);
     return check_launch();
 }
 

@@ -502,6 +502,7 @@ int asx_plan_destroy(asx_plan *plan)
     int st = ASX_STATUS_SUCCESS;
     if (plan->d_meta) st = status_of(hipFree(plan->d_meta));
     if (plan->d_counters) (void)hipFree(plan->d_counters);
+    if (plan->d_checksum_parts) (void)hipFree(plan->d_checksum_parts);
     free_blocked(&plan->blocked);
     free_sliced(&plan->sliced);
     free_window(&plan->window);
@@ -596,7 +597,7 @@ struct KernelEstimates {
     // window_bands: with rings per band of diagonals, which only the build finds out
     double rows, sliced, window, window_bands;
 };
-static KernelEstimates estimate_kernels(const asx_plan *p, size_t sv, const ColumnSample &cs, bool window_ok)
+static KernelEstimates estimate_kernels(const asx_plan *p, size_t sv, const ColumnSample &cs, bool window_ok, bool checked)
 {
     const double inf = 1e30;
     const double nnz = (double)p->nnz, m = (double)p->m, n = (double)p->n, dsv = (double)sv;
@@ -618,6 +619,12 @@ static KernelEstimates estimate_kernels(const asx_plan *p, size_t sv, const Colu
     const bool uncut = p->stats[0] <= 16;
     e.window = !window_ok ? inf : 8e-6 + (wslots * (dsv + 2) + n * dsv + 2 * m * dsv) / (uncut ? 5.6e12 : 4.8e12);
     e.window_bands = !window_ok ? inf : 8e-6 + (wslots * (dsv + 2) + 1.5 * n * dsv + 2 * m * dsv) / (uncut ? 4.6e12 : 3.9e12);
+    if (checked) {
+        // a checked plan reads the caller's values once more in every call (a stream of its own
+        // kernel: 6.3 TB/s measured) and launches three small kernels
+        const double check = 10e-6 + nnz * dsv / 6.0e12;
+        e.sliced += check, e.window += check, e.window_bands += check;
+    }
     return e;
 }
 
@@ -702,10 +709,23 @@ static bool window_may_pay(const asx_plan *p, int row_kernel)
            2 * p->hist[0] + p->hist[1] <= (int64_t)p->nnz / 4;
 }
 
-extern "C" {
+// the checksum words of a plan: of the values as they are now (2), of the values its copy holds (2)
+static unsigned long long *checksum_words(const asx_plan *p) { return reinterpret_cast<unsigned long long *>(p->d_counters + 44); }
 
-int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
-                         const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, void *stream)
+// Takes the checksum of d_val and keeps it as the checksum of the plan's copy (which was just made
+// or refreshed from d_val).
+static int keep_checksum(asx_plan *p, const void *d_val, hipStream_t s)
+{
+    unsigned long long *w = checksum_words(p);
+    int st = ASX_STATUS_SUCCESS;
+    if (!p->d_checksum_parts) st = status_of(hipMalloc((void **)&p->d_checksum_parts, sizeof(unsigned long long) * 2 * checksum_parts()));
+    if (!st) st = launch_checksum(d_val, (size_t)p->nnz * vsize(p->value_type), p->d_checksum_parts, w, s);
+    if (!st) st = launch_checksum_commit(w, w + 2, s);
+    return st;
+}
+
+static int spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
+                            const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, bool checked, void *stream)
 {
     if (!out) return ASX_STATUS_INVALID_POINTER;
     *out = nullptr;
@@ -754,7 +774,7 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
             // the row-block kernel needs columns near each other; whether they fit its windows the
             // build finds out (NOT_SUPPORTED when some 256 rows reach further)
             const bool window_ok = window_may_pay(p, row_kernel) && cs.spread < kScatteredMinSpread;
-            const KernelEstimates e = estimate_kernels(p, sv, cs, window_ok);
+            const KernelEstimates e = estimate_kernels(p, sv, cs, window_ok, checked);
             const bool sliced_pays = e.sliced < 0.97 * e.rows, window_pays = e.window < 0.97 * e.rows;
             if (window_pays && e.window < e.sliced / 1.05) done = add_window() == ASX_STATUS_SUCCESS;
             if (done && p->window.nbands > 1 && sliced_pays && !(e.window_bands < e.sliced / 1.05)) {
@@ -771,6 +791,17 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
         }
     }
     if (!done) st = plan_row_ordered(p, row_kernel, s);
+    if (!st && checked && asx_plan_holds_values(p)) {
+        // the values must lie on a 16-byte boundary for the checksum's loads (every allocation does);
+        // a view that does not keeps an unchecked plan out: row-ordered instead
+        if (((uintptr_t)d_val % 16) == 0) {
+            st = keep_checksum(p, d_val, s);
+            p->checked = st == ASX_STATUS_SUCCESS;
+        } else {
+            asx_plan_destroy(p);
+            return spmv_plan_create(out, alg, value_type, m, n, nnz, d_row_ptr, nullptr, nullptr, false, stream);
+        }
+    }
     if (st) {
         asx_plan_destroy(p);
         return st;
@@ -779,17 +810,58 @@ int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
     return ASX_STATUS_SUCCESS;
 }
 
+extern "C" {
+
+int asx_spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
+                         const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, void *stream)
+{
+    return spmv_plan_create(out, alg, value_type, m, n, nnz, d_row_ptr, d_col, d_val, false, stream);
+}
+
+int asx_spmv_plan_create_checked(asx_plan **out, int alg, int value_type, int32_t m, int32_t n, int32_t nnz,
+                                 const int32_t *d_row_ptr, const int32_t *d_col, const void *d_val, void *stream)
+{
+    return spmv_plan_create(out, alg, value_type, m, n, nnz, d_row_ptr, d_col, d_val, true, stream);
+}
+
+int asx_plan_is_checked(const asx_plan *plan) { return plan && plan->checked ? 1 : 0; }
+
+int asx_plan_refresh_if_changed(asx_plan *plan, const void *d_val, void *stream)
+{
+    if (!plan) return ASX_STATUS_INVALID_POINTER;
+    if (!plan->checked) return ASX_STATUS_SUCCESS;  // reads the caller's values in every call, or was made unchecked
+    if (plan->nnz > 0 && !d_val) return ASX_STATUS_INVALID_POINTER;
+    if (((uintptr_t)d_val % 16) != 0) return ASX_STATUS_INVALID_VALUE;
+    hipStream_t s = (hipStream_t)stream;
+    unsigned long long *w = checksum_words(plan);
+    int st = launch_checksum(d_val, (size_t)plan->nnz * vsize(plan->value_type), plan->d_checksum_parts, w, s);
+    if (st) return st;
+    if (plan->alg == ASX_SPMV_SLICED)
+        st = plan->value_type == ASX_R_64F ? sliced_update_values<double>(&plan->sliced, (const double *)d_val, s, w)
+                                           : sliced_update_values<float>(&plan->sliced, (const float *)d_val, s, w);
+    else if (plan->alg == ASX_SPMV_WINDOW)
+        st = plan->value_type == ASX_R_64F ? window_update_values<double>(&plan->window, (const double *)d_val, s, w)
+                                           : window_update_values<float>(&plan->window, (const float *)d_val, s, w);
+    if (st) return st;
+    return launch_checksum_commit(w, w + 2, s);
+}
+
 int asx_plan_update_values(asx_plan *plan, const void *d_val, void *stream)
 {
     if (!plan) return ASX_STATUS_INVALID_POINTER;
     if (plan->nnz > 0 && !d_val) return ASX_STATUS_INVALID_POINTER;
     hipStream_t s = (hipStream_t)stream;
-    if (!plan->is_spmm && plan->alg == ASX_SPMV_SLICED)
-        return plan->value_type == ASX_R_64F ? sliced_update_values<double>(&plan->sliced, (const double *)d_val, s)
-                                             : sliced_update_values<float>(&plan->sliced, (const float *)d_val, s);
-    if (!plan->is_spmm && plan->alg == ASX_SPMV_WINDOW)
-        return plan->value_type == ASX_R_64F ? window_update_values<double>(&plan->window, (const double *)d_val, s)
-                                             : window_update_values<float>(&plan->window, (const float *)d_val, s);
+    if (!plan->is_spmm && (plan->alg == ASX_SPMV_SLICED || plan->alg == ASX_SPMV_WINDOW)) {
+        int st;
+        if (plan->alg == ASX_SPMV_SLICED)
+            st = plan->value_type == ASX_R_64F ? sliced_update_values<double>(&plan->sliced, (const double *)d_val, s)
+                                               : sliced_update_values<float>(&plan->sliced, (const float *)d_val, s);
+        else
+            st = plan->value_type == ASX_R_64F ? window_update_values<double>(&plan->window, (const double *)d_val, s)
+                                               : window_update_values<float>(&plan->window, (const float *)d_val, s);
+        if (!st && plan->checked) st = ((uintptr_t)d_val % 16) == 0 ? keep_checksum(plan, d_val, s) : ASX_STATUS_INVALID_VALUE;
+        return st;
+    }
     if (plan->is_spmm && plan->alg == ASX_SPMM_BLOCKED)
         return plan->value_type == ASX_R_64F ? blocked_update_values<double>(&plan->blocked, (const double *)d_val, s)
                                              : blocked_update_values<float>(&plan->blocked, (const float *)d_val, s);

@@ -53,6 +53,12 @@ int launch_stream_row_blocks(const int32_t *d_row_ptr, int32_t m, int32_t nnz, i
                              hipStream_t s);
 int launch_copy_bytes(const void *d_src, void *d_dst, size_t bytes, hipStream_t s);
 int launch_fill_i32(int32_t *d_dst, int64_t n, int32_t value, hipStream_t s);
+// d_now[0..1] = two 64-bit checksums of `bytes` bytes (a multiple of 4, from a 16-byte boundary);
+// d_partials: 2 * checksum_parts() words of scratch
+int checksum_parts();
+int launch_checksum(const void *d_data, size_t bytes, unsigned long long *d_partials, unsigned long long *d_now, hipStream_t s);
+// kept = now
+int launch_checksum_commit(const unsigned long long *d_now, unsigned long long *d_kept, hipStream_t s);
 int launch_sample_columns(const int32_t *d_col, int64_t stride, int shift, const int32_t *d_row_ptr, int32_t m,
                           int32_t width, int32_t samples, int32_t *d_out, hipStream_t s);
 int launch_gather_lines(const void *d_buf, size_t bytes, int group_lanes, int per_lane, void *d_out, int *nthreads,
@@ -156,7 +162,7 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
                  const int32_t *row_ptr, const int32_t *col, const T *val, SlicedMatrix *out, hipStream_t s);
 void free_sliced(SlicedMatrix *p);
 template <typename T>
-int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s);
+int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s, const unsigned long long *unless_equal = nullptr);
 template <typename T>
 int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, const T *x, T beta, T *y, T *partial,
                        hipStream_t s);
@@ -194,7 +200,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
                  const T *val, WindowMatrix *out, hipStream_t s);
 void free_window(WindowMatrix *p);
 template <typename T>
-int window_update_values(const WindowMatrix *wm, const T *val, hipStream_t s);
+int window_update_values(const WindowMatrix *wm, const T *val, hipStream_t s, const unsigned long long *unless_equal = nullptr);
 template <typename T>
 int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, T *carry,
                        hipStream_t s);
@@ -215,7 +221,10 @@ struct asx_plan {
     int value_type;
     int32_t m, n, nnz, ncols;
     const int32_t *row_ptr;  // the device array the plan was built from (identity check only)
-    int64_t *d_counters;     // kPlanCounters words on the device: histogram (33), stats (4), a flag (40), 64 sample counts (64..95)
+    int64_t *d_counters;     // kPlanCounters words on the device: histogram (33), stats (4), a flag (40), checksums of the values:
+                             // of this call (44, 45) and of the copy the plan holds (46, 47), 64 sample counts (64..95)
+    int checked;             // the plan holds a copy of A's values and a checksum of them (asx_spmv_plan_create_checked)
+    unsigned long long *d_checksum_parts;  // checked plans: the workgroups' partial sums of one checksum run
     int32_t *d_meta;         // split points / row blocks (layout depends on alg)
     size_t meta_bytes;
     int32_t nunits;  // tiles / row blocks / segments

@@ -355,14 +355,18 @@ __global__ __launch_bounds__(kBlock) void k_sliced_empty_slices(const int32_t *_
     if (tile_off[s] == tile_off[s + 1]) chunk_lo[i] = tile_base[tile_off[s]];
 }
 
+// Copies the values again from where they came from.  `unless_equal` (may be null): four words, two
+// checksums of the values now and two of the values the copy holds; where they agree nothing is done.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_sliced_regather(const int32_t *__restrict__ perm, int64_t slots,
-                                                            const T *__restrict__ val, T *__restrict__ val_out)
+                                                            const T *__restrict__ val, T *__restrict__ val_out,
+                                                            const unsigned long long *unless_equal)
 {
-    const int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (d >= slots) return;
-    const int32_t src = perm[d];
-    val_out[d] = src >= 0 ? val[src] : T(0);
+    if (unless_equal && unless_equal[0] == unless_equal[2] && unless_equal[1] == unless_equal[3]) return;  // uniform
+    for (int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; d < slots; d += (int64_t)gridDim.x * blockDim.x) {
+        const int32_t src = perm[d];
+        val_out[d] = src >= 0 ? val[src] : T(0);
+    }
 }
 
 
@@ -813,12 +817,13 @@ done:
 
 
 template <typename T>
-int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s)
+int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s, const unsigned long long *unless_equal)
 {
     const int64_t slots = (int64_t)sm->ntiles * kSlicedTile;
     if (slots == 0) return ASX_STATUS_SUCCESS;
-    hipLaunchKernelGGL((k_sliced_regather<T>), dim3((unsigned)ceil_div64(slots, kBlock)), dim3(kBlock), 0, s, sm->perm,
-                       slots, val, (T *)sm->val);
+    // a bounded grid: where the checksums agree the kernel has nothing to do but to end
+    const unsigned grid = (unsigned)std::min<int64_t>(ceil_div64(slots, kBlock), 8192);
+    hipLaunchKernelGGL((k_sliced_regather<T>), dim3(grid), dim3(kBlock), 0, s, sm->perm, slots, val, (T *)sm->val, unless_equal);
     return check_launch();
 }
 
@@ -858,7 +863,7 @@ int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, co
 #define ASX_INST(T)                                                                                              \
     template int build_sliced<T>(int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, const int32_t *,          \
                                  const int32_t *, const T *, SlicedMatrix *, hipStream_t);                       \
-    template int sliced_update_values<T>(const SlicedMatrix *, const T *, hipStream_t);                          \
+    template int sliced_update_values<T>(const SlicedMatrix *, const T *, hipStream_t, const unsigned long long *);                          \
     template int launch_spmv_sliced<T>(int32_t, int32_t, T, const SlicedMatrix *, const T *, T, T *, T *, hipStream_t);
 ASX_INST(float)
 ASX_INST(double)

@@ -92,7 +92,7 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
                                        (alphasparseSpMVAlg_t)alg, &bytes);
         if (s) return 10 + (int)s;
         HIP_OK(hipMalloc(&buffer, bytes ? bytes : 1));
-        if (analysis) {
+        if (analysis && analysis != 5) {
             s = alphasparseSpMV_analysis(handle, opA, A, (alphasparseSpMVAlg_t)alg);
             if (s) return 30 + (int)s;
         }
@@ -101,7 +101,7 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
             s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
         }
-        if (!analysis) {
+        if (!analysis || analysis == 5) {
             // analysis on first use: unless ALPHASPARSE_AMD_AUTO_ANALYSIS=0, the calls above left kept
             // analysis on the descriptor although alphasparseSpMV_analysis was never called ("1": the
             // full one, which may regroup A; unset: only what reads the caller's values in every call)
@@ -121,6 +121,18 @@ static int run_case(const std::string &dir, const char *op, long m, long n, long
             HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
             s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
             if (s) return 50 + (int)s;
+        }
+        if (analysis == 5) {
+            // a caller written for the reference: it never calls the analysis, changes A's values in
+            // place (same pattern) and multiplies again; the product must use the new values, twice
+            auto val2 = read_bin<T>(dir + "/val2.bin", nnz);
+            HIP_OK(hipStreamSynchronize(handle->stream));
+            HIP_OK(hipMemcpy(d_val, val2.data(), val2.size() * sizeof(T), hipMemcpyHostToDevice));
+            for (int rep = 0; rep < 2; ++rep) {
+                HIP_OK(hipMemcpy(d_y, yin.data(), yin.size() * sizeof(T), hipMemcpyHostToDevice));
+                s = alphasparseSpMV(handle, opA, &alpha, A, X, &beta, Y, dt, (alphasparseSpMVAlg_t)alg, buffer);
+                if (s) return 50 + (int)s;
+            }
         }
         if (analysis == 3) {
             // a second descriptor that shares A's row offsets and columns but has its own values

@@ -257,10 +257,13 @@ def test_two_streams_share_one_analysed_descriptor(tmp_path, oracle):
 
 def test_analysis_on_first_use(tmp_path, oracle):
     """A caller that never calls alphasparseSpMV_analysis / alphasparseSpMM_preprocess (the reference's
-    own test loops do not) gets kept analysis from its first call on: by default only analysis that
-    reads the caller's values in every call (a row-ordered kernel's split points), with
-    ALPHASPARSE_AMD_AUTO_ANALYSIS=1 the full one (column slices on this matrix), with =0 none.  The
-    caller program prints the kept kernel and checks that the descriptor ends up analysed or not."""
+    own test loops do not) gets kept analysis from its first call on.  SpMV by default: the full
+    analysis (column slices on this matrix) with a copy of the values that every call checks against
+    the caller's values by checksum, so that values changed in place between two calls are picked up
+    without a word from the caller; ALPHASPARSE_AMD_AUTO_ANALYSIS=structure: only analysis that reads
+    the caller's values in every call (a row-ordered kernel's split points); =1: the full one,
+    unchecked; =0: none.  The caller program prints the kept kernel and checks that the descriptor
+    ends up analysed or not."""
     from library_amd import workloads as W
     rp, col, val = W.csr_zipf(1 << 20, 1 << 20, 20, 1.0, 5000, 0.01, np.float64, 5)
     n = 1 << 20
@@ -268,15 +271,38 @@ def test_analysis_on_first_use(tmp_path, oracle):
     x = rng.uniform(-1, 1, n)
     y0 = rng.uniform(-1, 1, rp.size - 1)
     ref, scale = oracle.spmv(rp, col, val, x, 2.1, 3.2, y0, 8), spmv_scale(rp, col, val, x, 2.1, 3.2, y0)
-    for env, kernels in ((None, ("kernel flat", "kernel merge")), ({"ALPHASPARSE_AMD_AUTO_ANALYSIS": "1"}, ("kernel sliced",)),
+    for env, kernels in ((None, ("kernel sliced",)), ({"ALPHASPARSE_AMD_AUTO_ANALYSIS": "structure"}, ("kernel flat", "kernel merge")),
+                         ({"ALPHASPARSE_AMD_AUTO_ANALYSIS": "1"}, ("kernel sliced",)),
                          ({"ALPHASPARSE_AMD_AUTO_ANALYSIS": "0"}, ("kernel none",))):
         said = []
         if env is None and "ALPHASPARSE_AMD_AUTO_ANALYSIS" in os.environ:
-            env = {"ALPHASPARSE_AMD_AUTO_ANALYSIS": "structure"}
+            env = {"ALPHASPARSE_AMD_AUTO_ANALYSIS": "checked"}
         got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, 2.1, 3.2, 0, env=env, said=said,
                         tag="" if env is None else "_" + list(env.values())[0])
         assert_close(got, ref, scale, np.float64, f"SpMV, analysis on first use, {env}")
         assert any(k in said[0] for k in kernels), (env, said[0])
+    # values changed in place between calls, no analysis call: a few of them, all of them, two of
+    # them swapped, one sign flipped
+    few = val.copy()
+    few[rng.integers(0, val.size, 5)] *= 3.0
+    swapped = val.copy()
+    i, j = 12345, val.size - 7
+    swapped[i], swapped[j] = val[j], val[i]
+    sign = val.copy()
+    sign[val.size // 2] = -sign[val.size // 2]
+    for name, val2 in (("few", few), ("all", rng.uniform(-1, 1, val.size)), ("swapped", swapped), ("sign", sign)):
+        for env in (None, {"ALPHASPARSE_AMD_AUTO_ANALYSIS": "structure"}):
+            if env is None and "ALPHASPARSE_AMD_AUTO_ANALYSIS" in os.environ:
+                env = {"ALPHASPARSE_AMD_AUTO_ANALYSIS": "checked"}
+            said = []
+            got = _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, 2.1, 3.2, 5, env=env, said=said, val2=val2,
+                            tag=f"_{name}" + ("" if env is None else "_" + list(env.values())[0]))
+            ref2, scale2 = oracle.spmv(rp, col, val2, x, 2.1, 3.2, y0, 8), spmv_scale(rp, col, val2, x, 2.1, 3.2, y0)
+            assert_close(got, ref2, scale2, np.float64, f"values changed in place ({name}), no analysis call, {env}")
+            if name in ("swapped", "sign"):  # the change is one the tolerance alone would not show
+                assert not np.array_equal(got, _run_case(tmp_path, "spmv", np.float64, rp, col, val, x, y0, 1, 0, 2.1, 3.2, 0, env=env,
+                                                         tag=f"_{name}_before" + ("" if env is None else "_s")))
+            assert ("kernel sliced" in said[0]) == (env is None or env["ALPHASPARSE_AMD_AUTO_ANALYSIS"] == "checked"), said[0]
     from test_gpu_parity import _block_structured
     m, k, nc = 700, 640, 64
     rp, col, val = _block_structured(rng, m, k, np.float32)

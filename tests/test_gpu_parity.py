@@ -1131,3 +1131,80 @@ def test_calibration_copy_runs(torch, capi):
         assert int(out.min()) == 16 and int(out.max()) == 16  # 16 loads of the value 1 per lane
     assert L.asx_gather_lines(capi._ptr(buf), buf.numel() * 4, 3, 16, capi._ptr(out), None, stream) == 3
     assert L.asx_gather_lines(capi._ptr(buf), buf.numel() * 4, 1, 12, capi._ptr(out), None, stream) == 3
+
+
+# ------------------------------------------------------------------ checked plans (values changed in place)
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_checked_plans_follow_values_changed_in_place(torch, capi, oracle, dtype):
+    """asx_spmv_plan_create_checked + asx_plan_refresh_if_changed: a plan that holds a copy of A's
+    values notices, by two checksums taken on the device before every call, that the caller changed
+    values in place, and refreshes its copy; with unchanged values the call gives the same bits as
+    before.  Sliced plan (scattered columns) and window plan (a band), DEFAULT's choice; a single
+    changed value, two swapped values (same multiset: only position-dependent sums see it), a flipped
+    sign, all values; a small matrix stays row-ordered and unchecked."""
+    from library_amd import workloads as W
+    rng = np.random.default_rng(77)
+    cases = []
+    rp, col, val = W.csr_fixed(1 << 18, 1 << 20, 12, dtype, 3)
+    cases.append(("scattered", rp, col, val, 1 << 20, capi.SPMV_SLICED))
+    rp, col, val = W.csr_banded(1 << 19, 4, dtype, 5)
+    cases.append(("band of 9", rp, col, val, 1 << 19, capi.SPMV_WINDOW))
+    for name, rp, col, val, n, want_alg in cases:
+        m, nnz = rp.size - 1, col.size
+        x = rng.uniform(-1, 1, n).astype(dtype)
+        y0 = rng.uniform(-1, 1, m).astype(dtype)
+        d_rp, d_col, d_val, d_x = (dev(torch, a) for a in (rp, col, val, x))
+        for alg in (want_alg, capi.SPMV_DEFAULT):
+            d_val.copy_(torch.from_numpy(val))
+            plan = capi.Plan(False, alg, np.dtype(dtype), m, n, nnz, d_rp, col=d_col, val=d_val, checked=True)
+            if alg == capi.SPMV_DEFAULT and plan.alg != want_alg:
+                # DEFAULT counted the price of checking and stayed with a kernel that reads the caller's values
+                assert not plan.checked and not plan.holds_values, (name, plan.alg)
+                plan.destroy()
+                continue
+            assert plan.alg == want_alg and plan.checked and plan.holds_values, (name, plan.alg)
+
+            def product(values):
+                ref = oracle.spmv(rp, col, values, x, dtype(1.5), dtype(0.5), y0, 4)
+                y = dev(torch, y0)
+                plan.refresh_if_changed(d_val)
+                capi.spmv(d_rp, d_col, d_val, d_x, y, 1.5, 0.5, alg=alg, plan=plan)
+                torch.cuda.synchronize()
+                got = y.cpu().numpy()
+                assert_close(got, ref, spmv_scale(rp, col, values, x, 1.5, 0.5, y0), dtype, f"{name} alg={alg}")
+                return got
+            first = product(val)
+            assert np.array_equal(first, product(val)), "unchanged values: the same bits"
+            cur = val.copy()
+            cur[nnz // 3] += dtype(0.25)  # one value
+            d_val.copy_(torch.from_numpy(cur))
+            one = product(cur)
+            assert not np.array_equal(one, first)
+            i, j = 17, nnz - 5            # two values swapped
+            cur[i], cur[j] = cur[j], cur[i]
+            d_val.copy_(torch.from_numpy(cur))
+            swapped = product(cur)
+            assert not np.array_equal(swapped, one)
+            cur[nnz // 2] = -cur[nnz // 2]  # one sign
+            d_val.copy_(torch.from_numpy(cur))
+            assert not np.array_equal(product(cur), swapped)
+            cur = rng.uniform(-1, 1, nnz).astype(dtype)  # all of them
+            d_val.copy_(torch.from_numpy(cur))
+            product(cur)
+            d_val.copy_(torch.from_numpy(val))  # and back: the first product again, bit for bit
+            assert np.array_equal(product(val), first)
+            # the explicit refresh keeps the checksums in step: nothing to do in the next check
+            cur = rng.uniform(-1, 1, nnz).astype(dtype)
+            d_val.copy_(torch.from_numpy(cur))
+            plan.update_values(d_val)
+            product(cur)
+            plan.destroy()
+    # a matrix too small to regroup: row-ordered, reads the caller's values, nothing to check
+    rp, col, val = csr_from_lengths(rng.integers(0, 9, 3000), 5000, 7, dtype)
+    d = [dev(torch, a) for a in (rp, col, val)]
+    plan = capi.Plan(False, capi.SPMV_DEFAULT, np.dtype(dtype), rp.size - 1, 5000, col.size, d[0], col=d[1], val=d[2], checked=True)
+    assert not plan.checked and not plan.holds_values
+    plan.refresh_if_changed(d[2])
+    plan.destroy()
+    L = capi.lib()
+    assert L.asx_plan_refresh_if_changed(None, None, None) == 7 and L.asx_plan_is_checked(None) == 0
