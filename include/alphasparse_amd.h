@@ -199,7 +199,10 @@ int asx_spmm_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, in
  * alone, not on timings.  Otherwise as asx_plan_create.  No counterpart in the reference (its
  * alphasparseSpMV_analysis is a stub).  alg = ASX_SPMV_WINDOW builds the row-block copy for the
  * kernel that keeps sliding windows of x in LDS (again a COPY of columns and values, and the
- * carry slots of a call); DEFAULT picks it, when the sliced kernel is not chosen, for nnz >= 2^21
+ * carry slots of a call; a matrix without rows of fewer than two stored elements needs no copy of
+ * the values: an fp32 plan, or a plan made by asx_spmv_plan_create_checked, then reads A's values
+ * in every call, ASX_PLAN_INFO_BY_REFERENCE = 1, and holds 2 bytes per stored element instead of
+ * 14 or 10); DEFAULT picks it, when the sliced kernel is not chosen, for nnz >= 2^21
  * and rows no longer than 2048 whenever the matrix qualifies: every 256 consecutive rows reach
  * over fewer than 16376 columns, or the stored elements lie on at most 4 bands of diagonals whose
  * windows fit the LDS together (stencils on three-dimensional grids); otherwise
@@ -219,8 +222,12 @@ int asx_plan_holds_values(const asx_plan *plan);
  * that a plan which ends up holding a copy of the values also keeps two 64-bit checksums of
  * them (position-dependent sums over their 32-bit words; a single changed word always changes
  * them, several changes escape with probability 2^-128) and that DEFAULT's choice counts what
- * checking costs.  d_val must lie on a 16-byte boundary for such a plan (otherwise the plan is made
- * row-ordered).  asx_plan_refresh_if_changed, called before every SpMV through the plan with the
+ * checking costs.  d_val must lie on a 16-byte boundary for such a plan (otherwise DEFAULT makes
+ * the plan row-ordered, and ASX_SPMV_SLICED / ASX_SPMV_WINDOW return ASX_STATUS_INVALID_VALUE).  A
+ * window plan over a matrix without rows of fewer than two stored elements keeps no copy of the
+ * values at all and so needs neither checksums nor refreshes (fp64: 5-point stencil on 4096^2,
+ * 210 us a multiply in place, 201 from a copy that the caller keeps up to date, 285 from a checked
+ * copy).  asx_plan_refresh_if_changed, called before every SpMV through the plan with the
  * values as they are now, takes their checksums (one read of the values: 42 us for 34 M fp64
  * values) and brings the copy up to date where they differ from the kept ones; all on the device,
  * asynchronous on `stream`, nothing is read back.  It does nothing for a plan that was made
@@ -262,8 +269,11 @@ enum {
     ASX_PLAN_INFO_WIDTH = 10,         /* columns per slice (sliced), columns the rings hold together (window) */
     ASX_PLAN_INFO_WORKGROUPS = 11,    /* workgroups of pass 1 (sliced), chains (window) */
     ASX_PLAN_INFO_PIECES = 12,        /* pieces of x fetched over all blocks (window) */
-    ASX_PLAN_INFO_STACKED_ROWS = 13   /* rows of a plane when the three bands share rotating regions of LDS and the
+    ASX_PLAN_INFO_STACKED_ROWS = 13,  /* rows of a plane when the three bands share rotating regions of LDS and the
                                          blocks are stored plane above plane (window; 0 otherwise) */
+    ASX_PLAN_INFO_BY_REFERENCE = 14   /* 1 when the plan keeps no copy of A's values (window: no row of A holds fewer than two
+                                         stored elements, so the stored elements of a tile are consecutive in A's val, which
+                                         every call reads in place; asx_plan_holds_values is 0 then) */
 };
 int64_t asx_plan_info(const asx_plan *plan, int what);
 /* Frees the buffer a sliced or window plan keeps for the partial sums / carries of a call.  Calls
@@ -280,10 +290,12 @@ size_t asx_plan_own_scratch_bytes(const asx_plan *plan);
  * that.  ASX_STATUS_INVALID_VALUE when the plan's kernel has no such array.  No counterpart in the
  * reference. */
 enum {
-    ASX_PLAN_ARRAY_VAL = 0,          /* slots x value: the regrouped values, in the order the loads deliver them */
+    ASX_PLAN_ARRAY_VAL = 0,          /* slots x value: the regrouped values, in the order the loads deliver them
+                                      * (with PERM: absent, ASX_STATUS_INVALID_VALUE, in a plan that reads A's values in place) */
     ASX_PLAN_ARRAY_CF = 1,           /* slots x u16: local column | first-of-run << 15 */
     ASX_PLAN_ARRAY_PERM = 2,         /* slots x i32: position in A's values of each stored copy (-1: pad) */
-    ASX_PLAN_ARRAY_TILE_WORDS = 3,   /* sliced: (tiles + 1) x i32 first partial sum of each tile; window: tiles x 2 i32 */
+    ASX_PLAN_ARRAY_TILE_WORDS = 3,   /* sliced: (tiles + 1) x i32 first partial sum of each tile; window: tiles x 4 i32
+                                      * (first row | starts-inside-a-row << 31, rows, first stored element in A, stored elements) */
     ASX_PLAN_ARRAY_WORKGROUPS = 4,   /* sliced: workgroups x 4 i32 (slice, first tile, end tile, 0); window: chains x 2 i32 */
     ASX_PLAN_ARRAY_PARTIAL_ROWS = 5, /* sliced: partial sums x u16 row inside the row block | may-repeat << 15 */
     ASX_PLAN_ARRAY_RANGES = 6,       /* sliced: (row blocks + 1) x slices i32: first partial sum of block b in slice s */

@@ -317,7 +317,7 @@ class Plan:
 
     INFO = {"tiles": 0, "slices": 1, "partial_sums": 2, "rows_per_wave": 3, "rows_per_block": 4, "bands": 5,
             "chains": 6, "carry_pass": 7, "row_blocks": 8, "steps": 9, "width": 10, "workgroups": 11, "pieces": 12,
-            "stacked_rows": 13}
+            "stacked_rows": 13, "by_reference": 14}
     # asx_plan_export: name -> (id, element type; "value" = the plan's value type)
     ARRAYS = {"val": (0, "value"), "cf": (1, np.uint16), "perm": (2, np.int32), "tile_words": (3, np.int32),
               "workgroups": (4, np.int32), "partial_rows": (5, np.uint16), "ranges": (6, np.int32),

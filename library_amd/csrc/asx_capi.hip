@@ -217,14 +217,15 @@ int spmv_impl(const asx_plan *plan, int alg, int32_t m, int32_t n, int32_t nnz, 
         return launch_spmv_sliced<T>(m, n, alpha, &plan->sliced, x, beta, y, scratch, s);
     }
     case ASX_SPMV_WINDOW: {
-        // the row blocks hold a copy of A's columns and values and are built by asx_spmv_plan_create;
-        // the carries of the call (plans with cut rows only) go where the sliced kernel's partial sums go
+        // the row blocks hold a copy of A's columns (and of its values, unless they can be read in
+        // place) and are built by asx_spmv_plan_create; the carries of the call (plans with cut rows
+        // only) go where the sliced kernel's partial sums go
         if (!plan || !plan->window.cf) return ASX_STATUS_NOT_INITIALIZED;
         if (plan->n != n) return ASX_STATUS_INVALID_VALUE;
         const size_t need = window_scratch_bytes(&plan->window, sizeof(T));
         T *scratch = ws && ws_bytes >= need ? (T *)ws : (T *)plan->window.carry;
         if (need && !scratch) return ws ? ASX_STATUS_INVALID_SIZE : ASX_STATUS_INVALID_POINTER;
-        return launch_spmv_window<T>(m, n, alpha, &plan->window, x, beta, y, scratch, s);
+        return launch_spmv_window<T>(m, n, alpha, &plan->window, val, x, beta, y, scratch, s);
     }
     default: return ASX_STATUS_NOT_SUPPORTED;
     }
@@ -623,7 +624,11 @@ static KernelEstimates estimate_kernels(const asx_plan *p, size_t sv, const Colu
         // a checked plan reads the caller's values once more in every call (a stream of its own
         // kernel: 6.3 TB/s measured) and launches three small kernels
         const double check = 10e-6 + nnz * dsv / 6.0e12;
-        e.sliced += check, e.window += check, e.window_bands += check;
+        e.sliced += check;
+        if (p->hist[0] + p->hist[1] > 0)
+            e.window += check, e.window_bands += check;
+        else if (sv == 8)  // reads A's values in place: no check; two scans a tile and loads off 16-byte boundaries
+            e.window *= 1.08, e.window_bands *= 1.08;
     }
     return e;
 }
@@ -665,14 +670,20 @@ int plan_add_slices(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
 // Builds the row-block copy onto a plan that already holds the histogram.
 constexpr int32_t kWindowMaxRow = 2048;  // longer rows would make the ordered carry pass serial
 template <typename T>
-int plan_add_window(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, hipStream_t s)
+int plan_add_window(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, bool follows_values, hipStream_t s)
 {
     if (p->stats[0] > kWindowMaxRow) return ASX_STATUS_NOT_SUPPORTED;
     int cus = 256;
     (void)asx_device_info(&cus, nullptr);
     WindowMatrix wm{};
     // one chain of row blocks per compute unit for fp64 (128 KiB of LDS each), two for fp32
-    const int st = build_window<T>(p->m, p->n, p->nnz, cus * (sizeof(T) == 4 ? 2 : 1), d_row_ptr, d_col, d_val, &wm, s);
+    // Reading A's values in place costs a multiply in fp32 nothing and in fp64 a twentieth to a
+    // tenth (two scans a tile instead of one; 5-point stencil on 4096^2: 201 us from the copy, 210 to
+    // 220 in place; a refresh of the copy takes more than a multiply): fp32 plans always do where
+    // they can, fp64 plans when the caller wants values changed in place to be followed (a checked
+    // plan), which then takes no check at all.
+    const int st = build_window<T>(p->m, p->n, p->nnz, cus * (sizeof(T) == 4 ? 2 : 1), sizeof(T) == 4 || follows_values, d_row_ptr,
+                                   d_col, d_val, &wm, s);
     if (st) return st;
     if (p->d_meta) (void)hipFree(p->d_meta);
     p->d_meta = nullptr;
@@ -753,8 +764,8 @@ static int spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, 
                    : plan_add_slices<float>(p, d_row_ptr, d_col, (const float *)d_val, pairs, s);
     };
     const auto add_window = [&]() {
-        return f64 ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, s)
-                   : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, s);
+        return f64 ? plan_add_window<double>(p, d_row_ptr, d_col, (const double *)d_val, checked, s)
+                   : plan_add_window<float>(p, d_row_ptr, d_col, (const float *)d_val, checked, s);
     };
     const bool can_regroup = alg == ASX_SPMV_DEFAULT && d_col && d_val && m > 0 && n > 0 && nnz >= kSlicedMinNnz &&
                              regrouped_copy_fits(p, sv);
@@ -799,6 +810,7 @@ static int spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, 
             p->checked = st == ASX_STATUS_SUCCESS;
         } else {
             asx_plan_destroy(p);
+            if (want) return ASX_STATUS_INVALID_VALUE;  // the kernel was asked for by name
             return spmv_plan_create(out, alg, value_type, m, n, nnz, d_row_ptr, nullptr, nullptr, false, stream);
         }
     }
@@ -871,7 +883,7 @@ int asx_plan_update_values(asx_plan *plan, const void *d_val, void *stream)
 int asx_plan_holds_values(const asx_plan *plan)
 {
     if (!plan) return 0;
-    return (!plan->is_spmm && (plan->alg == ASX_SPMV_SLICED || plan->alg == ASX_SPMV_WINDOW)) ||
+    return (!plan->is_spmm && (plan->alg == ASX_SPMV_SLICED || (plan->alg == ASX_SPMV_WINDOW && !plan->window.by_reference))) ||
            (plan->is_spmm && plan->alg == ASX_SPMM_BLOCKED);
 }
 
@@ -934,10 +946,10 @@ static bool plan_array(const asx_plan *p, int what, const void **ptr, size_t *by
         const WindowMatrix &m = p->window;
         const size_t slots = (size_t)m.ntiles * kSlicedTile;
         switch (what) {
-        case ASX_PLAN_ARRAY_VAL: *ptr = m.val, *bytes = slots * sv; return true;
+        case ASX_PLAN_ARRAY_VAL: *ptr = m.val, *bytes = slots * sv; return m.val != nullptr;
         case ASX_PLAN_ARRAY_CF: *ptr = m.cf, *bytes = slots * 2; return true;
-        case ASX_PLAN_ARRAY_PERM: *ptr = m.perm, *bytes = slots * 4; return true;
-        case ASX_PLAN_ARRAY_TILE_WORDS: *ptr = m.tile_info, *bytes = (size_t)m.ntiles * 8; return true;
+        case ASX_PLAN_ARRAY_PERM: *ptr = m.perm, *bytes = slots * 4; return m.perm != nullptr;
+        case ASX_PLAN_ARRAY_TILE_WORDS: *ptr = m.tile_info, *bytes = (size_t)m.ntiles * 16; return true;
         case ASX_PLAN_ARRAY_WORKGROUPS: *ptr = m.chains, *bytes = (size_t)m.nchains * 8; return true;
         case ASX_PLAN_ARRAY_BLOCKS: *ptr = m.blocks, *bytes = (size_t)m.nblocks * 16; return true;
         case ASX_PLAN_ARRAY_PIECES: *ptr = m.pieces, *bytes = (size_t)m.npieces * 16; return true;
@@ -1002,6 +1014,7 @@ int64_t asx_plan_info(const asx_plan *plan, int what)
     case ASX_PLAN_INFO_WORKGROUPS: return sliced ? plan->sliced.nwg : window ? plan->window.nchains : -1;
     case ASX_PLAN_INFO_PIECES: return window ? plan->window.npieces : -1;
     case ASX_PLAN_INFO_STACKED_ROWS: return window ? plan->window.stack_rows : -1;
+    case ASX_PLAN_INFO_BY_REFERENCE: return window ? plan->window.by_reference : -1;
     default: return -1;
     }
 }

@@ -125,6 +125,22 @@ __device__ __forceinline__ T wave_shift_up1(T v)
     return dpp0<0x138, 0xF>(v);
 }
 
+// value of one lane (a constant), in every lane
+template <typename T>
+__device__ __forceinline__ T wave_readlane(T v, int lane);
+template <>
+__device__ __forceinline__ float wave_readlane<float>(float v, int lane)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+template <>
+__device__ __forceinline__ double wave_readlane<double>(double v, int lane)
+{
+    const int lo = __builtin_amdgcn_readlane(__double2loint(v), lane);
+    const int hi = __builtin_amdgcn_readlane(__double2hiint(v), lane);
+    return __hiloint2double(hi, lo);
+}
+
 template <typename T>
 __device__ __forceinline__ T fma_t(T a, T b, T c);
 template <>

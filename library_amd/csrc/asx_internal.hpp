@@ -184,25 +184,29 @@ struct WindowMatrix {
     int32_t nbands;          // 1: one window per block; 2..kWindowBands: bands of diagonals
     int32_t stack_rows;      // > 0: three bands on stacked planes of this many rows, the blocks stored column by column
     int has_carry;           // some tile starts inside a row: the ordered carry pass is needed
-    void *store;             // one allocation: val, perm, cf, tile_info
+    int by_reference;        // every row holds two stored elements or more: the stored elements of a tile are consecutive in
+                             // A's val, which the kernel reads in place (no val, no perm)
+    void *store;             // one allocation: val, perm (unless by_reference), cf, tile_info
     void *tables;            // one allocation: blocks, pieces, chains
     void *val;               // ntiles * kSlicedTile values (a copy of A's; pads are 0)
     void *carry;             // ntiles values: the carries of one call, for callers that bring no buffer (null once released)
     uint16_t *cf;            // ntiles * kSlicedTile: LDS slot of the column, bit 15 = first slot of a row (or tile)
     int32_t *perm;           // where each stored copy comes from in A's val (-1 for pads)
-    int32_t *tile_info;      // ntiles x 2: row of the tile's first slot (bit 31: the tile starts inside it), rows in the tile
+    int32_t *tile_info;      // ntiles x 4: row of the tile's first slot (bit 31: the tile starts inside it), rows in the tile,
+                             // by_reference: index of the tile's first stored element in A's val, stored elements in the tile
     int32_t *blocks;         // nblocks x 4: first tile, end tile, first piece, end piece
     int32_t *pieces;         // x 4: columns of x to fetch before a block (from, to), first LDS slot and size of their ring
     int32_t *chains;         // nchains x 2: first block, end block
 };
+// in_place: where no row holds fewer than two stored elements, keep no copy of the values and read A's in every call
 template <typename T>
-int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const int32_t *row_ptr, const int32_t *col,
-                 const T *val, WindowMatrix *out, hipStream_t s);
+int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, bool in_place, const int32_t *row_ptr,
+                 const int32_t *col, const T *val, WindowMatrix *out, hipStream_t s);
 void free_window(WindowMatrix *p);
 template <typename T>
 int window_update_values(const WindowMatrix *wm, const T *val, hipStream_t s, const unsigned long long *unless_equal = nullptr);
 template <typename T>
-int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, T *carry,
+int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *val, const T *x, T beta, T *y, T *carry,
                        hipStream_t s);
 inline size_t window_scratch_bytes(const WindowMatrix *wm, size_t sv) { return wm->has_carry ? (size_t)wm->ntiles * sv : 0; }
 

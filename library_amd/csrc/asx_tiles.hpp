@@ -18,6 +18,14 @@ __host__ __device__ __forceinline__ int tile_val_pos(int e)
     return e;  // one load of 4 floats
 }
 
+// Where the column | flag word of the tile's p-th slot (in the order of A's stored elements) lies
+// in a tile whose lanes hold two pairs of consecutive slots, 2 lane .. 2 lane + 1 and
+// 128 + 2 lane .. 128 + 2 lane + 1 (tile_reduce_halves): the lane's four words are consecutive.
+__host__ __device__ __forceinline__ int tile_halves_pos(int p)
+{
+    return ((p & 127) >> 1) * 4 + (p >> 7) * 2 + (p & 1);
+}
+
 template <typename T>
 struct TileValues;
 template <>
@@ -99,6 +107,43 @@ __device__ __forceinline__ int tile_reduce(const Tile<T> &tl, int lane, const T 
     hb += f2;
     emit(f3, hb - 1, (f0 | f1 | f2) ? r2 : cin + r2);
     emit(lane == kWave - 1, total - 1, open);
+    return total;
+}
+
+// tile_reduce for a tile whose lane l holds slots 2l, 2l + 1 (c01, v[0..1]) and 128 + 2l,
+// 128 + 2l + 1 (c23, v[2..3]): two 16-byte loads per lane that each read 1 KiB of consecutive
+// values, where four consecutive doubles a lane would take two loads that each skip every other
+// 16 bytes.  The halves are summed side by side (two scans over the wave, independent of one
+// another); the run that the first half leaves open goes on through the lanes of the second half
+// below its first run start.  Same calls of `emit`, same return value.
+template <typename T, typename Emit>
+__device__ __forceinline__ int tile_reduce_halves(const Tile<T> &tl, int lane, const T *xs, Emit emit)
+{
+    const bool f0 = (tl.c01 >> 15) & 1, f1 = tl.c01 >> 31, f2 = (tl.c23 >> 15) & 1, f3 = tl.c23 >> 31;
+    const T p0 = tl.v[0] * xs[tl.c01 & 0x7fff], p1 = tl.v[1] * xs[(tl.c01 >> 16) & 0x7fff];
+    const T p2 = tl.v[2] * xs[tl.c23 & 0x7fff], p3 = tl.v[3] * xs[(tl.c23 >> 16) & 0x7fff];
+    const T r1 = f1 ? p1 : p0 + p1;
+    const T r3 = f3 ? p3 : p2 + p3;
+    const unsigned long long m0 = __ballot(f0), m1 = __ballot(f1), m2 = __ballot(f2), m3 = __ballot(f3);
+    const int first_half = __popcll(m0) + __popcll(m1);  // run starts in slots 0 .. 127
+    const int total = first_half + __popcll(m2) + __popcll(m3);
+    // per half: sum of the run that is open at the end of each lane's pair, over the lanes it spans
+    // (lane 0 of the second half counts as a start: nothing of that half lies below it)
+    const T open0 = wave_segsum_dpp<T>(r1, f0 | f1);
+    const T open1 = wave_segsum_dpp<T>(r3, f2 | f3 | (lane == 0));
+    const T left = wave_readlane<T>(open0, kWave - 1);  // what the first half leaves open
+    const bool joined = lanes_below(m2 | m3) == 0;      // no run starts in the second half below this lane
+    const T cin0 = wave_shift_up1<T>(open0);
+    const T cin1 = wave_shift_up1<T>(open1) + (joined ? left : T(0));
+    int hb = lanes_below(m0) + lanes_below(m1);
+    emit(f0 && hb > 0, hb - 1, cin0);
+    hb += f0;
+    emit(f1, hb - 1, f0 ? p0 : cin0 + p0);
+    hb = first_half + lanes_below(m2) + lanes_below(m3);  // >= 1: a tile starts with a run start
+    emit(f2, hb - 1, cin1);
+    hb += f2;
+    emit(f3, hb - 1, f2 ? p2 : cin1 + p2);
+    emit(lane == kWave - 1, total - 1, joined && !(f2 | f3) ? open1 + left : open1);
     return total;
 }
 

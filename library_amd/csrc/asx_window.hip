@@ -38,6 +38,7 @@ namespace {
 constexpr int32_t kNoCol = 0x7fffffff;
 constexpr int kWindowCols = 16384;    // ring size in columns: 128 KiB of fp64, 64 KiB of fp32
 constexpr int kWindowSlack = 8;       // a block's window is kept this much narrower (aligned fetches)
+constexpr int kFetchCols = 8192;     // columns of x a block past the first of its chain may fetch
 constexpr int kWindowWaves = 16;
 constexpr int32_t kAlignRowLen = 16;  // rows up to this length are not cut by tile starts
 constexpr int32_t kMinRowSlots = 2;   // slots a row takes at least
@@ -52,17 +53,21 @@ constexpr int window_depth(int rings, bool beta)
 constexpr int kSpanGroup = 128;  // rows per group of the column-span table; every block size is a multiple
 
 // first and last column of every group of kSpanGroup consecutive rows (gmin = kNoCol, gmax = -1 for
-// a group without stored elements); one wave per group reads the group's columns in order
+// a group without stored elements); one wave per group reads the group's columns in order.
+// *any_short (preset to 0) becomes 1 when a row holds fewer than kMinRowSlots stored elements.
 __global__ __launch_bounds__(kBlock) void k_window_group_span(const int32_t *__restrict__ row_ptr,
                                                               const int32_t *__restrict__ col, int32_t m,
                                                               int32_t ngroups, int32_t *__restrict__ gmin,
-                                                              int32_t *__restrict__ gmax)
+                                                              int32_t *__restrict__ gmax, int32_t *__restrict__ any_short)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t g = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
     if (g >= ngroups) return;  // whole waves leave
     int32_t lo = kNoCol, hi = -1;
     const int64_t r1 = (g + 1) * kSpanGroup < m ? (g + 1) * kSpanGroup : m;
+    bool is_short = false;  // a row of fewer than kMinRowSlots stored elements: it will be padded
+    for (int64_t r = g * kSpanGroup + lane; r < r1; r += kWave) is_short |= row_ptr[r + 1] - row_ptr[r] < kMinRowSlots;
+    if (is_short) *any_short = 1;
     for (int32_t k = row_ptr[g * kSpanGroup] + lane, end = row_ptr[r1]; k < end; k += kWave) {
         const int32_t c = col[k];
         lo = c < lo ? c : lo;
@@ -168,7 +173,7 @@ __global__ __launch_bounds__(kBlock) void k_window_pads(const int32_t *__restric
                                                         const int32_t *__restrict__ tile_off,
                                                         const int32_t *__restrict__ block_tiles, uint16_t pad,
                                                         uint16_t *__restrict__ cf, T *__restrict__ val,
-                                                        int32_t *__restrict__ perm)
+                                                        int32_t *__restrict__ perm, bool halves)
 {
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= m) return;
@@ -182,9 +187,12 @@ __global__ __launch_bounds__(kBlock) void k_window_pads(const int32_t *__restric
     for (int32_t o = from; o < to; ++o) {
         const int64_t d = base + o;
         const int64_t phys = d / kSlicedTile * kSlicedTile + tile_val_pos<T>((int)(d % kSlicedTile));
-        cf[d] = o < own && o > row_start[r] ? (uint16_t)(pad & 0x7fff) : pad;
-        val[phys] = T(0);
-        perm[phys] = -1;
+        cf[halves ? d / kSlicedTile * kSlicedTile + tile_halves_pos((int)(d % kSlicedTile)) : d] =
+            o < own && o > row_start[r] ? (uint16_t)(pad & 0x7fff) : pad;
+        if (val) {  // uniform: no copy of the values when the kernel reads A's in place
+            val[phys] = T(0);
+            perm[phys] = -1;
+        }
     }
 }
 
@@ -282,7 +290,7 @@ __global__ __launch_bounds__(kBlock) void k_window_place(const int32_t *__restri
                                                          const int32_t *__restrict__ seg_row,
                                                          const int32_t *__restrict__ row_start,
                                                          const int32_t *__restrict__ tile_off, uint16_t *__restrict__ cf,
-                                                         T *__restrict__ val_out, int32_t *__restrict__ perm)
+                                                         T *__restrict__ val_out, int32_t *__restrict__ perm, bool halves)
 {
     __shared__ int32_t s_rp[kBlock + 1];
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -307,21 +315,27 @@ __global__ __launch_bounds__(kBlock) void k_window_place(const int32_t *__restri
     } else {
         slot = bands.base[k] + c % bands.width[k];
     }
-    cf[d] = (uint16_t)(slot | (head ? 0x8000 : 0));
-    const int64_t phys = d / kSlicedTile * kSlicedTile + tile_val_pos<T>((int)(d % kSlicedTile));
-    val_out[phys] = val[i];
-    perm[phys] = (int32_t)i;
+    cf[halves ? d / kSlicedTile * kSlicedTile + tile_halves_pos((int)(d % kSlicedTile)) : d] = (uint16_t)(slot | (head ? 0x8000 : 0));
+    if (val_out) {  // uniform
+        const int64_t phys = d / kSlicedTile * kSlicedTile + tile_val_pos<T>((int)(d % kSlicedTile));
+        val_out[phys] = val[i];
+        perm[phys] = (int32_t)i;
+    }
 }
 
 // per tile: x = the row its first slot belongs to, bit 31 set when the tile starts inside that
-// row; y = the number of runs of the tile that are rows (the slots behind them are padding).
+// row; y = the number of runs of the tile that are rows (the slots behind them are padding); where
+// no row is padded (every row holds kMinRowSlots stored elements or more) the stored elements of a
+// tile are consecutive in A: z = the index of the first, w = how many (the tile's other slots,
+// behind them, are padding).
 // The blocks are stored in the order the chains walk them: stored_off[i] = first tile of the i-th
 // stored block, which holds the rows of block order[i] (of block i without an order).
 __global__ __launch_bounds__(kBlock) void k_window_tile_info(const int32_t *__restrict__ row_start, int32_t m,
                                                              int32_t rows, int32_t nblocks,
                                                              const int32_t *__restrict__ stored_off,
                                                              const int32_t *__restrict__ order, int32_t ntiles,
-                                                             int2 *__restrict__ tile_info, int32_t *__restrict__ any_cont)
+                                                             const int32_t *__restrict__ row_ptr,
+                                                             int4 *__restrict__ tile_info, int32_t *__restrict__ any_cont)
 {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= ntiles) return;
@@ -354,7 +368,9 @@ __global__ __launch_bounds__(kBlock) void k_window_tile_info(const int32_t *__re
             v = mid;
     }
     const bool cont = row_start[a] != o;
-    tile_info[t] = make_int2(a | (cont ? (int32_t)0x80000000 : 0), u - a);
+    const int32_t first = row_ptr[a] + (o - row_start[a]);
+    const int32_t end = row_start[u - 1] + (row_ptr[u] - row_ptr[u - 1]) - o;  // end of the last row's stored elements
+    tile_info[t] = make_int4(a | (cont ? (int32_t)0x80000000 : 0), u - a, first, end < kSlicedTile ? end : kSlicedTile);
     if (cont) *any_cont = 1;
 }
 
@@ -436,16 +452,50 @@ struct WindowTile : Tile<T> {
     int32_t limit;             // base, limit: the tile's two words, uniform
     T yv[kStageRows / kWave];  // BETA: y in rows (first row) + lane + 64 k
 };
-// the loads of tile t, whose words are `info`
-template <typename T, bool BETA>
-__device__ __forceinline__ void window_tile_load(WindowTile<T, BETA> &tl, int32_t t, int2 info, int lane,
+// A tile's four values per lane, read in place from A's val: the tile's stored elements are
+// `count` consecutive ones from `first` on (no row of the plan is padded), and what lies past them
+// is padding, which the buffer's range check reads as 0.  fp32: lane l holds the 4l-th to the
+// (4l+3)-th; fp64: the 2l-th, the next, the (128+2l)-th and the next (tile_reduce_halves).
+template <typename T>
+struct ValuesInPlace;
+template <>
+struct ValuesInPlace<double> {
+    static __device__ __forceinline__ void load(const double *val, int32_t first, int32_t count, int lane, double v[4])
+    {
+        typedef double f64x2 __attribute__((ext_vector_type(2)));
+        const __amdgpu_buffer_rsrc_t r =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<double *>(val) + first, 0, count * (int32_t)sizeof(double), 0x00020000);
+        // slots 2 lane, 2 lane + 1 and 128 + 2 lane, 128 + 2 lane + 1: each load reads 1 KiB of consecutive values
+        const f64x2 a = __builtin_bit_cast(f64x2, __builtin_amdgcn_raw_buffer_load_b128(r, (uint32_t)lane * 16u, 0, 2));
+        const f64x2 b = __builtin_bit_cast(f64x2, __builtin_amdgcn_raw_buffer_load_b128(r, 1024u + (uint32_t)lane * 16u, 0, 2));
+        v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
+    }
+};
+template <>
+struct ValuesInPlace<float> {
+    static __device__ __forceinline__ void load(const float *val, int32_t first, int32_t count, int lane, float v[4])
+    {
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        const __amdgpu_buffer_rsrc_t r =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(val) + first, 0, count * (int32_t)sizeof(float), 0x00020000);
+        const f32x4 a = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (uint32_t)lane * 16u, 0, 2));
+        v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w;
+    }
+};
+
+// the loads of tile t, whose words are `info`; INPLACE: the values from A's val, else from the plan's copy
+template <typename T, bool BETA, bool INPLACE>
+__device__ __forceinline__ void window_tile_load(WindowTile<T, BETA> &tl, int32_t t, int4 info, int lane,
                                                  const uint16_t *__restrict__ cf, const T *__restrict__ val, T *y)
 {
     typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
     const u32x2 cw = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(cf + (int64_t)t * kSlicedTile) + lane);
     tl.c01 = cw.x;
     tl.c23 = cw.y;
-    TileValues<T>::load(val + (int64_t)t * kSlicedTile, lane, tl.v);
+    if (INPLACE)
+        ValuesInPlace<T>::load(val, info.z, info.w, lane, tl.v);
+    else
+        TileValues<T>::load(val + (int64_t)t * kSlicedTile, lane, tl.v);
     tl.base = info.x;
     tl.limit = info.y;
     if (BETA) {
@@ -470,22 +520,25 @@ template <typename T>
 struct WindowStep {
     const uint16_t *__restrict__ cf;
     const T *__restrict__ val;
-    const int2 *__restrict__ tile_info;
+    const int4 *__restrict__ tile_info;
     T *y, *carry;
     const T *xs;
     T *stage;
     T alpha, beta;
     int32_t chain_last;
     int lane;
-    int2 info_next;  // the words of the tile the next step will request
+    int4 info_next;  // the words of the tile the next step will request
 };
 // One tile: its rows' sums into the staging area and from there to y, then the loads of the tile
 // `ahead` tiles further on (past the end of the chain: the last tile again) into the registers this
 // one has just left, and the words of the tile after that.
-template <typename T, bool BETA>
+template <typename T, bool BETA, bool INPLACE>
 __device__ __forceinline__ void window_step(WindowTile<T, BETA> &tl, int32_t t, int32_t ahead, int32_t stride, WindowStep<T> &w)
 {
-    tile_reduce<T>(tl, w.lane, w.xs, StageRows<T>{w.stage, w.lane});
+    if (INPLACE && sizeof(T) == 8)
+        tile_reduce_halves<T>(tl, w.lane, w.xs, StageRows<T>{w.stage, w.lane});
+    else
+        tile_reduce<T>(tl, w.lane, w.xs, StageRows<T>{w.stage, w.lane});
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the wave's LDS writes and reads execute in order
     __builtin_amdgcn_wave_barrier();
     const int32_t row0 = tl.base & 0x7fffffff, limit = tl.limit;
@@ -504,20 +557,20 @@ __device__ __forceinline__ void window_step(WindowTile<T, BETA> &tl, int32_t t, 
     if (cont) w.carry[t] = w.stage[0];  // uniform; every lane stores the same value
     __builtin_amdgcn_wave_barrier();
     const int32_t t1 = t + ahead < w.chain_last ? t + ahead : w.chain_last;
-    window_tile_load<T, BETA>(tl, t1, w.info_next, w.lane, w.cf, w.val, w.y);
+    window_tile_load<T, BETA, INPLACE>(tl, t1, w.info_next, w.lane, w.cf, w.val, w.y);
     const int32_t t2 = t + ahead + stride < w.chain_last ? t + ahead + stride : w.chain_last;
     w.info_next = w.tile_info[t2];
 }
 // `cnt` tiles of one wave in turn, the first in buffer P; a loop of its own for every P, with one
 // way out (a loop left from the middle is rebuilt with flags too), so that on every path through
 // it a buffer is used D - 1 steps after it was requested
-template <typename T, bool BETA, int D, int NW, int P>
+template <typename T, bool BETA, bool INPLACE, int D, int NW, int P>
 __device__ __forceinline__ void window_steps(WindowTile<T, BETA> (&tl)[D], int32_t &t, int32_t cnt, WindowStep<T> &w)
 {
     for (int32_t i = cnt / D; i > 0; --i) {
 #pragma unroll
         for (int j = 0; j < D; ++j) {
-            window_step<T, BETA>(tl[(P + j) % D], t, D * NW, NW, w);
+            window_step<T, BETA, INPLACE>(tl[(P + j) % D], t, D * NW, NW, w);
             t += NW;
         }
     }
@@ -525,7 +578,7 @@ __device__ __forceinline__ void window_steps(WindowTile<T, BETA> (&tl)[D], int32
 #pragma unroll
     for (int j = 0; j + 1 < D; ++j) {
         if (j < rest) {
-            window_step<T, BETA>(tl[(P + j) % D], t, D * NW, NW, w);
+            window_step<T, BETA, INPLACE>(tl[(P + j) % D], t, D * NW, NW, w);
             t += NW;
         }
     }
@@ -538,18 +591,23 @@ __device__ __forceinline__ void window_steps(WindowTile<T, BETA> (&tl)[D], int32
 // by word, so a unit may straddle the end, and x needs no more than the alignment of its elements.
 // With several pieces (NB > 1) every piece starts at a multiple of 64 units: the 64 lanes of a wave
 // then work on one piece, and which one is found with scalar compares; the builder keeps the
-// pieces of a block, each rounded up to 64 units, within what the registers hold (kWindowCols
-// columns).  NB = 1: one piece, ring of kWindowCols slots from slot 0 (constant modulus).
+// pieces of a block, each rounded up to 64 units, within what the registers hold: kFetchCols
+// columns a round.  The first block of a chain, which fetches whole windows, takes as many rounds as
+// it needs; every other block's pieces fit one (the builder starts a new chain otherwise), so the
+// registers that carry x through a block are half of what a whole window would take.
+// NB = 1: one piece, ring of kWindowCols slots from slot 0 (constant modulus).
 template <typename T, int THREADS, int NB>
 struct XFetch {
     static constexpr int V = 16 / sizeof(T);
-    static constexpr int PER = kWindowCols / (THREADS * V);
+    static constexpr int PER = kFetchCols / (THREADS * V);
+    static constexpr int kRound = PER * THREADS;  // units a round moves
     typedef T vec_t __attribute__((ext_vector_type(V)));
     typedef uint32_t bits_t __attribute__((ext_vector_type(4)));
     vec_t buf[PER];
     // the pending fetch (uniform values): its pieces, the first unit of each, the ring slot of its
     // first column and how many of its columns lie inside x
     int32_t from[NB], len[NB], inside[NB], base[NB], width[NB], ustart[NB], fslot[NB];
+    int32_t units;  // of the pending fetch, the padding between its pieces included
 
     __device__ __forceinline__ void set(const int4 *__restrict__ pieces, int32_t lo, int32_t hi, int32_t n)
     {
@@ -569,6 +627,7 @@ struct XFetch {
             u += (len[q] + V - 1) / V;
             if (NB > 1) u = (u + kWave - 1) & ~(kWave - 1);
         }
+        units = u;
     }
     // the piece the 64 units from `first_unit` on belong to (all values uniform)
     struct Piece {
@@ -590,23 +649,24 @@ struct XFetch {
         }
         return p;
     }
-    __device__ __forceinline__ void load(const T *__restrict__ x, int wave)
+    // round `u0 / kRound` of the pending fetch: units u0 .. u0 + kRound - 1
+    __device__ __forceinline__ void load(const T *__restrict__ x, int wave, int32_t u0 = 0)
     {
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
-            const Piece p = piece_of(k * THREADS + wave * kWave);
-            const int32_t u = k * THREADS + (int)threadIdx.x - p.ustart;  // unit inside the piece
+            const Piece p = piece_of(u0 + k * THREADS + wave * kWave);
+            const int32_t u = u0 + k * THREADS + (int)threadIdx.x - p.ustart;  // unit inside the piece
             const __amdgpu_buffer_rsrc_t cols =
                 __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(x) + p.from, 0, p.inside * (int32_t)sizeof(T), 0x00020000);
             buf[k] = __builtin_bit_cast(vec_t, __builtin_amdgcn_raw_buffer_load_b128(cols, (uint32_t)u * 16u, 0, 0));
         }
     }
-    __device__ __forceinline__ void store(T *xs, int wave) const
+    __device__ __forceinline__ void store(T *xs, int wave, int32_t u0 = 0) const
     {
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
-            const Piece p = piece_of(k * THREADS + wave * kWave);
-            const int32_t e = (k * THREADS + (int)threadIdx.x - p.ustart) * V;  // column inside the piece
+            const Piece p = piece_of(u0 + k * THREADS + wave * kWave);
+            const int32_t e = (u0 + k * THREADS + (int)threadIdx.x - p.ustart) * V;  // column inside the piece
             if (e < p.len) {
                 const int32_t sl = p.fslot + e;  // a piece is no longer than its ring: one wrap at most
                 *reinterpret_cast<vec_t *>(xs + p.base + (sl >= p.width ? sl - p.width : sl)) = buf[k];
@@ -615,12 +675,12 @@ struct XFetch {
     }
 };
 
-template <typename T, int NW, int NB, int D, bool BETA>
+template <typename T, int NW, int NB, int D, bool BETA, bool INPLACE>
 __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T beta, const int2 *__restrict__ chains,
                                                            const int4 *__restrict__ blocks,
                                                            const int4 *__restrict__ pieces,
                                                            const uint16_t *__restrict__ cf, const T *__restrict__ val,
-                                                           const int2 *__restrict__ tile_info,
+                                                           const int4 *__restrict__ tile_info,
                                                            const T *__restrict__ x, T *y, T *__restrict__ carry)
 {
     static_assert(D >= 1 && D <= 3, "one loop per starting buffer is written out for up to three buffers");
@@ -631,7 +691,7 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
     // the wave's number as a scalar: the tile counters and every loop condition below are uniform
     const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     WindowStep<T> w{cf, val, tile_info, y, carry, xs, stage_all + wave * kStageSlots, alpha, beta,
-                    blocks[chain.y - 1].y - 1, lane, make_int2(0, 0)};
+                    blocks[chain.y - 1].y - 1, lane, make_int4(0, 0, 0, 0)};
     // this wave's tiles are those congruent to its number, across the blocks of the chain; D are
     // in flight (requested D steps ahead; past the end of the chain the last tile is re-read)
     WindowTile<T, BETA> tl[D];
@@ -639,25 +699,26 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
 #pragma unroll
     for (int d = 0; d < D; ++d) {
         const int32_t td = t + d * NW < w.chain_last ? t + d * NW : w.chain_last;
-        window_tile_load<T, BETA>(tl[d], td, tile_info[td], lane, cf, val, y);
+        window_tile_load<T, BETA, INPLACE>(tl[d], td, tile_info[td], lane, cf, val, y);
     }
     w.info_next = tile_info[t + D * NW < w.chain_last ? t + D * NW : w.chain_last];
     if (threadIdx.x == 0) xs[kWindowCols] = T(0);
     XFetch<T, NW * kWave, NB> xf;
     int4 blk = blocks[chain.x];  // first tile, end tile, pieces of x to fetch before the block: first, end
+    // the first block's columns (whole windows), a round of registers at a time
     xf.set(pieces, blk.z, blk.w, n);
-    xf.load(x, wave);
+    for (int32_t u0 = 0; u0 < xf.units; u0 += xf.kRound) {
+        xf.load(x, wave, u0);
+        xf.store(xs, wave, u0);
+    }
     int32_t first = 0;  // the buffer that holds the wave's next tile
-    // Every wave passes the start of every block of the chain (the barriers count all waves),
-    // whether it has tiles in the block or not.  All conditions are uniform over the wave.
+    // Every wave passes the start and the end of every block of the chain (the barriers count all
+    // waves), whether it has tiles in the block or not.  All conditions are uniform over the wave.
     for (int32_t b = chain.x; b < chain.y; ++b) {
-        // the columns fetched for the block go into the ring once every wave is done with the block
-        // before; the next block's new columns are fetched while this one is multiplied
-        __syncthreads();
-        xf.store(xs, wave);
-        __syncthreads();
+        __syncthreads();  // the block's columns are in the rings
         const int32_t tile_hi = blk.y;
-        if (b + 1 < chain.y) {
+        const bool more = b + 1 < chain.y;
+        if (more) {  // the next block's new columns are fetched while this one is multiplied
             blk = blocks[b + 1];
             xf.set(pieces, blk.z, blk.w, n);
             xf.load(x, wave);
@@ -665,19 +726,21 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
         const int32_t cnt = t < tile_hi ? (tile_hi - t + NW - 1) / NW : 0;  // this wave's tiles in the block
         // the D tile buffers take turns without changing places
         if (D == 1 || first == 0)
-            window_steps<T, BETA, D, NW, 0>(tl, t, cnt, w);
+            window_steps<T, BETA, INPLACE, D, NW, 0>(tl, t, cnt, w);
         else if (D == 2 || first == 1)
-            window_steps<T, BETA, D, NW, 1 % D>(tl, t, cnt, w);
+            window_steps<T, BETA, INPLACE, D, NW, 1 % D>(tl, t, cnt, w);
         else
-            window_steps<T, BETA, D, NW, 2 % D>(tl, t, cnt, w);
+            window_steps<T, BETA, INPLACE, D, NW, 2 % D>(tl, t, cnt, w);
         first = (first + cnt) % D;
+        __syncthreads();  // every wave is done with the block: its columns may go
+        if (more) xf.store(xs, wave);
     }
 }
 
 // Adds the carries to their rows, in tile order: the thread of the first tile of a run of tiles
 // that start inside the same row sums the run's carries and adds the total once.
 template <typename T>
-__global__ __launch_bounds__(kBlock) void k_window_fixup(int32_t ntiles, T alpha, const int2 *__restrict__ tile_info,
+__global__ __launch_bounds__(kBlock) void k_window_fixup(int32_t ntiles, T alpha, const int4 *__restrict__ tile_info,
                                                          const T *__restrict__ carry, T *__restrict__ y)
 {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -703,8 +766,8 @@ void free_window(WindowMatrix *p)
 }
 
 template <typename T>
-int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const int32_t *row_ptr, const int32_t *col,
-                 const T *val, WindowMatrix *out, hipStream_t s)
+int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, bool in_place, const int32_t *row_ptr,
+                 const int32_t *col, const T *val, WindowMatrix *out, hipStream_t s)
 {
     WindowMatrix wm{};
     if (m <= 0 || nnz <= 0 || n <= 0) return ASX_STATUS_INVALID_SIZE;
@@ -715,7 +778,7 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     int32_t *bmin = nullptr, *bmax = nullptr, *btiles = nullptr, *tile_off = nullptr, *d_small = nullptr;
     std::vector<int32_t> h_bmin, h_bmax, h_bt, h_off, h_soff, h_order, blk, pcs, chains;
     int64_t stack_ulo = 0, stack_uhi = 0;
-    bool stacked = false;
+    bool stacked = false, halves = false;
     std::vector<uint32_t> h_bits;
     uint32_t *d_bits = nullptr;
     BandTable bands{};
@@ -747,11 +810,11 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     }
 
     // 1. column span of every group of rows
+    hipLaunchKernelGGL(k_window_fill_i32, dim3(1), dim3(kBlock), 0, s, d_small, (int64_t)16, 0);
     hipLaunchKernelGGL(k_window_group_span, dim3((unsigned)ceil_div64((int64_t)ngroups * kWave, kBlock)), dim3(kBlock), 0, s,
-                       row_ptr, col, m, ngroups, gmin, gmax);
+                       row_ptr, col, m, ngroups, gmin, gmax, d_small + 13);
     // 2. the largest block of rows whose widest window fits the ring: the widest window of every
     //    candidate size, all read back at once
-    hipLaunchKernelGGL(k_window_fill_i32, dim3(1), dim3(kBlock), 0, s, d_small, (int64_t)16, 0);
     for (int k = 0; k < kCandidates; ++k) {
         const int32_t rows = kBlockRows[k];
         if (rows > 256 && ceil_div64(m, rows) < min_blocks) continue;  // too few blocks to share out
@@ -761,8 +824,13 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     }
     st = launch_nnz_split_rows(row_ptr, m, nnz, kBlock, seg_row, s);  // for step 4; runs while the host waits
     if (st) goto done;
-    ASX_TRY(hipMemcpyAsync(h_small, d_small, sizeof(int32_t) * kCandidates, hipMemcpyDeviceToHost, s));
+    ASX_TRY(hipMemcpyAsync(h_small, d_small, sizeof(int32_t) * 14, hipMemcpyDeviceToHost, s));
     ASX_TRY(hipStreamSynchronize(s));
+    // no row shorter than kMinRowSlots: no slot between the stored elements of a tile is padding, and
+    // the kernel can read A's values in place; fp64 ones two 16-byte loads a lane, a pair of slots
+    // from either half of the tile (tile_reduce_halves; the lane's four column words lie together)
+    wm.by_reference = in_place && h_small[13] == 0;
+    halves = wm.by_reference && sizeof(T) == 8;
     wm.rows_per_block = 0;
     for (int k = 0; k < kCandidates; ++k) {
         const int32_t rows = kBlockRows[k];
@@ -950,27 +1018,29 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
         ASX_TRY(hipMemcpyAsync(bmin, h_soff.data(), sizeof(int32_t) * h_soff.size(), hipMemcpyHostToDevice, s));
         ASX_TRY(hipMemcpyAsync(bmax, h_order.data(), sizeof(int32_t) * h_order.size(), hipMemcpyHostToDevice, s));
     }
-    {   // the regrouped copy in one allocation
-        const size_t o_val = 0, o_perm = align_up(sizeof(T) * (size_t)slots, 256);
-        const size_t o_cf = o_perm + align_up(sizeof(int32_t) * (size_t)slots, 256);
+    {   // the regrouped copy in one allocation (values and their source indices only when they are copied)
+        const size_t o_val = 0, o_perm = wm.by_reference ? 0 : align_up(sizeof(T) * (size_t)slots, 256);
+        const size_t o_cf = o_perm + (wm.by_reference ? 0 : align_up(sizeof(int32_t) * (size_t)slots, 256));
         const size_t o_info = o_cf + align_up(sizeof(uint16_t) * (size_t)slots, 256);
-        ASX_TRY(hipMalloc(&wm.store, o_info + sizeof(int2) * (size_t)wm.ntiles));
+        ASX_TRY(hipMalloc(&wm.store, o_info + sizeof(int4) * (size_t)wm.ntiles));
         char *base = static_cast<char *>(wm.store);
-        wm.val = base + o_val, wm.perm = (int32_t *)(base + o_perm), wm.cf = (uint16_t *)(base + o_cf);
+        wm.val = wm.by_reference ? nullptr : base + o_val;
+        wm.perm = wm.by_reference ? nullptr : (int32_t *)(base + o_perm);
+        wm.cf = (uint16_t *)(base + o_cf);
         wm.tile_info = (int32_t *)(base + o_info);
     }
     ASX_TRY(hipMalloc(&wm.carry, sizeof(T) * (size_t)wm.ntiles));
     // 4. every stored element to its slot; every other slot becomes a zero that points at the zero
     //    behind the rings and opens a run of its own
     hipLaunchKernelGGL((k_window_place<T>), dim3((unsigned)ceil_div64(nnz, kBlock)), dim3(kBlock), 0, s, row_ptr, col, val,
-                       m, n, nnz, wm.rows_per_block, bands, seg_row, row_start, tile_off, wm.cf, (T *)wm.val, wm.perm);
+                       m, n, nnz, wm.rows_per_block, bands, seg_row, row_start, tile_off, wm.cf, (T *)wm.val, wm.perm, halves);
     hipLaunchKernelGGL((k_window_pads<T>), dim3(mgrid), dim3(kBlock), 0, s, row_ptr, m, wm.rows_per_block, row_start, tile_off,
-                       btiles, (uint16_t)(0x8000 | kWindowCols), wm.cf, (T *)wm.val, wm.perm);
+                       btiles, (uint16_t)(0x8000 | kWindowCols), wm.cf, (T *)wm.val, wm.perm, halves);
     // 5. first row and number of rows of every tile
     hipLaunchKernelGGL(k_window_fill_i32, dim3(1), dim3(kBlock), 0, s, d_small, (int64_t)2, 0);
     hipLaunchKernelGGL(k_window_tile_info, dim3((unsigned)ceil_div64(wm.ntiles, kBlock)), dim3(kBlock), 0, s, row_start, m,
                        wm.rows_per_block, wm.nblocks, stacked ? bmin : tile_off, stacked ? bmax : (int32_t *)nullptr,
-                       wm.ntiles, (int2 *)wm.tile_info, d_small);
+                       wm.ntiles, row_ptr, (int4 *)wm.tile_info, d_small);
     ASX_TRY(hipMemcpyAsync(h_small, d_small, sizeof(int32_t), hipMemcpyDeviceToHost, s));
     // 6. chains of blocks, one per workgroup, of about equal numbers of tiles.  Inside a chain a
     //    block fetches, per band, only the columns behind those already in the band's ring; a block
@@ -978,6 +1048,10 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
     //    whole windows).
     {
     const int64_t per_chain = std::max<int64_t>(1, ceil_div64(wm.ntiles, target_wgs));
+    const auto fetch_unit = [](int64_t columns) {  // several pieces: each takes whole waves of 64 16-byte units
+        constexpr int64_t unit = kWave * (16 / (int64_t)sizeof(T));
+        return (columns + unit - 1) / unit * unit;
+    };
     blk.resize((size_t)wm.nblocks * 4);
     if (stacked) {
         // A chain stays inside one column of blocks and climbs the planes.  Region g holds, for one
@@ -1043,10 +1117,15 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, const in
             }
             bool fresh = false;
             if (b != chain_lo) {
-                for (int k = 0; k < bands.nbands; ++k)  // columns never fetched in this chain, or already overwritten
+                int64_t fetch = 0;  // what the block would fetch as the chain's next one, as the kernel counts it
+                for (int k = 0; k < bands.nbands; ++k) {  // columns never fetched in this chain, or already overwritten
                     if (hi[k] > lo[k] && have[k] >= 0 &&
                         (lo[k] < low[k] || lo[k] < std::max(have[k], hi[k]) - bands.width[k] + kWindowSlack))
                         fresh = true;
+                    const int64_t piece = hi[k] <= lo[k] ? 0 : have[k] < 0 || lo[k] >= have[k] ? hi[k] - lo[k] : std::max(have[k], hi[k]) - have[k];
+                    fetch += bands.nbands > 1 ? fetch_unit(piece) : piece;
+                }
+                if (fetch > kFetchCols) fresh = true;  // more than one round of the fetch registers: only a chain's first block may
                 if (chain_tiles >= per_chain) fresh = true;
             }
             if (fresh) {
@@ -1115,7 +1194,7 @@ template <typename T>
 int window_update_values(const WindowMatrix *wm, const T *val, hipStream_t s, const unsigned long long *unless_equal)
 {
     const int64_t slots = (int64_t)wm->ntiles * kSlicedTile;
-    if (slots == 0) return ASX_STATUS_SUCCESS;
+    if (slots == 0 || wm->by_reference) return ASX_STATUS_SUCCESS;  // nothing copied: nothing to bring up to date
     // a bounded grid: where the checksums agree the kernel has nothing to do but to end
     const unsigned grid = (unsigned)std::min<int64_t>(ceil_div64(slots, kBlock), 8192);
     hipLaunchKernelGGL((k_window_regather<T>), dim3(grid), dim3(kBlock), 0, s, wm->perm, slots, val, (T *)wm->val, unless_equal);
@@ -1123,33 +1202,37 @@ int window_update_values(const WindowMatrix *wm, const T *val, hipStream_t s, co
 }
 
 template <typename T>
-int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *x, T beta, T *y, T *carry,
+int launch_spmv_window(int32_t m, int32_t n, T alpha, const WindowMatrix *wm, const T *val, const T *x, T beta, T *y, T *carry,
                        hipStream_t s)
 {
     if (m <= 0) return ASX_STATUS_SUCCESS;
     if (wm->has_carry && !carry) return ASX_STATUS_INVALID_POINTER;
-    // a kernel of its own for beta != 0, which loads y ahead with the tiles
-    const bool bands = wm->nbands != 1, b0 = beta == T(0);
-#define ASX_PICK(NB)                                                                 \
-    (b0 ? k_spmv_window<T, kWindowWaves, NB, window_depth<T>(NB, false), false>      \
-        : k_spmv_window<T, kWindowWaves, NB, window_depth<T>(NB, true), true>)
+    if (wm->by_reference && !val) return ASX_STATUS_INVALID_POINTER;
+    // kernels of their own for beta != 0 (y is loaded ahead with the tiles) and for values read in
+    // place from A's val (else from the plan's copy)
+    const bool bands = wm->nbands != 1, b0 = beta == T(0), in_place = wm->by_reference != 0;
+#define ASX_PICK2(NB, BETA) \
+    (in_place ? k_spmv_window<T, kWindowWaves, NB, window_depth<T>(NB, BETA), BETA, true> \
+              : k_spmv_window<T, kWindowWaves, NB, window_depth<T>(NB, BETA), BETA, false>)
+#define ASX_PICK(NB) (b0 ? ASX_PICK2(NB, false) : ASX_PICK2(NB, true))
     const auto kernel = bands ? ASX_PICK(kWindowBands) : ASX_PICK(1);
 #undef ASX_PICK
+#undef ASX_PICK2
     hipLaunchKernelGGL(kernel, dim3((unsigned)wm->nchains), dim3(kWindowWaves * kWave), 0, s, n, alpha, beta,
                        reinterpret_cast<const int2 *>(wm->chains), reinterpret_cast<const int4 *>(wm->blocks),
-                       reinterpret_cast<const int4 *>(wm->pieces), wm->cf, (const T *)wm->val,
-                       reinterpret_cast<const int2 *>(wm->tile_info), x, y, carry);
+                       reinterpret_cast<const int4 *>(wm->pieces), wm->cf, in_place ? val : (const T *)wm->val,
+                       reinterpret_cast<const int4 *>(wm->tile_info), x, y, carry);
     if (wm->has_carry)
         hipLaunchKernelGGL((k_window_fixup<T>), dim3((unsigned)ceil_div64(wm->ntiles, kBlock)), dim3(kBlock), 0, s,
-                           wm->ntiles, alpha, reinterpret_cast<const int2 *>(wm->tile_info), (const T *)carry, y);
+                           wm->ntiles, alpha, reinterpret_cast<const int4 *>(wm->tile_info), (const T *)carry, y);
     return check_launch();
 }
 
 #define ASX_INST(T)                                                                                               \
-    template int build_window<T>(int32_t, int32_t, int32_t, int32_t, const int32_t *, const int32_t *, const T *, \
+    template int build_window<T>(int32_t, int32_t, int32_t, int32_t, bool, const int32_t *, const int32_t *, const T *, \
                                  WindowMatrix *, hipStream_t);                                                    \
     template int window_update_values<T>(const WindowMatrix *, const T *, hipStream_t, const unsigned long long *);                           \
-    template int launch_spmv_window<T>(int32_t, int32_t, T, const WindowMatrix *, const T *, T, T *, T *, hipStream_t);
+    template int launch_spmv_window<T>(int32_t, int32_t, T, const WindowMatrix *, const T *, const T *, T, T *, T *, hipStream_t);
 ASX_INST(float)
 ASX_INST(double)
 #undef ASX_INST

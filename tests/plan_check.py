@@ -18,6 +18,7 @@ import numpy as np
 
 TILE = 256
 WINDOW_COLS = 16384
+FETCH_COLS = 8192     # columns a block past the first of its chain may fetch
 PAD_ROW = 0x7FFFFFFF
 MIN_ROW_SLOTS = 2    # slots a row takes at least in a window plan
 MAX_TILE_ROWS = 128  # so a tile of 256 slots holds at most this many rows
@@ -39,6 +40,13 @@ def val_pos(itemsize):
         lane, j = e >> 2, e & 3
         return (j >> 1) * 128 + lane * 2 + (j & 1)
     return e
+
+
+def halves_pos():
+    """Where the column word of a tile's p-th slot lies in a plan that reads fp64 values in place:
+    lane l holds slots 2l, 2l + 1, 128 + 2l, 128 + 2l + 1 and its four words lie together."""
+    p = np.arange(TILE)
+    return ((p & 127) >> 1) * 4 + (p >> 7) * 2 + (p & 1)
 
 
 def logical_order(a, itemsize):
@@ -245,12 +253,13 @@ def sliced_plan_arrays(rp, col, n, width, rows_per_wave, itemsize):
 
 # ------------------------------------------------------------------------------------- window
 def check_window(arrays, rp, col, n, rows_per_block, nbands, itemsize):
-    """arrays: perm, cf, tile_words (tiles x 2), blocks (x 4), pieces (x 4), workgroups = chains (x 2)."""
+    """arrays: perm (absent in a plan that reads A's values in place), cf, tile_words (tiles x 4),
+    blocks (x 4), pieces (x 4), workgroups = chains (x 2)."""
     rp = np.asarray(rp, np.int64)
     col = np.asarray(col, np.int64)
     m, nnz = rp.size - 1, col.size
     R = rows_per_block
-    info = np.asarray(arrays["tile_words"], np.int64).reshape(-1, 2)
+    info = np.asarray(arrays["tile_words"], np.int64).reshape(-1, 4)
     ntiles = info.shape[0]
     blocks = np.asarray(arrays["blocks"], np.int64).reshape(-1, 4)
     pieces = np.asarray(arrays["pieces"], np.int64).reshape(-1, 4)
@@ -280,15 +289,28 @@ def check_window(arrays, rp, col, n, rows_per_block, nbands, itemsize):
     _need(np.all(ring[1:, 0] >= ring[:-1, 0] + ring[:-1, 1]) and ring[-1, 0] + ring[-1, 1] <= WINDOW_COLS, "rings overlap or leave the LDS window")
     unit = 16 // itemsize * (64 if nbands > 1 else 1)  # several pieces: each starts a wave's 64 units
     fetched = (-(-(pieces[:, 1] - pieces[:, 0]) // unit) * unit).reshape(-1, nbands).sum(axis=1)
-    _need(np.all(fetched <= WINDOW_COLS), "a block fetches more columns than the fetch registers hold")
+    _need(np.all(fetched <= WINDOW_COLS), "a block fetches more columns than the rings hold")
+    later = np.ones(nblocks, bool)
+    later[chains[:, 0]] = False  # a chain's first block takes as many rounds as it needs
+    _need(np.all(fetched[later] <= FETCH_COLS), "a block past the first of its chain fetches more than one round of the fetch registers")
 
     # stored elements: each placed once; the blocks may be stored in another order than their rows'
     # (block i of the tables holds the rows of row block order[i]), the elements of one block in order
     slots = ntiles * TILE
-    perm = np.asarray(arrays["perm"], np.int64)
-    _need(perm.size == slots, f"perm holds {perm.size} slots for {ntiles} tiles")
-    perm = logical_order(perm, itemsize)
+    if arrays.get("perm") is None:
+        # values read in place: slot e of a tile holds stored element (word 2) + e for e < (word 3)
+        _need(np.all(rp[1:] - rp[:-1] >= MIN_ROW_SLOTS), "values can be read in place only where every row fills its slots")
+        _need(np.all(info[:, 3] >= 1) and np.all(info[:, 3] <= TILE), "a tile's count of stored elements leaves 1 .. 256")
+        _need(np.all(info[:, 2] >= 0) and np.all(info[:, 2] + info[:, 3] <= nnz), "a tile's stored elements leave the matrix")
+        e = np.arange(TILE)[None, :]
+        perm = np.where(e < info[:, 3:4], info[:, 2:3] + e, -1).reshape(-1)
+    else:
+        perm = np.asarray(arrays["perm"], np.int64)
+        _need(perm.size == slots, f"perm holds {perm.size} slots for {ntiles} tiles")
+        perm = logical_order(perm, itemsize)
     cf = np.asarray(arrays["cf"], np.int64)
+    if arrays.get("perm") is None and itemsize == 8:
+        cf = cf.reshape(-1, TILE)[:, halves_pos()].reshape(-1)  # into the order of the slots
     real = np.nonzero(perm >= 0)[0]
     src = perm[real]
     if src.size != nnz or not np.array_equal(np.sort(src), np.arange(nnz)):
@@ -375,18 +397,22 @@ def check_window(arrays, rp, col, n, rows_per_block, nbands, itemsize):
 
 
 def window_plan_arrays(rp, col, n, rows_per_block, itemsize, tiles_per_chain=1 << 30, fresh_check=True, stack=None,
-                       rotate=0):
+                       rotate=0, in_place=None):
     """A window plan built on the host from its definition, in the layout Plan.export gives: one
     band, or, with stack = (P, lowest, highest offset from the diagonal once the bands P below
     and above it are shifted onto it), three bands on stacked planes of P rows (square matrix, P a
     multiple of rows_per_block and a divisor of the number of rows).  fresh_check=False leaves out
     the rule that a block whose columns start below what its chain has fetched begins a new chain,
     rotate != 0 turns the regions of stacked planes the wrong way (the mistakes a replay of the
-    rings must catch)."""
+    rings must catch).  in_place (default: wherever every row has two stored elements or more)
+    leaves perm out, as a plan does that reads A's values where they are."""
     rp = np.asarray(rp, np.int64)
     col = np.asarray(col, np.int64)
     m, nnz, R = rp.size - 1, col.size, rows_per_block
     nblocks = -(-m // R)
+    lens = rp[1:] - rp[:-1]
+    if in_place is None:
+        in_place = bool(np.all(lens >= MIN_ROW_SLOTS))
     row_start = np.zeros(m, np.int64)
     btiles = np.zeros(nblocks, np.int64)
     for b in range(nblocks):
@@ -419,7 +445,6 @@ def window_plan_arrays(rp, col, n, rows_per_block, itemsize, tiles_per_chain=1 <
     perm = np.full(slots, -1, np.int64)
     perm[d] = np.arange(nnz)
     cf = np.full(slots, 0x8000 | WINDOW_COLS, np.int64)
-    lens = rp[1:] - rp[:-1]
     short_rows = np.nonzero(lens < MIN_ROW_SLOTS)[0]
     cf[tile_off[short_rows // R] * TILE + row_start[short_rows] + 1] = WINDOW_COLS  # continues the row's run
     head = (np.arange(nnz) == rp[erow]) | (o % TILE == 0)
@@ -430,7 +455,7 @@ def window_plan_arrays(rp, col, n, rows_per_block, itemsize, tiles_per_chain=1 <
         cf[d] = (((q + rotate) % 3) * size + col % size) | (head.astype(np.int64) << 15)
     else:
         cf[d] = (col % WINDOW_COLS) | (head.astype(np.int64) << 15)
-    info = np.zeros((ntiles, 2), np.int64)
+    info = np.zeros((ntiles, 4), np.int64)
     for b in range(nblocks):
         r0, r1 = b * R, min(m, (b + 1) * R)
         rs = row_start[r0:r1]
@@ -438,7 +463,8 @@ def window_plan_arrays(rp, col, n, rows_per_block, itemsize, tiles_per_chain=1 <
             off = (t - tile_off[b]) * TILE
             a = r0 + int(np.searchsorted(rs, off, side="right")) - 1
             u = r0 + int(np.searchsorted(rs, off + TILE, side="left"))
-            info[t] = (a | ((1 << 31) if row_start[a] != off else 0), u - a)
+            end = row_start[u - 1] + (rp[u] - rp[u - 1]) - off  # behind the last row's stored elements
+            info[t] = (a | ((1 << 31) if row_start[a] != off else 0), u - a, rp[a] + (off - row_start[a]), min(end, TILE))
     blocks, pieces, chains = [], [], []
     chain_lo, chain_tiles = 0, 0
     if stack:
@@ -471,6 +497,9 @@ def window_plan_arrays(rp, col, n, rows_per_block, itemsize, tiles_per_chain=1 <
             if b != chain_lo:
                 if fresh_check and hi > lo and have >= 0 and (lo < low or lo < max(have, hi) - WINDOW_COLS + 8):
                     fresh = True
+                piece = 0 if hi <= lo else (hi - lo if have < 0 or lo >= have else max(have, hi) - have)
+                if piece > FETCH_COLS:
+                    fresh = True
                 if chain_tiles >= tiles_per_chain:
                     fresh = True
             if fresh:
@@ -489,14 +518,19 @@ def window_plan_arrays(rp, col, n, rows_per_block, itemsize, tiles_per_chain=1 <
     chains.append([chain_lo, nblocks])
     perm_phys = np.empty_like(perm).reshape(-1, TILE)
     perm_phys[:, val_pos(itemsize)] = perm.reshape(-1, TILE)
-    return dict(perm=perm_phys.reshape(-1).astype(np.int32), cf=cf.astype(np.uint16),
+    if in_place and itemsize == 8:
+        stored = np.empty_like(cf).reshape(-1, TILE)
+        stored[:, halves_pos()] = cf.reshape(-1, TILE)
+        cf = stored.reshape(-1)
+    return dict(perm=None if in_place else perm_phys.reshape(-1).astype(np.int32), cf=cf.astype(np.uint16),
                 tile_words=(info & 0xFFFFFFFF).astype(np.uint32).view(np.int32).reshape(-1),
                 blocks=np.array(blocks, np.int32).reshape(-1), pieces=np.array(pieces, np.int32).reshape(-1),
                 workgroups=np.array(chains, np.int32).reshape(-1))
 
 
 def export_all(plan, names, value_dtype=None):
-    return {k: plan.export(k, value_dtype) for k in names}
+    held = [k for k in names if not (k == "perm" and plan.info("by_reference") == 1)]
+    return {k: plan.export(k, value_dtype) for k in held}
 
 
 SLICED_ARRAYS = ("perm", "cf", "tile_words", "workgroups", "partial_rows", "ranges", "step_ptr", "steps")

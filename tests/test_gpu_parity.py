@@ -381,7 +381,9 @@ def test_benchmark_configs_full_size(torch, capi, oracle):
             across_plans = []
             for alg in (capi.SPMV_WINDOW, capi.SPMV_DEFAULT):
                 plan = capi.Plan(False, alg, w.val.dtype, w.m, w.n, w.nnz, d[0], col=d[1], val=d[2])
-                assert plan.alg == capi.SPMV_WINDOW and plan.holds_values and plan.workspace_bytes == 0  # no row is cut
+                assert plan.alg == capi.SPMV_WINDOW and plan.workspace_bytes == 0  # no row is cut
+                # every row holds two elements or more: fp32 values are read where the caller keeps them
+                assert plan.info("by_reference") == int(w.val.dtype == np.float32) and plan.holds_values == (w.val.dtype != np.float32)
                 outs = []
                 for rep in range(2):
                     y = dev(torch, w.y)
@@ -676,6 +678,9 @@ def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
     for (m, n, half, dens, lr) in ((3000, 3000, 40, 0.3, None), (5000, 9000, 700, 0.02, 2500), (700, 700, 300, 0.9, 10),
                                    (20000, 20000, 3, 1.0, None), (257, 300, 100, 0.2, None), (1, 5, 2, 1.0, None)):
         cases.append((f"band {m}x{n} +-{half}", _banded_random(rng, m, n, half, dens, dtype, longrow=lr), n))
+    # without empty rows (and no row of one element): plans that read A's values in place
+    for (m, n, half, dens, lr) in ((3000, 3000, 40, 0.3, None), (5000, 9000, 700, 0.02, 2500), (2000, 2000, 2, 1.0, None)):
+        cases.append((f"full rows {m}x{n} +-{half}", _banded_random(rng, m, n, half, dens, dtype, empty=0.0, longrow=lr), n))
     st = W.stencil5_f64(300, 200)
     cases.append(("stencil 300x200", (st.row_ptr, st.col, st.val.astype(dtype)), st.n))
     # windows that move backwards from one block of rows to the next, inside what a ring could still
@@ -698,30 +703,37 @@ def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
         x = rng.uniform(-1, 1, n).astype(dtype)
         y0 = rng.uniform(-1, 1, m).astype(dtype)
         d = [dev(torch, a) for a in (rp, col, val, x)]
-        plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
-        assert plan.alg == capi.SPMV_WINDOW and plan.holds_values
-        plan_check.check_plan(plan, capi, rp, col, n, np.dtype(dtype).itemsize)
-        assert plan.workspace_bytes == plan.info("carry_pass") * plan.info("tiles") * np.dtype(dtype).itemsize
-        assert plan.info("bands") == 1 and plan.info("rows_per_block") % 256 == 0 and plan.info("tiles") > 0
-        if name == "windows moving backwards":
-            assert plan.info("chains") < -(-m // plan.info("rows_per_block")), "chains of several blocks expected"
-        for alpha, beta in ((1.5, 0.5), (1.0, 0.0), (-2.0, 1.0)):
-            ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 2)
-            scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
-            for rep in range(2):
-                y = dev(torch, y0 if beta else np.full(m, np.nan, dtype=dtype))
-                capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_WINDOW, plan=plan)
-                torch.cuda.synchronize()
-                assert_close(y.cpu().numpy(), ref, scale, dtype, f"{name} a={alpha} b={beta} rep={rep}")
-        val2 = rng.uniform(-1, 1, val.size).astype(dtype)
-        d2 = dev(torch, val2)
-        plan.update_values(d2)
-        y = dev(torch, y0)
-        capi.spmv(d[0], d[1], d2, d[3], y, 1.5, 0.5, alg=capi.SPMV_WINDOW, plan=plan)
-        torch.cuda.synchronize()
-        assert_close(y.cpu().numpy(), oracle.spmv(rp, col, val2, x, dtype(1.5), dtype(0.5), y0, 2),
-                     spmv_scale(rp, col, val2, x, 1.5, 0.5, y0), dtype, f"{name} updated values")
-        plan.destroy()
+        full_rows = bool(np.diff(rp).min() >= 2)  # rows that fill their two slots: the values can be read in place
+        assert full_rows == name.startswith(("full rows", "stencil", "band 1x5")), name  # the one-row matrix: 3 elements
+        # fp32 plans read the values in place wherever they can; fp64 ones when the plan is to follow
+        # values changed in place (a checked plan), and then check nothing
+        for checked in ((False, True) if full_rows else (False,)):
+            plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2], checked=checked)
+            assert plan.alg == capi.SPMV_WINDOW
+            in_place = int(full_rows and (checked or dtype == np.float32))
+            assert plan.info("by_reference") == in_place and plan.holds_values == (not in_place) and not plan.checked, name
+            plan_check.check_plan(plan, capi, rp, col, n, np.dtype(dtype).itemsize)
+            assert plan.workspace_bytes == plan.info("carry_pass") * plan.info("tiles") * np.dtype(dtype).itemsize
+            assert plan.info("bands") == 1 and plan.info("rows_per_block") % 256 == 0 and plan.info("tiles") > 0
+            if name == "windows moving backwards":
+                assert plan.info("chains") < -(-m // plan.info("rows_per_block")), "chains of several blocks expected"
+            for alpha, beta in ((1.5, 0.5), (1.0, 0.0), (-2.0, 1.0)):
+                ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 2)
+                scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
+                for rep in range(2):
+                    y = dev(torch, y0 if beta else np.full(m, np.nan, dtype=dtype))
+                    capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_WINDOW, plan=plan)
+                    torch.cuda.synchronize()
+                    assert_close(y.cpu().numpy(), ref, scale, dtype, f"{name} a={alpha} b={beta} rep={rep} checked={checked}")
+            val2 = rng.uniform(-1, 1, val.size).astype(dtype)
+            d2 = dev(torch, val2)
+            plan.update_values(d2)  # nothing to do for a plan that reads the values in place
+            y = dev(torch, y0)
+            capi.spmv(d[0], d[1], d2, d[3], y, 1.5, 0.5, alg=capi.SPMV_WINDOW, plan=plan)
+            torch.cuda.synchronize()
+            assert_close(y.cpu().numpy(), oracle.spmv(rp, col, val2, x, dtype(1.5), dtype(0.5), y0, 2),
+                         spmv_scale(rp, col, val2, x, 1.5, 0.5, y0), dtype, f"{name} updated values")
+            plan.destroy()
     # rows that reach far (uniform random columns over 200 000) are not this kernel's matrix; a row
     # longer than 2048 is not either
     L = capi.lib()
@@ -833,32 +845,38 @@ def test_spmv_window_kernel_bands_of_diagonals(torch, capi, oracle, dtype):
         x = rng.uniform(-1, 1, n).astype(dtype)
         y0 = rng.uniform(-1, 1, m).astype(dtype)
         d = [dev(torch, a) for a in (rp, col, val, x)]
-        plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
-        assert plan.alg == capi.SPMV_WINDOW and plan.holds_values
-        plan_check.check_plan(plan, capi, rp, col, n, np.dtype(dtype).itemsize)
-        assert plan.workspace_bytes == plan.info("carry_pass") * plan.info("tiles") * np.dtype(dtype).itemsize
-        assert 2 <= plan.info("bands") <= 4 and plan.info("slices") == -1, (name, plan.info("bands"))
-        # the stencils' three bands lie whole planes apart: their blocks are stored plane above plane
-        # and x is fetched about once (a ring per band: three times)
-        want_planes = {"stencil 7 points": plane, "stencil 27 points": plane, "stencil 7 points, planes of 9025": 9025}.get(name, 0)
-        assert plan.info("stacked_rows") == want_planes, (name, plan.info("stacked_rows"))
-        if want_planes:  # past the first block of a chain a block fetches the plane above it only
-            pcs = plan.export("pieces").reshape(-1, 3, 4)
-            fetches = (pcs[:, :, 1] > pcs[:, :, 0]).sum(axis=1)
-            first = np.zeros(fetches.size, bool)
-            first[plan.export("workgroups").reshape(-1, 2)[:, 0]] = True
-            assert np.all(fetches[~first] <= 1) and np.all(fetches[first] >= 2), name
-        if name in ("stencil 7 points", "long rows"):  # rows of at most 16 are never cut by tiles
-            assert plan.info("carry_pass") == (1 if name == "long rows" else 0), name
-        for alpha, beta in ((1.5, 0.5), (1.0, 0.0)):
-            ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 2)
-            scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
-            for rep in range(2):
-                y = dev(torch, y0 if beta else np.full(m, np.nan, dtype=dtype))
-                capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_WINDOW, plan=plan)
-                torch.cuda.synchronize()
-                assert_close(y.cpu().numpy(), ref, scale, dtype, f"{name} a={alpha} b={beta} rep={rep}")
-        plan.destroy()
+        # the grids without dropped elements have no row of fewer than two elements: fp32 plans read
+        # their values in place, fp64 plans when they are to follow values changed in place
+        full_rows = bool(np.diff(rp).min() >= 2)
+        for checked in ((False, True) if full_rows else (False,)):
+            plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2], checked=checked)
+            assert plan.alg == capi.SPMV_WINDOW
+            in_place = int(full_rows and (checked or dtype == np.float32))
+            assert plan.info("by_reference") == in_place and plan.holds_values == (not in_place) and not plan.checked, name
+            plan_check.check_plan(plan, capi, rp, col, n, np.dtype(dtype).itemsize)
+            assert plan.workspace_bytes == plan.info("carry_pass") * plan.info("tiles") * np.dtype(dtype).itemsize
+            assert 2 <= plan.info("bands") <= 4 and plan.info("slices") == -1, (name, plan.info("bands"))
+            # the stencils' three bands lie whole planes apart: their blocks are stored plane above plane
+            # and x is fetched about once (a ring per band: three times)
+            want_planes = {"stencil 7 points": plane, "stencil 27 points": plane, "stencil 7 points, planes of 9025": 9025}.get(name, 0)
+            assert plan.info("stacked_rows") == want_planes, (name, plan.info("stacked_rows"))
+            if want_planes:  # past the first block of a chain a block fetches the plane above it only
+                pcs = plan.export("pieces").reshape(-1, 3, 4)
+                fetches = (pcs[:, :, 1] > pcs[:, :, 0]).sum(axis=1)
+                first = np.zeros(fetches.size, bool)
+                first[plan.export("workgroups").reshape(-1, 2)[:, 0]] = True
+                assert np.all(fetches[~first] <= 1) and np.all(fetches[first] >= 2), name
+            if name in ("stencil 7 points", "long rows"):  # rows of at most 16 are never cut by tiles
+                assert plan.info("carry_pass") == (1 if name == "long rows" else 0), name
+            for alpha, beta in ((1.5, 0.5), (1.0, 0.0)):
+                ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 2)
+                scale = spmv_scale(rp, col, val, x, alpha, beta, y0)
+                for rep in range(2):
+                    y = dev(torch, y0 if beta else np.full(m, np.nan, dtype=dtype))
+                    capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_WINDOW, plan=plan)
+                    torch.cuda.synchronize()
+                    assert_close(y.cpu().numpy(), ref, scale, dtype, f"{name} a={alpha} b={beta} rep={rep} checked={checked}")
+            plan.destroy()
     # three bands of 9000 diagonals each: 27000 columns a block, more than the LDS holds
     rp, col, val = _diagonal_bands(rng, 30000, 90000, [(-40000, -31000), (0, 9000), (30000, 39000)], 0.002, dtype)
     d = [dev(torch, a) for a in (rp, col, val)]
@@ -1139,7 +1157,8 @@ def test_checked_plans_follow_values_changed_in_place(torch, capi, oracle, dtype
     """asx_spmv_plan_create_checked + asx_plan_refresh_if_changed: a plan that holds a copy of A's
     values notices, by two checksums taken on the device before every call, that the caller changed
     values in place, and refreshes its copy; with unchanged values the call gives the same bits as
-    before.  Sliced plan (scattered columns) and window plan (a band), DEFAULT's choice; a single
+    before.  Sliced plan (scattered columns) and window plans (a band whose values are read in
+    place: nothing kept, nothing checked; a band with empty rows: a checked copy), DEFAULT's choice; a single
     changed value, two swapped values (same multiset: only position-dependent sums see it), a flipped
     sign, all values; a small matrix stays row-ordered and unchecked."""
     from library_amd import workloads as W
@@ -1149,6 +1168,8 @@ def test_checked_plans_follow_values_changed_in_place(torch, capi, oracle, dtype
     cases.append(("scattered", rp, col, val, 1 << 20, capi.SPMV_SLICED))
     rp, col, val = W.csr_banded(1 << 19, 4, dtype, 5)
     cases.append(("band of 9", rp, col, val, 1 << 19, capi.SPMV_WINDOW))
+    rp, col, val = _banded_random(rng, 60000, 60000, 30, 0.3, dtype)  # one row in ten is empty
+    cases.append(("band with empty rows", rp, col, val, 60000, capi.SPMV_WINDOW))
     for name, rp, col, val, n, want_alg in cases:
         m, nnz = rp.size - 1, col.size
         x = rng.uniform(-1, 1, n).astype(dtype)
@@ -1162,7 +1183,11 @@ def test_checked_plans_follow_values_changed_in_place(torch, capi, oracle, dtype
                 assert not plan.checked and not plan.holds_values, (name, plan.alg)
                 plan.destroy()
                 continue
-            assert plan.alg == want_alg and plan.checked and plan.holds_values, (name, plan.alg)
+            # a window plan over rows of two elements or more keeps no copy: nothing to check or refresh,
+            # and the same sequence of in-place changes must come out right all the same
+            by_ref = plan.alg == capi.SPMV_WINDOW and plan.info("by_reference") == 1
+            assert plan.alg == want_alg and by_ref == (name == "band of 9"), (name, plan.alg)
+            assert plan.checked == (not by_ref) and plan.holds_values == (not by_ref), name
 
             def product(values):
                 ref = oracle.spmv(rp, col, values, x, dtype(1.5), dtype(0.5), y0, 4)
@@ -1208,3 +1233,28 @@ def test_checked_plans_follow_values_changed_in_place(torch, capi, oracle, dtype
     plan.destroy()
     L = capi.lib()
     assert L.asx_plan_refresh_if_changed(None, None, None) == 7 and L.asx_plan_is_checked(None) == 0
+    # values off a 16-byte boundary (a view one element into an allocation): no checksums can be
+    # taken, so a kernel asked for by name that would copy them is refused (INVALID_VALUE) ...
+    rp, col, val = csr_from_lengths(rng.integers(0, 9, 3000), 5000, 7, dtype)
+    d_rp, d_col = dev(torch, rp), dev(torch, col)
+    room = torch.zeros(col.size + 1, dtype=torch.float64 if dtype == np.float64 else torch.float32, device="cuda")
+    room[1:] = torch.from_numpy(val)
+    h = capi.C.c_void_p()
+    for alg in (capi.SPMV_SLICED, capi.SPMV_WINDOW):
+        assert L.asx_spmv_plan_create_checked(capi.C.byref(h), alg, capi.value_type(np.dtype(dtype)), rp.size - 1, 5000, col.size,
+                                              capi._ptr(d_rp), capi._ptr(d_col), capi._ptr(room[1:]), None) == 3
+        assert not h.value
+    # ... while a window plan that reads them in place takes them as they are
+    rp, col, val = W.csr_banded(20000, 4, dtype, 5)
+    room = torch.zeros(col.size + 1, dtype=room.dtype, device="cuda")
+    room[1:] = torch.from_numpy(val)
+    d_rp, d_col = dev(torch, rp), dev(torch, col)
+    x = rng.uniform(-1, 1, 20000).astype(dtype)
+    plan = capi.Plan(False, capi.SPMV_WINDOW, np.dtype(dtype), 20000, 20000, col.size, d_rp, col=d_col, val=room[1:], checked=True)
+    assert plan.info("by_reference") == 1 and not plan.checked
+    y = torch.zeros(20000, dtype=room.dtype, device="cuda")
+    capi.spmv(d_rp, d_col, room[1:], dev(torch, x), y, 1.0, 0.0, alg=capi.SPMV_WINDOW, plan=plan)
+    torch.cuda.synchronize()
+    assert_close(y.cpu().numpy(), oracle.spmv(rp, col, val, x, dtype(1.0), dtype(0.0), np.zeros(20000, dtype), 4),
+                 spmv_scale(rp, col, val, x, 1.0, 0.0, np.zeros(20000, dtype)), dtype, "values in place off a 16-byte boundary")
+    plan.destroy()

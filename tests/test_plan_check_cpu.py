@@ -112,7 +112,7 @@ def test_window_plan_from_its_definition_passes(itemsize):
     rp, col = _banded(11, 3000, 3000, 150, 0.05)
     for tiles_per_chain in (1 << 30, 40):
         plan = pc.window_plan_arrays(rp, col, 3000, 256, itemsize, tiles_per_chain)
-        assert (plan["tile_words"].reshape(-1, 2)[:, 0] < 0).any(), "the matrix should have rows cut by tile starts"
+        assert (plan["tile_words"].reshape(-1, 4)[:, 0] < 0).any(), "the matrix should have rows cut by tile starts"
         pc.check_window(plan, rp, col, 3000, 256, 1, itemsize)
     rp, col, n = _windows_moving_backwards()
     plan = pc.window_plan_arrays(rp, col, n, 256, itemsize)
@@ -130,13 +130,48 @@ def test_window_corruptions_are_rejected():
         pc.check_window(bad, rp, col, n, 256, 1, 8)
 
     rp, col = _banded(13, 3000, 3000, 150, 0.05)
-    good = pc.window_plan_arrays(rp, col, 3000, 256, 8, 40)
+    good = pc.window_plan_arrays(rp, col, 3000, 256, 8, 40, in_place=False)
 
     def corrupt(fn, match=None):
         p = {k: v.copy() for k, v in good.items()}
         fn(p)
         with pytest.raises(pc.PlanError, match=match):
             pc.check_window(p, rp, col, 3000, 256, 1, 8)
+
+    # a matrix whose values are read in place (no row of fewer than two stored elements): the words
+    # that say where a tile's values lie
+    rng = np.random.default_rng(17)
+    lens = rng.integers(2, 40, 3000)
+    rp2 = np.r_[0, np.cumsum(lens)].astype(np.int32)
+    col2 = np.concatenate([np.sort(rng.choice(np.arange(max(0, r - 150), min(3000, r + 151)), k, replace=False))
+                           for r, k in enumerate(lens)]).astype(np.int32)
+    in_place = pc.window_plan_arrays(rp2, col2, 3000, 256, 8, 40)
+    assert in_place["perm"] is None
+    pc.check_window(in_place, rp2, col2, 3000, 256, 1, 8)
+
+    def corrupt_in_place(fn, match):
+        p = {k: None if v is None else v.copy() for k, v in in_place.items()}
+        fn(p)
+        with pytest.raises(pc.PlanError, match=match):
+            pc.check_window(p, rp2, col2, 3000, 256, 1, 8)
+
+    pc.check_window(pc.window_plan_arrays(rp2, col2, 3000, 256, 4, 40), rp2, col2, 3000, 256, 1, 4)
+
+    def words_in_slot_order(p):  # fp64 in place: a lane's four words lie together, two slots from either half
+        p["cf"] = p["cf"].reshape(-1, pc.TILE)[:, pc.halves_pos()].reshape(-1)
+    corrupt_in_place(words_in_slot_order, "holds column|flag|a pad does not point")
+
+    def first_value_off_by_one(p):
+        p["tile_words"].reshape(-1, 4)[5, 2] += 1
+    corrupt_in_place(first_value_off_by_one, "placed|out of order|another block")
+
+    def one_value_fewer(p):
+        p["tile_words"].reshape(-1, 4)[5, 3] -= 1
+    corrupt_in_place(one_value_fewer, "placed")
+
+    def one_value_more(p):  # the kernel would multiply the next tile's first value by the zero
+        p["tile_words"].reshape(-1, 4)[5, 3] += 1
+    corrupt_in_place(one_value_more, "placed|leaves 1 .. 256")
 
     def dup_perm(p):
         real = np.nonzero(p["perm"] >= 0)[0]
@@ -161,11 +196,11 @@ def test_window_corruptions_are_rejected():
     corrupt(flag, "flag|fewer than two stored elements")
 
     def tile_rows(p):  # a tile that claims one row fewer: that row would never be written
-        p["tile_words"].reshape(-1, 2)[3, 1] -= 1
+        p["tile_words"].reshape(-1, 4)[3, 1] -= 1
     corrupt(tile_rows)
 
     def tile_first_row(p):
-        p["tile_words"].reshape(-1, 2)[3, 0] += 1
+        p["tile_words"].reshape(-1, 4)[3, 0] += 1
     corrupt(tile_first_row)
 
     def chain_gap(p):
@@ -227,7 +262,7 @@ def test_stacked_planes_corruptions_are_rejected():
     good = pc.window_plan_arrays(rp, col, n, 256, 8, 30, stack=(1024, -32, 32))
 
     def corrupt(fn, match):
-        p = {k: v.copy() for k, v in good.items()}
+        p = {k: None if v is None else v.copy() for k, v in good.items()}
         fn(p)
         with pytest.raises(pc.PlanError, match=match):
             pc.check_window(p, rp, col, n, 256, 3, 8)
@@ -247,7 +282,7 @@ def test_stacked_planes_corruptions_are_rejected():
 
     def swap_two_blocks_tiles(p):  # the tables name another block's tiles
         blk = p["blocks"].reshape(-1, 4)
-        info = p["tile_words"].reshape(-1, 2)
+        info = p["tile_words"].reshape(-1, 4)
         t0, t1 = int(blk[0, 0]), int(blk[1, 0])
         info[t0, 0], info[t1, 0] = info[t1, 0], info[t0, 0]
     corrupt(swap_two_blocks_tiles, "block")
