@@ -54,10 +54,10 @@ MEASURED_TRAFFIC_BYTES = {
     "uniform16_f32": 256_450_608,  # profiles/spmv_sliced_uniform16_f32.md
     "uniform16_f64": 477_788_284,  # profiles/spmv_sliced_uniform16_f64.md
     "powerlaw_f64": 728_906_293,  # profiles/spmv_sliced_powerlaw_f64.md
-    "stencil5_f64": 1_137_229_657,  # profiles/spmv_window_stencil5_f64.md
+    "stencil5_f64": 1_142_530_786,  # profiles/spmv_window_stencil5_f64.md
     "spmm_zipf_f32": 4_965_331_333,  # profiles/spmm_merge_spmm_zipf_f32.md
     "spmm_banded_f32": 1_870_263_890,  # profiles/spmm_blocked_spmm_banded_f32.md
-    "stencil7_f64": 1_622_985_065,  # profiles/spmv_window_stencil7_256_f64.md
+    "stencil7_f64": 1_630_404_585,  # profiles/spmv_window_stencil7_256_f64.md
 }
 
 
