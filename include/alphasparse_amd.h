@@ -57,7 +57,7 @@ enum {
     ASX_SPMV_WINDOW = 102 /* not a reference id: chains of blocks of consecutive rows with a sliding window of x
                              in LDS and 16-bit columns, for matrices whose rows reach only nearby columns
                              (needs a plan from asx_spmv_plan_create; NOT_SUPPORTED when some 256 rows reach
-                             over 16376 columns or more, or a row is longer than 2048) */
+                             over 16376 columns or more) */
 };
 
 /* SpMM kernels (alphasparseSpMMAlg_t values, include/alphasparse/spdef.h:390-402) */
@@ -203,7 +203,7 @@ int asx_spmm_plan_create(asx_plan **plan, int alg, int value_type, int32_t m, in
  * the values: an fp32 plan, or a plan made by asx_spmv_plan_create_checked, then reads A's values
  * in every call, ASX_PLAN_INFO_BY_REFERENCE = 1, and holds 2 bytes per stored element instead of
  * 14 or 10); DEFAULT picks it, when the sliced kernel is not chosen, for nnz >= 2^21
- * and rows no longer than 2048 whenever the matrix qualifies: every 256 consecutive rows reach
+ * whenever the matrix qualifies: every 256 consecutive rows reach
  * over fewer than 16376 columns, or the stored elements lie on at most 4 bands of diagonals whose
  * windows fit the LDS together (stencils on three-dimensional grids); otherwise
  * ASX_STATUS_NOT_SUPPORTED for the explicit id, the row-ordered plan for DEFAULT.  Synchronises

@@ -668,11 +668,9 @@ int plan_add_slices(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
 }
 
 // Builds the row-block copy onto a plan that already holds the histogram.
-constexpr int32_t kWindowMaxRow = 2048;  // longer rows would make the ordered carry pass serial
 template <typename T>
 int plan_add_window(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col, const T *d_val, bool follows_values, hipStream_t s)
 {
-    if (p->stats[0] > kWindowMaxRow) return ASX_STATUS_NOT_SUPPORTED;
     int cus = 256;
     (void)asx_device_info(&cus, nullptr);
     WindowMatrix wm{};
@@ -716,7 +714,7 @@ static bool regrouped_copy_fits(const asx_plan *p, size_t sv)
 
 static bool window_may_pay(const asx_plan *p, int row_kernel)
 {
-    return p->stats[0] <= kWindowMaxRow && (row_kernel == ASX_SPMV_FLAT || row_kernel == ASX_SPMV_MERGE) &&
+    return (row_kernel == ASX_SPMV_FLAT || row_kernel == ASX_SPMV_MERGE) &&
            2 * p->hist[0] + p->hist[1] <= (int64_t)p->nnz / 4;
 }
 

@@ -737,21 +737,48 @@ __global__ __launch_bounds__(NW *kWave) void k_spmv_window(int32_t n, T alpha, T
     }
 }
 
-// Adds the carries to their rows, in tile order: the thread of the first tile of a run of tiles
-// that start inside the same row sums the run's carries and adds the total once.
+// Adds the carries to their rows: the thread of the first tile of a run of tiles that start inside
+// the same row sums the run's carries and adds the total once.  Up to kSerialCarries of them it
+// sums itself, in tile order; what a longer run holds beyond those (a row of several thousand
+// stored elements) the 64 lanes of its wave sum together, 64 tiles a round, combined in a fixed
+// order: the same bits in every call.
+constexpr int32_t kSerialCarries = 8;
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_window_fixup(int32_t ntiles, T alpha, const int4 *__restrict__ tile_info,
                                                          const T *__restrict__ carry, T *__restrict__ y)
 {
+    const int lane = threadIdx.x & (kWave - 1);
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= ntiles) return;
-    const int32_t w = tile_info[t].x;
-    if (w >= 0) return;                            // starts at a row start
-    if (t > 0 && tile_info[t - 1].x == w) return;  // a later tile of its run
-    T s = carry[t];
-    for (int64_t j = t + 1; j < ntiles && tile_info[j].x == w; ++j) s += carry[j];
-    const int32_t r = w & 0x7fffffff;
-    y[r] = fma_t<T>(alpha, s, y[r]);
+    const int32_t w = t < ntiles ? tile_info[t].x : 0;
+    // a tile that starts inside a row and is the first of its run
+    const bool head = w < 0 && !(t > 0 && tile_info[t - 1].x == w);
+    T s = T(0);
+    int32_t taken = 0;
+    if (head) {
+        for (int64_t j = t; taken < kSerialCarries && j < ntiles && tile_info[j].x == w; ++j, ++taken) s += carry[j];
+    }
+    const bool more = head && taken == kSerialCarries && t + taken < ntiles && tile_info[t + taken].x == w;
+    unsigned long long todo = __ballot(more);
+    while (todo) {  // uniform over the wave
+        const int f = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const int32_t wf = __builtin_amdgcn_readlane(w, f);
+        const int64_t tf = ((int64_t)blockIdx.x * blockDim.x + (threadIdx.x & ~(kWave - 1)) + f) + kSerialCarries;
+        T part = T(0);
+        for (int64_t j0 = tf;; j0 += kWave) {
+            const int64_t j = j0 + lane;
+            const bool in = j < ntiles && tile_info[j].x == wf;
+            if (in) part += carry[j];
+            if (__ballot(in) != ~0ull) break;  // the run ended inside these 64 tiles
+        }
+#pragma unroll
+        for (int d = kWave / 2; d > 0; d >>= 1) part += __shfl_xor(part, d, kWave);
+        if (lane == f) s += part;
+    }
+    if (head) {
+        const int32_t r = w & 0x7fffffff;
+        y[r] = fma_t<T>(alpha, s, y[r]);
+    }
 }
 
 }  // namespace

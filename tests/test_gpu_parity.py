@@ -669,7 +669,7 @@ def _banded_random(rng, m, n, half, dens, dtype, empty=0.1, longrow=None):
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
     """The row-block kernel forced on banded matrices: empty rows (a slot of their own), rows cut by
-    tile starts (carry pass), a row of 1401 spanning six tiles, a block whose last tile is mostly
+    tile starts (carry pass), a row of 1401 spanning six tiles and one of 13001 spanning 51, a block whose last tile is mostly
     padding, a rectangular matrix, the 5-point stencil, beta = 0 over NaN, two calls through one
     plan, a value update; and NOT_SUPPORTED for rows that reach further than a window."""
     rng = np.random.default_rng(93)
@@ -681,6 +681,8 @@ def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
     # without empty rows (and no row of one element): plans that read A's values in place
     for (m, n, half, dens, lr) in ((3000, 3000, 40, 0.3, None), (5000, 9000, 700, 0.02, 2500), (2000, 2000, 2, 1.0, None)):
         cases.append((f"full rows {m}x{n} +-{half}", _banded_random(rng, m, n, half, dens, dtype, empty=0.0, longrow=lr), n))
+    # a row of 13001 stored elements: 51 tiles whose carries the lanes of a wave add up together
+    cases.append(("band 9000x14000 +-6500", _banded_random(rng, 9000, 14000, 6500, 0.02, dtype, longrow=4000), 14000))
     st = W.stencil5_f64(300, 200)
     cases.append(("stencil 300x200", (st.row_ptr, st.col, st.val.astype(dtype)), st.n))
     # windows that move backwards from one block of rows to the next, inside what a ring could still
@@ -735,9 +737,9 @@ def test_spmv_window_kernel_shapes(torch, capi, oracle, dtype):
                          spmv_scale(rp, col, val2, x, 1.5, 0.5, y0), dtype, f"{name} updated values")
             plan.destroy()
     # rows that reach far (uniform random columns over 200 000) are not this kernel's matrix; a row
-    # longer than 2048 is not either
+    # that alone reaches over more columns than the ring holds is not either
     L = capi.lib()
-    for lens, ncols in ((rng.integers(1, 9, 2000), 200000), (np.r_[np.full(50, 3), 2500, np.full(50, 3)], 2600)):
+    for lens, ncols in ((rng.integers(1, 9, 2000), 200000), (np.r_[np.full(50, 3), 17000, np.full(50, 3)], 20000)):
         rp, col, val = csr_from_lengths(lens, ncols, 5, dtype)
         d = [dev(torch, a) for a in (rp, col, val)]
         h = capi.C.c_void_p()
