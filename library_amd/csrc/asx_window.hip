@@ -492,8 +492,9 @@ __device__ __forceinline__ void window_tile_load(WindowTile<T, BETA> &tl, int32_
     const u32x2 cw = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(cf + (int64_t)t * kSlicedTile) + lane);
     tl.c01 = cw.x;
     tl.c23 = cw.y;
-    if (INPLACE)
-        ValuesInPlace<T>::load(val, info.z, info.w, lane, tl.v);
+    if (INPLACE)  // the buffer's words as scalars by name: left to itself the compiler keeps the count in a vector
+                  // register and wraps every load into a loop over the distinct values of the lanes
+        ValuesInPlace<T>::load(val, __builtin_amdgcn_readfirstlane(info.z), __builtin_amdgcn_readfirstlane(info.w), lane, tl.v);
     else
         TileValues<T>::load(val + (int64_t)t * kSlicedTile, lane, tl.v);
     tl.base = info.x;
