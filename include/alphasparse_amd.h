@@ -296,13 +296,16 @@ enum {
     ASX_PLAN_ARRAY_PERM = 2,         /* slots x i32: position in A's values of each stored copy (-1: pad) */
     ASX_PLAN_ARRAY_TILE_WORDS = 3,   /* sliced: (tiles + 1) x i32 first partial sum of each tile; window: tiles x 4 i32
                                       * (first row | starts-inside-a-row << 31, rows, first stored element in A, stored elements) */
-    ASX_PLAN_ARRAY_WORKGROUPS = 4,   /* sliced: workgroups x 4 i32 (slice, first tile, end tile, 0); window: chains x 2 i32 */
+    ASX_PLAN_ARRAY_WORKGROUPS = 4,   /* sliced: pieces x 4 i32 (slice, first tile, end tile, 0): what the workgroups of pass 1
+                                      * work off; window: chains x 2 i32 */
     ASX_PLAN_ARRAY_PARTIAL_ROWS = 5, /* sliced: partial sums x u16 row inside the row block | may-repeat << 15 */
     ASX_PLAN_ARRAY_RANGES = 6,       /* sliced: (row blocks + 1) x slices i32: first partial sum of block b in slice s */
     ASX_PLAN_ARRAY_STEP_PTR = 7,     /* sliced: (row blocks + 1) x i32: first step of each row block */
     ASX_PLAN_ARRAY_STEPS = 8,        /* sliced: steps x 4 i32 */
     ASX_PLAN_ARRAY_BLOCKS = 9,       /* window: blocks x 4 i32 (first tile, end tile, first piece, end piece) */
-    ASX_PLAN_ARRAY_PIECES = 10       /* window: pieces x 4 i32 (from column, to column, ring base, ring size) */
+    ASX_PLAN_ARRAY_PIECES = 10,      /* window: pieces x 4 i32 (from column, to column, ring base, ring size) */
+    ASX_PLAN_ARRAY_WG_PIECES = 11    /* sliced: workgroups x 8 i32 (first, end entry of ASX_PLAN_ARRAY_WORKGROUPS, 0, 0,
+                                      * the first of those entries again) */
 };
 int asx_plan_export(const asx_plan *plan, int what, void *h_dst, size_t cap, size_t *bytes, void *stream);
 /* Copies the plan's histogram (33 bins) and stats (4) to host arrays. */

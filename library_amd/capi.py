@@ -321,7 +321,8 @@ class Plan:
     # asx_plan_export: name -> (id, element type; "value" = the plan's value type)
     ARRAYS = {"val": (0, "value"), "cf": (1, np.uint16), "perm": (2, np.int32), "tile_words": (3, np.int32),
               "workgroups": (4, np.int32), "partial_rows": (5, np.uint16), "ranges": (6, np.int32),
-              "step_ptr": (7, np.int32), "steps": (8, np.int32), "blocks": (9, np.int32), "pieces": (10, np.int32)}
+              "step_ptr": (7, np.int32), "steps": (8, np.int32), "blocks": (9, np.int32), "pieces": (10, np.int32),
+              "wg_pieces": (11, np.int32)}
 
     def export(self, name, value_dtype=None):
         """One array of a sliced or window plan as a flat numpy array (asx_plan_export)."""

@@ -595,8 +595,9 @@ int asx_spmm_plan_create(asx_plan **out, int alg, int value_type, int32_t m, int
 constexpr int32_t kSlicedMinNnz = 1 << 21;
 struct KernelEstimates {
     // seconds; infinity where the kernel does not apply.  window: with one ring of x per block;
-    // window_bands: with rings per band of diagonals, which only the build finds out
-    double rows, sliced, window, window_bands;
+    // window_bands: with rings per band of diagonals, window_stacked: with three bands on stacked
+    // planes; which of the three it is only the build finds out
+    double rows, sliced, window, window_bands, window_stacked;
 };
 static KernelEstimates estimate_kernels(const asx_plan *p, size_t sv, const ColumnSample &cs, bool window_ok, bool checked)
 {
@@ -620,15 +621,21 @@ static KernelEstimates estimate_kernels(const asx_plan *p, size_t sv, const Colu
     const bool uncut = p->stats[0] <= 16;
     e.window = !window_ok ? inf : 8e-6 + (wslots * (dsv + 2) + n * dsv + 2 * m * dsv) / (uncut ? 5.6e12 : 4.8e12);
     e.window_bands = !window_ok ? inf : 8e-6 + (wslots * (dsv + 2) + 1.5 * n * dsv + 2 * m * dsv) / (uncut ? 4.6e12 : 3.9e12);
+    // three bands on stacked planes (x fetched about 1.3 times): 7-point stencil on 160^3 5.6e12 in
+    // fp64 but 3.5e12 in fp32, where the time goes with the slots and not with the bytes; 27-point
+    // on 96^3 (rows of 27, cut by tiles) 4.2e12
+    e.window_stacked = !window_ok ? inf
+                                  : 8e-6 + (wslots * (dsv + 2) + 1.3 * n * dsv + 2 * m * dsv) /
+                                               (sv == 8 ? (uncut ? 5.6e12 : 4.2e12) : (uncut ? 3.5e12 : 3.0e12));
     if (checked) {
         // a checked plan reads the caller's values once more in every call (a stream of its own
         // kernel: 6.3 TB/s measured) and launches three small kernels
         const double check = 10e-6 + nnz * dsv / 6.0e12;
         e.sliced += check;
         if (p->hist[0] + p->hist[1] > 0)
-            e.window += check, e.window_bands += check;
-        else if (sv == 8)  // reads A's values in place: no check; two scans a tile and loads off 16-byte boundaries
-            e.window *= 1.08, e.window_bands *= 1.08;
+            e.window += check, e.window_bands += check, e.window_stacked += check;
+        else if (sv == 8)  // reads A's values in place: no check, but two scans a tile
+            e.window *= 1.06, e.window_bands *= 1.06, e.window_stacked *= 1.06;
     }
     return e;
 }
@@ -786,7 +793,8 @@ static int spmv_plan_create(asx_plan **out, int alg, int value_type, int32_t m, 
             const KernelEstimates e = estimate_kernels(p, sv, cs, window_ok, checked);
             const bool sliced_pays = e.sliced < 0.97 * e.rows, window_pays = e.window < 0.97 * e.rows;
             if (window_pays && e.window < e.sliced / 1.05) done = add_window() == ASX_STATUS_SUCCESS;
-            if (done && p->window.nbands > 1 && sliced_pays && !(e.window_bands < e.sliced / 1.05)) {
+            if (done && p->window.nbands > 1 && sliced_pays &&
+                !((p->window.stack_rows > 0 ? e.window_stacked : e.window_bands) < e.sliced / 1.05)) {
                 // the build needed a ring per band of diagonals; with those the slices are ahead
                 WindowMatrix built = p->window;
                 p->window = WindowMatrix{};
@@ -932,7 +940,8 @@ static bool plan_array(const asx_plan *p, int what, const void **ptr, size_t *by
         case ASX_PLAN_ARRAY_CF: *ptr = m.cf, *bytes = slots * 2; return true;
         case ASX_PLAN_ARRAY_PERM: *ptr = m.perm, *bytes = slots * 4; return true;
         case ASX_PLAN_ARRAY_TILE_WORDS: *ptr = m.tile_base, *bytes = ((size_t)m.ntiles + 1) * 4; return true;
-        case ASX_PLAN_ARRAY_WORKGROUPS: *ptr = m.wg_tab, *bytes = (size_t)m.nwg * 16; return true;
+        case ASX_PLAN_ARRAY_WORKGROUPS: *ptr = m.wg_tab, *bytes = (size_t)m.npieces * 16; return true;
+        case ASX_PLAN_ARRAY_WG_PIECES: *ptr = m.wg_pieces, *bytes = (size_t)m.nwg * 32; return true;
         case ASX_PLAN_ARRAY_PARTIAL_ROWS: *ptr = m.prow, *bytes = (size_t)m.npartials * 2; return true;
         case ASX_PLAN_ARRAY_RANGES: *ptr = m.chunk_lo, *bytes = ((size_t)m.nrb + 1) * (size_t)m.nslices * 4; return true;
         case ASX_PLAN_ARRAY_STEP_PTR: *ptr = m.pstep_ptr, *bytes = ((size_t)m.nrb + 1) * 4; return true;

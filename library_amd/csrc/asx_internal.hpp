@@ -139,6 +139,7 @@ struct SlicedMatrix {
     int32_t ntiles;         // all slices; every slice starts a new tile and is padded to whole tiles
     int32_t npartials;      // partial sums written per call
     int32_t nwg;            // workgroups of pass 1
+    int32_t npieces;        // what they work off: runs of tiles inside one slice
     int32_t rows_per_wave;  // pass 2
     int32_t nrb;            // ceil(m / rows_per_wave)
     void *store;            // one allocation: val, perm, cf, tile_base, wg_tab, chunk_lo, pstep_ptr
@@ -148,7 +149,9 @@ struct SlicedMatrix {
     uint16_t *cf;           // ntiles * kSlicedTile: column inside the slice, bit 15 = first element of a run
     int32_t *perm;          // where each stored copy comes from in A's val (-1 for pads)
     int32_t *tile_base;     // ntiles + 1: index of the first partial sum of each tile
-    int32_t *wg_tab;        // nwg x 4: slice, first tile, end tile, 0
+    int32_t *wg_tab;        // npieces x 4: slice, first tile, end tile, 0
+    int32_t *wg_pieces;     // nwg x 8: first piece, end piece of each workgroup, 0, 0, then the first piece's four
+                            // words again (behind wg_tab in the store)
     uint16_t *prow;         // npartials + kSlicedReducePad: row of each partial sum inside its row block
     int32_t *chunk_lo;      // (nrb + 1) x nslices: first partial sum of row block b in slice s
     int32_t npsteps;        // steps of pass 2, all row blocks

@@ -397,8 +397,13 @@ __device__ __forceinline__ void store_staged(const T *stage, int lane, int total
     __builtin_amdgcn_wave_barrier();
 }
 
+// A workgroup takes the pieces wg_pieces[2 blockIdx.x].x .. .y - 1 of `pieces` in turn: tiles .y .. .z - 1
+// of slice .x each (nearly always one piece; two where the workgroup's share of the tiles reaches
+// over the end of a slice).  wg_pieces[2 blockIdx.x + 1] repeats the first of them, so that the
+// kernel's first loads wait for one read of a table, not two.
 template <typename T, int WIDTH, int NW, int D>
-__global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const int4 *__restrict__ wg_tab,
+__global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const int4 *__restrict__ wg_pieces,
+                                                               const int4 *__restrict__ pieces,
                                                                const uint16_t *__restrict__ cf,
                                                                const T *__restrict__ val,
                                                                const int32_t *__restrict__ tile_base,
@@ -406,33 +411,37 @@ __global__ __launch_bounds__(NW *kWave) void k_sliced_products(int32_t n, const 
 {
     __shared__ T xs[WIDTH];
     __shared__ T stage_all[NW * kStageRuns];
-    const int4 wg = wg_tab[blockIdx.x];
-    const int64_t c0 = (int64_t)wg.x * WIDTH;
-    const int32_t cnt = n - c0 < WIDTH ? (int32_t)(n - c0) : WIDTH;
+    const int4 mine = wg_pieces[2 * blockIdx.x];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     T *stage = stage_all + wave * kStageRuns;
-    // the first tiles' loads go out before the slice of x is fetched (they do not need it)
-    const int32_t last = wg.z - 1;
-    Tile<T> tl[D];
-    int32_t t = wg.y + wave;
+    for (int32_t pc = mine.x; pc < mine.y; ++pc) {  // uniform over the workgroup
+        const int4 wg = pc == mine.x ? wg_pieces[2 * blockIdx.x + 1] : pieces[pc];
+        const int64_t c0 = (int64_t)wg.x * WIDTH;
+        const int32_t cnt = n - c0 < WIDTH ? (int32_t)(n - c0) : WIDTH;
+        // the first tiles' loads go out before the slice of x is fetched (they do not need it)
+        const int32_t last = wg.z - 1;
+        Tile<T> tl[D];
+        int32_t t = wg.y + wave;
 #pragma unroll
-    for (int d = 0; d < D; ++d) tile_load<T>(tl[d], t + d * NW < last ? t + d * NW : last, lane, cf, val, tile_base);
-    load_x_window<T, WIDTH, NW * kWave>(xs, x, c0, cnt);
-    __syncthreads();
-    // D tiles in turn; a tile's loads are issued D steps ahead, right after the stores of the tile
-    // that used the buffer before it.  The loads are unconditional (past the end they re-read the
-    // last tile), so that the number of memory operations issued after them is known and a step
-    // waits for its own loads only.
-    while (t < wg.z) {  // uniform over the wave
+        for (int d = 0; d < D; ++d) tile_load<T>(tl[d], t + d * NW < last ? t + d * NW : last, lane, cf, val, tile_base);
+        if (pc != mine.x) __syncthreads();  // every wave is done with the slice before
+        load_x_window<T, WIDTH, NW * kWave>(xs, x, c0, cnt);
+        __syncthreads();
+        // D tiles in turn; a tile's loads are issued D steps ahead, right after the stores of the tile
+        // that used the buffer before it.  The loads are unconditional (past the end they re-read the
+        // last tile), so that the number of memory operations issued after them is known and a step
+        // waits for its own loads only.
+        while (t < wg.z) {  // uniform over the wave
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
-            if (t + d * NW < wg.z) {
-                const int total = tile_reduce<T>(tl[d], lane, xs, StageRun<T>{stage});
-                store_staged<T>(stage, lane, total, partial + tl[d].base);
+            for (int d = 0; d < D; ++d) {
+                if (t + d * NW < wg.z) {
+                    const int total = tile_reduce<T>(tl[d], lane, xs, StageRun<T>{stage});
+                    store_staged<T>(stage, lane, total, partial + tl[d].base);
+                }
+                tile_load<T>(tl[d], t + (D + d) * NW < last ? t + (D + d) * NW : last, lane, cf, val, tile_base);
             }
-            tile_load<T>(tl[d], t + (D + d) * NW < last ? t + (D + d) * NW : last, lane, cf, val, tile_base);
+            t += D * NW;
         }
-        t += D * NW;
     }
 }
 
@@ -623,7 +632,7 @@ void free_sliced(SlicedMatrix *p)
         if (q) (void)hipFree(q);
     p->store = p->val = p->partial = nullptr;
     p->cf = p->prow = nullptr;
-    p->perm = p->tile_base = p->wg_tab = p->chunk_lo = p->pstep_ptr = p->psteps = nullptr;
+    p->perm = p->tile_base = p->wg_tab = p->wg_pieces = p->chunk_lo = p->pstep_ptr = p->psteps = nullptr;
 }
 
 template <typename T>
@@ -657,7 +666,7 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
     int32_t *lrow = nullptr, *tile_cnt = nullptr, *step_cnt = nullptr;
     int32_t *tmp = nullptr;
     std::vector<int32_t> pstart((size_t)sm.nslices + 1), tile_off((size_t)sm.nslices + 1, 0);
-    std::vector<int32_t> tab;
+    std::vector<int32_t> tab, wgs;
     int64_t slots = 0;
     bool empty_slice = false;
     const size_t max_tiles = (size_t)ceil_div64(cap64, kSlicedTile);
@@ -707,35 +716,60 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
     sm.ntiles = tile_off[sm.nslices];
     slots = (int64_t)sm.ntiles * kSlicedTile;
     ASX_TRY(hipMemcpyAsync(d_tile_off, tile_off.data(), sizeof(int32_t) * tile_off.size(), hipMemcpyHostToDevice, s));
-    //    workgroups of pass 1: every slice gets its share of about `target_wgs` workgroups (at
-    //    least one, and no workgroup smaller than 32 tiles unless the slice is), its tiles in equal
-    //    pieces
+    //    workgroups of pass 1: about `target_wgs` equal shares of the tiles, whatever slices they lie
+    //    in (a share per slice, rounded, left 270 workgroups for 256 compute units where 54 slices
+    //    wanted 4.7 each: two rounds).  A cut that falls within 32 tiles of the start of a slice
+    //    moves there; a share that still reaches over such a start is worked off as two pieces,
+    //    one slice of x after the other.  No share smaller than 32 tiles unless there is only one.
     {
-        for (int32_t sl = 0; sl < sm.nslices; ++sl) {
-            const int32_t tiles = tile_off[sl + 1] - tile_off[sl];
-            if (tiles == 0) continue;
-            int32_t pieces = (int32_t)(((int64_t)tiles * target_wgs + sm.ntiles / 2) / sm.ntiles);
-            pieces = std::min<int32_t>(pieces, tiles / 32);
-            pieces = std::max<int32_t>(pieces, 1);
-            for (int32_t k = 0; k < pieces; ++k) {
-                tab.push_back(sl);
-                tab.push_back(tile_off[sl] + (int32_t)((int64_t)tiles * k / pieces));
-                tab.push_back(tile_off[sl] + (int32_t)((int64_t)tiles * (k + 1) / pieces));
-                tab.push_back(0);
-            }
+        const int64_t nt = sm.ntiles;
+        const int32_t shares = (int32_t)std::max<int64_t>(1, std::min<int64_t>(target_wgs, nt / 32));
+        std::vector<int32_t> cuts((size_t)shares + 1);
+        for (int32_t k = 0; k <= shares; ++k) {
+            int32_t c = (int32_t)(nt * k / shares);
+            // the start of a slice nearest to c, when fewer than 32 tiles away
+            const auto at = std::lower_bound(tile_off.begin(), tile_off.end(), c);
+            const int32_t above = at != tile_off.end() ? *at - c : 32, below = at != tile_off.begin() ? c - *(at - 1) : 32;
+            if (above < 32 && above <= below)
+                c += above;
+            else if (below < 32)
+                c -= below;
+            cuts[(size_t)k] = k == 0 ? 0 : k == shares ? (int32_t)nt : std::max(c, cuts[(size_t)k - 1]);
         }
-        sm.nwg = (int32_t)(tab.size() / 4);
-        // The workgroups of a slice all fetch that slice of x: keep them on one XCD, whose L2 then
-        // fetches it once (workgroup i runs on XCD i mod kXcds; entry j of the list above goes to
-        // position (j mod per_xcd) * kXcds + j / per_xcd, so consecutive entries share an XCD).
-        if (sm.nwg > sm.nslices && sm.nwg % kXcds == 0) {
+        int32_t sl = 0;
+        for (int32_t k = 0; k < shares; ++k) {
+            const int32_t lo = cuts[(size_t)k], hi = cuts[(size_t)k + 1];
+            if (hi <= lo) continue;
+            const int32_t first_piece = (int32_t)(tab.size() / 4);
+            while (tile_off[(size_t)sl + 1] <= lo) ++sl;  // the slice that holds tile lo
+            for (int32_t a = lo; a < hi;) {
+                while (tile_off[(size_t)sl + 1] <= a) ++sl;
+                const int32_t z = std::min(hi, tile_off[(size_t)sl + 1]);
+                tab.push_back(sl);
+                tab.push_back(a);
+                tab.push_back(z);
+                tab.push_back(0);
+                a = z;
+            }
+            wgs.push_back(first_piece);
+            wgs.push_back((int32_t)(tab.size() / 4));
+            wgs.push_back(0);
+            wgs.push_back(0);
+            for (int q = 0; q < 4; ++q) wgs.push_back(tab[(size_t)first_piece * 4 + q]);  // the first piece again
+        }
+        sm.npieces = (int32_t)(tab.size() / 4);
+        sm.nwg = (int32_t)(wgs.size() / 8);
+        // Workgroups next to each other in this list share slices of x: keep them on one XCD, whose
+        // L2 then fetches a slice once (workgroup i runs on XCD i mod kXcds; entry j of the list goes
+        // to position (j mod per_xcd) * kXcds + j / per_xcd, so consecutive entries share an XCD).
+        if (sm.nwg % kXcds == 0 && sm.nwg > 0) {
             const int32_t per_xcd = sm.nwg / kXcds;
-            std::vector<int32_t> placed(tab.size());
+            std::vector<int32_t> placed(wgs.size());
             for (int32_t j = 0; j < sm.nwg; ++j) {
                 const int32_t i = (j % per_xcd) * kXcds + j / per_xcd;
-                for (int q = 0; q < 4; ++q) placed[(size_t)i * 4 + q] = tab[(size_t)j * 4 + q];
+                for (int q = 0; q < 8; ++q) placed[(size_t)i * 8 + q] = wgs[(size_t)j * 8 + q];
             }
-            tab.swap(placed);
+            wgs.swap(placed);
         }
     }
     {   // what the plan keeps and whose size is known by now, in one allocation
@@ -747,14 +781,16 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
         };
         const size_t o_val = take(sizeof(T) * (size_t)slots), o_perm = take(sizeof(int32_t) * (size_t)slots);
         const size_t o_cf = take(sizeof(uint16_t) * (size_t)slots), o_tb = take(sizeof(int32_t) * ((size_t)sm.ntiles + 1));
-        const size_t o_wg = take(sizeof(int32_t) * std::max<size_t>(tab.size(), 4));
+        const size_t o_wg = take(sizeof(int32_t) * std::max<size_t>(tab.size() + wgs.size(), 4));
         const size_t o_cl = take(sizeof(int32_t) * (size_t)ncells), o_sp = take(sizeof(int32_t) * ((size_t)sm.nrb + 1));
         ASX_TRY(hipMalloc(&sm.store, off));
         char *base = static_cast<char *>(sm.store);
         sm.val = base + o_val, sm.perm = (int32_t *)(base + o_perm), sm.cf = (uint16_t *)(base + o_cf);
         sm.tile_base = (int32_t *)(base + o_tb), sm.wg_tab = (int32_t *)(base + o_wg);
         sm.chunk_lo = (int32_t *)(base + o_cl), sm.pstep_ptr = (int32_t *)(base + o_sp);
+        sm.wg_pieces = sm.wg_tab + tab.size();
         ASX_TRY(hipMemcpyAsync(sm.wg_tab, tab.data(), sizeof(int32_t) * tab.size(), hipMemcpyHostToDevice, s));
+        ASX_TRY(hipMemcpyAsync(sm.wg_pieces, wgs.data(), sizeof(int32_t) * wgs.size(), hipMemcpyHostToDevice, s));
     }
     // 3. every stored element to its slot; the pads behind every slice
     {
@@ -837,8 +873,8 @@ int launch_spmv_sliced(int32_t m, int32_t n, T alpha, const SlicedMatrix *sm, co
     const int4 *tab = reinterpret_cast<const int4 *>(sm->wg_tab);
     constexpr int kDepth = 2;  // tiles in flight per wave (3 and 4 measured the same or slower)
 #define ASX_PROD(W)                                                                                                 \
-    hipLaunchKernelGGL((k_sliced_products<T, W, 16, kDepth>), dim3((unsigned)sm->nwg), dim3(16 * kWave), 0, s, n, tab, \
-                       sm->cf, (const T *)sm->val, sm->tile_base, x, partial)
+    hipLaunchKernelGGL((k_sliced_products<T, W, 16, kDepth>), dim3((unsigned)sm->nwg), dim3(16 * kWave), 0, s, n,      \
+                       reinterpret_cast<const int4 *>(sm->wg_pieces), tab, sm->cf, (const T *)sm->val, sm->tile_base, x, partial)
     if (sm->nwg > 0) {
         if (sm->width == kLarge)
             ASX_PROD(kLarge);

@@ -165,15 +165,23 @@ def check_sliced(arrays, rp, col, n, width, rows_per_wave, itemsize):
     if bad.size:
         b, s = map(int, bad[0])
         raise PlanError(f"range start of row block {b} in slice {s} is {int(ranges[b, s])}, expected {int(ref['ranges'][b, s])}")
-    # workgroups of pass 1: every tile of every slice in exactly one
+    # pass 1: every tile of every slice in exactly one piece, every piece inside one slice, every
+    # piece worked off by exactly one workgroup
     wg = np.asarray(arrays["workgroups"], np.int64).reshape(-1, 4)
-    _need(np.all(wg[:, 2] > wg[:, 1]), "a workgroup of pass 1 without tiles")
+    _need(np.all(wg[:, 2] > wg[:, 1]), "a piece of pass 1 without tiles")
+    wp = np.asarray(arrays["wg_pieces"], np.int64).reshape(-1, 8)
+    _need(np.all(wp[:, 1] > wp[:, 0]) and np.all(wp[:, 0] >= 0) and np.all(wp[:, 1] <= wg.shape[0]), "a workgroup of pass 1 without pieces")
+    _need(np.array_equal(wp[:, 4:8], wg[wp[:, 0]]), "a workgroup's copy of its first piece differs from the piece")
+    taken = np.zeros(wg.shape[0] + 1, np.int64)
+    np.add.at(taken, wp[:, 0], 1)
+    np.add.at(taken, wp[:, 1], -1)
+    _need(np.all(np.cumsum(taken)[:-1] == 1), "the workgroups of pass 1 do not take every piece exactly once")
     covered = np.zeros(ref["ntiles"] + 1, np.int64)
     np.add.at(covered, wg[:, 1], 1)
     np.add.at(covered, wg[:, 2], -1)
-    _need(np.all(np.cumsum(covered)[:-1] == 1), "the workgroups of pass 1 do not cover every tile exactly once")
+    _need(np.all(np.cumsum(covered)[:-1] == 1), "the pieces of pass 1 do not cover every tile exactly once")
     _need(np.all(ref["tile_off"][wg[:, 0]] <= wg[:, 1]) and np.all(wg[:, 2] <= ref["tile_off"][wg[:, 0] + 1]),
-          "a workgroup's tiles leave its slice")
+          "a piece's tiles leave its slice")
     check_sliced_steps(arrays["step_ptr"], arrays["steps"], ranges)
 
 
@@ -247,6 +255,7 @@ def sliced_plan_arrays(rp, col, n, width, rows_per_wave, itemsize):
     wg = [[s, to[s], to[s + 1], 0] for s in range(nslices) if to[s + 1] > to[s]]
     return dict(perm=perm_phys.reshape(-1).astype(np.int32), cf=ref["cf"].astype(np.uint16),
                 tile_words=ref["tile_base"].astype(np.int32), workgroups=np.array(wg, np.int32).reshape(-1),
+                wg_pieces=np.array([[i, i + 1, 0, 0] + wg[i] for i in range(len(wg))], np.int32).reshape(-1),
                 partial_rows=ref["prow"].astype(np.uint16), ranges=ref["ranges"].astype(np.int32).reshape(-1),
                 step_ptr=step_ptr, steps=steps.reshape(-1))
 
@@ -533,7 +542,7 @@ def export_all(plan, names, value_dtype=None):
     return {k: plan.export(k, value_dtype) for k in held}
 
 
-SLICED_ARRAYS = ("perm", "cf", "tile_words", "workgroups", "partial_rows", "ranges", "step_ptr", "steps")
+SLICED_ARRAYS = ("perm", "cf", "tile_words", "workgroups", "wg_pieces", "partial_rows", "ranges", "step_ptr", "steps")
 WINDOW_ARRAYS = ("perm", "cf", "tile_words", "blocks", "pieces", "workgroups")
 
 

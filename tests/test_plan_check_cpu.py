@@ -79,6 +79,14 @@ def test_sliced_corruptions_are_rejected():
         p["workgroups"].reshape(-1, 4)[0, 2] -= 1
     corrupt("workgroups", workgroups)
 
+    def piece_taken_twice(p):  # two workgroups of pass 1 would write the same partial sums; another piece is left out
+        p["wg_pieces"].reshape(-1, 8)[1] = p["wg_pieces"].reshape(-1, 8)[0]
+    corrupt("every piece exactly once", piece_taken_twice)
+
+    def stale_copy_of_the_first_piece(p):
+        p["wg_pieces"].reshape(-1, 8)[2, 6] -= 1
+    corrupt("copy of the first piece", stale_copy_of_the_first_piece)
+
 
 def _banded(seed, m, n, half, dens, cut_rows=True):
     rng = np.random.default_rng(seed)
