@@ -778,6 +778,35 @@ def test_spmv_sliced_wide_steps(torch, capi, oracle):
         plan.destroy()
 
 
+def test_spmv_sliced_workgroups_that_reach_over_the_end_of_a_slice(torch, capi, oracle):
+    """Pass 1 hands its workgroups equal shares of all tiles; a share that reaches over the start
+    of a slice (further than 32 tiles on either side) is worked off as two pieces with two slices of x,
+    one after the other.  Three slices and about a hundred tiles per share: workgroups of two pieces,
+    and every workgroup's share within a tile or so of the others'."""
+    W = pytest.importorskip("library_amd.workloads")
+    rng = np.random.default_rng(181)
+    for dtype, m, n, k in ((np.float64, 400000, 40000, 16), (np.float32, 400000, 90000, 16)):
+        rp, col, val = W.csr_fixed(m, n, k, dtype, seed=5)
+        x = rng.uniform(-1, 1, n).astype(dtype)
+        y0 = rng.uniform(-1, 1, m).astype(dtype)
+        d = [dev(torch, a) for a in (rp, col, val, x)]
+        plan = capi.Plan(False, capi.SPMV_SLICED, np.dtype(dtype), m, n, col.size, d[0], col=d[1], val=d[2])
+        plan_check.check_plan(plan, capi, rp, col, n, np.dtype(dtype).itemsize)
+        assert plan.info("slices") == 3
+        pieces = plan.export("workgroups").reshape(-1, 4)
+        wgs = plan.export("wg_pieces").reshape(-1, 8)
+        assert wgs.shape[0] == plan.info("workgroups") and (wgs[:, 1] - wgs[:, 0]).max() == 2, "a workgroup of two pieces expected"
+        share = np.array([(pieces[a:b, 2] - pieces[a:b, 1]).sum() for a, b in wgs[:, :2]])
+        assert share.max() - share.min() <= 64 and share.sum() == plan.info("tiles"), (share.min(), share.max())
+        for alpha, beta in ((1.5, 0.5), (1.0, 0.0)):
+            ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 4)
+            y = dev(torch, y0 if beta else np.full(m, np.nan, dtype=dtype))
+            capi.spmv(d[0], d[1], d[2], d[3], y, alpha, beta, alg=capi.SPMV_SLICED, plan=plan)
+            torch.cuda.synchronize()
+            assert_close(y.cpu().numpy(), ref, spmv_scale(rp, col, val, x, alpha, beta, y0), dtype, f"{np.dtype(dtype).name} a={alpha} b={beta}")
+        plan.destroy()
+
+
 def _diagonal_bands(rng, m, n, bands, dens, dtype, empty=0.05):
     """Rows whose columns lie on bands of diagonals: for every (lo, hi) in `bands` the columns
     centre + lo .. centre + hi (centre = r n // m) that fall inside the matrix, a fraction `dens`
