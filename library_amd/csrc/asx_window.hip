@@ -860,15 +860,31 @@ int build_window(int32_t m, int32_t n, int32_t nnz, int32_t target_wgs, bool in_
     wm.by_reference = in_place && h_small[13] == 0;
     halves = wm.by_reference && sizeof(T) == 8;
     wm.rows_per_block = 0;
-    for (int k = 0; k < kCandidates; ++k) {
-        const int32_t rows = kBlockRows[k];
-        if (rows > 256 && ceil_div64(m, rows) < min_blocks) continue;
-        if (h_small[k] <= kWindowCols - kWindowSlack) {
+    {
+        // Of the sizes whose windows fit, the one with the shortest longest chain: a workgroup walks
+        // ceil(blocks / workgroups) blocks, each of which costs its rows (at a workgroup's share of
+        // 5.6 TB/s) and about 1.1 us to start.  4.5 M rows of a 5-point stencil on 256 workgroups:
+        // 1099 blocks of 4096 rows make chains of 5 (20480 rows), 1465 blocks of 3072 chains of 6
+        // (18432 rows).  A block past the first of a chain may fetch kFetchCols columns at most, so
+        // sizes that advance further than that along the columns are left out.
+        const double row_bytes = (double)nnz / (double)m * (double)(sizeof(T) + 2) + 3.0 * (double)sizeof(T);
+        const double row_time = row_bytes / (5.6e12 / (double)target_wgs), start_time = 1.1e-6;
+        double best = 0.0;
+        int best_k = -1;
+        for (int k = 0; k < kCandidates; ++k) {
+            const int32_t rows = kBlockRows[k];
+            if (rows > 256 && ceil_div64(m, rows) < min_blocks) continue;
+            if (h_small[k] > kWindowCols - kWindowSlack) continue;
+            if (rows > 256 && (double)rows * (double)n / (double)m > (double)kFetchCols) continue;
+            const double chain = (double)ceil_div64(ceil_div64(m, rows), target_wgs) * ((double)rows * row_time + start_time);
+            if (best_k < 0 || chain < best * 0.98) best = chain, best_k = k;  // a larger size unless a smaller one is clearly ahead
+        }
+        if (best_k >= 0) {
+            const int32_t rows = kBlockRows[best_k];
             wm.rows_per_block = rows;
             wm.nblocks = (int32_t)ceil_div64(m, rows);
             hipLaunchKernelGGL(k_window_block_span, dim3((unsigned)ceil_div64(wm.nblocks, kBlock)), dim3(kBlock), 0, s, gmin,
                                gmax, ngroups, rows / kSpanGroup, wm.nblocks, bmin, bmax, d_small + 15);
-            break;
         }
     }
     bands.nbands = 1;
