@@ -241,9 +241,43 @@ def _step_words(base, first, fill):
     return [b[0], b[1], b[2], f[1] | f[2] << 8 | fill << 16]
 
 
-def sliced_plan_arrays(rp, col, n, width, rows_per_wave, itemsize):
+def split_tiles(tile_off, shares):
+    """Pass 1's work: `shares` equal shares of the tiles (no share below 32 tiles unless there is
+    one only), a cut within 32 tiles of the start of a slice moved there, every share cut into
+    pieces at the starts of slices.  Returns (pieces x 4, workgroups x 8) as a plan holds them."""
+    tile_off = np.asarray(tile_off, np.int64)
+    nt = int(tile_off[-1])
+    shares = max(1, min(shares, nt // 32))
+    cuts = [0]
+    for k in range(1, shares + 1):
+        c = nt * k // shares
+        at = int(np.searchsorted(tile_off, c, side="left"))
+        above = int(tile_off[at]) - c if at < tile_off.size else 32
+        below = c - int(tile_off[at - 1]) if at > 0 else 32
+        if above < 32 and above <= below:
+            c += above
+        elif below < 32:
+            c -= below
+        cuts.append(nt if k == shares else max(c, cuts[-1]))
+    pieces, wgs = [], []
+    for lo, hi in zip(cuts[:-1], cuts[1:]):
+        if hi <= lo:
+            continue
+        first = len(pieces)
+        a = lo
+        while a < hi:
+            sl = int(np.searchsorted(tile_off, a, side="right")) - 1
+            z = min(hi, int(tile_off[sl + 1]))
+            pieces.append([sl, a, z, 0])
+            a = z
+        wgs.append([first, len(pieces), 0, 0] + pieces[first])
+    return np.array(pieces, np.int32).reshape(-1), np.array(wgs, np.int32).reshape(-1)
+
+
+def sliced_plan_arrays(rp, col, n, width, rows_per_wave, itemsize, shares=None):
     """A whole sliced plan built on the host from its definition, in the layout Plan.export gives
-    (one workgroup of pass 1 per slice that has tiles)."""
+    (one workgroup of pass 1 per slice that has tiles, or, with `shares`, that many equal shares
+    of the tiles as the library's builder hands them out)."""
     rp = np.asarray(rp, np.int64)
     col = np.asarray(col, np.int64)
     nslices = -(-n // width)
@@ -253,9 +287,11 @@ def sliced_plan_arrays(rp, col, n, width, rows_per_wave, itemsize):
     step_ptr, steps = pack_steps(ref["ranges"])
     to = ref["tile_off"]
     wg = [[s, to[s], to[s + 1], 0] for s in range(nslices) if to[s + 1] > to[s]]
+    pieces, wgs = np.array(wg, np.int32).reshape(-1), np.array([[i, i + 1, 0, 0] + wg[i] for i in range(len(wg))], np.int32).reshape(-1)
+    if shares:
+        pieces, wgs = split_tiles(to, shares)
     return dict(perm=perm_phys.reshape(-1).astype(np.int32), cf=ref["cf"].astype(np.uint16),
-                tile_words=ref["tile_base"].astype(np.int32), workgroups=np.array(wg, np.int32).reshape(-1),
-                wg_pieces=np.array([[i, i + 1, 0, 0] + wg[i] for i in range(len(wg))], np.int32).reshape(-1),
+                tile_words=ref["tile_base"].astype(np.int32), workgroups=pieces, wg_pieces=wgs,
                 partial_rows=ref["prow"].astype(np.uint16), ranges=ref["ranges"].astype(np.int32).reshape(-1),
                 step_ptr=step_ptr, steps=steps.reshape(-1))
 

@@ -798,6 +798,14 @@ def test_spmv_sliced_workgroups_that_reach_over_the_end_of_a_slice(torch, capi, 
         assert wgs.shape[0] == plan.info("workgroups") and (wgs[:, 1] - wgs[:, 0]).max() == 2, "a workgroup of two pieces expected"
         share = np.array([(pieces[a:b, 2] - pieces[a:b, 1]).sum() for a, b in wgs[:, :2]])
         assert share.max() - share.min() <= 64 and share.sum() == plan.info("tiles"), (share.min(), share.max())
+        # the same pieces as the rule restated on the host gives for one share per compute unit
+        cus = capi.C.c_int(0)
+        assert capi.lib().asx_device_info(capi.C.byref(cus), None) == 0
+        width = 131072 // np.dtype(dtype).itemsize
+        tile_off = np.r_[0, np.cumsum(-(-np.bincount(col // width, minlength=3) // 256))]
+        want_pieces, want_wgs = plan_check.split_tiles(tile_off, cus.value)
+        assert np.array_equal(pieces.reshape(-1), want_pieces)
+        assert sorted(map(tuple, wgs.tolist())) == sorted(map(tuple, want_wgs.reshape(-1, 8).tolist()))
         for alpha, beta in ((1.5, 0.5), (1.0, 0.0)):
             ref = oracle.spmv(rp, col, val, x, dtype(alpha), dtype(beta), y0 if beta else np.zeros_like(y0), 4)
             y = dev(torch, y0 if beta else np.full(m, np.nan, dtype=dtype))

@@ -22,6 +22,32 @@ def test_sliced_plan_from_its_definition_passes(itemsize, width):
     pc.check_sliced(plan, rp, col, n, width, 256, itemsize)
 
 
+def test_sliced_shares_of_tiles_across_slices():
+    """Pass 1's workgroups as equal shares of the tiles: shares that reach over the start of a slice
+    become two pieces, cuts near such a start move onto it, and the plan still passes."""
+    rng = np.random.default_rng(5)
+    m, n, width = 30000, 40000, 16384  # three slices
+    lens = np.full(m, 12)
+    rp = np.r_[0, np.cumsum(lens)].astype(np.int32)
+    col = np.sort(rng.integers(0, n, (m, 12)), axis=1).reshape(-1).astype(np.int32)
+    for shares in (1, 3, 7, 10, 40):
+        plan = pc.sliced_plan_arrays(rp, col, n, width, 256, 8, shares=shares)
+        pc.check_sliced(plan, rp, col, n, width, 256, 8)
+        wgs, pieces = plan["wg_pieces"].reshape(-1, 8), plan["workgroups"].reshape(-1, 4)
+        ntiles = int(pieces[:, 2].max())
+        size = np.array([(pieces[a:b, 2] - pieces[a:b, 1]).sum() for a, b in wgs[:, :2]])
+        assert size.sum() == ntiles
+        if shares <= 10:  # shares of more than 64 tiles: none vanishes when its cuts move, and they stay alike
+            assert wgs.shape[0] == shares and size.max() - size.min() <= 64
+        else:
+            assert wgs.shape[0] <= min(shares, ntiles // 32)
+    assert (pc.sliced_plan_arrays(rp, col, n, width, 256, 8, shares=7)["wg_pieces"].reshape(-1, 8)[:, 1:2]
+            - pc.sliced_plan_arrays(rp, col, n, width, 256, 8, shares=7)["wg_pieces"].reshape(-1, 8)[:, 0:1]).max() == 2
+    # a cut 10 tiles behind the start of a slice moves onto it
+    pieces, wgs = pc.split_tiles(np.array([0, 110, 400]), 4)  # cuts at 100, 200, 300
+    assert pieces.reshape(-1, 4)[:, 1:3].tolist() == [[0, 110], [110, 200], [200, 300], [300, 400]]
+
+
 def test_sliced_corruptions_are_rejected():
     rp, col, n = _scattered()
     good = pc.sliced_plan_arrays(rp, col, n, 16384, 256, 8)
