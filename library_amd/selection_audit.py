@@ -103,6 +103,13 @@ def families():
     fams.append(("hypersparse: 1 in 4 of 12M rows holds 1 element near the diagonal, float64", np.float64,
                  lambda: _near_diagonal(12 << 20, 12 << 20, 1, 100, rng, keep=0.25) + (12 << 20,)))
     fams.append(("2 scattered per row, 4M x 4M, float64", np.float64, lambda: fixed(1 << 22, 1 << 22, 2, np.float64)))
+    # sizes that are no powers of two: slices that do not divide the workgroups, blocks that do not divide the rows
+    fams.append(("uniform 16/row, 1048576 x 1300000 (80 slices), float64", np.float64, lambda: fixed(1 << 20, 1300000, 16, np.float64)))
+    fams.append(("uniform 16/row, 1500000 x 700000 (22 slices), float32", np.float32, lambda: fixed(1500000, 700000, 16, np.float32)))
+    fams.append(("uniform 16/row, 700001 x 2500000 (153 slices), float64", np.float64, lambda: fixed(700001, 2500000, 16, np.float64)))
+    fams.append(("5-point stencil 3000 x 1500, float64", np.float64, lambda: W.csr_stencil5(3000, 1500)[:2] + (3000 * 1500,)))
+    fams.append(("7-point stencil 200 x 150 x 100, float64", np.float64, lambda: _stencil3d(200, 150, 100, 7) + (200 * 150 * 100,)))
+    fams.append(("band of 9, 3000001 rows, float64", np.float64, lambda: W.csr_banded(3000001, 4, np.float64, seed=3)[:2] + (3000001,)))
     return fams
 
 
