@@ -23,6 +23,9 @@ Per workload, on the GPU:
   unchanged_caller_ms   SpMV: what a caller that never calls the analysis gets by default through the
                   generic API: a plan made on first use that may hold a copy of the values, checked
                   against the caller's values by checksum in every call (unchanged_caller_kernel)
+  changing_caller_ms    the same caller when the values do change in place before every call (the copy,
+                  where the plan holds one, is brought up to date inside the call)
+  update_values_ms      asx_plan_update_values on the plan of ms_per_step (0 where it holds no values)
 and on the host (unless --no-cpu), the reference's own CPU kernels (oracle/_ref, kind
 "reference") or their C restatement (kind "port") on the same inputs: all physical cores of the
 box's share, and one thread.
@@ -170,7 +173,7 @@ def measure(w, steps, warmup, alg):
     #     change in place): analysis on first use that may keep a copy of the values, and in every
     #     call two checksums of the caller's values on the device with a refresh of the copy where
     #     they differ.  DEFAULT's choice counts that read, so the kernel may be another one.
-    checked_ms, checked_kernel = None, None
+    checked_ms, checked_kernel, changing_ms, update_ms = None, None, None, None
     if not spmm:
         cplan = capi.Plan(False, alg, w.val.dtype, w.m, w.n, w.nnz, d_rp, col=d_col, val=d_val, checked=True)
         checked_kernel = KERNEL_NAMES.get(cplan.alg, str(cplan.alg)) + (" + checksum" if cplan.checked else "")
@@ -189,7 +192,38 @@ def measure(w, steps, warmup, alg):
         e1.record()
         torch.cuda.synchronize()
         checked_ms = e0.elapsed_time(e1) / nrep
+        # the same with values that differ from one call to the next (two arrays that differ in one
+        # element, passed in turn: what the plan sees is its values changed in place)
+        d_val2 = d_val.clone()
+        d_val2[w.nnz // 2] += 1.0
+        vals = (d_val2, d_val)
+
+        def step_changing(i):
+            cplan.refresh_if_changed(vals[i & 1])
+            capi.spmv(d_rp, d_col, vals[i & 1], d_x, d_y, w.alpha, w.beta, plan=cplan, workspace=ws3)
+
+        for i in range(4):
+            step_changing(i)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(nrep):
+            step_changing(i)
+        e1.record()
+        torch.cuda.synchronize()
+        changing_ms = e0.elapsed_time(e1) / nrep
+        cplan.refresh_if_changed(d_val)
         cplan.destroy()
+        del d_val2
+        # and what the caller of an explicit analysis pays to say that the values changed
+        for _ in range(3):
+            plan.update_values(d_val)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(nrep):
+            plan.update_values(d_val)
+        e1.record()
+        torch.cuda.synchronize()
+        update_ms = e0.elapsed_time(e1) / nrep if plan.holds_values else 0.0
     nbytes = w.bytes_algorithmic()
     res = {
         "workload": w.name, "kind": w.kind, "dtype": "f64" if w.dtype.itemsize == 8 else "f32",
@@ -204,6 +238,8 @@ def measure(w, steps, warmup, alg):
         "cold_ms_median": float(np.median(cold)),
         "noplan_ms": float(noplan_ms),
         "unchanged_caller_ms": None if checked_ms is None else float(checked_ms), "unchanged_caller_kernel": checked_kernel,
+        "changing_caller_ms": None if changing_ms is None else float(changing_ms),
+        "update_values_ms": None if update_ms is None else float(update_ms),
     }
     res["gbs"] = nbytes / (wall_ms * 1e-3) / 1e9
     res["gflops"] = w.flops / (wall_ms * 1e-3) / 1e9

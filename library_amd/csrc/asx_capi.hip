@@ -707,15 +707,16 @@ int plan_add_window(asx_plan *p, const int32_t *d_row_ptr, const int32_t *d_col,
 // call), so a matrix where that padding exceeds a quarter of its stored elements stays with the
 // other kernels.
 // A regrouped copy roughly doubles what the matrix takes on the device (per stored element: the
-// value, 2 bytes of column, 4 bytes of source index; the sliced kernel also keeps a buffer for the
-// partial sums of a call), and its build needs about 4 bytes per stored element more for a while.
+// value, 2 bytes of column, 4 bytes of source index; the sliced kernel also 2 bytes for bringing
+// the values up to date and a buffer for the partial sums of a call), and its build needs about 4
+// bytes per stored element more for a while.
 // DEFAULT only makes one while twice that is free: a caller who sized the device for one copy of A
 // is not pushed to the edge by an analysis call.
 static bool regrouped_copy_fits(const asx_plan *p, size_t sv)
 {
     size_t free_b = 0, total_b = 0;
     if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) return false;
-    const double copy = (double)p->nnz * (double)(sv + 6) + (double)p->nnz * (double)(sv + 2) + (double)p->nnz * 4.0;
+    const double copy = (double)p->nnz * (double)(sv + 8) + (double)p->nnz * (double)(sv + 2) + (double)p->nnz * 4.0;
     return (double)free_b >= 2.0 * copy;
 }
 

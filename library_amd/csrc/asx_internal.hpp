@@ -150,6 +150,9 @@ struct SlicedMatrix {
     int32_t *perm;          // where each stored copy comes from in A's val (-1 for pads)
     int32_t *tile_base;     // ntiles + 1: index of the first partial sum of each tile
     int32_t *wg_tab;        // npieces x 4: slice, first tile, end tile, 0
+    int32_t nnz, nsort_blocks;  // stored elements; blocks of 4096 of them, as the build sorted them
+    uint16_t *pos;          // nnz: position of each stored element among its block's elements in slice order
+    int32_t *block_base;    // (nsort_blocks + 1) x nslices: slot of a block's first element of each slice (last row: the slices' ends)
     int32_t *wg_pieces;     // nwg x 8: first piece, end piece of each workgroup, 0, 0, then the first piece's four
                             // words again (behind wg_tab in the store)
     uint16_t *prow;         // npartials + kSlicedReducePad: row of each partial sum inside its row block

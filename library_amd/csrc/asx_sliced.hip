@@ -123,7 +123,8 @@ __global__ __launch_bounds__(kSortThreads) void k_sliced_scatter(
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col, const T *__restrict__ val,
     const int32_t *__restrict__ seg_row, int32_t m, int32_t nnz, int32_t width, int32_t nslices, int32_t nbits,
     int32_t nblocks, const int32_t *__restrict__ offs, const int32_t *__restrict__ tile_off, int32_t *__restrict__ lrow,
-    uint16_t *__restrict__ cf, T *__restrict__ val_out, int32_t *__restrict__ perm)
+    uint16_t *__restrict__ cf, T *__restrict__ val_out, int32_t *__restrict__ perm, uint16_t *__restrict__ pos,
+    int32_t *__restrict__ block_base)
 {
     __shared__ int32_t cnt[kSortWaves * MAXS];  // per wave and slice: count, then first rank of the wave's elements
     __shared__ int32_t lofs[MAXS];              // per slice: the block's count, then its first position in slice order
@@ -178,6 +179,11 @@ __global__ __launch_bounds__(kSortThreads) void k_sliced_scatter(
         }
         lofs[s] = run;
         gbase[s] = tile_off[s] * kSlicedTile + offs[(int64_t)s * nblocks + b] - offs[(int64_t)s * nblocks];
+        // for k_sliced_rescatter: where the block's elements of every slice start (row nblocks: where the slice's end)
+        block_base[(int64_t)b * nslices + s] = gbase[s];
+        if (b == nblocks - 1)
+            block_base[(int64_t)nblocks * nslices + s] =
+                tile_off[s] * kSlicedTile + offs[(int64_t)s * nblocks + nblocks] - offs[(int64_t)s * nblocks];
     }
     __syncthreads();
     block_exclusive_sum(lofs, nslices, wave_tot);
@@ -198,6 +204,7 @@ __global__ __launch_bounds__(kSortThreads) void k_sliced_scatter(
             const int32_t in_slice = mycnt[key] + rk[k];
             const int32_t p = lofs[key] + in_slice;
             rk[k] = p;
+            pos[i] = (uint16_t)p;
             dest[p] = gbase[key] + in_slice;
             row_s[p] = row_holding(row_ptr, r_lo, r_hi, (int32_t)i);
             src_s[p] = (int32_t)i;
@@ -355,20 +362,65 @@ __global__ __launch_bounds__(kBlock) void k_sliced_empty_slices(const int32_t *_
     if (tile_off[s] == tile_off[s + 1]) chunk_lo[i] = tile_base[tile_off[s]];
 }
 
-// Copies the values again from where they came from.  `unless_equal` (may be null): four words, two
-// checksums of the values now and two of the values the copy holds; where they agree nothing is done.
-template <typename T>
-__global__ __launch_bounds__(kBlock) void k_sliced_regather(const int32_t *__restrict__ perm, int64_t slots,
-                                                            const T *__restrict__ val, T *__restrict__ val_out,
-                                                            const unsigned long long *unless_equal)
+
+// The values of A once more into a plan's slots (asx_plan_update_values), from the side of A: a
+// workgroup reads kSortElems consecutive values and, for each, its position among the block's
+// elements in slice order (kept from the build: 2 bytes), orders them so in LDS, and writes them
+// out as the build did, a run of consecutive slots per slice (where each run starts: block_base,
+// also kept).  Reading through the slots' source indices instead (one thread per slot) takes a
+// 32-byte sector of A's values for every value: 371 us on the power-law matrix, three multiplies.
+// `unless_equal` (may be null): four words, two checksums of the values now and two of the values
+// the copy holds; where they agree nothing is done.
+template <typename T, int MAXS>
+__global__ __launch_bounds__(kSortThreads) void k_sliced_rescatter(const T *__restrict__ val, int32_t nnz, int32_t nslices,
+                                                                   int32_t nblocks, const uint16_t *__restrict__ pos,
+                                                                   const int32_t *__restrict__ block_base,
+                                                                   T *__restrict__ val_out,
+                                                                   const unsigned long long *unless_equal)
 {
+    __shared__ int32_t lofs[MAXS];      // per slice: the block's count, then its first position in slice order
+    __shared__ int32_t gbase[MAXS];     // per slice: slot of the block's first element of the slice
+    __shared__ int32_t wave_tot[kSortWaves];
+    __shared__ T val_s[kSortElems];
     if (unless_equal && unless_equal[0] == unless_equal[2] && unless_equal[1] == unless_equal[3]) return;  // uniform
-    for (int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; d < slots; d += (int64_t)gridDim.x * blockDim.x) {
-        const int32_t src = perm[d];
-        val_out[d] = src >= 0 ? val[src] : T(0);
+    const int tid = threadIdx.x;
+    const int32_t per_xcd = (int32_t)gridDim.x / kXcds;  // as in k_sliced_scatter: neighbouring blocks on one XCD
+    const int32_t b = ((int32_t)blockIdx.x % kXcds) * per_xcd + (int32_t)blockIdx.x / kXcds;
+    if (b >= nblocks) return;  // the whole workgroup leaves
+    const int64_t base = (int64_t)b * kSortElems;
+    const int64_t left = (int64_t)nnz - base;
+    const int32_t count = left < kSortElems ? (int32_t)left : kSortElems;
+    T v[kSortPerLane];
+    uint16_t p[kSortPerLane];
+#pragma unroll
+    for (int k = 0; k < kSortPerLane; ++k) {
+        const int32_t j = k * kSortThreads + tid;
+        v[k] = j < count ? val[base + j] : T(0);
+        p[k] = j < count ? pos[base + j] : (uint16_t)0;
+    }
+    for (int s = tid; s < nslices; s += kSortThreads) {
+        const int32_t g = block_base[(int64_t)b * nslices + s];
+        gbase[s] = g;
+        lofs[s] = block_base[(int64_t)(b + 1) * nslices + s] - g;
+    }
+    __syncthreads();
+    block_exclusive_sum(lofs, nslices, wave_tot);
+#pragma unroll
+    for (int k = 0; k < kSortPerLane; ++k)
+        if (k * kSortThreads + tid < count) val_s[p[k]] = v[k];
+    __syncthreads();
+    for (int j = tid; j < count; j += kSortThreads) {
+        int lo = 0, hi = nslices - 1;  // the slice of position j: the last one that starts at or before j
+        while (lo < hi) {
+            const int mid = lo + (hi - lo + 1) / 2;
+            if (lofs[mid] <= j)
+                lo = mid;
+            else
+                hi = mid - 1;
+        }
+        val_out[slot_val_pos<T>((int64_t)gbase[lo] + (j - lofs[lo]))] = val_s[j];
     }
 }
-
 
 // ---- pass 1 ------------------------------------------------------------------------------
 // A run's sum goes, at the run's rank, into the wave's staging area in LDS; the tile's sums then
@@ -632,7 +684,8 @@ void free_sliced(SlicedMatrix *p)
         if (q) (void)hipFree(q);
     p->store = p->val = p->partial = nullptr;
     p->cf = p->prow = nullptr;
-    p->perm = p->tile_base = p->wg_tab = p->wg_pieces = p->chunk_lo = p->pstep_ptr = p->psteps = nullptr;
+    p->perm = p->tile_base = p->wg_tab = p->wg_pieces = p->chunk_lo = p->pstep_ptr = p->psteps = p->block_base = nullptr;
+    p->pos = nullptr;
 }
 
 template <typename T>
@@ -783,12 +836,16 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
         const size_t o_cf = take(sizeof(uint16_t) * (size_t)slots), o_tb = take(sizeof(int32_t) * ((size_t)sm.ntiles + 1));
         const size_t o_wg = take(sizeof(int32_t) * std::max<size_t>(tab.size() + wgs.size(), 4));
         const size_t o_cl = take(sizeof(int32_t) * (size_t)ncells), o_sp = take(sizeof(int32_t) * ((size_t)sm.nrb + 1));
+        const size_t o_pos = take(sizeof(uint16_t) * (size_t)nnz);
+        const size_t o_bb = take(sizeof(int32_t) * ((size_t)nblocks + 1) * (size_t)sm.nslices);
         ASX_TRY(hipMalloc(&sm.store, off));
         char *base = static_cast<char *>(sm.store);
         sm.val = base + o_val, sm.perm = (int32_t *)(base + o_perm), sm.cf = (uint16_t *)(base + o_cf);
         sm.tile_base = (int32_t *)(base + o_tb), sm.wg_tab = (int32_t *)(base + o_wg);
         sm.chunk_lo = (int32_t *)(base + o_cl), sm.pstep_ptr = (int32_t *)(base + o_sp);
         sm.wg_pieces = sm.wg_tab + tab.size();
+        sm.pos = (uint16_t *)(base + o_pos), sm.block_base = (int32_t *)(base + o_bb);
+        sm.nnz = nnz, sm.nsort_blocks = nblocks;
         ASX_TRY(hipMemcpyAsync(sm.wg_tab, tab.data(), sizeof(int32_t) * tab.size(), hipMemcpyHostToDevice, s));
         ASX_TRY(hipMemcpyAsync(sm.wg_pieces, wgs.data(), sizeof(int32_t) * wgs.size(), hipMemcpyHostToDevice, s));
     }
@@ -797,7 +854,8 @@ int build_sliced(int32_t m, int32_t n, int32_t nnz, int32_t width, int32_t rows_
         const unsigned sgrid = (unsigned)(ceil_div64(nblocks, kXcds) * kXcds);
 #define ASX_SCATTER(MAXS)                                                                                              \
     hipLaunchKernelGGL((k_sliced_scatter<T, MAXS>), dim3(sgrid), dim3(kSortThreads), 0, s, row_ptr, col, val, seg_row, m, \
-                       nnz, width, sm.nslices, nbits, nblocks, offs, d_tile_off, lrow, sm.cf, (T *)sm.val, sm.perm)
+                       nnz, width, sm.nslices, nbits, nblocks, offs, d_tile_off, lrow, sm.cf, (T *)sm.val, sm.perm, sm.pos,     \
+                       sm.block_base)
         if (sm.nslices <= 256)
             ASX_SCATTER(256);
         else
@@ -857,9 +915,14 @@ int sliced_update_values(const SlicedMatrix *sm, const T *val, hipStream_t s, co
 {
     const int64_t slots = (int64_t)sm->ntiles * kSlicedTile;
     if (slots == 0) return ASX_STATUS_SUCCESS;
-    // a bounded grid: where the checksums agree the kernel has nothing to do but to end
-    const unsigned grid = (unsigned)std::min<int64_t>(ceil_div64(slots, kBlock), 8192);
-    hipLaunchKernelGGL((k_sliced_regather<T>), dim3(grid), dim3(kBlock), 0, s, sm->perm, slots, val, (T *)sm->val, unless_equal);
+    // the pads keep the zeros the build gave them; where the checksums agree the kernel has nothing to do but to end
+    const unsigned grid = (unsigned)(ceil_div64(sm->nsort_blocks, kXcds) * kXcds);
+    if (sm->nslices <= 256)
+        hipLaunchKernelGGL((k_sliced_rescatter<T, 256>), dim3(grid), dim3(kSortThreads), 0, s, val, sm->nnz, sm->nslices,
+                           sm->nsort_blocks, sm->pos, sm->block_base, (T *)sm->val, unless_equal);
+    else
+        hipLaunchKernelGGL((k_sliced_rescatter<T, kSlicedMaxSlices>), dim3(grid), dim3(kSortThreads), 0, s, val, sm->nnz,
+                           sm->nslices, sm->nsort_blocks, sm->pos, sm->block_base, (T *)sm->val, unless_equal);
     return check_launch();
 }
 

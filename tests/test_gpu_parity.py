@@ -604,6 +604,9 @@ def test_spmv_sliced_kernel_shapes(torch, capi, oracle, dtype):
     n70 = 69 * width + 5
     lens = np.r_[rng.integers(0, 4, 500), np.full(40, 300), 0, 0, 9000]
     cases.append(("slices70", csr_from_lengths(lens, n70, 9, dtype), n70))
+    # 300 slices: the builder's and the value update's tables for more than 256 slices
+    n300 = 299 * width + 77
+    cases.append(("slices300", csr_from_lengths(np.r_[rng.integers(0, 30, 3000), np.full(20, 700)], n300, 13, dtype), n300))
     for name, (rp, col, val), n in cases:
         m = rp.size - 1
         x = rng.uniform(-1, 1, n).astype(dtype)
