@@ -54,9 +54,9 @@ KERNEL_NAMES = {3: "k_spmv_stream", 6: "k_spmv_vector", 9: "k_spmv_merge", 15: "
 # warm and with cold caches.
 MEASURED_TRAFFIC_BYTES = {
     "banded_f64": 458_624,  # profiles/spmv_vector_banded_f64.md
-    "uniform16_f32": 256_509_003,  # profiles/spmv_sliced_uniform16_f32.md
-    "uniform16_f64": 477_824_736,  # profiles/spmv_sliced_uniform16_f64.md
-    "powerlaw_f64": 729_603_217,  # profiles/spmv_sliced_powerlaw_f64.md
+    "uniform16_f32": 256_483_686,  # profiles/spmv_sliced_uniform16_f32.md
+    "uniform16_f64": 478_017_157,  # profiles/spmv_sliced_uniform16_f64.md
+    "powerlaw_f64": 730_483_835,  # profiles/spmv_sliced_powerlaw_f64.md
     "stencil5_f64": 1_142_530_786,  # profiles/spmv_window_stencil5_f64.md
     "spmm_zipf_f32": 4_965_331_333,  # profiles/spmm_merge_spmm_zipf_f32.md
     "spmm_banded_f32": 1_870_263_890,  # profiles/spmm_blocked_spmm_banded_f32.md
