@@ -999,6 +999,48 @@ def test_sliced_and_window_calls_replay_in_a_hip_graph(torch, capi, oracle):
             assert np.array_equal(y.cpu().numpy(), eager), f"alg {alg} replay {rep}"
         del graph
         plan.destroy()
+    # checked plans: the check of the values, the update of the copy and the multiply are kernels
+    # only as well; captured together they follow values changed in place between two replays.
+    # A sliced plan (checksums, copy brought up to date) and a window plan over full rows (values
+    # read in place: nothing but the multiply)
+    cases = [(capi.SPMV_SLICED, csr_from_lengths(lens, 90000, 7, np.float64), 90000),
+             (capi.SPMV_WINDOW, _banded_random(rng, 20000, 20000, 300, 0.05, np.float64, empty=0.0, longrow=700), 20000)]
+    for alg, (rp, col, val), n in cases:
+        m = rp.size - 1
+        x = rng.uniform(-1, 1, n)
+        y0 = rng.uniform(-1, 1, m)
+        d = [dev(torch, a) for a in (rp, col, val, x)]
+        plan = capi.Plan(False, alg, val.dtype, m, n, col.size, d[0], col=d[1], val=d[2], checked=True)
+        assert plan.checked == (alg == capi.SPMV_SLICED) and plan.holds_values == (alg == capi.SPMV_SLICED)
+        ws = torch.empty(max(plan.workspace_bytes, 256), dtype=torch.uint8, device="cuda")
+        y = dev(torch, y0)
+        plan.refresh_if_changed(d[2])  # once outside: whatever the first call sets up is set up
+        capi.spmv(d[0], d[1], d[2], d[3], y, 1.5, 0.5, alg=alg, plan=plan, workspace=ws)
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                plan.refresh_if_changed(d[2])
+                capi.spmv(d[0], d[1], d[2], d[3], y, 1.5, 0.5, alg=alg, plan=plan, workspace=ws)
+        torch.cuda.synchronize()
+        cur = val.copy()
+        for rep in range(4):
+            if rep:  # the caller overwrites values in place: one, then many, then the first ones again
+                cur = val.copy() if rep == 3 else cur
+                if rep == 1:
+                    cur[col.size // 3] += 0.5
+                elif rep == 2:
+                    cur = rng.uniform(-1, 1, col.size)
+                d[2].copy_(torch.from_numpy(cur))
+            y.copy_(dev(torch, y0))
+            graph.replay()
+            torch.cuda.synchronize()
+            assert_close(y.cpu().numpy(), oracle.spmv(rp, col, cur, x, 1.5, 0.5, y0, 2), spmv_scale(rp, col, cur, x, 1.5, 0.5, y0),
+                         np.float64, f"checked alg {alg} replay {rep}")
+        del graph
+        plan.destroy()
 
 
 def test_one_plan_two_streams_two_workspaces(torch, capi, oracle):
